@@ -1,0 +1,362 @@
+// The decode weight matvec for gfx950: y[m][r] = sum_c W[r][c] * x[m][c], M = 1..4 rows of x on the vector ALUs
+// (M = 8..32 take the MFMA kernel in gemv_mfma.hip). Memory-bound: every weight byte is read once, with 16-byte
+// per-lane non-temporal loads, a wave covering 1 KiB of a row per load instruction and keeping RPW * U of them in
+// flight; x is staged once per workgroup in LDS (optionally through the SwiGLU fold) and read from there with
+// ds_read_b128, shared by the RPW rows a lane works on. A row is summed by LPR lanes (64, 32 or 16, chosen from the
+// row length alone), each lane running its units in ascending column order with one fma per weight, then a fixed
+// DPP tree over the lanes: the sequence for (m, r) depends on neither M nor the launch, so row m of a wide pass
+// equals the one-row pass bit for bit - the law the reference's card kernels keep (native/cuda/btb_kernels.cu:84-88).
+//
+// The same loop serves every stored form through a policy (btb_widen.hpp semantics, vector forms here): the bytes a
+// lane loads are widened in its registers, never through a dequantised copy in memory.
+
+#include "btb_common.hpp"
+#include "btb_tuning.hpp"
+#include "btb_widen.hpp"
+
+#include "../../include/btb_hip.h"
+
+namespace btb {
+
+// ------------------------------------------------------------------------------------------------------------
+// policies
+// ------------------------------------------------------------------------------------------------------------
+
+// bf16 rows: a unit is 8 weights, one 16-byte load
+struct FmtBf16 {
+    static constexpr int UW = 8;
+    struct Params {
+        const uint4* w;
+    };
+    struct Raw {
+        uint4 v;
+    };
+    struct RowCtx {
+        const uint4* row;
+    };
+    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
+        return RowCtx{p.w + r * (size_t)units};
+    }
+    __device__ static __forceinline__ Raw load(const RowCtx& c, int unit) { return Raw{load_stream16(c.row + unit)}; }
+    __device__ static __forceinline__ Raw zero() { return Raw{make_uint4(0, 0, 0, 0)}; }
+    __device__ static __forceinline__ void widen(const RowCtx&, const Raw& r, int /*unit*/, float (&w)[UW]) {
+        w[0] = bf16lo_f32(r.v.x);
+        w[1] = bf16hi_f32(r.v.x);
+        w[2] = bf16lo_f32(r.v.y);
+        w[3] = bf16hi_f32(r.v.y);
+        w[4] = bf16lo_f32(r.v.z);
+        w[5] = bf16hi_f32(r.v.z);
+        w[6] = bf16lo_f32(r.v.w);
+        w[7] = bf16hi_f32(r.v.w);
+    }
+    // nothing past the stream
+    __device__ static __forceinline__ float tail(const Params&, const RowCtx&, size_t, int, int, int, const uint32_t*,
+                                                 int) {
+        return 0.f;
+    }
+};
+
+// ------------------------------------------------------------------------------------------------------------
+// x staging: [M, C] bf16 into LDS as packed pairs, plain or through the SwiGLU fold
+// ------------------------------------------------------------------------------------------------------------
+
+enum XMode { X_PLAIN = 0, X_SILU = 1 };
+
+// the fold the reference's btb_gemv_silu_bf16 makes in its x load (native/cuda/btb_kernels.cu:168-209):
+// x = bf16(bf16(silu(g)) * u), g and u the two halves of a [M, 2C] row
+__device__ __forceinline__ uint32_t silu_pair(uint32_t g2, uint32_t u2) {
+    const float s0 = bfround(bf16lo_f32(g2) / (1.f + expf(-bf16lo_f32(g2))));
+    const float s1 = bfround(bf16hi_f32(g2) / (1.f + expf(-bf16hi_f32(g2))));
+    const uint32_t lo = f32_bf16(s0 * bf16lo_f32(u2));
+    const uint32_t hi = f32_bf16(s1 * bf16hi_f32(u2));
+    return lo | (hi << 16);
+}
+
+template <int XMODE>
+__device__ __forceinline__ void stage_x(uint32_t* xs, const uint16_t* x, int M, int C) {
+    const int tid = threadIdx.x, nt = blockDim.x;
+    if (XMODE == X_PLAIN) {
+        const uint4* src = reinterpret_cast<const uint4*>(x);
+        uint4* dst = reinterpret_cast<uint4*>(xs);
+        const int n = M * C / 8;
+        for (int i = tid; i < n; i += nt) dst[i] = src[i];
+    } else {
+        const int half = C / 2;  // pairs per row
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(x);
+        for (int i = tid; i < M * half; i += nt) {
+            const int m = i / half, c = i - m * half;
+            xs[i] = silu_pair(src[(size_t)m * 2 * half + c], src[(size_t)m * 2 * half + half + c]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// the kernel
+// ------------------------------------------------------------------------------------------------------------
+
+// one unit of every one of the RPW rows against the M rows of x: x read once from LDS, eight at a time, in index order
+template <class F, int M, int RPW>
+__device__ __forceinline__ void fma_unit(const typename F::RowCtx (&ctx)[RPW], const typename F::Raw (&raw)[RPW],
+                                         int unit, const uint4* xs4, int xrow4, float (&acc)[RPW][M]) {
+    constexpr int UW = F::UW;
+    constexpr int H = UW / 8;
+    uint4 xv[H][M];
+#pragma unroll
+    for (int h = 0; h < H; ++h)
+#pragma unroll
+        for (int m = 0; m < M; ++m) xv[h][m] = xs4[m * xrow4 + unit * H + h];
+#pragma unroll
+    for (int j = 0; j < RPW; ++j) {
+        float w[UW];
+        F::widen(ctx[j], raw[j], unit, w);
+#pragma unroll
+        for (int h = 0; h < H; ++h)
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                float a = acc[j][m];
+                a = fmaf(w[h * 8 + 0], bf16lo_f32(xv[h][m].x), a);
+                a = fmaf(w[h * 8 + 1], bf16hi_f32(xv[h][m].x), a);
+                a = fmaf(w[h * 8 + 2], bf16lo_f32(xv[h][m].y), a);
+                a = fmaf(w[h * 8 + 3], bf16hi_f32(xv[h][m].y), a);
+                a = fmaf(w[h * 8 + 4], bf16lo_f32(xv[h][m].z), a);
+                a = fmaf(w[h * 8 + 5], bf16hi_f32(xv[h][m].z), a);
+                a = fmaf(w[h * 8 + 6], bf16lo_f32(xv[h][m].w), a);
+                a = fmaf(w[h * 8 + 7], bf16hi_f32(xv[h][m].w), a);
+                acc[j][m] = a;
+            }
+    }
+}
+
+// where the kernel reads x from: LDS (staged once per workgroup) or straight from global memory through the caches
+enum XSrc { XS_LDS = 0, XS_GLOBAL = 1 };
+
+// the loads of one span: U units of each of the RPW rows; a unit past the row's end is not loaded
+template <class F, int LPR, int RPW, int U, bool GUARD>
+__device__ __forceinline__ void load_span(typename F::Raw (&raw)[U][RPW], const typename F::RowCtx (&ctx)[RPW], int k0,
+                                          int sl, int units) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int unit = k0 + u * LPR + sl;
+        if (!GUARD || unit < units) {
+#pragma unroll
+            for (int j = 0; j < RPW; ++j) raw[u][j] = F::load(ctx[j], unit);
+        }
+    }
+}
+
+template <class F, int M, int LPR, int RPW, int U, bool GUARD>
+__device__ __forceinline__ void fma_span(const typename F::Raw (&raw)[U][RPW], const typename F::RowCtx (&ctx)[RPW],
+                                         int k0, int sl, int units, const uint4* xs4, int xrow4,
+                                         float (&acc)[RPW][M]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int unit = k0 + u * LPR + sl;
+        if (!GUARD || unit < units) fma_unit<F, M, RPW>(ctx, raw[u], unit, xs4, xrow4, acc);
+    }
+}
+
+template <class F, int M, int LPR, int RPW, int U, int XMODE, int XSRC>
+__global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, const uint16_t* __restrict__ x,
+                                                   uint16_t* __restrict__ y, int R, int C) {
+    extern __shared__ __align__(16) uint32_t xs[];  // [M][C / 2] packed bf16 pairs
+    constexpr int UW = F::UW;
+    constexpr int G = WAVE / LPR;        // rows a wave covers per set
+    constexpr int ROWS = G * RPW;        // rows a wave covers per tile
+    const int units = C / UW;            // units per row
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int sl = lane % LPR;           // the lane's place among its row's lanes
+    const int wave = blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
+    const int nwaves = gridDim.x * (blockDim.x / WAVE);
+    const int ntiles = (R + ROWS - 1) / ROWS;
+    const int span = U * LPR;
+    const int xrow4 = C / 8;  // uint4 per row of x
+
+    // the first span of the wave's first tile is requested before x is staged: the weights do not wait for x
+    typename F::Raw raw[U][RPW];
+    typename F::RowCtx ctx[RPW];
+    int rows[RPW];
+    int tile = wave;
+    if (tile < ntiles) {
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) {
+            rows[j] = tile * ROWS + j * G + lane / LPR;
+            // a row past the end reads the last row again (no divergence in the stream) and is not written
+            ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
+        }
+        if (span <= units)
+            load_span<F, LPR, RPW, U, false>(raw, ctx, 0, sl, units);
+        else
+            load_span<F, LPR, RPW, U, true>(raw, ctx, 0, sl, units);
+    }
+    const uint4* xs4;
+    if (XSRC == XS_LDS) {
+        stage_x<XMODE>(xs, x, M, C);
+        __syncthreads();
+        xs4 = reinterpret_cast<const uint4*>(xs);
+    } else {
+        xs4 = reinterpret_cast<const uint4*>(x);
+    }
+
+    bool primed = true;
+    for (; tile < ntiles; tile += nwaves) {
+        if (!primed) {
+#pragma unroll
+            for (int j = 0; j < RPW; ++j) {
+                rows[j] = tile * ROWS + j * G + lane / LPR;
+                ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
+            }
+        }
+        float acc[RPW][M];
+#pragma unroll
+        for (int j = 0; j < RPW; ++j)
+#pragma unroll
+            for (int m = 0; m < M; ++m) acc[j][m] = 0.f;
+
+        for (int k0 = 0; k0 < units; k0 += span) {
+            if (k0 + span <= units) {
+                if (!primed) load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
+                fma_span<F, M, LPR, RPW, U, false>(raw, ctx, k0, sl, units, xs4, xrow4, acc);
+            } else {
+                if (!primed) load_span<F, LPR, RPW, U, true>(raw, ctx, k0, sl, units);
+                fma_span<F, M, LPR, RPW, U, true>(raw, ctx, k0, sl, units, xs4, xrow4, acc);
+            }
+            primed = false;
+        }
+#pragma unroll
+        for (int j = 0; j < RPW; ++j)
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                const float s = group_sum<LPR>(acc[j][m]);
+                if (sl == 0 && rows[j] < R) y[(size_t)m * R + rows[j]] = f32_bf16(s);
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// launch
+// ------------------------------------------------------------------------------------------------------------
+
+// lanes a row is summed by: from the row length alone, so a row's bits do not depend on M or on R
+static int lanes_per_row(int units) {
+    if (units % 64 == 0 || units >= 256) return 64;
+    if (units % 32 == 0 || units >= 96) return 32;
+    return 16;
+}
+
+template <class F, int M, int LPR, int RPW, int U, int XMODE, int XSRC>
+static int32_t launch_variant(const typename F::Params& p, const void* x, void* y, int R, int C, hipStream_t st) {
+    constexpr int G = WAVE / LPR;
+    const DeviceInfo& dev = device_info();
+    const size_t lds = XSRC == XS_LDS ? (size_t)M * C * 2 : 0;
+    if (lds > (size_t)dev.lds_bytes) {
+        set_error("gemv: the x rows do not fit LDS");
+        return ERR_DOMAIN;
+    }
+    const int ntiles = (R + G * RPW - 1) / (G * RPW);
+    int per_cu = tuning("gemv_wgs_per_cu");
+    if (per_cu <= 0) per_cu = 16;  // past this many workgroups a CU the waves loop over tiles
+    int grid = (ntiles + 3) / 4;
+    const int cap = dev.cus * per_cu;
+    if (grid > cap) grid = cap;
+    if (grid < 1) grid = 1;
+    auto kern = gemv_stream<F, M, LPR, RPW, U, XMODE, XSRC>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, p, static_cast<const uint16_t*>(x),
+                       static_cast<uint16_t*>(y), R, C);
+    return hip_status(hipGetLastError(), "gemv launch");
+}
+
+template <class F, int M, int LPR, int XMODE>
+static int32_t launch_stream(const typename F::Params& p, const void* x, void* y, int R, int C, hipStream_t st) {
+    // Rows per wave tile (RPW) and units in flight per row (U), measured on MI355X at the Qwen3-4B shapes: two rows
+    // by four units where the matrix has rows enough to give every SIMD several waves that way, else one row by
+    // eight units. Neither changes a result bit (a lane's units stay in ascending order).
+    const int v = tuning("gemv_variant");
+    const bool tall = v >= 0 ? (v == 1) : (R >= 4096 * (WAVE / LPR));
+    if (M <= 2) {
+        if (tall) return launch_variant<F, M, LPR, 2, 4, XMODE, XS_LDS>(p, x, y, R, C, st);
+        return launch_variant<F, M, LPR, 1, 8, XMODE, XS_LDS>(p, x, y, R, C, st);
+    }
+    if (tall) return launch_variant<F, M, LPR, 2, 2, XMODE, XS_LDS>(p, x, y, R, C, st);
+    return launch_variant<F, M, LPR, 1, 4, XMODE, XS_LDS>(p, x, y, R, C, st);
+}
+
+template <class F, int M, int XMODE>
+static int32_t launch_by_lanes(const typename F::Params& p, const void* x, void* y, int R, int C, hipStream_t st) {
+    switch (lanes_per_row(C / F::UW)) {
+        case 64:
+            return launch_stream<F, M, 64, XMODE>(p, x, y, R, C, st);
+        case 32:
+            return launch_stream<F, M, 32, XMODE>(p, x, y, R, C, st);
+        default:
+            return launch_stream<F, M, 16, XMODE>(p, x, y, R, C, st);
+    }
+}
+
+template <class F, int XMODE>
+static int32_t launch_by_m(const typename F::Params& p, const void* x, void* y, int R, int C, int M, hipStream_t st) {
+    switch (M) {
+        case 1:
+            return launch_by_lanes<F, 1, XMODE>(p, x, y, R, C, st);
+        case 2:
+            return launch_by_lanes<F, 2, XMODE>(p, x, y, R, C, st);
+        case 3:
+            return launch_by_lanes<F, 3, XMODE>(p, x, y, R, C, st);
+        case 4:
+            return launch_by_lanes<F, 4, XMODE>(p, x, y, R, C, st);
+        default:
+            return ERR_DOMAIN;
+    }
+}
+
+// wider passes run as passes of at most four rows: each row's bits are those of its own one-row pass
+template <class F, int XMODE>
+static int32_t run_rows(const typename F::Params& p, const void* x, void* y, size_t R, size_t C, size_t M,
+                        size_t x_row_elems, hipStream_t st) {
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    uint16_t* yp = static_cast<uint16_t*>(y);
+    for (size_t m0 = 0; m0 < M; m0 += 4) {
+        const int mm = (int)(M - m0 < 4 ? M - m0 : 4);
+        int32_t rc = launch_by_m<F, XMODE>(p, xp + m0 * x_row_elems, yp + m0 * R, (int)R, (int)C, mm, st);
+        if (rc != OK) return rc;
+    }
+    return OK;
+}
+
+static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+
+static int32_t check_dims(size_t R, size_t C, size_t M, size_t uw) {
+    if (R == 0 || C == 0 || M == 0) return ERR_DOMAIN;
+    if (R > 0x7FFFFFFFu / 4 || C > (1u << 24) || M > 1024 || C % uw != 0) return ERR_DOMAIN;
+    return OK;
+}
+
+}  // namespace btb
+
+using namespace btb;
+
+extern "C" {
+
+int32_t btb_hip_gemv_bf16(const void* w, const void* x, void* y, size_t R, size_t C, size_t M, void* stream) {
+    if (w == nullptr || x == nullptr || y == nullptr) return ERR_NULL;
+    int32_t rc = check_dims(R, C, M, FmtBf16::UW);
+    if (rc != OK) return rc;
+    if (!aligned16(w) || !aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 1u)) return ERR_DOMAIN;
+    FmtBf16::Params p{static_cast<const uint4*>(w)};
+    return run_rows<FmtBf16, X_PLAIN>(p, x, y, R, C, M, C, static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_gemv_silu_bf16(const void* w, const void* gu, void* y, size_t R, size_t C, size_t M, void* stream) {
+    if (w == nullptr || gu == nullptr || y == nullptr) return ERR_NULL;
+    int32_t rc = check_dims(R, C, M, FmtBf16::UW);
+    if (rc != OK) return rc;
+    if (!aligned16(w) || !aligned16(gu) || (reinterpret_cast<uintptr_t>(y) & 1u)) return ERR_DOMAIN;
+    FmtBf16::Params p{static_cast<const uint4*>(w)};
+    return run_rows<FmtBf16, X_SILU>(p, gu, y, R, C, M, 2 * C, static_cast<hipStream_t>(stream));
+}
+
+}  // extern "C"

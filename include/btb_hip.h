@@ -1,0 +1,71 @@
+/*
+ * libbtb_hip: the decode weight-matvec path of btb for one AMD MI355X (gfx950), as a C ABI.
+ *
+ * Conventions, kept from the reference's native crate (native/src/lib.rs:1-9, 17-33):
+ *   - every function returns 0 on success or a negative code; buffers are caller-owned and written in place; a
+ *     refused call writes nothing and launches nothing;
+ *   - BTB_ERR_NULL is checked before BTB_ERR_DOMAIN;
+ *   - all sizes are size_t, all pointers are plain device pointers (hipMalloc'd or torch-owned), `stream` is a
+ *     hipStream_t passed as void* (NULL is the default stream). Work is queued on that stream and the call
+ *     returns without waiting, so every entry point may be recorded into a hipGraph capture;
+ *   - re-entrant; the result for an output row depends on neither the number of x rows in the call nor on the
+ *     launch geometry.
+ *
+ * Two faces are exported, as in the reference: the device twins of the crate's CPU entry points (f32 x and y, the
+ * host's summation order, bit for bit: btb_hip_gemv_*_rows) and the card operators the CUDA backend launches by
+ * kernel name (bf16 x and y: btb_hip_gemv_bf16 and friends, also reachable through btb_hip_launch).
+ */
+#ifndef BTB_HIP_H
+#define BTB_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define BTB_OK 0
+#define BTB_ERR_NULL (-1)
+#define BTB_ERR_OVERFLOW (-5)
+#define BTB_ERR_DOMAIN (-6)
+#define BTB_ERR_PANIC (-7) /* a HIP runtime failure at the boundary; btb_hip_last_error() names it */
+
+/* ---- process ------------------------------------------------------------------------------------------- */
+
+/* Binds the calling process to `device` (hipSetDevice) and reads its compute-unit count and LDS size. Optional:
+ * the first operator call does the same for the current device. Replaces the module load of the reference's
+ * `_Cuda.__init__` (btb/engine/native.py:1263-1300). */
+int32_t btb_hip_init(int32_t device);
+
+/* The GPU architecture the kernels were compiled for ("gfx950"): the tier a benchmark's numbers belong to.
+ * Replaces btb_isa (native/src/lib.rs:43-50). Static NUL-terminated string. */
+const char* btb_hip_arch(void);
+
+/* Compute units of the bound device: `_Cuda.sms` (btb/engine/native.py:1297). */
+int32_t btb_hip_sms(void);
+
+/* The message of the last BTB_ERR_PANIC / refused call on this thread (static storage, never NULL). */
+const char* btb_hip_last_error(void);
+
+/* Overrides a launch-tuning knob (e.g. "gemv_wgs_per_cu"); value < 0 restores the default. Unknown keys are
+ * BTB_ERR_DOMAIN. For measurement only: no knob changes any result bit. No counterpart in the reference. */
+int32_t btb_hip_set_tuning(const char* key, int32_t value);
+
+/* ---- card operators: bf16 activations in, f32 accumulate, bf16 out ------------------------------------- */
+
+/* y[m][r] = bf16(sum_c w[r][c] * x[m][c]).  w [R, C] bf16 row-major, x [M, C] bf16, y [M, R] bf16; C a multiple
+ * of 8, w and x 16-byte aligned. Replaces the kernels btb_gemv_bf16_m{1,2,4,8,16,32}
+ * (native/cuda/btb_kernels.cu:84-155) and btb_gemv_mma_bf16 (native/cuda/btb_gemv_mma.cuh:196-200); M is an
+ * argument, any value from 1 to 1024. */
+int32_t btb_hip_gemv_bf16(const void* w, const void* x, void* y, size_t R, size_t C, size_t M, void* stream);
+
+/* The down projection with the SwiGLU fold in its x load: gu [M, 2C] bf16 (gate then up),
+ * x[m][c] = bf16(bf16(silu(g)) * u). Replaces btb_gemv_silu_bf16_m{M} (native/cuda/btb_kernels.cu:168-227). */
+int32_t btb_hip_gemv_silu_bf16(const void* w, const void* gu, void* y, size_t R, size_t C, size_t M, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+
+#endif /* BTB_HIP_H */

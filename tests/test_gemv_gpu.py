@@ -1,0 +1,105 @@
+"""The bf16 decode matvec on the GPU (through the C ABI) against the CPU oracle on the same seeded inputs.
+
+Bar (BASELINE.json north_star): max |y_gpu - y_ref| / max |y_ref| <= 1e-2 on the bf16 outputs, y_ref the oracle's f32
+result rounded to bf16. Both sides accumulate in f32 with one fused multiply-add per weight; they differ only in the
+order of the additions (<= ~sqrt(C) * 2^-24 relative to sum |w x|, far below a bf16 ulp), so what is seen is at most a
+bf16 rounding flip: 2^-8 relative to the output. The reference's own card bar, one bf16 ulp of the largest output
+(tests/kernels/test_card_kernels.py:135-148), is asserted too.
+"""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+import oracle
+from oracle import codecs
+
+from .helpers import acts_bf16, bits16, weights_bf16
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-2
+
+
+def oracle_bf16_out(w: torch.Tensor, x: torch.Tensor) -> np.ndarray:
+    """the CPU path's answer as the card stores it: f32 lane sums, rounded to bf16 (kept as f32)"""
+    y = oracle.gemv_bf16(bits16(w), x.float().numpy(), threads=0)
+    return codecs.round_bf16(y)
+
+
+def check(y: torch.Tensor, ref: np.ndarray) -> None:
+    got = y.float().cpu().numpy()
+    peak = np.abs(ref).max()
+    err = np.abs(got - ref).max()
+    assert err <= REL_TOL * peak, (err, peak)
+    assert err <= peak * 2.0**-7, (err, peak)
+
+
+@pytest.mark.parametrize("R,C", [(9728, 2560), (2560, 9728), (6144, 2560), (2560, 4096), (2048, 768), (1536, 2048),
+                                 (128, 2048), (1000, 264), (7, 8), (3, 1032)])
+@pytest.mark.parametrize("M", [1, 4])
+def test_gemv_bf16_matches_oracle(card, R, C, M):
+    w = weights_bf16(R, C, seed=100)
+    x = acts_bf16(M, C, seed=101)
+    y = card.gemv(w.cuda(), x.cuda())
+    check(y, oracle_bf16_out(w, x))
+
+
+@pytest.mark.parametrize("M", [2, 3, 5, 8, 16, 32])
+def test_row_of_a_wide_pass_is_its_one_row_pass(card, M):
+    """native/cuda/btb_kernels.cu:84-88 and tests/kernels/test_card_kernels.py:145-148: row m does not depend on M"""
+    R, C = 2560, 4096
+    w = weights_bf16(R, C, seed=110).cuda()
+    x = acts_bf16(M, C, seed=111).cuda()
+    y = card.gemv(w, x)
+    check(y, oracle_bf16_out(w.cpu(), x.cpu()))
+    for m in (0, M - 1):
+        solo = card.gemv(w, x[m : m + 1].contiguous())
+        assert torch.equal(solo[0].view(torch.int16), y[m].view(torch.int16))
+
+
+def test_repeat_runs_are_bit_stable(card):
+    w = weights_bf16(9728, 2560, seed=120).cuda()
+    x = acts_bf16(1, 2560, seed=121).cuda()
+    a = card.gemv(w, x).clone()
+    for _ in range(5):
+        assert torch.equal(card.gemv(w, x).view(torch.int16), a.view(torch.int16))
+
+
+@pytest.mark.parametrize("M", [1, 4])
+def test_silu_fold_equals_two_steps(card, M):
+    """tests/kernels/test_card_kernels.py:376-391: the folded down projection equals act-mul then the plain matvec"""
+    R, C = 2560, 9728
+    w = weights_bf16(R, C, seed=130).cuda()
+    gu = acts_bf16(M, 2 * C, seed=131).cuda()
+    g, u = gu[:, :C].float(), gu[:, C:].float()
+    s = (g / (1 + torch.exp(-g))).to(torch.bfloat16).float()
+    x = (s * u).to(torch.bfloat16)
+    folded = card.gemv_silu(w, gu)
+    plain = card.gemv(w, x.contiguous())
+    # the activation's exp may differ from torch's in the last bit, which can flip a bf16 rounding of x here and there
+    ref = oracle_bf16_out(w.cpu(), x.cpu())
+    check(folded, ref)
+    frac = (folded != plain).float().mean().item()
+    assert frac < 0.02, frac
+
+
+def test_refusals_launch_nothing(card):
+    w = weights_bf16(16, 64, seed=140).cuda()
+    x = acts_bf16(1, 64, seed=141).cuda()
+    with pytest.raises(ValueError):
+        card.gemv(w.float(), x)
+    with pytest.raises(ValueError):
+        card.gemv(w, x.cpu())
+    with pytest.raises(ValueError):
+        card.gemv(w, x, torch.empty(3, dtype=torch.bfloat16, device="cuda"))
+    L = card.lib
+    y = torch.full((1, 16), 7.0, dtype=torch.bfloat16, device="cuda")
+    assert L.btb_hip_gemv_bf16(None, card.ptr(x), card.ptr(y), 16, 64, 1, None) == -1
+    assert L.btb_hip_gemv_bf16(card.ptr(w), card.ptr(x), card.ptr(y), 0, 64, 1, None) == -6
+    assert L.btb_hip_gemv_bf16(card.ptr(w), card.ptr(x), card.ptr(y), 16, 60, 1, None) == -6  # C % 8
+    assert L.btb_hip_gemv_bf16(None, card.ptr(x), card.ptr(y), 0, 64, 1, None) == -1  # null before domain
+    torch.cuda.synchronize()
+    assert torch.all(y == 7.0)
