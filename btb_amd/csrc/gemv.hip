@@ -11,50 +11,12 @@
 // lane loads are widened in its registers, never through a dequantised copy in memory.
 
 #include "btb_common.hpp"
+#include "btb_formats.hpp"
 #include "btb_tuning.hpp"
-#include "btb_widen.hpp"
 
 #include "../../include/btb_hip.h"
 
 namespace btb {
-
-// ------------------------------------------------------------------------------------------------------------
-// policies
-// ------------------------------------------------------------------------------------------------------------
-
-// bf16 rows: a unit is 8 weights, one 16-byte load
-struct FmtBf16 {
-    static constexpr int UW = 8;
-    struct Params {
-        const uint4* w;
-    };
-    struct Raw {
-        uint4 v;
-    };
-    struct RowCtx {
-        const uint4* row;
-    };
-    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
-        return RowCtx{p.w + r * (size_t)units};
-    }
-    __device__ static __forceinline__ Raw load(const RowCtx& c, int unit) { return Raw{load_stream16(c.row + unit)}; }
-    __device__ static __forceinline__ Raw zero() { return Raw{make_uint4(0, 0, 0, 0)}; }
-    __device__ static __forceinline__ void widen(const RowCtx&, const Raw& r, int /*unit*/, float (&w)[UW]) {
-        w[0] = bf16lo_f32(r.v.x);
-        w[1] = bf16hi_f32(r.v.x);
-        w[2] = bf16lo_f32(r.v.y);
-        w[3] = bf16hi_f32(r.v.y);
-        w[4] = bf16lo_f32(r.v.z);
-        w[5] = bf16hi_f32(r.v.z);
-        w[6] = bf16lo_f32(r.v.w);
-        w[7] = bf16hi_f32(r.v.w);
-    }
-    // nothing past the stream
-    __device__ static __forceinline__ float tail(const Params&, const RowCtx&, size_t, int, int, int, const uint32_t*,
-                                                 int) {
-        return 0.f;
-    }
-};
 
 // ------------------------------------------------------------------------------------------------------------
 // x staging: [M, C] bf16 into LDS as packed pairs, plain or through the SwiGLU fold
@@ -224,6 +186,10 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, const u
         }
 #pragma unroll
         for (int j = 0; j < RPW; ++j)
+            F::template tail<M>(p, ctx[j], (size_t)min(rows[j], R - 1), sl, LPR, C,
+                                reinterpret_cast<const uint32_t*>(xs4), acc[j]);
+#pragma unroll
+        for (int j = 0; j < RPW; ++j)
 #pragma unroll
             for (int m = 0; m < M; ++m) {
                 const float s = group_sum<LPR>(acc[j][m]);
@@ -357,6 +323,51 @@ int32_t btb_hip_gemv_silu_bf16(const void* w, const void* gu, void* y, size_t R,
     if (!aligned16(w) || !aligned16(gu) || (reinterpret_cast<uintptr_t>(y) & 1u)) return ERR_DOMAIN;
     FmtBf16::Params p{static_cast<const uint4*>(w)};
     return run_rows<FmtBf16, X_SILU>(p, gu, y, R, C, M, 2 * C, static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
+                         size_t n_esc, const void* row_ptr, const void* x, void* y, size_t R, size_t C, size_t M,
+                         void* stream) {
+    if (lo == nullptr || hi4 == nullptr || table == nullptr || row_ptr == nullptr || x == nullptr || y == nullptr)
+        return ERR_NULL;
+    if (n_esc > 0 && (esc_idx == nullptr || esc_val == nullptr)) return ERR_NULL;
+    int32_t rc = check_dims(R, C, M, FmtP12::UW);
+    if (rc != OK) return rc;
+    if (R * C > 0x7FFFFFFFull) return ERR_DOMAIN;  // the escape indices are int32
+    if (!aligned16(lo) || (reinterpret_cast<uintptr_t>(hi4) & 7u) || !aligned16(x) ||
+        (reinterpret_cast<uintptr_t>(row_ptr) & 3u) || (reinterpret_cast<uintptr_t>(esc_idx) & 3u) ||
+        (reinterpret_cast<uintptr_t>(y) & 1u))
+        return ERR_DOMAIN;
+    FmtP12::Params p{static_cast<const uint8_t*>(lo),       static_cast<const uint8_t*>(hi4),
+                     static_cast<const uint8_t*>(table),    static_cast<const int32_t*>(esc_idx),
+                     static_cast<const uint8_t*>(esc_val),  static_cast<const int32_t*>(row_ptr)};
+    return run_rows<FmtP12, X_PLAIN>(p, x, y, R, C, M, C, static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_gemv_fp8(const void* w, const void* scales, size_t sr, size_t sc, const void* x, void* y, size_t R,
+                         size_t C, size_t M, void* stream) {
+    if (w == nullptr || scales == nullptr || x == nullptr || y == nullptr) return ERR_NULL;
+    if (sr == 0 || sc == 0) return ERR_DOMAIN;
+    int32_t rc = check_dims(R, C, M, FmtF8::UW);
+    if (rc != OK) return rc;
+    if (R % sr != 0 || C % sc != 0 || (C / sc) % FmtF8::UW != 0) return ERR_DOMAIN;
+    if (!aligned16(w) || !aligned16(x) || (reinterpret_cast<uintptr_t>(scales) & 3u) ||
+        (reinterpret_cast<uintptr_t>(y) & 1u))
+        return ERR_DOMAIN;
+    const uint32_t upb = (uint32_t)(C / sc / FmtF8::UW);
+    FmtF8::Params p{static_cast<const uint8_t*>(w), static_cast<const float*>(scales), (int)sc, (int)(R / sr),
+                    (int)upb, upb > 1 ? (uint32_t)(0x100000000ull / upb + 1) : 0u};
+    return run_rows<FmtF8, X_PLAIN>(p, x, y, R, C, M, C, static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_gemv_mxfp4(const void* blocks, const void* scales, const void* x, void* y, size_t R, size_t C, size_t M,
+                           void* stream) {
+    if (blocks == nullptr || scales == nullptr || x == nullptr || y == nullptr) return ERR_NULL;
+    int32_t rc = check_dims(R, C, M, FmtMx4::UW);
+    if (rc != OK) return rc;
+    if (!aligned16(blocks) || !aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 1u)) return ERR_DOMAIN;
+    FmtMx4::Params p{static_cast<const uint8_t*>(blocks), static_cast<const uint8_t*>(scales)};
+    return run_rows<FmtMx4, X_PLAIN>(p, x, y, R, C, M, C, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -34,6 +34,13 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_set_tuning": (_i32, [ctypes.c_char_p, _i32]),
     "btb_hip_gemv_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_gemv_silu_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_gemv_p12": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_p12_row_ptr": (_i32, [_vp, _sz, _sz, _sz, _vp, _vp]),
+    "btb_hip_p12_widen": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _vp, _vp]),
+    "btb_hip_gemv_fp8": (_i32, [_vp, _vp, _sz, _sz, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_fp8_widen": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _i32, _vp]),
+    "btb_hip_gemv_mxfp4": (_i32, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_mx4_widen": (_i32, [_vp, _vp, _vp, _sz, ctypes.c_int64, _vp, _i32, _vp]),
 }
 
 
@@ -128,6 +135,117 @@ class HipCard:
                 raise ValueError(f"[hip] gemv_silu: y holds {y.numel()} elements, the product has {M * R}")
         self._call("btb_hip_gemv_silu_bf16", self.ptr(w), self.ptr(g2), self.ptr(y), R, C, M, _stream())
         return y
+
+
+    # -- the stored forms ---------------------------------------------------------------------------------------
+
+    def _out(self, y: torch.Tensor | None, M: int, R: int, dev: torch.device, what: str) -> torch.Tensor:
+        if y is None:
+            return torch.empty(M, R, dtype=torch.bfloat16, device=dev)
+        self._need(y, torch.bfloat16, "y")
+        if y.numel() != M * R:
+            raise ValueError(f"[hip] {what}: y holds {y.numel()} elements, the product has {M * R}")
+        return y
+
+    def p12_row_ptr(self, esc_idx: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
+        """int32 [rows + 1]: the first escape at or past each row's first weight (built once at upload)"""
+        self._need(esc_idx, torch.int32, "esc_idx")
+        out = torch.empty(rows + 1, dtype=torch.int32, device=esc_idx.device)
+        self._call("btb_hip_p12_row_ptr", self.ptr(esc_idx) if esc_idx.numel() else None, esc_idx.numel(), rows, cols,
+                   self.ptr(out), _stream())
+        return out
+
+    def gemv_p12(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
+        """y [M, R] = x [M, C] over a `P12Weight`, the 12-bit form widened in registers"""
+        R, C = w.shape
+        self._need(x, torch.bfloat16, "x")
+        x2 = x.reshape(-1, C)
+        M = int(x2.shape[0])
+        y = self._out(y, M, R, x.device, "gemv_p12")
+        ne = int(w.esc_idx.numel())
+        self._call("btb_hip_gemv_p12", self.ptr(w.lo), self.ptr(w.hi4), self.ptr(w.table),
+                   self.ptr(w.esc_idx) if ne else None, self.ptr(w.esc_val) if ne else None, ne, self.ptr(w.row_ptr),
+                   self.ptr(x2), self.ptr(y), R, C, M, _stream())
+        return y
+
+    def p12_widen(self, lo, hi4, table, esc_idx, esc_val, n: int, shape: Sequence[int]) -> torch.Tensor:
+        """a packed tensor back to bf16 on the GPU (`unpack_bf16`), through the matvec's own in-register widen"""
+        for t, what in ((lo, "lo"), (hi4, "hi4"), (table, "table")):
+            self._need(t, torch.uint8, what)
+        out = torch.empty(tuple(shape), dtype=torch.bfloat16, device=lo.device)
+        ne = 0 if esc_idx is None else int(esc_idx.numel())
+        if ne:
+            self._need(esc_idx, torch.int32, "esc_idx")
+            self._need(esc_val, torch.uint8, "esc_val")
+        self._call("btb_hip_p12_widen", self.ptr(lo), self.ptr(hi4), self.ptr(table), self.ptr(esc_idx) if ne else None,
+                   self.ptr(esc_val) if ne else None, ne, n, self.ptr(out), _stream())
+        return out
+
+    def gemv_fp8(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
+        """y [M, R] = x [M, C] over an `F8Weight`: each weight bf16(e4m3 * scale), made in registers"""
+        R, C = w.shape
+        sr, sc = w.grid
+        self._need(w.w, torch.uint8, "w")
+        self._need(w.scales, torch.float32, "scales")
+        self._need(x, torch.bfloat16, "x")
+        x2 = x.reshape(-1, C)
+        M = int(x2.shape[0])
+        y = self._out(y, M, R, x.device, "gemv_fp8")
+        self._call("btb_hip_gemv_fp8", self.ptr(w.w), self.ptr(w.scales), sr, sc, self.ptr(x2), self.ptr(y), R, C, M,
+                   _stream())
+        return y
+
+    def fp8_widen(self, w: Any, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+        """an `F8Weight` as the held matrix (`fp8.held`), bf16 or the same values as f32"""
+        R, C = w.shape
+        sr, sc = w.grid
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError("[hip] fp8_widen writes bf16 or float32")
+        out = torch.empty(R, C, dtype=dtype, device=w.w.device)
+        self._call("btb_hip_fp8_widen", self.ptr(w.w), self.ptr(w.scales), R, C, sr, sc, self.ptr(out),
+                   int(dtype == torch.float32), _stream())
+        return out
+
+    def gemv_mx4(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
+        """y [M, R] = x [M, C] over an `MxWeight` (checkpoint layout), fp4 * 2^(scale - 127) made in registers"""
+        R, C = w.shape
+        self._need(w.blocks, torch.uint8, "blocks")
+        self._need(w.scales, torch.uint8, "scales")
+        self._need(x, torch.bfloat16, "x")
+        x2 = x.reshape(-1, C)
+        M = int(x2.shape[0])
+        y = self._out(y, M, R, x.device, "gemv_mx4")
+        self._call("btb_hip_gemv_mxfp4", self.ptr(w.blocks), self.ptr(w.scales), self.ptr(x2), self.ptr(y), R, C, M,
+                   _stream())
+        return y
+
+    def mx4_widen(self, blocks: torch.Tensor, scales: torch.Tensor, seats: torch.Tensor | None = None,
+                  out: torch.Tensor | None = None, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+        """MXFP4 experts at `seats` of the stacks `blocks` [S, .., 16] and `scales` [S, ..] widened to
+        [len(seats), groups * 32] in one pass (the reference's `_Cuda.mx4_widen`, btb/engine/native.py:1494-1530);
+        `dtype` float32 keeps the unrounded f32 product the CPU matvec multiplies"""
+        groups = int(scales[0].numel())
+        if (blocks.dtype != torch.uint8 or scales.dtype != torch.uint8
+                or not (blocks.is_contiguous() and scales.is_contiguous())
+                or int(blocks[0].numel()) != 16 * groups or blocks.device != scales.device or not blocks.is_cuda):
+            raise ValueError(f"[hip] mx4_widen: blocks {tuple(blocks.shape)} {blocks.dtype} and scales "
+                             f"{tuple(scales.shape)} {scales.dtype} are not a contiguous uint8 stack of 16-byte "
+                             f"blocks and their scales on the GPU")
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError("[hip] mx4_widen writes bf16 or float32")
+        if seats is not None:
+            seats = seats.to(blocks.device, torch.int32).contiguous()
+            n = int(seats.numel())
+        else:
+            n = int(scales.shape[0])
+        if out is None:
+            out = torch.empty(n, groups * 32, dtype=dtype, device=blocks.device)
+        elif out.dtype != dtype or not out.is_contiguous() or out.numel() != n * groups * 32:
+            raise ValueError(f"[hip] mx4_widen: out must be {n * groups * 32} contiguous {dtype}")
+        if n:
+            self._call("btb_hip_mx4_widen", self.ptr(blocks), self.ptr(scales), None if seats is None else self.ptr(seats),
+                       n, groups, self.ptr(out), int(dtype == torch.float32), _stream())
+        return out
 
 
 class Native:

@@ -64,6 +64,51 @@ int32_t btb_hip_gemv_bf16(const void* w, const void* x, void* y, size_t R, size_
  * x[m][c] = bf16(bf16(silu(g)) * u). Replaces btb_gemv_silu_bf16_m{M} (native/cuda/btb_kernels.cu:168-227). */
 int32_t btb_hip_gemv_silu_bf16(const void* w, const void* gu, void* y, size_t R, size_t C, size_t M, void* stream);
 
+/* ---- the stored weight forms, widened in registers inside the matvec ------------------------------------ */
+
+/* The matvec over a pack12 matrix (n = R * C weights): lo u8[n], hi4 u8[(n + 1) / 2] (weight 2k in the low nibble
+ * of byte k), table u8[16], esc_idx i32[n_esc] strictly ascending, esc_val u8[n_esc] - the arrays of
+ * btb_gemv_p12_rows (native/src/lib.rs:114-135), on the device - plus row_ptr i32[R + 1] from btb_hip_p12_row_ptr.
+ * x [M, C] bf16, y [M, R] bf16; C a multiple of 16, lo 16-byte and hi4 8-byte aligned. The reference has no card
+ * kernel for this form (it widens a packed layer to bf16 before the card holds it: btb/engine/tiers.py:1200-1216). */
+int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
+                         size_t n_esc, const void* row_ptr, const void* x, void* y, size_t R, size_t C, size_t M,
+                         void* stream);
+
+/* row_ptr[r] = how many escapes lie below weight r * cols, r = 0..rows: the per-row slices of the escape list the
+ * matvec reads. Run once when a packed matrix is uploaded; replaces the per-call search of p12_cursors
+ * (native/src/gemv.rs:719-734). */
+int32_t btb_hip_p12_row_ptr(const void* esc_idx, size_t n_esc, size_t rows, size_t cols, void* row_ptr, void* stream);
+
+/* A packed tensor of n weights back to bf16 [n], escapes applied: unpack_bf16 (btb/pack12.py:70-97) on the device,
+ * through the same in-register widen the matvec uses. out 16-byte aligned. */
+int32_t btb_hip_p12_widen(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
+                          size_t n_esc, size_t n, void* out, void* stream);
+
+/* The matvec over an FP8 matrix: w u8[R * C] e4m3fn, scales f32[sr * sc] row-major (one per block of R / sr rows by
+ * C / sc columns), weight = bf16(e4m3 * scale) - btb_gemv_fp8_rows (native/src/lib.rs:511-526) with bf16 x and y.
+ * sr divides R, sc divides C, and a block is a multiple of 16 columns wide. */
+int32_t btb_hip_gemv_fp8(const void* w, const void* scales, size_t sr, size_t sc, const void* x, void* y, size_t R,
+                         size_t C, size_t M, void* stream);
+
+/* An FP8 matrix widened to the held weights bf16(e4m3 * scale): bf16 [rows, cols] (out_f32 == 0) or the same values
+ * as f32 (out_f32 != 0). fp8.held (btb/fp8.py:97-100) on the device. */
+int32_t btb_hip_fp8_widen(const void* w, const void* scales, size_t rows, size_t cols, size_t sr, size_t sc, void* out,
+                          int32_t out_f32, void* stream);
+
+/* The matvec over an MXFP4 matrix in the checkpoint's layout: blocks u8[R * C / 32 * 16], scales u8[R * C / 32],
+ * weight = fp4(code) * 2^(scale - 127) - btb_gemv_mxfp4_rows (native/src/lib.rs:147-160) with bf16 x and y. C a
+ * multiple of 32. */
+int32_t btb_hip_gemv_mxfp4(const void* blocks, const void* scales, const void* x, void* y, size_t R, size_t C, size_t M,
+                           void* stream);
+
+/* MXFP4 stacks widened block by block: for seat i (seats[i], or i when seats is NULL) the `groups` blocks at
+ * blocks[seat * groups ..] become out[i * groups * 32 ..], bf16 (out_f32 == 0: the kernel btb_mx4_widen,
+ * native/cuda/btb_kernels.cu:718-738) or the unrounded f32 product (out_f32 != 0: the CPU matvec's weight,
+ * native/src/gemv.rs:1090-1119). n_seats <= 65535. */
+int32_t btb_hip_mx4_widen(const void* blocks, const void* scales, const void* seats, size_t n_seats, int64_t groups,
+                          void* out, int32_t out_f32, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
