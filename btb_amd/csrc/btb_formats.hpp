@@ -1,7 +1,9 @@
 // The stored weight forms as policies of the streaming matvec (gemv.hip) and of the widen kernels (widen.hip): what
 // one lane loads in one step - a "unit" of UW consecutive weights of a row - and how those bytes become f32 weights
-// in its registers. The vector forms here must equal the scalar definitions of btb_widen.hpp bit for bit; the widen
-// kernels expose them so the tests can check exactly that, over every byte value.
+// in its registers, as bf16 pairs (every form's weight is exactly a bf16: a stored one, a table byte over a low
+// byte, the nearest bf16 to e4m3 * scale, or an fp4 value times a power of two). The vector forms here must equal the
+// scalar definitions of btb_widen.hpp bit for bit; the widen kernels expose them so the tests can check exactly
+// that, over every byte value.
 #pragma once
 
 #include "btb_common.hpp"
@@ -27,15 +29,11 @@ struct FmtBf16 {
         return RowCtx{p.w + r * (size_t)units};
     }
     __device__ static __forceinline__ Raw load(const RowCtx& c, int unit) { return Raw{load_stream16(c.row + unit)}; }
-    __device__ static __forceinline__ void widen(const RowCtx&, const Raw& r, int /*unit*/, float (&w)[UW]) {
-        w[0] = bf16lo_f32(r.v.x);
-        w[1] = bf16hi_f32(r.v.x);
-        w[2] = bf16lo_f32(r.v.y);
-        w[3] = bf16hi_f32(r.v.y);
-        w[4] = bf16lo_f32(r.v.z);
-        w[5] = bf16hi_f32(r.v.z);
-        w[6] = bf16lo_f32(r.v.w);
-        w[7] = bf16hi_f32(r.v.w);
+    __device__ static __forceinline__ void widen(const RowCtx&, const Raw& r, int /*unit*/, uint32_t (&w)[UW / 2]) {
+        w[0] = r.v.x;
+        w[1] = r.v.y;
+        w[2] = r.v.z;
+        w[3] = r.v.w;
     }
     // nothing past the stream
     template <int M>
@@ -46,8 +44,8 @@ struct FmtBf16 {
 // ------------------------------------------------------------------------------------------------------------
 // pack12: a unit is 16 weights - 16 low bytes (one 16-byte load) and 16 four-bit codes (one 8-byte load). A code
 // becomes its high byte through the 16-entry table held in four registers: two byte-permutes pick from entries 0..7
-// and 8..15, a bit-select on the code's top bit chooses between them; a third permute per weight zips the high byte
-// over its low byte into the top half of an f32. An escaped weight (code 15) comes out of the stream with
+// and 8..15, a bit-select on the code's top bit chooses between them; one more permute per pair of weights zips the
+// high bytes over their low bytes into a bf16 pair. An escaped weight (code 15) comes out of the stream with
 // table[15]'s high byte; `tail` then replaces its term from the escape list: acc += (true - streamed) * x, two
 // fused multiply-adds per escape, found through the row's slice of the list (row_ptr).
 // ------------------------------------------------------------------------------------------------------------
@@ -100,24 +98,22 @@ struct FmtP12 {
         const uint32_t m = ((v >> 3) & 0x01010101u) * 0xFFu;      // 0xFF in the bytes whose code is 8..15
         return (b & m) | (a & ~m);
     }
-    // eight weights: codes c (weight k in nibble k), their low bytes l0 (weights 0..3) and l1 (4..7)
-    __device__ static __forceinline__ void widen8(const uint4& t, uint32_t c, uint32_t l0, uint32_t l1, float* w) {
-        const uint32_t he = lut16(t, c & 0x0F0F0F0Fu);         // high bytes of weights 0, 2, 4, 6
-        const uint32_t ho = lut16(t, (c >> 4) & 0x0F0F0F0Fu);  // of weights 1, 3, 5, 7
-        // f32 bits = high byte << 24 | low byte << 16: selector 4..7 takes a byte of the first operand, 0..3 of the
-        // second, 0x0c is zero
-        w[0] = bits_f32(__builtin_amdgcn_perm(he, l0, 0x04000c0cu));
-        w[1] = bits_f32(__builtin_amdgcn_perm(ho, l0, 0x04010c0cu));
-        w[2] = bits_f32(__builtin_amdgcn_perm(he, l0, 0x05020c0cu));
-        w[3] = bits_f32(__builtin_amdgcn_perm(ho, l0, 0x05030c0cu));
-        w[4] = bits_f32(__builtin_amdgcn_perm(he, l1, 0x06000c0cu));
-        w[5] = bits_f32(__builtin_amdgcn_perm(ho, l1, 0x06010c0cu));
-        w[6] = bits_f32(__builtin_amdgcn_perm(he, l1, 0x07020c0cu));
-        w[7] = bits_f32(__builtin_amdgcn_perm(ho, l1, 0x07030c0cu));
+    // eight weights as four bf16 pairs: codes c (weight k in nibble k), their low bytes l0 (weights 0..3), l1 (4..7).
+    // A byte-permute's selector 0..3 takes a byte of its second operand, 4..7 of its first.
+    __device__ static __forceinline__ void widen8(const uint4& t, uint32_t c, uint32_t l0, uint32_t l1, uint32_t* w) {
+        const uint32_t even = c & 0x0F0F0F0Fu;         // codes of weights 0, 2, 4, 6
+        const uint32_t odd = (c >> 4) & 0x0F0F0F0Fu;   // of weights 1, 3, 5, 7
+        const uint32_t c03 = __builtin_amdgcn_perm(odd, even, 0x05010400u);  // codes 0, 1, 2, 3 a byte each
+        const uint32_t c47 = __builtin_amdgcn_perm(odd, even, 0x07030602u);  // codes 4, 5, 6, 7
+        const uint32_t h03 = lut16(t, c03), h47 = lut16(t, c47);             // their high bytes
+        w[0] = __builtin_amdgcn_perm(h03, l0, 0x05010400u);  // lo0 hi0 lo1 hi1
+        w[1] = __builtin_amdgcn_perm(h03, l0, 0x07030602u);  // lo2 hi2 lo3 hi3
+        w[2] = __builtin_amdgcn_perm(h47, l1, 0x05010400u);
+        w[3] = __builtin_amdgcn_perm(h47, l1, 0x07030602u);
     }
-    __device__ static __forceinline__ void widen(const RowCtx& c, const Raw& r, int /*unit*/, float (&w)[UW]) {
+    __device__ static __forceinline__ void widen(const RowCtx& c, const Raw& r, int /*unit*/, uint32_t (&w)[UW / 2]) {
         widen8(c.table, r.codes.x, r.lo.x, r.lo.y, w);
-        widen8(c.table, r.codes.y, r.lo.z, r.lo.w, w + 8);
+        widen8(c.table, r.codes.y, r.lo.z, r.lo.w, w + 4);
     }
     // the row's escapes, spread over the row's lanes: the streamed term out, the true term in
     template <int M>
@@ -143,8 +139,9 @@ struct FmtP12 {
 // ------------------------------------------------------------------------------------------------------------
 // FP8 e4m3fn with an f32 scale per block of a [sr, sc] grid: a unit is 16 weights, one 16-byte load, under one
 // scale (the block's width is a multiple of 16). weight = bf16_rne(e4m3 * scale): the byte pair is converted by
-// v_cvt_pk_f32_fp8 (exact: every e4m3 value is an f32), multiplied by the scale once in f32, and rounded to bf16 by
-// the integer rule of btb_common.hpp.
+// v_cvt_pk_f32_fp8 (exact: every e4m3 value is an f32), multiplied by the scale once in f32, and rounded to bf16,
+// nearest even, by v_cvt_pk_bf16_f32 - the same bits as the integer rule of btb_common.hpp on every byte and scale
+// (the widen kernel's test sweeps them all).
 // ------------------------------------------------------------------------------------------------------------
 struct FmtF8 {
     static constexpr int UW = 16;
@@ -174,19 +171,20 @@ struct FmtF8 {
         const int blk = c.upb == 1 ? unit : (int)__umulhi((uint32_t)unit, c.magic);
         return Raw{load_stream16(c.row + unit), c.srow[blk]};
     }
-    __device__ static __forceinline__ void widen4(uint32_t q, float s, float* w) {
+    // four bytes to two bf16 pairs: exact conversion to f32, one f32 multiply by the scale, nearest-even to bf16
+    __device__ static __forceinline__ void widen4(uint32_t q, float s, uint32_t* w) {
         const f32x2 a = __builtin_amdgcn_cvt_pk_f32_fp8(q, false);
         const f32x2 b = __builtin_amdgcn_cvt_pk_f32_fp8(q, true);
-        w[0] = round_bf16_f32(a.x * s);
-        w[1] = round_bf16_f32(a.y * s);
-        w[2] = round_bf16_f32(b.x * s);
-        w[3] = round_bf16_f32(b.y * s);
+        const bf16x2 p0 = {(__bf16)(a.x * s), (__bf16)(a.y * s)};
+        const bf16x2 p1 = {(__bf16)(b.x * s), (__bf16)(b.y * s)};
+        w[0] = __builtin_bit_cast(uint32_t, p0);
+        w[1] = __builtin_bit_cast(uint32_t, p1);
     }
-    __device__ static __forceinline__ void widen(const RowCtx&, const Raw& r, int /*unit*/, float (&w)[UW]) {
+    __device__ static __forceinline__ void widen(const RowCtx&, const Raw& r, int /*unit*/, uint32_t (&w)[UW / 2]) {
         widen4(r.v.x, r.scale, w);
-        widen4(r.v.y, r.scale, w + 4);
-        widen4(r.v.z, r.scale, w + 8);
-        widen4(r.v.w, r.scale, w + 12);
+        widen4(r.v.y, r.scale, w + 2);
+        widen4(r.v.z, r.scale, w + 4);
+        widen4(r.v.w, r.scale, w + 6);
     }
     template <int M>
     __device__ static __forceinline__ void tail(const Params&, const RowCtx&, size_t, int, int, int, const uint32_t*,
@@ -195,8 +193,9 @@ struct FmtF8 {
 
 // ------------------------------------------------------------------------------------------------------------
 // MXFP4: a unit is one block of 32 weights - 16 bytes of packed e2m1 codes (the earlier weight of a pair in the low
-// nibble) and one e8m0 scale byte. weight = fp4 * 2^(scale - 127) in f32 (exact wherever it is a normal f32):
-// v_cvt_scalef32_pk_f32_fp4 converts a byte's two codes and applies the scale in one instruction.
+// nibble) and one e8m0 scale byte. weight = fp4 * 2^(scale - 127): an fp4 value has two significant bits, so the
+// product is exact in bf16 for every scale below 255 (bf16 has f32's exponent range), and
+// v_cvt_scalef32_pk_bf16_fp4 converts a byte's two codes and applies the scale in one instruction.
 // ------------------------------------------------------------------------------------------------------------
 struct FmtMx4 {
     static constexpr int UW = 32;
@@ -218,39 +217,36 @@ struct FmtMx4 {
     __device__ static __forceinline__ Raw load(const RowCtx& c, int unit) {
         return Raw{load_stream16(c.row + unit), (uint32_t)__builtin_nontemporal_load(c.srow + unit)};
     }
-    __device__ static __forceinline__ void widen8(uint32_t q, float s, float* w) {
-        const f32x2 a = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q, s, 0);
-        const f32x2 b = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q, s, 1);
-        const f32x2 c = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q, s, 2);
-        const f32x2 d = __builtin_amdgcn_cvt_scalef32_pk_f32_fp4(q, s, 3);
-        w[0] = a.x;
-        w[1] = a.y;
-        w[2] = b.x;
-        w[3] = b.y;
-        w[4] = c.x;
-        w[5] = c.y;
-        w[6] = d.x;
-        w[7] = d.y;
+    // eight codes to four bf16 pairs
+    __device__ static __forceinline__ void widen8(uint32_t q, float s, uint32_t* w) {
+        w[0] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, s, 0));
+        w[1] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, s, 1));
+        w[2] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, s, 2));
+        w[3] = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, s, 3));
     }
-    __device__ static __forceinline__ void widen(const RowCtx&, const Raw& r, int /*unit*/, float (&w)[UW]) {
-        // the scale as an f32 power of two; 0 (2^-127) and 255 (inf) are not normal f32 exponents and take the
-        // scalar definition
-        const uint32_t s = r.s;
-        if (__builtin_expect(s == 0u || s == 255u, 0)) {
-            const uint32_t q[4] = {r.v.x, r.v.y, r.v.z, r.v.w};
-#pragma unroll
-            for (int j = 0; j < 16; ++j) {
-                const uint8_t byte = (uint8_t)(q[j >> 2] >> ((j & 3) * 8));
-                w[2 * j] = mx4_weight(byte, 0, (uint8_t)s);
-                w[2 * j + 1] = mx4_weight(byte, 1, (uint8_t)s);
-            }
-            return;
-        }
-        const float sf = bits_f32(s << 23);
+    // a pair under scale 255 (2^128, past f32: +inf): the CPU's product is +-inf, or NaN for a zero code
+    __device__ static __forceinline__ uint32_t inf_pair(uint32_t byte) {
+        const uint32_t lo = ((byte & 7u) ? 0x7F80u : 0x7FC0u) | ((byte & 8u) << 12);
+        const uint32_t hi = ((byte & 0x70u) ? 0x7F80u : 0x7FC0u) | ((byte & 0x80u) << 8);
+        return lo | (hi << 16);
+    }
+    __device__ static __forceinline__ void widen(const RowCtx&, const Raw& r, int /*unit*/, uint32_t (&w)[UW / 2]) {
+        // the instruction reads the scale's exponent field, so the e8m0 byte goes in as f32 bits s << 23 - for
+        // s == 0 too, which it takes as 2^-127 (the widen kernel's test covers every scale)
+        const float sf = bits_f32(r.s << 23);
         widen8(r.v.x, sf, w);
-        widen8(r.v.y, sf, w + 8);
-        widen8(r.v.z, sf, w + 16);
-        widen8(r.v.w, sf, w + 24);
+        widen8(r.v.y, sf, w + 4);
+        widen8(r.v.z, sf, w + 8);
+        widen8(r.v.w, sf, w + 12);
+    }
+    // Scale 255 is 2^128, not a finite f32; no quantizer writes it. The CPU's product there is +-inf (NaN for a
+    // zero code); the widen kernel patches its output to exactly that, the matvec leaves what the conversion
+    // instruction gives (non-finite either way).
+    __device__ static __forceinline__ void patch255(const Raw& r, uint32_t (&w)[UW / 2]) {
+        if (r.s != 255u) return;
+        const uint32_t q[4] = {r.v.x, r.v.y, r.v.z, r.v.w};
+#pragma unroll
+        for (int j = 0; j < 16; ++j) w[j] = inf_pair((q[j >> 2] >> ((j & 3) * 8)) & 0xFFu);
     }
     template <int M>
     __device__ static __forceinline__ void tail(const Params&, const RowCtx&, size_t, int, int, int, const uint32_t*,

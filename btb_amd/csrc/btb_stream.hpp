@@ -1,0 +1,114 @@
+// The streaming matvec's building blocks, shared by the dense kernels (gemv.hip) and the routed-expert kernels
+// (moe.hip): staging x in LDS, the span loads, and the pair-wise products of one unit against the rows of x.
+#pragma once
+
+#include "btb_common.hpp"
+#include "btb_formats.hpp"
+
+namespace btb {
+
+// ------------------------------------------------------------------------------------------------------------
+// x staging: [M, C] bf16 into LDS as packed pairs, plain or through the SwiGLU fold
+// ------------------------------------------------------------------------------------------------------------
+
+enum XMode { X_PLAIN = 0, X_SILU = 1 };
+
+// the fold the reference's btb_gemv_silu_bf16 makes in its x load (native/cuda/btb_kernels.cu:168-209):
+// x = bf16(bf16(silu(g)) * u), g and u the two halves of a [M, 2C] row
+__device__ __forceinline__ uint32_t silu_pair(uint32_t g2, uint32_t u2) {
+    const float s0 = bfround(bf16lo_f32(g2) / (1.f + expf(-bf16lo_f32(g2))));
+    const float s1 = bfround(bf16hi_f32(g2) / (1.f + expf(-bf16hi_f32(g2))));
+    const uint32_t lo = f32_bf16(s0 * bf16lo_f32(u2));
+    const uint32_t hi = f32_bf16(s1 * bf16hi_f32(u2));
+    return lo | (hi << 16);
+}
+
+template <int XMODE>
+__device__ __forceinline__ void stage_x(uint32_t* xs, const uint16_t* x, int M, int C) {
+    const int tid = threadIdx.x, nt = blockDim.x;
+    if (XMODE == X_PLAIN) {
+        const uint4* src = reinterpret_cast<const uint4*>(x);
+        uint4* dst = reinterpret_cast<uint4*>(xs);
+        const int n = M * C / 8;
+        for (int i = tid; i < n; i += nt) dst[i] = src[i];
+    } else {
+        const int half = C / 2;  // pairs per row
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(x);
+        for (int i = tid; i < M * half; i += nt) {
+            const int m = i / half, c = i - m * half;
+            xs[i] = silu_pair(src[(size_t)m * 2 * half + c], src[(size_t)m * 2 * half + half + c]);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// the kernel
+// ------------------------------------------------------------------------------------------------------------
+
+// one unit of every one of the RPW rows against the M rows of x. x is read once from LDS, eight values (four bf16
+// pairs) at a time; a weight pair meets its x pair in one v_dot2_f32_bf16: acc += w0 * x0 + w1 * x1 with the products
+// exact and the sum kept in f32, pairs in ascending column order.
+__device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {
+    return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, w), __builtin_bit_cast(bf16x2, x), acc, false);
+}
+
+template <class F, int M, int RPW>
+__device__ __forceinline__ void fma_unit(const typename F::RowCtx (&ctx)[RPW], const typename F::Raw (&raw)[RPW],
+                                         int unit, const uint4* xs4, int xrow4, float (&acc)[RPW][M]) {
+    constexpr int UW = F::UW;
+    constexpr int H = UW / 8;
+    uint4 xv[H][M];
+#pragma unroll
+    for (int h = 0; h < H; ++h)
+#pragma unroll
+        for (int m = 0; m < M; ++m) xv[h][m] = xs4[m * xrow4 + unit * H + h];
+#pragma unroll
+    for (int j = 0; j < RPW; ++j) {
+        uint32_t w[UW / 2];
+        F::widen(ctx[j], raw[j], unit, w);
+#pragma unroll
+        for (int h = 0; h < H; ++h)
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                float a = acc[j][m];
+                a = dot2(w[h * 4 + 0], xv[h][m].x, a);
+                a = dot2(w[h * 4 + 1], xv[h][m].y, a);
+                a = dot2(w[h * 4 + 2], xv[h][m].z, a);
+                a = dot2(w[h * 4 + 3], xv[h][m].w, a);
+                acc[j][m] = a;
+            }
+    }
+}
+
+// where the kernel reads x from: LDS (staged once per workgroup) or straight from global memory through the caches
+enum XSrc { XS_LDS = 0, XS_GLOBAL = 1 };
+
+// the loads of one span: U units of each of the RPW rows; a unit past the row's end is not loaded
+template <class F, int LPR, int RPW, int U, bool GUARD>
+__device__ __forceinline__ void load_span(typename F::Raw (&raw)[U][RPW], const typename F::RowCtx (&ctx)[RPW], int k0,
+                                          int sl, int units) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int unit = k0 + u * LPR + sl;
+        if (!GUARD || unit < units) {
+#pragma unroll
+            for (int j = 0; j < RPW; ++j) raw[u][j] = F::load(ctx[j], unit);
+        }
+    }
+}
+
+template <class F, int M, int LPR, int RPW, int U, bool GUARD>
+__device__ __forceinline__ void fma_span(const typename F::Raw (&raw)[U][RPW], const typename F::RowCtx (&ctx)[RPW],
+                                         int k0, int sl, int units, const uint4* xs4, int xrow4,
+                                         float (&acc)[RPW][M]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int unit = k0 + u * LPR + sl;
+        if (!GUARD || unit < units) fma_unit<F, M, RPW>(ctx, raw[u], unit, xs4, xrow4, acc);
+        // one unit's widening and products at a time: without the fence the scheduler hoists every unit's widening
+        // ahead of the first product and the live registers cost the kernel its occupancy
+        __builtin_amdgcn_sched_barrier(0);
+    }
+}
+
+}  // namespace btb

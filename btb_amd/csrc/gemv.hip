@@ -3,8 +3,8 @@
 // per-lane non-temporal loads, a wave covering 1 KiB of a row per load instruction and keeping RPW * U of them in
 // flight; x is staged once per workgroup in LDS (optionally through the SwiGLU fold) and read from there with
 // ds_read_b128, shared by the RPW rows a lane works on. A row is summed by LPR lanes (64, 32 or 16, chosen from the
-// row length alone), each lane running its units in ascending column order with one fma per weight, then a fixed
-// DPP tree over the lanes: the sequence for (m, r) depends on neither M nor the launch, so row m of a wide pass
+// row length alone), each lane running its units in ascending column order, a pair of weights per v_dot2_f32_bf16
+// (f32 accumulate), then a fixed DPP tree over the lanes: the sequence for (m, r) depends on neither M nor the launch, so row m of a wide pass
 // equals the one-row pass bit for bit - the law the reference's card kernels keep (native/cuda/btb_kernels.cu:84-88).
 //
 // The same loop serves every stored form through a policy (btb_widen.hpp semantics, vector forms here): the bytes a
@@ -12,6 +12,7 @@
 
 #include "btb_common.hpp"
 #include "btb_formats.hpp"
+#include "btb_stream.hpp"
 #include "btb_tuning.hpp"
 
 #include "../../include/btb_hip.h"
@@ -19,103 +20,8 @@
 namespace btb {
 
 // ------------------------------------------------------------------------------------------------------------
-// x staging: [M, C] bf16 into LDS as packed pairs, plain or through the SwiGLU fold
-// ------------------------------------------------------------------------------------------------------------
-
-enum XMode { X_PLAIN = 0, X_SILU = 1 };
-
-// the fold the reference's btb_gemv_silu_bf16 makes in its x load (native/cuda/btb_kernels.cu:168-209):
-// x = bf16(bf16(silu(g)) * u), g and u the two halves of a [M, 2C] row
-__device__ __forceinline__ uint32_t silu_pair(uint32_t g2, uint32_t u2) {
-    const float s0 = bfround(bf16lo_f32(g2) / (1.f + expf(-bf16lo_f32(g2))));
-    const float s1 = bfround(bf16hi_f32(g2) / (1.f + expf(-bf16hi_f32(g2))));
-    const uint32_t lo = f32_bf16(s0 * bf16lo_f32(u2));
-    const uint32_t hi = f32_bf16(s1 * bf16hi_f32(u2));
-    return lo | (hi << 16);
-}
-
-template <int XMODE>
-__device__ __forceinline__ void stage_x(uint32_t* xs, const uint16_t* x, int M, int C) {
-    const int tid = threadIdx.x, nt = blockDim.x;
-    if (XMODE == X_PLAIN) {
-        const uint4* src = reinterpret_cast<const uint4*>(x);
-        uint4* dst = reinterpret_cast<uint4*>(xs);
-        const int n = M * C / 8;
-        for (int i = tid; i < n; i += nt) dst[i] = src[i];
-    } else {
-        const int half = C / 2;  // pairs per row
-        const uint32_t* src = reinterpret_cast<const uint32_t*>(x);
-        for (int i = tid; i < M * half; i += nt) {
-            const int m = i / half, c = i - m * half;
-            xs[i] = silu_pair(src[(size_t)m * 2 * half + c], src[(size_t)m * 2 * half + half + c]);
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------------------------
 // the kernel
 // ------------------------------------------------------------------------------------------------------------
-
-// one unit of every one of the RPW rows against the M rows of x: x read once from LDS, eight at a time, in index order
-template <class F, int M, int RPW>
-__device__ __forceinline__ void fma_unit(const typename F::RowCtx (&ctx)[RPW], const typename F::Raw (&raw)[RPW],
-                                         int unit, const uint4* xs4, int xrow4, float (&acc)[RPW][M]) {
-    constexpr int UW = F::UW;
-    constexpr int H = UW / 8;
-    uint4 xv[H][M];
-#pragma unroll
-    for (int h = 0; h < H; ++h)
-#pragma unroll
-        for (int m = 0; m < M; ++m) xv[h][m] = xs4[m * xrow4 + unit * H + h];
-#pragma unroll
-    for (int j = 0; j < RPW; ++j) {
-        float w[UW];
-        F::widen(ctx[j], raw[j], unit, w);
-#pragma unroll
-        for (int h = 0; h < H; ++h)
-#pragma unroll
-            for (int m = 0; m < M; ++m) {
-                float a = acc[j][m];
-                a = fmaf(w[h * 8 + 0], bf16lo_f32(xv[h][m].x), a);
-                a = fmaf(w[h * 8 + 1], bf16hi_f32(xv[h][m].x), a);
-                a = fmaf(w[h * 8 + 2], bf16lo_f32(xv[h][m].y), a);
-                a = fmaf(w[h * 8 + 3], bf16hi_f32(xv[h][m].y), a);
-                a = fmaf(w[h * 8 + 4], bf16lo_f32(xv[h][m].z), a);
-                a = fmaf(w[h * 8 + 5], bf16hi_f32(xv[h][m].z), a);
-                a = fmaf(w[h * 8 + 6], bf16lo_f32(xv[h][m].w), a);
-                a = fmaf(w[h * 8 + 7], bf16hi_f32(xv[h][m].w), a);
-                acc[j][m] = a;
-            }
-    }
-}
-
-// where the kernel reads x from: LDS (staged once per workgroup) or straight from global memory through the caches
-enum XSrc { XS_LDS = 0, XS_GLOBAL = 1 };
-
-// the loads of one span: U units of each of the RPW rows; a unit past the row's end is not loaded
-template <class F, int LPR, int RPW, int U, bool GUARD>
-__device__ __forceinline__ void load_span(typename F::Raw (&raw)[U][RPW], const typename F::RowCtx (&ctx)[RPW], int k0,
-                                          int sl, int units) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const int unit = k0 + u * LPR + sl;
-        if (!GUARD || unit < units) {
-#pragma unroll
-            for (int j = 0; j < RPW; ++j) raw[u][j] = F::load(ctx[j], unit);
-        }
-    }
-}
-
-template <class F, int M, int LPR, int RPW, int U, bool GUARD>
-__device__ __forceinline__ void fma_span(const typename F::Raw (&raw)[U][RPW], const typename F::RowCtx (&ctx)[RPW],
-                                         int k0, int sl, int units, const uint4* xs4, int xrow4,
-                                         float (&acc)[RPW][M]) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const int unit = k0 + u * LPR + sl;
-        if (!GUARD || unit < units) fma_unit<F, M, RPW>(ctx, raw[u], unit, xs4, xrow4, acc);
-    }
-}
 
 template <class F, int M, int LPR, int RPW, int U, int XMODE, int XSRC>
 __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, const uint16_t* __restrict__ x,
@@ -133,23 +39,6 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, const u
     const int span = U * LPR;
     const int xrow4 = C / 8;  // uint4 per row of x
 
-    // the first span of the wave's first tile is requested before x is staged: the weights do not wait for x
-    typename F::Raw raw[U][RPW];
-    typename F::RowCtx ctx[RPW];
-    int rows[RPW];
-    int tile = wave;
-    if (tile < ntiles) {
-#pragma unroll
-        for (int j = 0; j < RPW; ++j) {
-            rows[j] = tile * ROWS + j * G + lane / LPR;
-            // a row past the end reads the last row again (no divergence in the stream) and is not written
-            ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
-        }
-        if (span <= units)
-            load_span<F, LPR, RPW, U, false>(raw, ctx, 0, sl, units);
-        else
-            load_span<F, LPR, RPW, U, true>(raw, ctx, 0, sl, units);
-    }
     const uint4* xs4;
     if (XSRC == XS_LDS) {
         stage_x<XMODE>(xs, x, M, C);
@@ -159,14 +48,14 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, const u
         xs4 = reinterpret_cast<const uint4*>(x);
     }
 
-    bool primed = true;
-    for (; tile < ntiles; tile += nwaves) {
-        if (!primed) {
+    for (int tile = wave; tile < ntiles; tile += nwaves) {
+        typename F::RowCtx ctx[RPW];
+        int rows[RPW];
 #pragma unroll
-            for (int j = 0; j < RPW; ++j) {
-                rows[j] = tile * ROWS + j * G + lane / LPR;
-                ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
-            }
+        for (int j = 0; j < RPW; ++j) {
+            rows[j] = tile * ROWS + j * G + lane / LPR;
+            // a row past the end reads the last row again (no divergence in the stream) and is not written
+            ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
         }
         float acc[RPW][M];
 #pragma unroll
@@ -175,14 +64,14 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, const u
             for (int m = 0; m < M; ++m) acc[j][m] = 0.f;
 
         for (int k0 = 0; k0 < units; k0 += span) {
+            typename F::Raw raw[U][RPW];
             if (k0 + span <= units) {
-                if (!primed) load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
+                load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
                 fma_span<F, M, LPR, RPW, U, false>(raw, ctx, k0, sl, units, xs4, xrow4, acc);
             } else {
-                if (!primed) load_span<F, LPR, RPW, U, true>(raw, ctx, k0, sl, units);
+                load_span<F, LPR, RPW, U, true>(raw, ctx, k0, sl, units);
                 fma_span<F, M, LPR, RPW, U, true>(raw, ctx, k0, sl, units, xs4, xrow4, acc);
             }
-            primed = false;
         }
 #pragma unroll
         for (int j = 0; j < RPW; ++j)
@@ -218,12 +107,15 @@ static int32_t launch_variant(const typename F::Params& p, const void* x, void* 
         set_error("gemv: the x rows do not fit LDS");
         return ERR_DOMAIN;
     }
+    // Every workgroup stages x once, so the grid is kept to a few workgroups a CU and each wave walks a whole number
+    // of tiles (the last wave of the grid may walk fewer): tiles_per_wave is the smallest count that fits the cap.
     const int ntiles = (R + G * RPW - 1) / (G * RPW);
     int per_cu = tuning("gemv_wgs_per_cu");
-    if (per_cu <= 0) per_cu = 16;  // past this many workgroups a CU the waves loop over tiles
-    int grid = (ntiles + 3) / 4;
-    const int cap = dev.cus * per_cu;
-    if (grid > cap) grid = cap;
+    if (per_cu <= 0) per_cu = 3;
+    const int cap_waves = dev.cus * per_cu * 4;
+    const int tiles_per_wave = (ntiles + cap_waves - 1) / cap_waves;
+    const int waves = (ntiles + tiles_per_wave - 1) / tiles_per_wave;
+    int grid = (waves + 3) / 4;
     if (grid < 1) grid = 1;
     auto kern = gemv_stream<F, M, LPR, RPW, U, XMODE, XSRC>;
     if (lds > 64 * 1024) {

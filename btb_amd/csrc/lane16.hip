@@ -1,0 +1,233 @@
+// The host matvec's bits on the GPU: the device twins of the reference crate's CPU entry points, f32 x and y, every
+// output computed in exactly the CPU's order so the result is bit-identical to btb_gemv_*_rows on the host
+// (native/src/gemv.rs:84-123, 45-58). Sixteen lanes work on a row: lane j runs the columns = j (mod 16) in ascending
+// order, one fused multiply-add each, and the sixteen lane sums fold pairwise ((l0+l1)+(l2+l3))+... - the same
+// tree as the host's reduce16, since every step adds the two halves of an aligned group. The reference's card has the
+// same pair of kernels for bf16 and MXFP4 (btb_gemv_lane16_f32_m*, btb_gemv_lane16_mx4_f32_m*:
+// native/cuda/btb_kernels.cu:1635-1766); here all four stored forms have one, each weight made by the scalar
+// definition of btb_widen.hpp. These are the parity and routing kernels (the router's logits must be the CPU's, bit
+// for bit, for the top-k picks to be); the bandwidth path is gemv.hip.
+
+#include "btb_common.hpp"
+#include "btb_tuning.hpp"
+#include "btb_widen.hpp"
+
+#include "../../include/btb_hip.h"
+
+namespace btb {
+
+struct W16Bf16 {
+    const uint16_t* w;
+    __device__ __forceinline__ float at(size_t r, size_t c, size_t cols) const { return bf16_f32(w[r * cols + c]); }
+};
+
+struct W16P12 {
+    const uint8_t* lo;
+    const uint8_t* hi4;
+    const uint8_t* table;
+    const int32_t* esc_idx;
+    const uint8_t* esc_val;
+    size_t n_esc;
+    __device__ __forceinline__ float at(size_t r, size_t c, size_t cols) const {
+        const size_t i = r * cols + c;
+        const uint8_t byte = hi4[i >> 1];
+        const unsigned code = (i & 1) ? (byte >> 4) : (byte & 0x0F);
+        uint32_t hi = table[code];
+        if (code == 15u && n_esc != 0) {
+            // an escaped weight: its high byte is in the list, found by its index
+            size_t a = 0, b = n_esc;
+            while (a < b) {
+                const size_t m = a + (b - a) / 2;
+                if ((size_t)esc_idx[m] < i)
+                    a = m + 1;
+                else
+                    b = m;
+            }
+            if (a < n_esc && (size_t)esc_idx[a] == i) hi = esc_val[a];
+        }
+        return bits_f32((hi << 24) | ((uint32_t)lo[i] << 16));
+    }
+};
+
+struct W16Mx4 {
+    const uint8_t* blocks;
+    const uint8_t* scales;
+    __device__ __forceinline__ float at(size_t r, size_t c, size_t cols) const {
+        const size_t i = r * cols + c;
+        const size_t g = i >> 5;
+        const unsigned k = (unsigned)(i & 31);
+        return mx4_weight(blocks[g * 16 + (k >> 1)], (int)(k & 1), scales[g]);
+    }
+};
+
+struct W16F8 {
+    const uint8_t* w;
+    const float* scales;
+    size_t sc, bm, bn;
+    __device__ __forceinline__ float at(size_t r, size_t c, size_t cols) const {
+        return f8_held(w[r * cols + c], scales[(r / bm) * sc + c / bn]);
+    }
+};
+
+// B rows of x per pass (the host walks up to 8 at a time; the order within one (row, vector) pair is the same)
+template <class W, int B>
+__global__ void __launch_bounds__(256) lane16_kernel(W w, const float* __restrict__ x, float* __restrict__ y, size_t rows,
+                                                     size_t cols, size_t b0, size_t btotal) {
+    const int j = threadIdx.x & 15;
+    const size_t r = (size_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
+    const bool live = r < rows;
+    const size_t rr = live ? r : rows - 1;
+    float acc[B];
+#pragma unroll
+    for (int i = 0; i < B; ++i) acc[i] = 0.f;
+    for (size_t c = (size_t)j; c < cols; c += 16) {
+        const float wv = w.at(rr, c, cols);
+#pragma unroll
+        for (int i = 0; i < B; ++i) {
+            if (b0 + i < btotal) acc[i] = fmaf(wv, x[(b0 + i) * cols + c], acc[i]);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < B; ++i) {
+        const float s = group_sum<16>(acc[i]);
+        if (j == 0 && live && b0 + i < btotal) y[(b0 + i) * rows + r] = s;
+    }
+}
+
+template <class W>
+static int32_t launch_lane16(const W& w, const float* x, float* y, size_t rows, size_t cols, size_t b, hipStream_t st) {
+    const unsigned grid = (unsigned)((rows + 15) / 16);
+    for (size_t b0 = 0; b0 < b; b0 += 4) {
+        const size_t left = b - b0;
+        if (left >= 4)
+            hipLaunchKernelGGL((lane16_kernel<W, 4>), dim3(grid), dim3(256), 0, st, w, x, y, rows, cols, b0, b);
+        else if (left >= 2)
+            hipLaunchKernelGGL((lane16_kernel<W, 3>), dim3(grid), dim3(256), 0, st, w, x, y, rows, cols, b0, b);
+        else
+            hipLaunchKernelGGL((lane16_kernel<W, 1>), dim3(grid), dim3(256), 0, st, w, x, y, rows, cols, b0, b);
+        int32_t rc = hip_status(hipGetLastError(), "lane16 launch");
+        if (rc != OK) return rc;
+    }
+    return OK;
+}
+
+static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+// the crate's shape rule (native/src/gemv.rs:4216-4222), with the grid's 2^31 limit on rows / 16
+static bool shape_ok(size_t rows, size_t cols, size_t b) {
+    const size_t cap = (size_t)INTPTR_MAX / 4;
+    size_t n;
+    if (__builtin_mul_overflow(rows, cols, &n) || n > cap) return false;
+    if (__builtin_mul_overflow(b, cols, &n) || n > cap) return false;
+    if (__builtin_mul_overflow(b, rows, &n) || n > cap) return false;
+    return rows / 16 < 0x7FFFFFFFull;
+}
+
+}  // namespace btb
+
+using namespace btb;
+
+extern "C" {
+
+int32_t btb_hip_gemv_bf16_rows(const uint16_t* w, size_t rows, size_t cols, const float* x, size_t b, float* y,
+                               void* stream) {
+    if (w == nullptr || x == nullptr || y == nullptr) return ERR_NULL;
+    if (rows == 0 || cols == 0 || b == 0) return ERR_DOMAIN;
+    if (!shape_ok(rows, cols, b) || !al(w, 2) || !al(x, 4) || !al(y, 4)) return ERR_DOMAIN;
+    return launch_lane16(W16Bf16{w}, x, y, rows, cols, b, static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_gemv_bf16_group(size_t n, const uint16_t* const* w, const size_t* rows, const size_t* cols,
+                                const float* const* x, const size_t* b, float* const* y, void* stream) {
+    if (w == nullptr || rows == nullptr || cols == nullptr || x == nullptr || b == nullptr || y == nullptr)
+        return ERR_NULL;
+    if (n == 0) return ERR_DOMAIN;
+    // every task is checked before the first is launched: a refused call launches nothing
+    for (size_t t = 0; t < n; ++t) {
+        if (w[t] == nullptr || x[t] == nullptr || y[t] == nullptr) return ERR_NULL;
+        if (rows[t] == 0 || cols[t] == 0 || b[t] == 0) return ERR_DOMAIN;
+        if (!shape_ok(rows[t], cols[t], b[t]) || !al(w[t], 2) || !al(x[t], 4) || !al(y[t], 4)) return ERR_DOMAIN;
+    }
+    for (size_t t = 0; t < n; ++t) {
+        int32_t rc = launch_lane16(W16Bf16{w[t]}, x[t], y[t], rows[t], cols[t], b[t], static_cast<hipStream_t>(stream));
+        if (rc != OK) return rc;
+    }
+    return OK;
+}
+
+int32_t btb_hip_gemv_p12_rows(const uint8_t* lo, const uint8_t* hi4, const uint8_t* table, const int32_t* esc_idx,
+                              const uint8_t* esc_val, size_t n_esc, size_t rows, size_t cols, const float* x, size_t b,
+                              float* y, void* stream) {
+    if (lo == nullptr || hi4 == nullptr || table == nullptr || x == nullptr || y == nullptr) return ERR_NULL;
+    if (n_esc > 0 && (esc_idx == nullptr || esc_val == nullptr)) return ERR_NULL;
+    if (rows == 0 || cols == 0 || b == 0) return ERR_DOMAIN;
+    if (!shape_ok(rows, cols, b) || !al(x, 4) || !al(y, 4)) return ERR_DOMAIN;
+    if (n_esc > 0 && (n_esc > rows * cols || !al(esc_idx, 4))) return ERR_DOMAIN;
+    // the list's order is the caller's to keep on the device (the host entry point walks it; here that would be a
+    // copy back): an index absent from the list leaves the table's byte in place
+    return launch_lane16(W16P12{lo, hi4, table, esc_idx, esc_val, n_esc}, x, y, rows, cols, b,
+                         static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_gemv_mxfp4_rows(const uint8_t* blocks, const uint8_t* scales, size_t rows, size_t cols, const float* x,
+                                size_t b, float* y, void* stream) {
+    if (blocks == nullptr || scales == nullptr || x == nullptr || y == nullptr) return ERR_NULL;
+    if (rows == 0 || cols == 0 || b == 0 || cols % 32 != 0 || !shape_ok(rows, cols, b) || !al(x, 4) || !al(y, 4))
+        return ERR_DOMAIN;
+    return launch_lane16(W16Mx4{blocks, scales}, x, y, rows, cols, b, static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_gemv_mxfp4_group(size_t n, const uint8_t* const* blocks, const uint8_t* const* scales,
+                                 const size_t* rows, const size_t* cols, const float* const* x, const size_t* b,
+                                 float* const* y, void* stream) {
+    if (blocks == nullptr || scales == nullptr || rows == nullptr || cols == nullptr || x == nullptr || b == nullptr ||
+        y == nullptr)
+        return ERR_NULL;
+    if (n == 0) return ERR_DOMAIN;
+    for (size_t t = 0; t < n; ++t) {
+        if (blocks[t] == nullptr || scales[t] == nullptr || x[t] == nullptr || y[t] == nullptr) return ERR_NULL;
+        if (rows[t] == 0 || cols[t] == 0 || b[t] == 0 || cols[t] % 32 != 0 || !shape_ok(rows[t], cols[t], b[t]) ||
+            !al(x[t], 4) || !al(y[t], 4))
+            return ERR_DOMAIN;
+    }
+    for (size_t t = 0; t < n; ++t) {
+        int32_t rc = launch_lane16(W16Mx4{blocks[t], scales[t]}, x[t], y[t], rows[t], cols[t], b[t],
+                                   static_cast<hipStream_t>(stream));
+        if (rc != OK) return rc;
+    }
+    return OK;
+}
+
+int32_t btb_hip_gemv_fp8_rows(const uint8_t* w, const float* scales, size_t rows, size_t cols, size_t sr, size_t sc,
+                              const float* x, size_t b, float* y, void* stream) {
+    if (w == nullptr || scales == nullptr || x == nullptr || y == nullptr) return ERR_NULL;
+    if (rows == 0 || cols == 0 || b == 0 || sr == 0 || sc == 0) return ERR_DOMAIN;
+    if (rows % sr != 0 || cols % sc != 0 || !shape_ok(rows, cols, b) || !al(scales, 4) || !al(x, 4) || !al(y, 4))
+        return ERR_DOMAIN;
+    return launch_lane16(W16F8{w, scales, sc, rows / sr, cols / sc}, x, y, rows, cols, b,
+                         static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_gemv_fp8_group(size_t n, const uint8_t* const* w, const float* const* scales, const size_t* rows,
+                               const size_t* cols, const size_t* sr, const size_t* sc, const float* const* x,
+                               const size_t* b, float* const* y, void* stream) {
+    if (w == nullptr || scales == nullptr || rows == nullptr || cols == nullptr || sr == nullptr || sc == nullptr ||
+        x == nullptr || b == nullptr || y == nullptr)
+        return ERR_NULL;
+    if (n == 0) return ERR_DOMAIN;
+    for (size_t t = 0; t < n; ++t) {
+        if (w[t] == nullptr || scales[t] == nullptr || x[t] == nullptr || y[t] == nullptr) return ERR_NULL;
+        if (rows[t] == 0 || cols[t] == 0 || b[t] == 0 || sr[t] == 0 || sc[t] == 0) return ERR_DOMAIN;
+        if (rows[t] % sr[t] != 0 || cols[t] % sc[t] != 0 || !shape_ok(rows[t], cols[t], b[t]) || !al(scales[t], 4) ||
+            !al(x[t], 4) || !al(y[t], 4))
+            return ERR_DOMAIN;
+    }
+    for (size_t t = 0; t < n; ++t) {
+        int32_t rc = launch_lane16(W16F8{w[t], scales[t], sc[t], rows[t] / sr[t], cols[t] / sc[t]}, x[t], y[t], rows[t],
+                                   cols[t], b[t], static_cast<hipStream_t>(stream));
+        if (rc != OK) return rc;
+    }
+    return OK;
+}
+
+}  // extern "C"

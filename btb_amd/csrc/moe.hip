@@ -1,0 +1,342 @@
+// The routed top-k MoE decode layer on the GPU, all experts resident in VRAM:
+//
+//   route      per token: f32 softmax over the E logits, the top k in the total order (p descending, index ascending),
+//              weights p / sum(top k) summed in rank order, rounded to bf16 - the reference's btb_moe_route
+//              (native/cuda/btb_kernels.cu:845-948) and Qwen4Router.forward (btb/engine/families/qwen4/router.py:43-51)
+//   gate_up    for every (token, pick): gu = W_gu[expert] . x[token], f32 accumulate, bf16 out; the experts' matrices
+//              are streamed once per pick with the dense matvec's loop (btb_stream.hpp)
+//   down       for every token and output row: the k experts in ASCENDING expert id, each d = bf16(W_dn[e] . h_e) with
+//              h_e = bf16(bf16(silu(g)) * u) folded into the x staging, then y = bf16(y + bf16(d * w_e)) - the dtype
+//              chain and the summation order of _Experts._one_row / _loop (btb/engine/host.py:508-569, 906-967)
+//
+// Nothing goes back to the host between the steps, so the layer records into a hipGraph.
+
+#include "btb_common.hpp"
+#include "btb_formats.hpp"
+#include "btb_stream.hpp"
+#include "btb_tuning.hpp"
+
+#include "../../include/btb_hip.h"
+
+namespace btb {
+
+constexpr int ROUTE_MAX_K = 32;  // the reference's ROUTE_MAX_K (native/cuda/btb_kernels.cu:859)
+
+// ------------------------------------------------------------------------------------------------------------
+// route: one wave per token
+// ------------------------------------------------------------------------------------------------------------
+
+template <bool F32>
+__device__ __forceinline__ float logit_at(const void* base, size_t i) {
+    return F32 ? static_cast<const float*>(base)[i] : bf16_f32(static_cast<const uint16_t*>(base)[i]);
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) v = fmaxf(v, __shfl_xor(v, s, WAVE));
+    return v;
+}
+
+// the (value, index) maximum over the wave in the total order: value descending, then index ascending; an index of
+// NONE is "nothing"
+constexpr int NONE = 0x7fffffff;
+__device__ __forceinline__ void wave_argmax(float& v, int& i) {
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) {
+        const float ov = __shfl_xor(v, s, WAVE);
+        const int oi = __shfl_xor(i, s, WAVE);
+        if (oi != NONE && (i == NONE || ov > v || (ov == v && oi < i))) {
+            v = ov;
+            i = oi;
+        }
+    }
+}
+
+template <bool F32>
+__global__ void __launch_bounds__(64) moe_route_kernel(const void* __restrict__ logits, size_t ls, int E, int k,
+                                                       int32_t* __restrict__ idx, uint16_t* __restrict__ w,
+                                                       float* __restrict__ w32) {
+    extern __shared__ float pr[];  // [E] the row's probabilities; a picked one is set below every live one
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const size_t base = (size_t)t * ls;
+    float m = bits_f32(0xff800000u);
+    for (int e = lane; e < E; e += WAVE) m = fmaxf(m, logit_at<F32>(logits, base + e));
+    m = wave_max(m);
+    float s = 0.f;
+    for (int e = lane; e < E; e += WAVE) {
+        const float p = expf(logit_at<F32>(logits, base + e) - m);
+        pr[e] = p;
+        s += p;
+    }
+    s = group_sum<64>(s);
+    s = __shfl(s, 0, WAVE);
+    for (int e = lane; e < E; e += WAVE) pr[e] = pr[e] / s;
+    __syncthreads();
+    // k rounds of the maximum; probabilities are >= 0, so -1 is below every live one and a pick is marked -2. A row of
+    // NaN probabilities compares below nothing: it still takes live experts, the first it meets, as the reference's
+    // kernel does (native/cuda/btb_kernels.cu:891-900)
+    float topv = 0.f;  // lane j keeps pick j
+    int topi = 0;
+    for (int j = 0; j < k; ++j) {
+        float bv = -1.f;
+        int bi = NONE;
+        for (int e = lane; e < E; e += WAVE) {
+            const float v = pr[e];
+            if (v > bv || (bi == NONE && v != -2.f)) {  // e ascends within the lane, so a tie keeps the lower index
+                bv = v;
+                bi = e;
+            }
+        }
+        wave_argmax(bv, bi);
+        if (lane == j) {
+            topv = bv;
+            topi = bi;
+        }
+        if (lane == 0 && bi != NONE) pr[bi] = -2.f;
+        __syncthreads();
+    }
+    // the weights: sum of the top k in rank order, each p / sum
+    float sum = 0.f;
+    for (int j = 0; j < k; ++j) sum += __shfl(topv, j, WAVE);
+    if (lane < k) {
+        const float wv = topv / sum;
+        const size_t o = (size_t)t * k + lane;
+        idx[o] = topi;
+        w[o] = f32_bf16(wv);
+        if (w32 != nullptr) w32[o] = wv;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// gate_up: the dense loop over (token, pick) pairs; blockIdx.y is the pair
+// ------------------------------------------------------------------------------------------------------------
+
+template <int LPR, int RPW, int U>
+__global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restrict__ stack, const uint16_t* __restrict__ x,
+                                                          const int32_t* __restrict__ idx, uint16_t* __restrict__ gu,
+                                                          int R, int C, int k, int E) {
+    extern __shared__ __align__(16) uint32_t xs[];
+    using F = FmtBf16;
+    constexpr int G = WAVE / LPR, ROWS = G * RPW;
+    const int pair = blockIdx.y;
+    const int token = pair / k;
+    int expert = idx[pair];
+    expert = expert < 0 ? 0 : (expert >= E ? E - 1 : expert);  // a bad id reads a real expert and is the caller's
+    const int units = C / F::UW;
+    const int lane = threadIdx.x & (WAVE - 1), sl = lane % LPR;
+    const int wave = blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
+    const int nwaves = gridDim.x * (blockDim.x / WAVE);
+    const int ntiles = (R + ROWS - 1) / ROWS;
+    const int span = U * LPR;
+    F::Params p{stack + (size_t)expert * R * units};
+    uint16_t* y = gu + (size_t)pair * R;
+
+    stage_x<X_PLAIN>(xs, x + (size_t)token * C, 1, C);
+    __syncthreads();
+    const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
+    for (int tile = wave; tile < ntiles; tile += nwaves) {
+        F::RowCtx ctx[RPW];
+        int rows[RPW];
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) {
+            rows[j] = tile * ROWS + j * G + lane / LPR;
+            ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
+        }
+        float acc[RPW][1];
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) acc[j][0] = 0.f;
+        for (int k0 = 0; k0 < units; k0 += span) {
+            F::Raw raw[U][RPW];
+            if (k0 + span <= units) {
+                load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
+                fma_span<F, 1, LPR, RPW, U, false>(raw, ctx, k0, sl, units, xs4, C / 8, acc);
+            } else {
+                load_span<F, LPR, RPW, U, true>(raw, ctx, k0, sl, units);
+                fma_span<F, 1, LPR, RPW, U, true>(raw, ctx, k0, sl, units, xs4, C / 8, acc);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) {
+            const float s = group_sum<LPR>(acc[j][0]);
+            if (sl == 0 && rows[j] < R) y[rows[j]] = f32_bf16(s);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// down + weighted sum: blockIdx.y is the token; the k experts of a row are walked in ascending expert id
+// ------------------------------------------------------------------------------------------------------------
+
+template <int LPR, int RPW, int U>
+__global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__ stack, const uint16_t* __restrict__ gu,
+                                                       const int32_t* __restrict__ idx, const uint16_t* __restrict__ wts,
+                                                       uint16_t* __restrict__ y, int R, int C, int k, int E) {
+    extern __shared__ __align__(16) uint32_t hs[];  // [k][C / 2] the k experts' h rows, in ascending expert order
+    __shared__ int s_expert[ROUTE_MAX_K];
+    __shared__ float s_weight[ROUTE_MAX_K];
+    using F = FmtBf16;
+    constexpr int G = WAVE / LPR, ROWS = G * RPW;
+    const int token = blockIdx.y;
+    const int units = C / F::UW;
+    const int lane = threadIdx.x & (WAVE - 1), sl = lane % LPR;
+    const int wave = blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
+    const int nwaves = gridDim.x * (blockDim.x / WAVE);
+    const int ntiles = (R + ROWS - 1) / ROWS;
+    const int span = U * LPR;
+
+    // the token's picks by ascending expert id: pick j goes to place #{i : id_i < id_j} (ids of a row are distinct; a
+    // repeated id keeps its rank order)
+    if (threadIdx.x < k) {
+        const int j = threadIdx.x;
+        const int mine = idx[(size_t)token * k + j];
+        int place = 0;
+        for (int i = 0; i < k; ++i) {
+            const int other = idx[(size_t)token * k + i];
+            place += (other < mine) || (other == mine && i < j);
+        }
+        s_expert[place] = mine < 0 ? 0 : (mine >= E ? E - 1 : mine);
+        s_weight[place] = bf16_f32(wts[(size_t)token * k + j]);
+        // the h row of this pick, staged at its place below
+        s_expert[place] |= j << 20;
+    }
+    __syncthreads();
+    for (int q = 0; q < k; ++q) {
+        const int j = s_expert[q] >> 20;
+        stage_x<X_SILU>(hs + (size_t)q * (C / 2), gu + ((size_t)token * k + j) * 2 * C, 1, C);
+    }
+    __syncthreads();
+    const uint4* hs4 = reinterpret_cast<const uint4*>(hs);
+
+    for (int tile = wave; tile < ntiles; tile += nwaves) {
+        int rows[RPW];
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) rows[j] = tile * ROWS + j * G + lane / LPR;
+        float out[RPW];
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) out[j] = 0.f;
+        for (int q = 0; q < k; ++q) {
+            const int expert = s_expert[q] & 0xFFFFF;
+            F::Params p{stack + (size_t)expert * R * units};
+            F::RowCtx ctx[RPW];
+#pragma unroll
+            for (int j = 0; j < RPW; ++j) ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
+            float acc[RPW][1];
+#pragma unroll
+            for (int j = 0; j < RPW; ++j) acc[j][0] = 0.f;
+            const uint4* xq = hs4 + (size_t)q * (C / 8);
+            for (int k0 = 0; k0 < units; k0 += span) {
+                F::Raw raw[U][RPW];
+                if (k0 + span <= units) {
+                    load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
+                    fma_span<F, 1, LPR, RPW, U, false>(raw, ctx, k0, sl, units, xq, C / 8, acc);
+                } else {
+                    load_span<F, LPR, RPW, U, true>(raw, ctx, k0, sl, units);
+                    fma_span<F, 1, LPR, RPW, U, true>(raw, ctx, k0, sl, units, xq, C / 8, acc);
+                }
+            }
+            const float wq = s_weight[q];
+#pragma unroll
+            for (int j = 0; j < RPW; ++j) {
+                const float d = bfround(group_sum<LPR>(acc[j][0]));  // the expert's down product, as the row's dtype
+                out[j] = bfround(out[j] + bfround(d * wq));          // times its weight, added in bf16
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < RPW; ++j)
+            if (sl == 0 && rows[j] < R) y[(size_t)token * R + rows[j]] = f32_bf16(out[j]);
+    }
+}
+
+static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+static int lanes_for(int units) {
+    if (units % 64 == 0 || units >= 256) return 64;
+    if (units % 32 == 0 || units >= 96) return 32;
+    return 16;
+}
+
+template <int LPR>
+static int32_t launch_gate_up(const void* stack, const void* x, const int32_t* idx, void* gu, int R, int C, int k, int E,
+                              int pairs, hipStream_t st) {
+    constexpr int RPW = 2, U = 4, G = WAVE / LPR;
+    const int ntiles = (R + G * RPW - 1) / (G * RPW);
+    const int grid = (ntiles + 3) / 4;
+    hipLaunchKernelGGL((moe_gate_up_kernel<LPR, RPW, U>), dim3(grid, pairs), dim3(256), (size_t)C * 2, st,
+                       static_cast<const uint4*>(stack), static_cast<const uint16_t*>(x), idx,
+                       static_cast<uint16_t*>(gu), R, C, k, E);
+    return hip_status(hipGetLastError(), "moe gate_up launch");
+}
+
+template <int LPR>
+static int32_t launch_down(const void* stack, const void* gu, const int32_t* idx, const void* w, void* y, int R, int C,
+                           int k, int E, int T, hipStream_t st) {
+    constexpr int RPW = 1, U = 4, G = WAVE / LPR;
+    const int ntiles = (R + G * RPW - 1) / (G * RPW);
+    const int grid = (ntiles + 3) / 4;
+    const size_t lds = (size_t)k * C * 2;
+    auto kern = moe_down_kernel<LPR, RPW, U>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
+    }
+    hipLaunchKernelGGL(kern, dim3(grid, T), dim3(256), lds, st, static_cast<const uint4*>(stack),
+                       static_cast<const uint16_t*>(gu), idx, static_cast<const uint16_t*>(w),
+                       static_cast<uint16_t*>(y), R, C, k, E);
+    return hip_status(hipGetLastError(), "moe down launch");
+}
+
+}  // namespace btb
+
+using namespace btb;
+
+extern "C" {
+
+int32_t btb_hip_moe_route(const void* logits, int32_t logits_f32, size_t ls, size_t E, size_t k, size_t T, int32_t* idx,
+                          void* w, float* w32, void* stream) {
+    if (logits == nullptr || idx == nullptr || w == nullptr) return ERR_NULL;
+    if (E == 0 || k == 0 || T == 0 || k > E || k > (size_t)ROUTE_MAX_K || ls < E || E > 8192 || T > 0x7FFFFFFFull)
+        return ERR_DOMAIN;
+    if (!al(logits, logits_f32 ? 4 : 2) || !al(idx, 4) || !al(w, 2) || !al(w32, 4)) return ERR_DOMAIN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    if (logits_f32)
+        hipLaunchKernelGGL(moe_route_kernel<true>, dim3((unsigned)T), dim3(64), E * 4, st, logits, ls, (int)E, (int)k, idx,
+                           static_cast<uint16_t*>(w), w32);
+    else
+        hipLaunchKernelGGL(moe_route_kernel<false>, dim3((unsigned)T), dim3(64), E * 4, st, logits, ls, (int)E, (int)k, idx,
+                           static_cast<uint16_t*>(w), w32);
+    return hip_status(hipGetLastError(), "moe_route launch");
+}
+
+int32_t btb_hip_moe_experts_bf16(const void* gate_up, const void* down, const void* x, const int32_t* idx, const void* w,
+                                 void* gu, void* y, size_t T, size_t k, size_t E, size_t H, size_t I, void* stream) {
+    if (gate_up == nullptr || down == nullptr || x == nullptr || idx == nullptr || w == nullptr || gu == nullptr ||
+        y == nullptr)
+        return ERR_NULL;
+    if (T == 0 || k == 0 || E == 0 || H == 0 || I == 0 || k > (size_t)ROUTE_MAX_K || T * k > 65535 || H % 8 != 0 ||
+        I % 8 != 0 || H > (1u << 20) || I > (1u << 20) || E > (1u << 20))
+        return ERR_DOMAIN;
+    if (!al(gate_up, 16) || !al(down, 16) || !al(x, 16) || !al(gu, 16) || !al(idx, 4) || !al(w, 2) || !al(y, 2))
+        return ERR_DOMAIN;
+    const DeviceInfo& dev = device_info();
+    if (k * I * 2 > (size_t)dev.lds_bytes || H * 2 > (size_t)dev.lds_bytes) {
+        set_error("moe: the staged rows do not fit LDS");
+        return ERR_DOMAIN;
+    }
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int R1 = (int)(2 * I), C1 = (int)H, R2 = (int)H, C2 = (int)I;
+    int32_t rc;
+    switch (lanes_for(C1 / 8)) {
+        case 64: rc = launch_gate_up<64>(gate_up, x, idx, gu, R1, C1, (int)k, (int)E, (int)(T * k), st); break;
+        case 32: rc = launch_gate_up<32>(gate_up, x, idx, gu, R1, C1, (int)k, (int)E, (int)(T * k), st); break;
+        default: rc = launch_gate_up<16>(gate_up, x, idx, gu, R1, C1, (int)k, (int)E, (int)(T * k), st); break;
+    }
+    if (rc != OK) return rc;
+    switch (lanes_for(C2 / 8)) {
+        case 64: return launch_down<64>(down, gu, idx, w, y, R2, C2, (int)k, (int)E, (int)T, st);
+        case 32: return launch_down<32>(down, gu, idx, w, y, R2, C2, (int)k, (int)E, (int)T, st);
+        default: return launch_down<16>(down, gu, idx, w, y, R2, C2, (int)k, (int)E, (int)T, st);
+    }
+}
+
+}  // extern "C"

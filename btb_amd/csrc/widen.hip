@@ -24,11 +24,8 @@ __global__ void __launch_bounds__(256) p12_widen_kernel(FmtP12::Params p, size_t
         c.e0 = c.e1 = 0;
         // plain (cached) loads: the matvec's own stream is non-temporal, the bytes are the same
         FmtP12::Raw raw{c.lo[unit], c.hi4[unit]};
-        float w[FmtP12::UW];
-        FmtP12::widen(c, raw, 0, w);
-        uint32_t packed[8];
-#pragma unroll
-        for (int k = 0; k < 8; ++k) packed[k] = (f32_bits(w[2 * k]) >> 16) | (f32_bits(w[2 * k + 1]) & 0xFFFF0000u);
+        uint32_t packed[FmtP12::UW / 2];
+        FmtP12::widen(c, raw, 0, packed);
         uint4* o = reinterpret_cast<uint4*>(out) + unit * 2;
         o[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]);
         o[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
@@ -75,24 +72,23 @@ __global__ void __launch_bounds__(256) fp8_widen_kernel(FmtF8::Params p, int R, 
     const FmtF8::RowCtx c = FmtF8::row_ctx(p, r, units);
     const int blk = c.upb == 1 ? unit : (int)__umulhi((uint32_t)unit, c.magic);
     FmtF8::Raw raw{c.row[unit], c.srow[blk]};
-    float w[FmtF8::UW];
-    FmtF8::widen(c, raw, unit, w);
+    uint32_t packed[FmtF8::UW / 2];
+    FmtF8::widen(c, raw, unit, packed);
     if (OUT_F32) {
         float4* o = reinterpret_cast<float4*>(out) + t * 4;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) o[k] = make_float4(w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3]);
+        for (int k = 0; k < 4; ++k)
+            o[k] = make_float4(bf16lo_f32(packed[2 * k]), bf16hi_f32(packed[2 * k]), bf16lo_f32(packed[2 * k + 1]),
+                               bf16hi_f32(packed[2 * k + 1]));
     } else {
-        uint32_t packed[8];
-#pragma unroll
-        for (int k = 0; k < 8; ++k) packed[k] = (f32_bits(w[2 * k]) >> 16) | (f32_bits(w[2 * k + 1]) & 0xFFFF0000u);
         uint4* o = reinterpret_cast<uint4*>(out) + t * 2;
         o[0] = make_uint4(packed[0], packed[1], packed[2], packed[3]);
         o[1] = make_uint4(packed[4], packed[5], packed[6], packed[7]);
     }
 }
 
-// one thread a block of 32 weights. OUT_F32: the CPU matvec's weight fp4 * 2^(s - 127) as f32; else that value
-// rounded to bf16 (the reference card's btb_mx4_widen, exact wherever the product is a normal bf16). `seats` picks
+// one thread a block of 32 weights: fp4 * 2^(s - 127) as bf16 (the reference card's btb_mx4_widen; exact for every
+// scale below 255), or with OUT_F32 the same values as f32 (the CPU matvec's weight). `seats` picks
 // the stacks (experts) to widen, or is null for the identity.
 template <bool OUT_F32>
 __global__ void __launch_bounds__(256) mx4_widen_kernel(FmtMx4::Params p, const int32_t* __restrict__ seats,
@@ -103,17 +99,17 @@ __global__ void __launch_bounds__(256) mx4_widen_kernel(FmtMx4::Params p, const 
     const long long at = seat * groups + g;
     FmtMx4::RowCtx c{reinterpret_cast<const uint4*>(p.blocks), p.scales};
     FmtMx4::Raw raw{c.row[at], (uint32_t)c.srow[at]};
-    float w[FmtMx4::UW];
-    FmtMx4::widen(c, raw, 0, w);
+    uint32_t packed[FmtMx4::UW / 2];
+    FmtMx4::widen(c, raw, 0, packed);
+    FmtMx4::patch255(raw, packed);
     const long long o0 = (long long)blockIdx.y * groups + g;
     if (OUT_F32) {
         float4* o = reinterpret_cast<float4*>(out) + o0 * 8;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) o[k] = make_float4(w[4 * k], w[4 * k + 1], w[4 * k + 2], w[4 * k + 3]);
+        for (int k = 0; k < 8; ++k)
+            o[k] = make_float4(bf16lo_f32(packed[2 * k]), bf16hi_f32(packed[2 * k]), bf16lo_f32(packed[2 * k + 1]),
+                               bf16hi_f32(packed[2 * k + 1]));
     } else {
-        uint32_t packed[16];
-#pragma unroll
-        for (int k = 0; k < 16; ++k) packed[k] = (uint32_t)f32_bf16(w[2 * k]) | ((uint32_t)f32_bf16(w[2 * k + 1]) << 16);
         uint4* o = reinterpret_cast<uint4*>(out) + o0 * 4;
 #pragma unroll
         for (int k = 0; k < 4; ++k) o[k] = make_uint4(packed[4 * k], packed[4 * k + 1], packed[4 * k + 2], packed[4 * k + 3]);

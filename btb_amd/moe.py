@@ -1,0 +1,63 @@
+"""The routed MoE decode layer on the GPU: the counterparts of the reference's `Qwen4Router`
+(btb/engine/families/qwen4/router.py:21-51) and `_Experts` (btb/engine/host.py:310-1107, its arithmetic only: every
+expert is resident in VRAM here, so there is no store, no wave and no host round trip).
+
+    router = Router(card, w_router, top_k)           # w_router bf16 [E, H]
+    experts = Experts(card, gate_up, down)           # bf16 stacks [E, 2I, H], [E, H, I]
+    logits, weights, picks = router(x)               # x bf16 [T, H]
+    y = experts(x, picks, weights)                   # bf16 [T, H], summed in ascending expert order
+"""
+
+from __future__ import annotations
+
+from typing import Any
+
+import torch
+
+
+class Router:
+    """f32 logits by the host's own matvec order on the card (so the picks are the CPU path's, bit for bit), then the
+    card's softmax / top-k / renormalise. Returns (logits in x's dtype, weights in x's dtype, picks int32)."""
+
+    def __init__(self, card: Any, weight: torch.Tensor, top_k: int, norm_topk_prob: bool = True) -> None:
+        if weight.dtype != torch.bfloat16 or weight.dim() != 2 or not weight.is_cuda:
+            raise ValueError("[moe] the router's weight is a bf16 [E, H] matrix on the GPU")
+        if not norm_topk_prob:
+            raise ValueError("[moe] the card's router renormalises the picked weights (norm_topk_prob)")
+        self.card = card
+        self.weight = weight.contiguous()
+        self.top_k = int(top_k)
+        self.num_experts, self.hidden_dim = (int(s) for s in weight.shape)
+
+    def __call__(self, hidden_states: torch.Tensor):
+        x = hidden_states.reshape(-1, self.hidden_dim)
+        logits = self.card.gemv_lane16(self.weight, x.float().contiguous())
+        picks, weights, _ = self.card.moe_route(logits, self.top_k)
+        return logits.to(hidden_states.dtype), weights.to(hidden_states.dtype), picks
+
+
+class Experts:
+    """The layer's experts as two bf16 stacks on the GPU. `__call__(x, picks, weights)` is `_Experts.forward`'s
+    result: [T, H] in the rows' dtype (bf16), every pick's product times its weight, summed in ascending expert
+    order with each step rounded to bf16."""
+
+    def __init__(self, card: Any, gate_up: torch.Tensor, down: torch.Tensor) -> None:
+        E, I2, H = (int(s) for s in gate_up.shape)
+        if tuple(down.shape) != (E, H, I2 // 2):
+            raise ValueError(f"[moe] gate_up {tuple(gate_up.shape)} and down {tuple(down.shape)} are not one layer's")
+        self.card = card
+        self.gate_up = gate_up.contiguous()
+        self.down = down.contiguous()
+        self.num_experts, self.hidden_dim, self.intermediate_dim = E, H, I2 // 2
+        self._gu: torch.Tensor | None = None
+
+    def __call__(self, hidden_states: torch.Tensor, top_k_index: torch.Tensor, top_k_weights: torch.Tensor,
+                 out: torch.Tensor | None = None) -> torch.Tensor:
+        x = hidden_states.reshape(-1, self.hidden_dim)
+        if x.dtype != torch.bfloat16:
+            raise ValueError("[moe] the card's experts take bf16 rows")
+        T, k = (int(s) for s in top_k_index.shape)
+        if self._gu is None or self._gu.shape[0] < T or self._gu.shape[1] != k:
+            self._gu = torch.empty(T, k, 2 * self.intermediate_dim, dtype=torch.bfloat16, device=x.device)
+        return self.card.moe_experts(self.gate_up, self.down, x.contiguous(), top_k_index.to(torch.int32).contiguous(),
+                                     top_k_weights.to(torch.bfloat16).contiguous(), out, self._gu[:T])

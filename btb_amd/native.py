@@ -41,6 +41,15 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_fp8_widen": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _i32, _vp]),
     "btb_hip_gemv_mxfp4": (_i32, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_mx4_widen": (_i32, [_vp, _vp, _vp, _sz, ctypes.c_int64, _vp, _i32, _vp]),
+    "btb_hip_gemv_bf16_rows": (_i32, [_vp, _sz, _sz, _vp, _sz, _vp, _vp]),
+    "btb_hip_gemv_bf16_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "btb_hip_gemv_p12_rows": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _sz, _vp, _vp]),
+    "btb_hip_gemv_mxfp4_rows": (_i32, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp]),
+    "btb_hip_gemv_mxfp4_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "btb_hip_gemv_fp8_rows": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _vp]),
+    "btb_hip_gemv_fp8_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "btb_hip_moe_route": (_i32, [_vp, _i32, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp]),
+    "btb_hip_moe_experts_bf16": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _vp]),
 }
 
 
@@ -246,6 +255,92 @@ class HipCard:
             self._call("btb_hip_mx4_widen", self.ptr(blocks), self.ptr(scales), None if seats is None else self.ptr(seats),
                        n, groups, self.ptr(out), int(dtype == torch.float32), _stream())
         return out
+
+
+    # -- the host's bits on the card: f32 rows in, f32 rows out ------------------------------------------------------
+
+    def _rows_io(self, x: torch.Tensor, y: torch.Tensor | None, R: int, C: int, what: str):
+        self._need(x, torch.float32, "x")
+        x2 = x.reshape(-1, C)
+        b = int(x2.shape[0])
+        if y is None:
+            y = torch.empty(b, R, dtype=torch.float32, device=x.device)
+        else:
+            self._need(y, torch.float32, "y")
+            if y.numel() != b * R:
+                raise ValueError(f"[hip] {what}: y holds {y.numel()} elements, the product has {b * R}")
+        return x2, b, y
+
+    def gemv_lane16(self, w: torch.Tensor, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
+        """the host's bf16 x f32 matvec to the bit (the reference's `_Cuda.gemv_lane16`, btb/engine/native.py:2342-2365):
+        w bf16 [R, C], x f32 [n, C] -> f32 [n, R]"""
+        self._need(w, torch.bfloat16, "w")
+        R, C = (int(s) for s in w.shape)
+        x2, b, y = self._rows_io(x, y, R, C, "gemv_lane16")
+        self._call("btb_hip_gemv_bf16_rows", self.ptr(w), R, C, self.ptr(x2), b, self.ptr(y), _stream())
+        return y
+
+    def gemv_lane16_p12(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
+        R, C = w.shape
+        x2, b, y = self._rows_io(x, y, R, C, "gemv_lane16_p12")
+        ne = int(w.esc_idx.numel())
+        self._call("btb_hip_gemv_p12_rows", self.ptr(w.lo), self.ptr(w.hi4), self.ptr(w.table),
+                   self.ptr(w.esc_idx) if ne else None, self.ptr(w.esc_val) if ne else None, ne, R, C, self.ptr(x2), b,
+                   self.ptr(y), _stream())
+        return y
+
+    def gemv_lane16_mx4(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
+        """the host's MXFP4 matvec to the bit (`_Cuda.gemv_lane16_mx4`, btb/engine/native.py:2367-2390)"""
+        R, C = w.shape
+        x2, b, y = self._rows_io(x, y, R, C, "gemv_lane16_mx4")
+        self._call("btb_hip_gemv_mxfp4_rows", self.ptr(w.blocks), self.ptr(w.scales), R, C, self.ptr(x2), b, self.ptr(y),
+                   _stream())
+        return y
+
+    def gemv_lane16_fp8(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
+        R, C = w.shape
+        sr, sc = w.grid
+        x2, b, y = self._rows_io(x, y, R, C, "gemv_lane16_fp8")
+        self._call("btb_hip_gemv_fp8_rows", self.ptr(w.w), self.ptr(w.scales), R, C, sr, sc, self.ptr(x2), b, self.ptr(y),
+                   _stream())
+        return y
+
+    # -- routed experts -----------------------------------------------------------------------------------------
+
+    def moe_route(self, logits: torch.Tensor, k: int, E: int | None = None):
+        """(idx int32 [T, k], weights bf16 [T, k], weights f32 [T, k]) of logits [T, ls] (bf16 or f32): softmax over
+        the first E, top k by (p descending, index ascending), renormalised (`btb_moe_route`)"""
+        if logits.dtype not in (torch.bfloat16, torch.float32) or not logits.is_cuda or logits.dim() != 2 \
+                or logits.stride(1) != 1:
+            raise ValueError("[hip] moe_route: logits must be a [T, ls] bf16 or f32 tensor on the GPU, rows contiguous")
+        T, ls = int(logits.shape[0]), int(logits.stride(0))
+        E = int(logits.shape[1]) if E is None else int(E)
+        idx = torch.empty(T, k, dtype=torch.int32, device=logits.device)
+        w = torch.empty(T, k, dtype=torch.bfloat16, device=logits.device)
+        w32 = torch.empty(T, k, dtype=torch.float32, device=logits.device)
+        self._call("btb_hip_moe_route", self.ptr(logits), int(logits.dtype == torch.float32), ls, E, k, T, self.ptr(idx),
+                   self.ptr(w), self.ptr(w32), _stream())
+        return idx, w, w32
+
+    def moe_experts(self, gate_up: torch.Tensor, down: torch.Tensor, x: torch.Tensor, idx: torch.Tensor,
+                    w: torch.Tensor, y: torch.Tensor | None = None, gu: torch.Tensor | None = None) -> torch.Tensor:
+        """y [T, H]: the routed experts of x [T, H] over the stacks gate_up [E, 2I, H] and down [E, H, I] (bf16),
+        picks idx int32 [T, k] and weights w bf16 [T, k], summed in ascending expert order"""
+        for t, what in ((gate_up, "gate_up"), (down, "down"), (x, "x"), (w, "w")):
+            self._need(t, torch.bfloat16, what)
+        self._need(idx, torch.int32, "idx")
+        E, I2, H = (int(s) for s in gate_up.shape)
+        if tuple(down.shape) != (E, H, I2 // 2) or x.shape[-1] != H or idx.shape != w.shape:
+            raise ValueError(f"[hip] moe_experts: gate_up {tuple(gate_up.shape)}, down {tuple(down.shape)}, x "
+                             f"{tuple(x.shape)}, idx {tuple(idx.shape)}, w {tuple(w.shape)} do not fit together")
+        T, k = (int(s) for s in idx.shape)
+        if gu is None:
+            gu = torch.empty(T, k, I2, dtype=torch.bfloat16, device=x.device)
+        if y is None:
+            y = torch.empty(T, H, dtype=torch.bfloat16, device=x.device)
+        self._call("btb_hip_moe_experts_bf16", self.ptr(gate_up), self.ptr(down), self.ptr(x), self.ptr(idx), self.ptr(w),
+                   self.ptr(gu), self.ptr(y), T, k, E, H, I2 // 2, _stream())
+        return y
 
 
 class Native:

@@ -109,6 +109,59 @@ int32_t btb_hip_gemv_mxfp4(const void* blocks, const void* scales, const void* x
 int32_t btb_hip_mx4_widen(const void* blocks, const void* scales, const void* seats, size_t n_seats, int64_t groups,
                           void* out, int32_t out_f32, void* stream);
 
+/* ---- the crate's CPU entry points on the device: f32 x and y, the host's bits ------------------------------ */
+
+/* y[i][r] = sum_c bf16(w[r][c]) * x[i][c] in f32, in the host's order (16 lane sums, lane j the columns = j mod 16,
+ * the pairwise fold): bit-identical to btb_gemv_bf16_rows on the CPU (native/src/lib.rs:69-80) for every b. w
+ * [rows, cols] bf16 bit patterns, x [b, cols] f32, y [b, rows] f32, all on the device; `threads` is replaced by the
+ * stream. Also the reference card's btb_gemv_lane16_f32_m* (native/cuda/btb_kernels.cu:1635-1699). */
+int32_t btb_hip_gemv_bf16_rows(const uint16_t* w, size_t rows, size_t cols, const float* x, size_t b, float* y,
+                               void* stream);
+
+/* n independent tasks (native/src/lib.rs:91-104): the arrays of pointers and sizes are host arrays, what they point
+ * to is on the device. Every task is checked before the first is launched. */
+int32_t btb_hip_gemv_bf16_group(size_t n, const uint16_t* const* w, const size_t* rows, const size_t* cols,
+                                const float* const* x, const size_t* b, float* const* y, void* stream);
+
+/* btb_gemv_p12_rows (native/src/lib.rs:114-135) on the device, bit-identical to it and so to the bf16 form. The
+ * escape list's ascending order is not re-checked here (that would copy it back to the host). */
+int32_t btb_hip_gemv_p12_rows(const uint8_t* lo, const uint8_t* hi4, const uint8_t* table, const int32_t* esc_idx,
+                              const uint8_t* esc_val, size_t n_esc, size_t rows, size_t cols, const float* x, size_t b,
+                              float* y, void* stream);
+
+/* btb_gemv_mxfp4_rows / _group (native/src/lib.rs:147-160, 193-209) on the device, bit-identical to them; the
+ * reference card's btb_gemv_lane16_mx4_f32_m* (native/cuda/btb_kernels.cu:1701-1766). */
+int32_t btb_hip_gemv_mxfp4_rows(const uint8_t* blocks, const uint8_t* scales, size_t rows, size_t cols, const float* x,
+                                size_t b, float* y, void* stream);
+int32_t btb_hip_gemv_mxfp4_group(size_t n, const uint8_t* const* blocks, const uint8_t* const* scales,
+                                 const size_t* rows, const size_t* cols, const float* const* x, const size_t* b,
+                                 float* const* y, void* stream);
+
+/* btb_gemv_fp8_rows / _group (native/src/lib.rs:511-552) on the device, bit-identical to them. */
+int32_t btb_hip_gemv_fp8_rows(const uint8_t* w, const float* scales, size_t rows, size_t cols, size_t sr, size_t sc,
+                              const float* x, size_t b, float* y, void* stream);
+int32_t btb_hip_gemv_fp8_group(size_t n, const uint8_t* const* w, const float* const* scales, const size_t* rows,
+                               const size_t* cols, const size_t* sr, const size_t* sc, const float* const* x,
+                               const size_t* b, float* const* y, void* stream);
+
+/* ---- routed experts ---------------------------------------------------------------------------------------- */
+
+/* Per row t of logits [T, ls] (bf16, or f32 when logits_f32 != 0): f32 softmax over the first E, the top k in the
+ * total order (p descending, index ascending), weights p / sum(top k) summed in rank order. idx i32 [T, k], w bf16
+ * [T, k], and the unrounded weights into w32 f32 [T, k] when it is not NULL. k <= 32. Replaces the kernel
+ * btb_moe_route (native/cuda/btb_kernels.cu:861-948; its host-publish arguments have no use with experts resident
+ * in VRAM) and the softmax / topk / renormalise of Qwen4Router.forward (btb/engine/families/qwen4/router.py:43-51). */
+int32_t btb_hip_moe_route(const void* logits, int32_t logits_f32, size_t ls, size_t E, size_t k, size_t T, int32_t* idx,
+                          void* w, float* w32, void* stream);
+
+/* The routed experts of T rows: gate_up [E, 2I, H] and down [E, H, I] bf16 stacks (gate rows then up rows), x [T, H]
+ * bf16, the picks idx [T, k] and weights w bf16 [T, k] of btb_hip_moe_route, gu [T, k, 2I] bf16 scratch the caller
+ * owns, y [T, H] bf16. Per pick: gu = bf16(W_gu x), h = bf16(bf16(silu(g)) * u), d = bf16(W_dn h); per row
+ * y = sum over the picks in ASCENDING expert id of bf16(d * w), each addition rounded to bf16: the arithmetic of
+ * _Experts._one_row / _loop (btb/engine/host.py:508-569, 906-967). T * k <= 65535. */
+int32_t btb_hip_moe_experts_bf16(const void* gate_up, const void* down, const void* x, const int32_t* idx, const void* w,
+                                 void* gu, void* y, size_t T, size_t k, size_t E, size_t H, size_t I, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

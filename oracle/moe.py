@@ -1,0 +1,73 @@
+"""TEST INFRASTRUCTURE - the routed MoE layer as the reference's CPU path computes it, in numpy over the oracle's C
+matvec. Follows:
+
+  router     btb/engine/families/qwen4/router.py:43-51: logits = W_r x (f32, the host matvec), f32 softmax over all
+             experts, top k (torch.topk: value descending; on equal values the lower index, the rule the card's
+             kernel states at native/cuda/btb_kernels.cu:848-851), weights / their sum, cast to the rows' dtype
+  experts    btb/engine/host.py:508-569 (one row) and :906-967 (several): per selected expert gu = W_gu x (f32) ->
+             rows' dtype -> silu(gate) * up on the two halves (host.py:439-441) -> f32 -> W_dn h (f32) -> rows' dtype
+             -> times the pick's weight -> summed into the row in ASCENDING expert order, every step in the rows'
+             dtype
+
+`dt` is the rows' dtype: "bf16" (the engine running bf16 rows, what the GPU path computes) or "f32".
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+import oracle
+from oracle import codecs
+
+
+def _as(dt: str, a: np.ndarray) -> np.ndarray:
+    a = np.asarray(a, dtype=np.float32)
+    return codecs.round_bf16(a) if dt == "bf16" else a
+
+
+def router(w_router_bits: np.ndarray, x: np.ndarray, k: int, dt: str = "bf16", norm_topk: bool = True):
+    """x [T, H] (values of the rows' dtype, as f32) -> (logits f32 [T, E], weights [T, k] in dt, experts int64 [T, k])"""
+    logits = oracle.gemv_bf16(w_router_bits, np.asarray(x, np.float32), threads=0)
+    m = logits.max(axis=-1, keepdims=True)
+    e = np.exp((logits - m).astype(np.float32)).astype(np.float32)
+    probs = (e / e.sum(axis=-1, keepdims=True, dtype=np.float32)).astype(np.float32)
+    # value descending, index ascending on ties: a stable sort of the negated values
+    order = np.argsort(-probs, axis=-1, kind="stable")[:, :k]
+    top = np.take_along_axis(probs, order, axis=-1)
+    if norm_topk:
+        s = np.zeros(top.shape[0], np.float32)
+        for j in range(k):
+            s = (s + top[:, j]).astype(np.float32)
+        top = (top / s[:, None]).astype(np.float32)
+    return logits, _as(dt, top), order.astype(np.int64)
+
+
+def silu(g: np.ndarray) -> np.ndarray:
+    g = np.asarray(g, np.float32)
+    return (g / (np.float32(1.0) + np.exp(-g).astype(np.float32))).astype(np.float32)
+
+
+def experts(gate_up_bits: np.ndarray, down_bits: np.ndarray, x: np.ndarray, picks: np.ndarray, weights: np.ndarray,
+            dt: str = "bf16") -> np.ndarray:
+    """gate_up [E, 2I, H] and down [E, H, I] as bf16 bit patterns, x [T, H], picks [T, k], weights [T, k] (values of
+    dt) -> [T, H] in dt"""
+    x = np.asarray(x, np.float32)
+    T, H = x.shape
+    I = down_bits.shape[2]
+    final = np.zeros((T, H), np.float32)
+    for e in sorted(set(int(v) for v in picks.reshape(-1))):
+        tok, pos = np.nonzero(picks == e)
+        cur = x[tok]
+        gu = _as(dt, oracle.gemv_bf16(gate_up_bits[e], cur, threads=0))
+        act = _as(dt, silu(gu[:, :I]))            # the activation is one op in the rows' dtype ...
+        h = _as(dt, act * gu[:, I:])               # ... and the product another
+        d = _as(dt, oracle.gemv_bf16(down_bits[e], h, threads=0))
+        contrib = _as(dt, d * np.asarray(weights, np.float32)[tok, pos, None])
+        for i, t in enumerate(tok):                # index_add_ in ascending expert order, each add in dt
+            final[t] = _as(dt, final[t] + contrib[i])
+    return final
+
+
+def layer(w_router_bits, gate_up_bits, down_bits, x, k: int, dt: str = "bf16"):
+    logits, w, picks = router(w_router_bits, x, k, dt)
+    return experts(gate_up_bits, down_bits, x, picks, w, dt), logits, w, picks

@@ -1,0 +1,90 @@
+"""The routed MoE decode layer on the GPU (Qwen3-30B-A3B shape: hidden 2048, 128 experts, top-8, intermediate 768)
+against the CPU path restated in oracle/moe.py, on the same seeded inputs.
+
+Bars (BASELINE.json north_star): the top-k picks, as ordered lists, are bit-exact; the router's f32 logits are
+bit-exact (they are made in the CPU's order); the routing weights agree to one bf16 ulp (the two sides' expf may
+differ in the last bit); the layer output agrees within max relative error 1e-2 of the largest output (bf16 rows; the
+expert matvecs accumulate in f32 in a different order than the CPU's, which can flip a bf16 rounding of gu, h or d)."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from btb_amd.moe import Experts, Router
+from oracle import codecs
+from oracle import moe as omoe
+
+from .helpers import acts_bf16, bits16, f32_bits, gen, weights_bf16
+
+pytestmark = pytest.mark.gpu
+
+E, K, H, I = 128, 8, 2048, 768
+
+
+@pytest.fixture(scope="module")
+def layer_weights():
+    g = gen(500)
+    wr = (torch.randn(E, H, generator=g) * 0.02).to(torch.bfloat16)
+    gu = (torch.randn(E, 2 * I, H, generator=g) * 0.02).to(torch.bfloat16)
+    dn = (torch.randn(E, H, I, generator=g) * 0.02).to(torch.bfloat16)
+    return wr, gu, dn
+
+
+@pytest.mark.parametrize("T", [1, 4, 8])
+def test_moe_layer_matches_cpu_path(card, layer_weights, T):
+    wr, gu, dn = layer_weights
+    x = acts_bf16(T, H, seed=510 + T)
+    router = Router(card, wr.cuda(), K)
+    experts = Experts(card, gu.cuda(), dn.cuda())
+    logits, weights, picks = router(x.cuda())
+    y = experts(x.cuda(), picks, weights)
+    torch.cuda.synchronize()
+
+    want, ologits, ow, opicks = omoe.layer(bits16(wr), bits16(gu), bits16(dn), x.float().numpy(), K, "bf16")
+    raw = card.gemv_lane16(wr.cuda(), x.float().cuda()).cpu().numpy()
+    assert np.array_equal(f32_bits(raw), f32_bits(ologits))                       # logits: the CPU's bits
+    assert np.array_equal(picks.cpu().numpy().astype(np.int64), opicks)           # picks: bit-exact, in rank order
+    dw = np.abs(weights.float().cpu().numpy() - ow)
+    assert np.all(dw <= np.abs(ow) * 2.0**-7)                                     # weights: within a bf16 ulp
+    got = y.float().cpu().numpy()
+    err = np.abs(got - want).max() / np.abs(want).max()
+    assert err <= 1e-2, err
+
+
+def test_experts_with_the_cpu_picks(card, layer_weights):
+    """the expert stage on its own, fed the oracle's picks and weights: only the matvecs' summation order differs"""
+    wr, gu, dn = layer_weights
+    T = 4
+    x = acts_bf16(T, H, seed=520)
+    _, ow, opicks = omoe.router(bits16(wr), x.float().numpy(), K, "bf16")
+    want = omoe.experts(bits16(gu), bits16(dn), x.float().numpy(), opicks, ow, "bf16")
+    experts = Experts(card, gu.cuda(), dn.cuda())
+    y = experts(x.cuda(), torch.from_numpy(opicks).to(torch.int32).cuda(),
+                torch.from_numpy(ow).to(torch.bfloat16).cuda())
+    got = y.float().cpu().numpy()
+    assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max()
+
+
+def test_route_tie_rule_and_bf16_logits(card):
+    """equal logits: the lower index wins (native/cuda/btb_kernels.cu:848-851, 900, 912); bf16 logits as the
+    reference's kernel takes them"""
+    logits = torch.zeros(2, 16)
+    logits[0, [3, 7, 11]] = 2.0      # three equal maxima, then thirteen equal zeros
+    logits[1] = torch.arange(16, 0, -1).float()
+    idx, w, w32 = card.moe_route(logits.cuda(), 5)
+    assert idx[0].tolist() == [3, 7, 11, 0, 1]
+    assert idx[1].tolist() == [0, 1, 2, 3, 4]
+    assert abs(float(w32[0].sum()) - 1.0) < 1e-6
+    idxb, wb, _ = card.moe_route(logits.to(torch.bfloat16).cuda(), 5)
+    assert torch.equal(idxb, idx) and torch.equal(wb, w)
+    # torch's own routing on distinct values agrees
+    g = torch.randn(6, 128, generator=gen(530))
+    p = torch.softmax(g, dim=-1)
+    top, ids = torch.topk(p, 8, dim=-1)
+    idx, w, w32 = card.moe_route(g.cuda(), 8)
+    assert torch.equal(idx.cpu().long(), ids)
+    assert torch.allclose(w32.cpu(), top / top.sum(-1, keepdim=True), rtol=1e-5, atol=0)
+    with pytest.raises(Exception):
+        card.moe_route(g.cuda(), 33)
