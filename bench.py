@@ -1,0 +1,192 @@
+"""Benchmark of the decode hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode|decode_p12] [--no-cpu]
+
+A step is one decode step of a random-init Qwen3-4B-shaped dense stack (36 layers, hidden 2560, 32 query / 8 kv heads
+of 128, SwiGLU 9728, vocab 151936; weights ~N(0, 0.02) in bf16, seeded N(0, 1) K/V for a 4096-token context), M = 1
+token, replayed as one captured hipGraph with every operand already resident in HBM. It prints ONE JSON line:
+`value` is the step's HBM stream in GB/s - the linear weights plus the K/V rows one step reads, divided by the step's
+time - next to tokens/s and the fraction of the 8 TB/s HBM3E peak; `roofline` prices the dominant kernel (the bf16
+streaming matvec at the qkv / gate_up / head shapes) from its own timed region, measured with device events on the
+launch stream; `cpu_baseline` times the CPU oracle's AVX-512 / AVX2 matvec (a port of the reference's CPU path) on the
+host's cores over a bounded sample of the same matrices.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+CTX = 4096
+METRIC = "decode GEMV HBM GB/s (% of peak) + decode tok/s, Qwen3-4B-shape bf16 M=1"
+
+
+def cpu_baseline(budget_s: float = 12.0) -> dict:
+    """the oracle's bf16 matvec (the reference's CPU arithmetic, ported) over gate_up-shaped matrices drawn from a
+    pool larger than 4x the last-level cache, every core, for about `budget_s` seconds"""
+    import numpy as np
+
+    import oracle
+
+    R, C = 19456, 2560
+    rng = np.random.default_rng(0x0B7B)
+    pool = [rng.integers(0x3A00, 0x3D00, (R, C), dtype=np.uint16) for _ in range(12)]  # 1.2 GB of bf16 patterns
+    x = rng.standard_normal((1, C)).astype(np.float32)
+    cores = os.cpu_count() or 1
+    oracle.gemv_bf16(pool[0], x, threads=0)
+    t0 = time.perf_counter()
+    calls = 0
+    while time.perf_counter() - t0 < budget_s:
+        oracle.gemv_bf16(pool[calls % len(pool)], x, threads=0)
+        calls += 1
+    dt = time.perf_counter() - t0
+    gbs = calls * (R * C * 2 + C * 4 + R * 4) / dt / 1e9
+    return {"value": round(gbs, 2), "unit": "GB/s", "cores": cores, "kind": "port", "isa": oracle.isa(),
+            "sample": f"{calls} bf16 matvecs [{R}x{C}] (the gate_up shape), 12 distinct matrices (1.2 GB) in rotation, "
+                      f"f32 x and y, all {cores} host threads, {dt:.1f} s"}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--workload", default="decode", choices=["decode", "decode_p12"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
+        return 2
+    if args.steps < 1 or args.warmup < 0 or args.steps + args.warmup > 480:
+        print("bench.py: steps + warmup must stay within the cache's 480 spare rows", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from btb_amd.decode import QWEN3_4B, DecodeStep, random_stack
+    from btb_amd.native import Native
+
+    card = Native.card_kernels()  # raises where the HIP library or the GPU is missing: there is no fallback
+    cfg = QWEN3_4B
+    packed = args.workload == "decode_p12"
+    weights = random_stack(card, cfg, packed=packed)
+    cap = CTX + 512
+    step = DecodeStep(card, cfg, weights, cap)
+    g = torch.Generator(device="cuda").manual_seed(0x0B7B0200)
+    for i in range(cfg.layers):  # seeded K/V ~ N(0, 1) for the context
+        step.kv[i, :, :, :CTX].copy_(torch.randn(2, cfg.kv_heads, CTX, cfg.head_dim, generator=g, device="cuda"))
+    step.reset(CTX, 0)
+    step.capture(warmup=2)
+    step.reset(CTX, 0)
+
+    stream = torch.cuda.current_stream()
+    for _ in range(args.warmup):
+        step.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    t0 = time.perf_counter()
+    e0.record(stream)
+    for _ in range(args.steps):
+        step.replay()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    wall = time.perf_counter() - t0
+    ms = e0.elapsed_time(e1) / args.steps
+    n_keys = CTX + args.warmup + (args.steps + 1) / 2.0  # the average context over the timed steps
+    wbytes, kvbytes = step.weight_bytes(), step.kv_bytes(int(n_keys))
+    gbs = (wbytes + kvbytes) / (ms * 1e-3) / 1e9
+
+    # -- the dominant kernel in a timed region of its own: the streaming matvec at the qkv, gate_up and head shapes
+    #    (5.5 of the step's 8.0 GB of bf16 weights), over the model's own matrices, so nothing repeats from cache
+    x = torch.randn(1, cfg.hidden, device="cuda").to(torch.bfloat16)
+    outs = {n: torch.empty(1, r, dtype=torch.bfloat16, device="cuda")
+            for n, r in (("qkv", cfg.qkv_rows), ("gu", 2 * cfg.intermediate), ("head", cfg.vocab))}
+
+    def dominant() -> tuple[int, int]:
+        launches = nbytes = 0
+        for i in range(cfg.layers):
+            for n in ("qkv", "gu"):
+                lin = weights[f"layers.{i}.{n}"]
+                lin.matvec(x, outs[n])
+                launches += 1
+                nbytes += lin.nbytes + cfg.hidden * 2 + lin.shape[0] * 2
+        weights["head"].matvec(x, outs["head"])
+        return launches + 1, nbytes + weights["head"].nbytes + cfg.hidden * 2 + cfg.vocab * 2
+
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        launches, dom_bytes = dominant()
+    torch.cuda.synchronize()
+    gd = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(gd):
+        dominant()
+    gd.replay()
+    torch.cuda.synchronize()
+    reps = 10
+    d0, d1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    d0.record(stream)
+    for _ in range(reps):
+        gd.replay()
+    d1.record(stream)
+    torch.cuda.synchronize()
+    dom_us = d0.elapsed_time(d1) * 1e3 / (reps * launches)
+    achieved = dom_bytes / launches / (dom_us * 1e-6) / 1e9
+    traffic = None
+    tpath = os.path.join(ROOT, "profiles", "traffic.json")
+    if os.path.exists(tpath):
+        with open(tpath) as f:
+            traffic = json.load(f).get(args.workload)
+
+    line = {
+        "metric": METRIC,
+        "value": round(gbs, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16 weights and activations, f32 accumulate" if not packed else
+                 "pack12 weights widened to bf16 in registers, f32 accumulate",
+        "data": "synthetic: random-init N(0, 0.02) weights, seeded N(0, 1) K/V",
+        "tokens_per_s": round(1e3 / ms, 1),
+        "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
+        "config": {
+            "workload": ("configs[1]: full decode step of a Qwen3-4B-shaped dense stack, M=1, ctx 4096, one hipGraph"
+                         if not packed else
+                         "configs[2]: the same stack with every linear in pack12, widened in registers"),
+            "layers": cfg.layers, "hidden": cfg.hidden, "q_heads": cfg.q_heads, "kv_heads": cfg.kv_heads,
+            "head_dim": cfg.head_dim, "intermediate": cfg.intermediate, "vocab": cfg.vocab, "context": CTX,
+            "weight_bytes_per_step": wbytes, "kv_bytes_per_step": kvbytes, "kernels_per_step": 2 + 8 * cfg.layers + 4,
+            "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
+        },
+        "roofline": {
+            "kernel": "gemv_stream (streaming matvec, M=1) at the qkv / gate_up / head shapes",
+            "bound": "hbm",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBS, 4),
+            "traffic": traffic,
+            "launches": launches,
+            "avg_launch_us": round(dom_us, 3),
+            "bytes_per_launch": int(dom_bytes / launches),
+        },
+        "cpu_baseline": None if args.no_cpu else cpu_baseline(),
+    }
+    print(json.dumps(line))
+    return 0
+
+
+if __name__ == "__main__":
+    raise SystemExit(main())

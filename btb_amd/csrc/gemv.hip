@@ -185,6 +185,9 @@ static int32_t run_rows(const typename F::Params& p, const void* x, void* y, siz
     return OK;
 }
 
+// the matrix-core form of the bf16 matvec (gemv_mfma.hip)
+int32_t gemv_mfma_bf16(const void* w, const void* x, void* y, int R, int C, int M, hipStream_t st);
+
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 static int32_t check_dims(size_t R, size_t C, size_t M, size_t uw) {
@@ -204,6 +207,17 @@ int32_t btb_hip_gemv_bf16(const void* w, const void* x, void* y, size_t R, size_
     int32_t rc = check_dims(R, C, M, FmtBf16::UW);
     if (rc != OK) return rc;
     if (!aligned16(w) || !aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 1u)) return ERR_DOMAIN;
+    // the verify widths go to the matrix cores, 32 rows of x a pass; narrower passes stay on the vector ALUs
+    if (M >= 8 && C % 32 == 0 && tuning("gemv_no_mfma") <= 0) {
+        const uint16_t* xp = static_cast<const uint16_t*>(x);
+        uint16_t* yp = static_cast<uint16_t*>(y);
+        for (size_t m0 = 0; m0 < M; m0 += 32) {
+            const int mm = (int)(M - m0 < 32 ? M - m0 : 32);
+            rc = gemv_mfma_bf16(w, xp + m0 * C, yp + m0 * R, (int)R, (int)C, mm, static_cast<hipStream_t>(stream));
+            if (rc != OK) return rc;
+        }
+        return OK;
+    }
     FmtBf16::Params p{static_cast<const uint4*>(w)};
     return run_rows<FmtBf16, X_PLAIN>(p, x, y, R, C, M, C, static_cast<hipStream_t>(stream));
 }

@@ -1,0 +1,449 @@
+// The decode step's kernels between the matvecs, each rounding to bf16 exactly where the reference's card kernels
+// do (native/cuda/btb_kernels.cu:250-423, 448-488; the attention's contract: native/cuda/btb_attn_flash.cuh):
+//
+//   embed           h[t] = table[ids[t]]
+//   add_rmsnorm     h = bf16(h + y); x = bf16(h * rsqrt(mean(h^2) + eps) * w)            (or * (1 + w))
+//   norm_rope_kv    q/k RMSNorm per head, rope, the row written into the K/V cache at its slot, q out
+//   attn_decode     softmax(q K^T * scale) V over the cached keys, split over the keys, last arriver folds
+//   silu_mul        m = bf16(bf16(silu(g)) * u) over a [T, 2I] block
+//   argmax          the largest logit's index, the lowest on ties (native/src/sample.rs:53-67)
+//   publish         token, clock and cache length into pinned host memory at the graph's end; the step's own
+//                   bookkeeping (the next token id, the cache length + 1) stays on the device
+//
+// Every reduction runs in an order fixed by the element's index alone, so a replayed graph repeats its bits.
+
+#include "btb_common.hpp"
+#include "btb_tuning.hpp"
+
+#include "../../include/btb_hip.h"
+
+namespace btb {
+
+// sum over a 256-thread block in a fixed order: each wave's DPP tree, then waves 0..3 in order
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+    v = group_sum<64>(v);
+    const int wv = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[wv] = v;
+    __syncthreads();
+    const float s = ((red[0] + red[1]) + red[2]) + red[3];
+    __syncthreads();
+    return s;
+}
+
+__global__ void __launch_bounds__(256) embed_kernel(const uint4* __restrict__ table, const int32_t* __restrict__ ids,
+                                                    uint4* __restrict__ h, int H8, int vocab) {
+    const int t = blockIdx.x;
+    int id = ids[t];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    for (int i = threadIdx.x; i < H8; i += 256) h[(size_t)t * H8 + i] = table[(size_t)id * H8 + i];
+}
+
+__global__ void __launch_bounds__(256) add_rmsnorm_kernel(uint16_t* __restrict__ h, const uint16_t* __restrict__ y,
+                                                          const uint16_t* __restrict__ w, float eps,
+                                                          uint16_t* __restrict__ x, int H, int centered) {
+    __shared__ float red[4];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    uint16_t* hr = h + (size_t)t * H;
+    const uint16_t* yr = y == nullptr ? nullptr : y + (size_t)t * H;
+    uint16_t* xr = x + (size_t)t * H;
+    float ss = 0.f;
+    for (int i = tid; i < H; i += 256) {
+        float hv = bf16_f32(hr[i]);
+        if (yr != nullptr) {
+            hv = bfround(hv + bf16_f32(yr[i]));
+            hr[i] = f32_bf16(hv);
+        }
+        ss = fmaf(hv, hv, ss);
+    }
+    const float rstd = rsqrtf(block_sum256(ss, red) / (float)H + eps);
+    for (int i = tid; i < H; i += 256) {
+        const float wv = bf16_f32(w[i]);
+        xr[i] = f32_bf16(bf16_f32(hr[i]) * rstd * (centered ? 1.f + wv : wv));
+    }
+}
+
+// one wave per (head, row): a lane holds D / 64 consecutive dims; the rotated half is D / 2 dims away, lane ^ 32
+template <int D>
+__global__ void __launch_bounds__(64) norm_rope_kv_kernel(const uint16_t* __restrict__ qkv, const uint16_t* __restrict__ wq,
+                                                          const uint16_t* __restrict__ wk, float eps,
+                                                          const uint16_t* __restrict__ cos_t,
+                                                          const uint16_t* __restrict__ sin_t, const int32_t* __restrict__ n0p,
+                                                          const int32_t* __restrict__ depth, uint16_t* __restrict__ K,
+                                                          uint16_t* __restrict__ V, uint16_t* __restrict__ qo, int Hq,
+                                                          int Hk, long long hs, long long rs, int centered) {
+    constexpr int E = D / 64;
+    const int head = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
+    const int n0 = *n0p;
+    const int slot = n0 + t;
+    const int pos = n0 + (depth != nullptr ? depth[t] : t);
+    const int width = (Hq + 2 * Hk) * D;
+    const uint16_t* src = qkv + (size_t)t * width + (size_t)head * D + lane * E;
+    if (head >= Hq + Hk) {
+        uint16_t* dst = V + (size_t)(head - Hq - Hk) * hs + (size_t)slot * rs + lane * E;
+#pragma unroll
+        for (int e = 0; e < E; ++e) dst[e] = src[e];
+        return;
+    }
+    const bool is_q = head < Hq;
+    const uint16_t* wn = is_q ? wq : wk;
+    float v[E];
+#pragma unroll
+    for (int e = 0; e < E; ++e) v[e] = bf16_f32(src[e]);
+    if (wn != nullptr) {
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < E; ++e) ss = fmaf(v[e], v[e], ss);
+        ss = group_sum<64>(ss);
+        const float rstd = rsqrtf(ss / (float)D + eps);
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            const float wv = bf16_f32(wn[lane * E + e]);
+            v[e] = bfround(v[e] * rstd * (centered ? 1.f + wv : wv));
+        }
+    }
+    // rope: out = bf16(fma(rot, sin, bf16(v * cos))), rot = -v[i + D/2] in the first half, v[i - D/2] in the second
+    const uint16_t* cp = cos_t + (size_t)pos * D + lane * E;
+    const uint16_t* sp = sin_t + (size_t)pos * D + lane * E;
+    const float sgn = lane < 32 ? -1.f : 1.f;
+    uint16_t* dst = is_q ? (qo + ((size_t)t * Hq + head) * D + lane * E)
+                         : (K + (size_t)(head - Hq) * hs + (size_t)slot * rs + lane * E);
+#pragma unroll
+    for (int e = 0; e < E; ++e) {
+        const float rot = __shfl_xor(v[e], 32, WAVE);
+        const float qc = bfround(v[e] * bf16_f32(cp[e]));
+        dst[e] = f32_bf16(fmaf(sgn * rot, bf16_f32(sp[e]), qc));
+    }
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// decode attention, D = 128. A workgroup takes one kv head and one span of the keys; its four waves take the span's
+// keys four at a time (16 lanes a key, 8 dims a lane: a wave's load covers four whole 256-byte rows). Each 16-lane
+// group keeps an online-softmax state (max, sum, 8 output dims) for each of the G query heads over its own keys, in
+// log2 units (the scale carries log2 e, exp is exp2). The groups' states fold through LDS in a fixed order, the
+// spans' through memory: every workgroup writes its state, and the last to arrive for a (row, kv head) folds the
+// spans in span order, writes bf16(O / L) and resets the arrival count, so the graph replays. G <= 8.
+// ------------------------------------------------------------------------------------------------------------
+constexpr int ATT_D = 128;
+constexpr int ATT_MAXG = 8;
+
+// a value another workgroup wrote in this launch: read at device scope, past this CU's vector cache
+__device__ __forceinline__ float peek(const float* p) {
+    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <int G>
+__global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ K,
+                                                          const uint16_t* __restrict__ V, uint16_t* __restrict__ att,
+                                                          const int32_t* __restrict__ n0p, int Hq, int Hk, long long hs,
+                                                          long long rs, float scale_log2, float* __restrict__ part_m,
+                                                          float* __restrict__ part_l, float* __restrict__ part_acc,
+                                                          unsigned* __restrict__ cnt, int span) {
+    constexpr int D = ATT_D;
+    __shared__ float s_m[16][G], s_l[16][G];
+    __shared__ float s_acc[16][G][D];
+    __shared__ unsigned s_last;
+    const int g = blockIdx.x, sp = blockIdx.y, t = blockIdx.z, S = gridDim.y;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int sub = lane >> 4, dl = lane & 15;   // the lane's key within a quad of keys, its 8 dims
+    const int grp = wv * 4 + sub;                // one of the workgroup's 16 key streams
+    const int n = *n0p + t + 1;                  // row t sees the cache's keys and the pass's rows up to itself
+    const int k_begin = sp * span, k_end = min(n, k_begin + span);
+
+    // the row's G query heads, scaled into log2 units, the lane's 8 dims of each
+    float qv[G][8];
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(q + ((size_t)t * Hq + (size_t)g * G + j) * D + dl * 8);
+        qv[j][0] = bf16lo_f32(raw.x) * scale_log2;
+        qv[j][1] = bf16hi_f32(raw.x) * scale_log2;
+        qv[j][2] = bf16lo_f32(raw.y) * scale_log2;
+        qv[j][3] = bf16hi_f32(raw.y) * scale_log2;
+        qv[j][4] = bf16lo_f32(raw.z) * scale_log2;
+        qv[j][5] = bf16hi_f32(raw.z) * scale_log2;
+        qv[j][6] = bf16lo_f32(raw.w) * scale_log2;
+        qv[j][7] = bf16hi_f32(raw.w) * scale_log2;
+    }
+    float m[G], l[G], acc[G][8];
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+        m[j] = bits_f32(0xff800000u);
+        l[j] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
+    }
+    const uint16_t* Kh = K + (size_t)g * hs + dl * 8;
+    const uint16_t* Vh = V + (size_t)g * hs + dl * 8;
+    for (int key = k_begin + grp; key < k_end; key += 16) {
+        const uint4 kr = *reinterpret_cast<const uint4*>(Kh + (size_t)key * rs);
+        const uint4 vr = *reinterpret_cast<const uint4*>(Vh + (size_t)key * rs);
+        const float kf[8] = {bf16lo_f32(kr.x), bf16hi_f32(kr.x), bf16lo_f32(kr.y), bf16hi_f32(kr.y),
+                             bf16lo_f32(kr.z), bf16hi_f32(kr.z), bf16lo_f32(kr.w), bf16hi_f32(kr.w)};
+        const float vf[8] = {bf16lo_f32(vr.x), bf16hi_f32(vr.x), bf16lo_f32(vr.y), bf16hi_f32(vr.y),
+                             bf16lo_f32(vr.z), bf16hi_f32(vr.z), bf16lo_f32(vr.w), bf16hi_f32(vr.w)};
+#pragma unroll
+        for (int j = 0; j < G; ++j) {
+            float s = 0.f;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) s = fmaf(qv[j][e], kf[e], s);
+            s = group_sum<16>(s);
+            const float mn = fmaxf(m[j], s);
+            const float corr = exp2f(m[j] - mn);   // 0 on the stream's first key (m = -inf)
+            const float p = exp2f(s - mn);
+            l[j] = fmaf(l[j], corr, p);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[j][e] = fmaf(p, vf[e], acc[j][e] * corr);
+            m[j] = mn;
+        }
+    }
+    // the 16 streams' states into LDS
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+        if (dl == 0) {
+            s_m[grp][j] = m[j];
+            s_l[grp][j] = l[j];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s_acc[grp][j][dl * 8 + e] = acc[j][e];
+    }
+    __syncthreads();
+    // fold them in stream order: thread (j, d) for d < D; G * D <= 1024 values over 256 threads
+    const size_t prow = ((size_t)t * Hk + g) * S + sp;  // this workgroup's slot among the partial states
+    for (int o = threadIdx.x; o < G * D; o += 256) {
+        const int j = o / D, d = o - j * D;
+        float M = bits_f32(0xff800000u);
+        for (int s2 = 0; s2 < 16; ++s2) M = fmaxf(M, s_m[s2][j]);
+        float L = 0.f, A = 0.f;
+        for (int s2 = 0; s2 < 16; ++s2) {
+            const float f = s_m[s2][j] == bits_f32(0xff800000u) ? 0.f : exp2f(s_m[s2][j] - M);
+            L = fmaf(s_l[s2][j], f, L);
+            A = fmaf(s_acc[s2][j][d], f, A);
+        }
+        part_acc[(prow * G + j) * D + d] = A;
+        if (d == 0) {
+            part_m[prow * G + j] = M;
+            part_l[prow * G + j] = L;
+        }
+    }
+    // the last workgroup in for this (row, kv head) folds the spans
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) s_last = atomicAdd(&cnt[(size_t)t * Hk + g], 1u);
+    __syncthreads();
+    if (s_last != (unsigned)(S - 1)) return;
+    __threadfence();
+    const size_t base = ((size_t)t * Hk + g) * S;
+    for (int o = threadIdx.x; o < G * D; o += 256) {
+        const int j = o / D, d = o - j * D;
+        float M = bits_f32(0xff800000u);
+        for (int s2 = 0; s2 < S; ++s2) M = fmaxf(M, peek(&part_m[(base + s2) * G + j]));
+        float L = 0.f, A = 0.f;
+        for (int s2 = 0; s2 < S; ++s2) {
+            const float pm = peek(&part_m[(base + s2) * G + j]);
+            const float f = pm == bits_f32(0xff800000u) ? 0.f : exp2f(pm - M);
+            L = fmaf(peek(&part_l[(base + s2) * G + j]), f, L);
+            A = fmaf(peek(&part_acc[((base + s2) * G + j) * D + d]), f, A);
+        }
+        att[((size_t)t * Hq + (size_t)g * G + j) * D + d] = f32_bf16(A * (1.f / L));
+    }
+    if (threadIdx.x == 0) cnt[(size_t)t * Hk + g] = 0u;
+}
+
+__global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ m,
+                                                       size_t T, size_t I) {
+    const size_t n = T * I;
+    for (size_t k = (size_t)blockIdx.x * 256 + threadIdx.x; k < n; k += (size_t)gridDim.x * 256) {
+        const size_t t = k / I, i = k - t * I;
+        const float g = bf16_f32(gu[t * 2 * I + i]);
+        const float u = bf16_f32(gu[t * 2 * I + I + i]);
+        const float s = bfround(g / (1.f + expf(-g)));
+        m[k] = f32_bf16(s * u);
+    }
+}
+
+// one workgroup of 1024 per row: each thread its own strided elements in ascending order (a tie keeps the earlier),
+// then the (value, index) maximum over the block in the total order value descending, index ascending
+__global__ void __launch_bounds__(1024) argmax_kernel(const uint16_t* __restrict__ logits, int32_t* __restrict__ out,
+                                                      int V) {
+    __shared__ float s_v[16];
+    __shared__ int s_i[16];
+    const int t = blockIdx.x, tid = threadIdx.x;
+    const uint16_t* row = logits + (size_t)t * V;
+    float bv = bits_f32(0xff800000u);
+    int bi = 0x7fffffff;
+    for (int i = tid; i < V; i += 1024) {
+        const float v = bf16_f32(row[i]);
+        if (v > bv || bi == 0x7fffffff) {
+            bv = v;
+            bi = i;
+        }
+    }
+#pragma unroll
+    for (int s = 32; s > 0; s >>= 1) {
+        const float ov = __shfl_xor(bv, s, WAVE);
+        const int oi = __shfl_xor(bi, s, WAVE);
+        if (ov > bv || (ov == bv && oi < bi)) {
+            bv = ov;
+            bi = oi;
+        }
+    }
+    if ((tid & 63) == 0) {
+        s_v[tid >> 6] = bv;
+        s_i[tid >> 6] = bi;
+    }
+    __syncthreads();
+    if (tid == 0) {
+        for (int k = 1; k < 16; ++k)
+            if (s_v[k] > bv || (s_v[k] == bv && s_i[k] < bi)) {
+                bv = s_v[k];
+                bi = s_i[k];
+            }
+        out[t] = bi;
+    }
+}
+
+// the step's end: the picked token becomes the next step's input and the cache grows by one on the device; with
+// pinned host buffers, the token, the GPU clock and then (after a system fence) the new length go to the host
+__global__ void publish_kernel(int32_t* __restrict__ n0, const int32_t* __restrict__ picked, int32_t* __restrict__ next_ids,
+                               int32_t* out_tok, int32_t* out_n0, long long* out_ts) {
+    if (threadIdx.x != 0 || blockIdx.x != 0) return;
+    const int tok = *picked;
+    const int len = *n0 + 1;
+    if (next_ids != nullptr) *next_ids = tok;
+    *n0 = len;
+    if (out_tok != nullptr) {
+        *out_tok = tok;
+        if (out_ts != nullptr) *out_ts = (long long)wall_clock64();
+        __threadfence_system();
+        if (out_n0 != nullptr) *out_n0 = len;
+    }
+}
+
+static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
+
+}  // namespace btb
+
+using namespace btb;
+
+extern "C" {
+
+int32_t btb_hip_embed(const void* table, const int32_t* ids, void* h, size_t T, size_t H, size_t vocab, void* stream) {
+    if (table == nullptr || ids == nullptr || h == nullptr) return ERR_NULL;
+    if (T == 0 || H == 0 || vocab == 0 || H % 8 != 0 || T > 65535 || vocab > 0x7FFFFFFFull) return ERR_DOMAIN;
+    if (!al(table, 16) || !al(h, 16) || !al(ids, 4)) return ERR_DOMAIN;
+    hipLaunchKernelGGL(embed_kernel, dim3((unsigned)T), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint4*>(table), ids, static_cast<uint4*>(h), (int)(H / 8), (int)vocab);
+    return hip_status(hipGetLastError(), "embed launch");
+}
+
+int32_t btb_hip_add_rmsnorm(void* h, const void* y, const void* w, float eps, void* x, size_t T, size_t H,
+                            int32_t centered, void* stream) {
+    if (h == nullptr || w == nullptr || x == nullptr) return ERR_NULL;
+    if (T == 0 || H == 0 || T > 0x7FFFFFFFull || H > 0x7FFFFFFFull || !(eps >= 0.f)) return ERR_DOMAIN;
+    if (!al(h, 2) || !al(y, 2) || !al(w, 2) || !al(x, 2)) return ERR_DOMAIN;
+    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3((unsigned)T), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<uint16_t*>(h), static_cast<const uint16_t*>(y), static_cast<const uint16_t*>(w), eps,
+                       static_cast<uint16_t*>(x), (int)H, centered);
+    return hip_status(hipGetLastError(), "add_rmsnorm launch");
+}
+
+int32_t btb_hip_norm_rope_kv(const void* qkv, const void* wq, const void* wk, float eps, const void* cos_t,
+                             const void* sin_t, const int32_t* n0, const int32_t* depth, void* K, void* V, void* q,
+                             size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered,
+                             void* stream) {
+    if (qkv == nullptr || cos_t == nullptr || sin_t == nullptr || n0 == nullptr || K == nullptr || V == nullptr ||
+        q == nullptr)
+        return ERR_NULL;
+    if (T == 0 || Hq == 0 || Hk == 0 || T > 65535 || Hq + 2 * Hk > 0x7FFFFFFFull || hs <= 0 || rs <= 0 ||
+        !(eps >= 0.f))
+        return ERR_DOMAIN;
+    if (D != 64 && D != 128 && D != 256) return ERR_DOMAIN;
+    const dim3 grid((unsigned)(Hq + 2 * Hk), (unsigned)T);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define NRK(DD)                                                                                                      \
+    hipLaunchKernelGGL(norm_rope_kv_kernel<DD>, grid, dim3(64), 0, st, static_cast<const uint16_t*>(qkv),             \
+                       static_cast<const uint16_t*>(wq), static_cast<const uint16_t*>(wk), eps,                      \
+                       static_cast<const uint16_t*>(cos_t), static_cast<const uint16_t*>(sin_t), n0, depth,          \
+                       static_cast<uint16_t*>(K), static_cast<uint16_t*>(V), static_cast<uint16_t*>(q), (int)Hq,      \
+                       (int)Hk, (long long)hs, (long long)rs, centered)
+    if (D == 64)
+        NRK(64);
+    else if (D == 128)
+        NRK(128);
+    else
+        NRK(256);
+#undef NRK
+    return hip_status(hipGetLastError(), "norm_rope_kv launch");
+}
+
+size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, size_t S) {
+    // part_m and part_l [T, Hk, S, G], part_acc [T, Hk, S, G, D]
+    return T * Hq * S * (2 + D);
+}
+
+int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0, size_t T,
+                            size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap, size_t S,
+                            float* scratch, uint32_t* cnt, void* stream) {
+    if (q == nullptr || K == nullptr || V == nullptr || att == nullptr || n0 == nullptr || scratch == nullptr ||
+        cnt == nullptr)
+        return ERR_NULL;
+    if (T == 0 || Hq == 0 || Hk == 0 || S == 0 || cap == 0 || T > 65535 || S > 65535 || Hq % Hk != 0 || hs <= 0 ||
+        rs <= 0 || !(scale == scale))
+        return ERR_DOMAIN;
+    const size_t G = Hq / Hk;
+    if (D != (size_t)ATT_D || G > (size_t)ATT_MAXG) {
+        set_error("attn_decode: head_dim 128 and at most 8 query heads per kv head");
+        return ERR_DOMAIN;
+    }
+    if (!al(q, 16) || !al(K, 16) || !al(V, 16) || (rs % 8) != 0 || (hs % 8) != 0) return ERR_DOMAIN;
+    const int span = (int)((cap + S - 1) / S);
+    float* part_m = scratch;
+    float* part_l = scratch + T * Hq * S;
+    float* part_acc = scratch + 2 * T * Hq * S;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    const dim3 grid((unsigned)Hk, (unsigned)S, (unsigned)T);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+#define ATT(GG)                                                                                                      \
+    hipLaunchKernelGGL(attn_decode_kernel<GG>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(q),              \
+                       static_cast<const uint16_t*>(K), static_cast<const uint16_t*>(V), static_cast<uint16_t*>(att), \
+                       n0, (int)Hq, (int)Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, cnt,   \
+                       span)
+    switch (G) {
+        case 1: ATT(1); break;
+        case 2: ATT(2); break;
+        case 4: ATT(4); break;
+        case 8: ATT(8); break;
+        default:
+            set_error("attn_decode: 1, 2, 4 or 8 query heads per kv head");
+            return ERR_DOMAIN;
+    }
+#undef ATT
+    return hip_status(hipGetLastError(), "attn_decode launch");
+}
+
+int32_t btb_hip_silu_mul(const void* gu, void* m, size_t T, size_t I, void* stream) {
+    if (gu == nullptr || m == nullptr) return ERR_NULL;
+    if (T == 0 || I == 0) return ERR_DOMAIN;
+    size_t blocks = (T * I + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    hipLaunchKernelGGL(silu_mul_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t*>(gu), static_cast<uint16_t*>(m), T, I);
+    return hip_status(hipGetLastError(), "silu_mul launch");
+}
+
+int32_t btb_hip_argmax(const void* logits, int32_t* out, size_t T, size_t V, void* stream) {
+    if (logits == nullptr || out == nullptr) return ERR_NULL;
+    if (T == 0 || V == 0 || T > 0x7FFFFFFFull || V > 0x7FFFFFFEull) return ERR_DOMAIN;
+    hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)T), dim3(1024), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t*>(logits), out, (int)V);
+    return hip_status(hipGetLastError(), "argmax launch");
+}
+
+int32_t btb_hip_publish(int32_t* n0, const int32_t* picked, int32_t* next_ids, int32_t* out_tok, int32_t* out_n0,
+                        int64_t* out_ts, void* stream) {
+    if (n0 == nullptr || picked == nullptr) return ERR_NULL;
+    hipLaunchKernelGGL(publish_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), n0, picked, next_ids,
+                       out_tok, out_n0, reinterpret_cast<long long*>(out_ts));
+    return hip_status(hipGetLastError(), "publish launch");
+}
+
+}  // extern "C"

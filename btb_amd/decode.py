@@ -1,0 +1,225 @@
+"""The dense decode step on the GPU as one hipGraph: the counterpart of the reference's card graph
+(`_card_buffers` btb/engine/cuda.py:1491-1562, `_card_body` :1601-1837, `_capture` :988-999, `_card_step_graph` :2101)
+for a Qwen3-shaped stack with every weight resident in VRAM, in bf16 or in the 12-bit packed form.
+
+Per layer, as the reference sequences it: add_rmsnorm -> qkv matvec -> q/k norm + rope + cache write -> decode
+attention -> o matvec -> add_rmsnorm -> gate_up matvec -> down matvec with the SwiGLU fold in its x load; then the
+final norm, the head matvec, the greedy pick and the publish. `DecodeStep.capture()` records the whole step with
+torch's graph capture (a hipGraph on ROCm); afterwards the host only replays it and reads the token from pinned
+memory.
+"""
+
+from __future__ import annotations
+
+import math
+from dataclasses import dataclass
+from typing import Any
+
+import torch
+
+from .pack12 import P12Weight
+
+
+@dataclass(frozen=True)
+class StackConfig:
+    """the shape of a dense decoder stack (Qwen3-4B: 36, 2560, 32, 8, 128, 9728, 151936)"""
+
+    layers: int = 36
+    hidden: int = 2560
+    q_heads: int = 32
+    kv_heads: int = 8
+    head_dim: int = 128
+    intermediate: int = 9728
+    vocab: int = 151936
+    eps: float = 1e-6
+    rope_theta: float = 1_000_000.0
+
+    @property
+    def qkv_rows(self) -> int:
+        return (self.q_heads + 2 * self.kv_heads) * self.head_dim
+
+    def weight_elements(self) -> int:
+        """the linear weights' element count per step: 4 matrices a layer and the head"""
+        per = (self.qkv_rows * self.hidden + self.hidden * self.q_heads * self.head_dim
+               + 2 * self.intermediate * self.hidden + self.hidden * self.intermediate)
+        return self.layers * per + self.vocab * self.hidden
+
+
+QWEN3_4B = StackConfig()
+
+
+def rope_tables(cfg: StackConfig, positions: int, device: Any) -> tuple[torch.Tensor, torch.Tensor]:
+    """the model's rotary tables as the card kernels read them: cos / sin [positions, D] bf16 (the default rope:
+    angles pos * theta^(-2i/D) over the first half of the dims, repeated over the second)"""
+    half = cfg.head_dim // 2
+    inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, half, dtype=torch.float32, device=device) * 2.0 / cfg.head_dim))
+    ang = torch.arange(positions, dtype=torch.float32, device=device)[:, None] * inv[None, :]
+    emb = torch.cat([ang, ang], dim=-1)
+    return emb.cos().to(torch.bfloat16).contiguous(), emb.sin().to(torch.bfloat16).contiguous()
+
+
+class Linear:
+    """one linear's weight on the GPU in its stored form, multiplied as stored: a bf16 tensor or a `P12Weight`"""
+
+    __slots__ = ("card", "w")
+
+    def __init__(self, card: Any, w: Any) -> None:
+        self.card = card
+        self.w = w
+
+    @property
+    def shape(self) -> tuple[int, int]:
+        return (int(self.w.shape[0]), int(self.w.shape[1]))
+
+    @property
+    def nbytes(self) -> int:
+        return int(self.w.nbytes) if isinstance(self.w, P12Weight) else int(self.w.numel()) * 2
+
+    def matvec(self, x: torch.Tensor, y: torch.Tensor) -> None:
+        if isinstance(self.w, P12Weight):
+            self.card.gemv_p12(self.w, x, y)
+        else:
+            self.card.gemv(self.w, x, y)
+
+
+class DecodeStep:
+    """Buffers, caches and the kernel sequence of one decode step over `T` rows (1: the step; more: a chain of rows
+    verified in one pass). `weights` maps `layers.{i}.{ln1,ln2,wq,wk}` (bf16 vectors), `layers.{i}.{qkv,o,gu,down}`
+    (`Linear`), `embed` (bf16 [V, H]), `norm` and `head` (`Linear`)."""
+
+    def __init__(self, card: Any, cfg: StackConfig, weights: dict[str, Any], cap: int, T: int = 1,
+                 attn_spans: int | None = None, fold_silu: bool = True) -> None:
+        dev = torch.device("cuda")
+        self.card, self.cfg, self.w, self.cap, self.T = card, cfg, weights, int(cap), int(T)
+        H, D, Hq, Hk, I = cfg.hidden, cfg.head_dim, cfg.q_heads, cfg.kv_heads, cfg.intermediate
+        bf = dict(dtype=torch.bfloat16, device=dev)
+        self.h = torch.zeros(T, H, **bf)
+        self.x = torch.zeros(T, H, **bf)
+        self.y = torch.zeros(T, H, **bf)
+        self.qkv = torch.zeros(T, cfg.qkv_rows, **bf)
+        self.q = torch.zeros(T, Hq * D, **bf)
+        self.att = torch.zeros(T, Hq * D, **bf)
+        self.gu = torch.zeros(T, 2 * I, **bf)
+        self.m = torch.zeros(T, I, **bf)
+        self.logits = torch.zeros(T, cfg.vocab, **bf)
+        self.ids = torch.zeros(T, dtype=torch.int32, device=dev)
+        self.picked = torch.zeros(T, dtype=torch.int32, device=dev)
+        self.n0 = torch.zeros(1, dtype=torch.int32, device=dev)
+        # the caches: [layer, K/V, kv head, slot, dim], head-major so a key's row is one contiguous run
+        self.kv = torch.zeros(cfg.layers, 2, Hk, self.cap, D, **bf)
+        self.cos, self.sin = rope_tables(cfg, self.cap, dev)
+        self.scale = 1.0 / math.sqrt(D)
+        # key spans: enough workgroups (kv heads x spans) to cover the CUs about twice, a span at least 64 keys
+        if attn_spans is None:
+            attn_spans = max(1, min(self.cap // 64, (2 * card.sms + Hk - 1) // Hk))
+        self.S = int(attn_spans)
+        self.scratch, self.cnt = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
+        self.fold_silu = bool(fold_silu)
+        # the handoff to the host: token, cache length and the GPU's clock in pinned memory
+        self.host_tok = torch.zeros(1, dtype=torch.int32).pin_memory()
+        self.host_n0 = torch.zeros(1, dtype=torch.int32).pin_memory()
+        self.host_ts = torch.zeros(1, dtype=torch.int64).pin_memory()
+        self.graph: torch.cuda.CUDAGraph | None = None
+
+    # -- state ---------------------------------------------------------------------------------------------------
+
+    def reset(self, n0: int, token: int) -> None:
+        """the cache holds `n0` rows; `token` is the step's input"""
+        if not 0 <= n0 + self.T <= self.cap:
+            raise ValueError(f"[decode] {n0} cached rows and a pass of {self.T} do not fit a cache of {self.cap}")
+        self.n0.fill_(int(n0))
+        self.ids.fill_(int(token))
+
+    def weight_bytes(self) -> int:
+        """bytes of linear weights one step streams"""
+        n = sum(self.w[f"layers.{i}.{k}"].nbytes for i in range(self.cfg.layers) for k in ("qkv", "o", "gu", "down"))
+        return n + self.w["head"].nbytes
+
+    def kv_bytes(self, n: int) -> int:
+        """bytes of cache one step reads with `n` keys a head"""
+        return self.cfg.layers * 2 * self.cfg.kv_heads * n * self.cfg.head_dim * 2
+
+    # -- the kernel sequence ---------------------------------------------------------------------------------------
+
+    def body(self) -> None:
+        k, cfg, w = self.card, self.cfg, self.w
+        Hq, Hk, D = cfg.q_heads, cfg.kv_heads, cfg.head_dim
+        k.embed(w["embed"], self.ids, self.h)
+        y_prev = None
+        for i in range(cfg.layers):
+            L = f"layers.{i}."
+            K, V = self.kv[i, 0], self.kv[i, 1]
+            k.add_rmsnorm(self.h, y_prev, w[L + "ln1"], cfg.eps, self.x)
+            w[L + "qkv"].matvec(self.x, self.qkv)
+            k.norm_rope_kv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K, V,
+                           self.q, Hq, Hk, D)
+            k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch, self.cnt)
+            w[L + "o"].matvec(self.att, self.y)
+            k.add_rmsnorm(self.h, self.y, w[L + "ln2"], cfg.eps, self.x)
+            w[L + "gu"].matvec(self.x, self.gu)
+            down = w[L + "down"]
+            if self.fold_silu and isinstance(down.w, torch.Tensor):
+                k.gemv_silu(down.w, self.gu, self.y)
+            else:
+                k.silu_mul(self.gu, self.m)
+                down.matvec(self.m, self.y)
+            y_prev = self.y
+        k.add_rmsnorm(self.h, y_prev, w["norm"], cfg.eps, self.x)
+        w["head"].matvec(self.x, self.logits)
+        k.argmax(self.logits, self.picked)
+        k.publish(self.n0, self.picked, self.ids, self.host_tok, self.host_n0, self.host_ts)
+
+    def capture(self, warmup: int = 2) -> torch.cuda.CUDAGraph:
+        """run the step eagerly (on a side stream, as a capture requires), then record it: the hipGraph the host
+        replays. The warm-up steps advance the cache; `reset` before the first replay."""
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for _ in range(warmup):
+                self.body()
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            self.body()
+        self.graph = g
+        return g
+
+    def replay(self) -> None:
+        if self.graph is None:
+            raise RuntimeError("[decode] capture() the step before replaying it")
+        self.graph.replay()
+
+    def token(self) -> int:
+        """the last step's token as the host sees it (after a synchronize, or once host_n0 shows the new length)"""
+        return int(self.host_tok[0])
+
+
+def random_stack(card: Any, cfg: StackConfig, seed: int = 0x0B7B0000, packed: bool = False,
+                 std: float = 0.02) -> dict[str, Any]:
+    """random-init weights of the stack's shape on the GPU: linears ~ N(0, std) rounded to bf16 (drawn with the
+    device's generator, one seed per tensor), norm weights one. `packed`: every linear stored in the 12-bit form."""
+    dev = torch.device("cuda")
+    H, I = cfg.hidden, cfg.intermediate
+    n = [0]
+
+    def mat(rows: int, cols: int) -> Linear:
+        g = torch.Generator(device=dev).manual_seed(seed + n[0])
+        n[0] += 1
+        t = (torch.randn(rows, cols, generator=g, device=dev, dtype=torch.float32) * std).to(torch.bfloat16)
+        return Linear(card, P12Weight.pack(t, card) if packed else t)
+
+    w: dict[str, Any] = {}
+    for i in range(cfg.layers):
+        L = f"layers.{i}."
+        w[L + "qkv"] = mat(cfg.qkv_rows, H)
+        w[L + "o"] = mat(H, cfg.q_heads * cfg.head_dim)
+        w[L + "gu"] = mat(2 * I, H)
+        w[L + "down"] = mat(H, I)
+        for name, length in (("ln1", H), ("ln2", H), ("wq", cfg.head_dim), ("wk", cfg.head_dim)):
+            w[L + name] = torch.ones(length, dtype=torch.bfloat16, device=dev)
+    g = torch.Generator(device=dev).manual_seed(seed + 100_000)
+    w["embed"] = (torch.randn(cfg.vocab, H, generator=g, device=dev, dtype=torch.float32) * std).to(torch.bfloat16)
+    w["norm"] = torch.ones(H, dtype=torch.bfloat16, device=dev)
+    w["head"] = mat(cfg.vocab, H)
+    return w

@@ -50,6 +50,16 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_gemv_fp8_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_moe_route": (_i32, [_vp, _i32, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp]),
     "btb_hip_moe_experts_bf16": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _vp]),
+    "btb_hip_embed": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_add_rmsnorm": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _sz, _sz, _i32, _vp]),
+    "btb_hip_norm_rope_kv": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
+                                    _sz, ctypes.c_int64, ctypes.c_int64, _i32, _vp]),
+    "btb_hip_attn_scratch_floats": (_sz, [_sz, _sz, _sz, _sz, _sz]),
+    "btb_hip_attn_decode": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
+                                   ctypes.c_float, _sz, _sz, _vp, _vp, _vp]),
+    "btb_hip_silu_mul": (_i32, [_vp, _vp, _sz, _sz, _vp]),
+    "btb_hip_argmax": (_i32, [_vp, _vp, _sz, _sz, _vp]),
+    "btb_hip_publish": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
 }
 
 
@@ -341,6 +351,93 @@ class HipCard:
         self._call("btb_hip_moe_experts_bf16", self.ptr(gate_up), self.ptr(down), self.ptr(x), self.ptr(idx), self.ptr(w),
                    self.ptr(gu), self.ptr(y), T, k, E, H, I2 // 2, _stream())
         return y
+
+
+    # -- the decode step's kernels between the matvecs ------------------------------------------------------------
+
+    def embed(self, table: torch.Tensor, ids: torch.Tensor, h: torch.Tensor) -> torch.Tensor:
+        self._need(table, torch.bfloat16, "table")
+        self._need(ids, torch.int32, "ids")
+        self._need(h, torch.bfloat16, "h")
+        V, H = (int(s) for s in table.shape)
+        self._call("btb_hip_embed", self.ptr(table), self.ptr(ids), self.ptr(h), int(ids.numel()), H, V, _stream())
+        return h
+
+    def add_rmsnorm(self, h: torch.Tensor, y: torch.Tensor | None, w: torch.Tensor, eps: float, x: torch.Tensor,
+                    centered: bool = False) -> torch.Tensor:
+        """h += y in place (bf16 add), x = rmsnorm(h) * w (`btb_add_rmsnorm`)"""
+        for t, what in ((h, "h"), (w, "w"), (x, "x")):
+            self._need(t, torch.bfloat16, what)
+        if y is not None:
+            self._need(y, torch.bfloat16, "y")
+        H = int(w.numel())
+        T = int(h.numel()) // H
+        if h.numel() != T * H or x.numel() != T * H or (y is not None and y.numel() != T * H):
+            raise ValueError("[hip] add_rmsnorm: h, y and x are [T, H] with H the weight's length")
+        self._call("btb_hip_add_rmsnorm", self.ptr(h), None if y is None else self.ptr(y), self.ptr(w), float(eps),
+                   self.ptr(x), T, H, int(bool(centered)), _stream())
+        return x
+
+    def norm_rope_kv(self, qkv: torch.Tensor, wq: torch.Tensor | None, wk: torch.Tensor | None, eps: float,
+                     cos: torch.Tensor, sin: torch.Tensor, n0: torch.Tensor, K: torch.Tensor, V: torch.Tensor,
+                     q: torch.Tensor, Hq: int, Hk: int, D: int, depth: torch.Tensor | None = None,
+                     centered: bool = False) -> None:
+        """q/k norm, rope and the cache write for the pass's rows (`btb_norm_rope_kv_d{D}`); K, V are one layer's
+        [Hk, cap, D] views (any strides with D contiguous)"""
+        for t, what in ((qkv, "qkv"), (cos, "cos"), (sin, "sin"), (q, "q")):
+            self._need(t, torch.bfloat16, what)
+        self._need(n0, torch.int32, "n0")
+        if K.dtype != torch.bfloat16 or V.dtype != torch.bfloat16 or K.stride(2) != 1 or K.stride() != V.stride():
+            raise ValueError("[hip] norm_rope_kv: K and V are bf16 [Hk, cap, D] views with the same strides")
+        T = int(qkv.numel()) // ((Hq + 2 * Hk) * D)
+        self._call("btb_hip_norm_rope_kv", self.ptr(qkv), None if wq is None else self.ptr(wq),
+                   None if wk is None else self.ptr(wk), float(eps), self.ptr(cos), self.ptr(sin), self.ptr(n0),
+                   None if depth is None else self.ptr(depth), self.ptr(K), self.ptr(V), self.ptr(q), T, Hq, Hk, D,
+                   int(K.stride(0)), int(K.stride(1)), int(bool(centered)), _stream())
+
+    def attn_scratch(self, T: int, Hq: int, Hk: int, D: int, S: int, device: Any = "cuda"):
+        """(scratch f32, arrival counts u32) for `attn_decode` at these sizes; the counts start, and stay, zero"""
+        n = int(self.lib.btb_hip_attn_scratch_floats(T, Hq, Hk, D, S))
+        return (torch.empty(n, dtype=torch.float32, device=device),
+                torch.zeros(T * Hk, dtype=torch.int32, device=device))
+
+    def attn_decode(self, q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, att: torch.Tensor, n0: torch.Tensor,
+                    Hq: int, Hk: int, D: int, scale: float, S: int, scratch: torch.Tensor, cnt: torch.Tensor) -> None:
+        """att [T, Hq * D] = the rows' attention over the cache (row t sees keys 0 .. n0 + t)"""
+        self._need(q, torch.bfloat16, "q")
+        self._need(att, torch.bfloat16, "att")
+        self._need(n0, torch.int32, "n0")
+        if K.dtype != torch.bfloat16 or V.dtype != torch.bfloat16 or K.stride(2) != 1 or K.stride() != V.stride():
+            raise ValueError("[hip] attn_decode: K and V are bf16 [Hk, cap, D] views with the same strides")
+        T = int(q.numel()) // (Hq * D)
+        need = int(self.lib.btb_hip_attn_scratch_floats(T, Hq, Hk, D, S))
+        if scratch.numel() < need or cnt.numel() < T * Hk:
+            raise ValueError(f"[hip] attn_decode: scratch holds {scratch.numel()} floats, {need} are needed")
+        self._call("btb_hip_attn_decode", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0), T, Hq, Hk,
+                   D, int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S, self.ptr(scratch),
+                   self.ptr(cnt), _stream())
+
+    def silu_mul(self, gu: torch.Tensor, m: torch.Tensor) -> torch.Tensor:
+        self._need(gu, torch.bfloat16, "gu")
+        self._need(m, torch.bfloat16, "m")
+        I = int(gu.shape[-1]) // 2
+        self._call("btb_hip_silu_mul", self.ptr(gu), self.ptr(m), int(gu.numel()) // (2 * I), I, _stream())
+        return m
+
+    def argmax(self, logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        self._need(logits, torch.bfloat16, "logits")
+        self._need(out, torch.int32, "out")
+        V = int(logits.shape[-1])
+        self._call("btb_hip_argmax", self.ptr(logits), self.ptr(out), int(logits.numel()) // V, V, _stream())
+        return out
+
+    def publish(self, n0: torch.Tensor, picked: torch.Tensor, next_ids: torch.Tensor | None = None,
+                out_tok: torch.Tensor | None = None, out_n0: torch.Tensor | None = None,
+                out_ts: torch.Tensor | None = None) -> None:
+        """the step's end: next_ids = picked, n0 += 1, and the token / clock / length into pinned host tensors"""
+        p = lambda t: None if t is None else self.ptr(t)
+        self._call("btb_hip_publish", self.ptr(n0), self.ptr(picked), p(next_ids), p(out_tok), p(out_n0), p(out_ts),
+                   _stream())
 
 
 class Native:

@@ -162,6 +162,53 @@ int32_t btb_hip_moe_route(const void* logits, int32_t logits_f32, size_t ls, siz
 int32_t btb_hip_moe_experts_bf16(const void* gate_up, const void* down, const void* x, const int32_t* idx, const void* w,
                                  void* gu, void* y, size_t T, size_t k, size_t E, size_t H, size_t I, void* stream);
 
+/* ---- the decode step's kernels between the matvecs ---------------------------------------------------------- */
+
+/* h[t] = table[ids[t]]: the step's input row (the reference gathers it with torch before its graph). table
+ * [vocab, H] bf16, ids i32 [T] on the device, h [T, H] bf16; H a multiple of 8. */
+int32_t btb_hip_embed(const void* table, const int32_t* ids, void* h, size_t T, size_t H, size_t vocab, void* stream);
+
+/* h [T, H] bf16 in place: h = bf16(h + y) when y is not NULL; x = bf16(h * rsqrt(mean(h^2) + eps) * w), or
+ * * (1 + w) when centered. Replaces btb_add_rmsnorm (native/cuda/btb_kernels.cu:360-393). */
+int32_t btb_hip_add_rmsnorm(void* h, const void* y, const void* w, float eps, void* x, size_t T, size_t H,
+                            int32_t centered, void* stream);
+
+/* q/k RMSNorm per head (wq / wk [D], NULL: none), rope from the bf16 tables cos / sin [positions, D], row t of the
+ * pass written into the caches at slot *n0 + t and q [T, Hq, D] out. qkv [T, (Hq + 2 Hk) D] bf16; head g's slot j
+ * of K / V at g * hs + j * rs elements; row t's position is *n0 + depth[t] (depth NULL: *n0 + t). D 64, 128 or
+ * 256. Replaces btb_norm_rope_kv_d{D} (native/cuda/btb_kernels.cu:250-358). */
+int32_t btb_hip_norm_rope_kv(const void* qkv, const void* wq, const void* wk, float eps, const void* cos_t,
+                             const void* sin_t, const int32_t* n0, const int32_t* depth, void* K, void* V, void* q,
+                             size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered,
+                             void* stream);
+
+/* floats of scratch btb_hip_attn_decode needs for T rows and S key spans */
+size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, size_t S);
+
+/* Decode attention: att [T, Hq * D] = softmax(q K^T * scale) V, row t over the keys 0 .. *n0 + t, f32 throughout,
+ * bf16 out. The keys (capacity `cap`) are cut into S spans, a workgroup per (kv head, span, row); `scratch`
+ * (btb_hip_attn_scratch_floats) and cnt u32 [T * Hk] (zero before the first launch; every launch leaves it zero)
+ * carry the spans' partial states to the last arriver, which folds them in span order. head_dim 128, Hq / Hk in
+ * {1, 2, 4, 8}. Replaces btb_attn_flash_d128's decode form (native/cuda/btb_attn_flash.cuh:277-675) for a chain of
+ * rows. */
+int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0, size_t T,
+                            size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap, size_t S,
+                            float* scratch, uint32_t* cnt, void* stream);
+
+/* m [T, I] = bf16(bf16(silu(g)) * u) over gu [T, 2I] (gate then up). Replaces btb_silu_mul
+ * (native/cuda/btb_kernels.cu:467-484); the matvec btb_hip_gemv_silu_bf16 folds the same values into its x load. */
+int32_t btb_hip_silu_mul(const void* gu, void* m, size_t T, size_t I, void* stream);
+
+/* out[t] = the index of row t's largest logit, the lowest index on ties (native/src/sample.rs:53-67). logits
+ * [T, V] bf16. */
+int32_t btb_hip_argmax(const void* logits, int32_t* out, size_t T, size_t V, void* stream);
+
+/* The step's end, one thread: *next_ids = *picked (the next step's input, when not NULL), *n0 += 1, and with
+ * out_tok not NULL (pinned host memory) the token and the GPU's clock, then - after a system fence - the new
+ * length, so a host that sees the length sees the token. Replaces btb_publish (native/cuda/btb_kernels.cu:448-465). */
+int32_t btb_hip_publish(int32_t* n0, const int32_t* picked, int32_t* next_ids, int32_t* out_tok, int32_t* out_n0,
+                        int64_t* out_ts, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

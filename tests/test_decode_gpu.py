@@ -1,0 +1,129 @@
+"""The whole decode step on the GPU - eager and as a captured, replayed hipGraph - against the CPU restatement
+(oracle/decode.py) at a reduced Qwen3 shape, in bf16 and with every linear in the 12-bit packed form.
+
+Bars: the two sides share every rounding point and differ in the order of the f32 additions inside matvecs, norms and
+attention, so a bf16 rounding can flip here and there and travel through the layers: logits are held to 3e-2 of the
+largest logit, and the greedy token must agree whenever the oracle's top-2 margin exceeds that bar. The packed stack
+must reproduce the bf16 stack's GPU logits to the same bar (on the CPU the pair is bit-equal: native/tests/gemv.rs:297-299)
+and a replayed graph must reproduce the eager step bit for bit, replay after replay."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from btb_amd.decode import DecodeStep, Linear, StackConfig
+from btb_amd.pack12 import P12Weight
+from oracle import decode as od
+
+from .helpers import bits16, gen
+
+pytestmark = pytest.mark.gpu
+
+CFG = StackConfig(layers=3, hidden=256, q_heads=4, kv_heads=2, head_dim=128, intermediate=512, vocab=1000)
+CAP, N0, TOKEN = 96, 40, 17
+
+
+def make_weights(card, packed: bool):
+    g = gen(700)
+    W, dev = {}, {}
+
+    def mat(name, rows, cols):
+        t = (torch.randn(rows, cols, generator=g) * 0.05).to(torch.bfloat16)
+        W[name] = bits16(t)
+        dev[name] = Linear(card, P12Weight.pack(t.cuda(), card) if packed else t.cuda())
+
+    def vec(name, n):
+        t = (1.0 + 0.1 * torch.randn(n, generator=g)).to(torch.bfloat16)
+        W[name] = bits16(t)
+        dev[name] = t.cuda()
+
+    H, I = CFG.hidden, CFG.intermediate
+    for i in range(CFG.layers):
+        L = f"layers.{i}."
+        mat(L + "qkv", CFG.qkv_rows, H)
+        mat(L + "o", H, CFG.q_heads * CFG.head_dim)
+        mat(L + "gu", 2 * I, H)
+        mat(L + "down", H, I)
+        for n_, ln in (("ln1", H), ("ln2", H), ("wq", CFG.head_dim), ("wk", CFG.head_dim)):
+            vec(L + n_, ln)
+    emb = (torch.randn(CFG.vocab, H, generator=g)).to(torch.bfloat16)
+    W["embed"], dev["embed"] = bits16(emb), emb.cuda()
+    vec("norm", H)
+    mat("head", CFG.vocab, H)
+    kv = torch.randn(CFG.layers, 2, CFG.kv_heads, CAP, CFG.head_dim, generator=g).to(torch.bfloat16)
+    return W, dev, kv
+
+
+def run_gpu(card, dev, kv, graph: bool, fold: bool = True):
+    step = DecodeStep(card, CFG, dev, CAP, fold_silu=fold)
+    step.kv.copy_(kv.cuda())
+    step.reset(N0, TOKEN)
+    if graph:
+        step.capture(warmup=1)
+        step.kv.copy_(kv.cuda())
+        step.reset(N0, TOKEN)
+        step.replay()
+    else:
+        step.body()
+    torch.cuda.synchronize()
+    return step
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_decode_step_matches_cpu_path(card, packed):
+    W, dev, kv = make_weights(card, packed)
+    step = run_gpu(card, dev, kv, graph=False)
+    okv = kv.float().numpy().copy()
+    want, tok = od.step(CFG, W, TOKEN, okv, N0)
+    got = step.logits[0].float().cpu().numpy()
+    bar = 3e-2 * np.abs(want).max()
+    assert np.abs(got - want).max() <= bar
+    top2 = np.sort(want)[-2:]
+    if top2[1] - top2[0] > 2 * bar:
+        assert step.token() == tok
+    # the step wrote its K / V row at slot N0, advanced the cache and fed its token forward
+    assert int(step.n0[0]) == N0 + 1 and int(step.host_n0[0]) == N0 + 1 and int(step.ids[0]) == step.token()
+    krow = step.kv[:, 0, :, N0].float().cpu().numpy()
+    assert np.abs(krow - okv[:, 0, :, N0]).max() <= 3e-2 * np.abs(okv[:, 0, :, N0]).max()
+
+
+def test_packed_stack_tracks_the_bf16_stack(card):
+    _, dev_b, kv = make_weights(card, False)
+    _, dev_p, _ = make_weights(card, True)
+    a = run_gpu(card, dev_b, kv, graph=False, fold=False).logits.float()
+    b = run_gpu(card, dev_p, kv, graph=False).logits.float()
+    assert (a - b).abs().max() <= 3e-2 * a.abs().max()
+    c = run_gpu(card, dev_b, kv, graph=False, fold=True).logits.float()
+    assert (a - c).abs().max() <= 3e-2 * a.abs().max()   # the SwiGLU fold and the two-kernel form agree
+
+
+def test_graph_replays_equal_the_eager_step(card):
+    """several replays, with eager work and synchronisations between them, each checked against the eager result"""
+    W, dev, kv = make_weights(card, False)
+    eager = run_gpu(card, dev, kv, graph=False)
+    want_logits, want_tok = eager.logits.clone(), eager.token()
+    step = DecodeStep(card, CFG, dev, CAP)
+    step.kv.copy_(kv.cuda())
+    step.reset(N0, TOKEN)
+    step.capture(warmup=1)
+    for rep in range(4):
+        step.kv.copy_(kv.cuda())
+        step.reset(N0, TOKEN)
+        step.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(step.logits, want_logits), rep
+        assert step.token() == want_tok and int(step.host_n0[0]) == N0 + 1
+        junk = torch.randn(1 << 16, device="cuda").sum()   # unrelated eager work between the replays
+        torch.cuda.synchronize()
+        assert torch.isfinite(junk)
+    # consecutive replays decode a sequence: each step feeds its token and cache row to the next
+    step.kv.copy_(kv.cuda())
+    step.reset(N0, TOKEN)
+    toks = []
+    for _ in range(3):
+        step.replay()
+        torch.cuda.synchronize()
+        toks.append(step.token())
+    assert int(step.n0[0]) == N0 + 3 and toks[0] == want_tok

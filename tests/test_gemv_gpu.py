@@ -47,7 +47,7 @@ def test_gemv_bf16_matches_oracle(card, R, C, M):
     check(y, oracle_bf16_out(w, x))
 
 
-@pytest.mark.parametrize("M", [2, 3, 5, 8, 16, 32])
+@pytest.mark.parametrize("M", [2, 3, 4, 5, 7])
 def test_row_of_a_wide_pass_is_its_one_row_pass(card, M):
     """native/cuda/btb_kernels.cu:84-88 and tests/kernels/test_card_kernels.py:145-148: row m does not depend on M"""
     R, C = 2560, 4096
@@ -58,6 +58,28 @@ def test_row_of_a_wide_pass_is_its_one_row_pass(card, M):
     for m in (0, M - 1):
         solo = card.gemv(w, x[m : m + 1].contiguous())
         assert torch.equal(solo[0].view(torch.int16), y[m].view(torch.int16))
+
+
+@pytest.mark.parametrize("R,C", [(9728, 2560), (2560, 9728), (2560, 4096), (1000, 96), (18, 32)])
+@pytest.mark.parametrize("M", [8, 16, 32, 12, 40])
+def test_verify_widths_on_the_matrix_cores(card, R, C, M):
+    """M >= 8 runs on MFMA: within the oracle's bar, and a row's bits are the same at every verify width (the
+    reference's tensor-core matvec keeps that law within its family: tests/kernels/test_card_kernels.py:513-524)"""
+    w = weights_bf16(R, C, seed=112).cuda()
+    x = acts_bf16(M, C, seed=113).cuda()
+    y = card.gemv(w, x)
+    check(y, oracle_bf16_out(w.cpu(), x.cpu()))
+    y8 = card.gemv(w, x[:8].contiguous())
+    assert torch.equal(y8.view(torch.int16), y[:8].view(torch.int16))
+    # the vector-ALU form of the same pass agrees to the same bar and equals the one-row pass bit for bit
+    card.set_tuning("gemv_no_mfma", 1)
+    try:
+        v = card.gemv(w, x)
+        solo = card.gemv(w, x[M - 1 :].contiguous())
+    finally:
+        card.set_tuning("gemv_no_mfma", -1)
+    check(v, oracle_bf16_out(w.cpu(), x.cpu()))
+    assert torch.equal(solo[0].view(torch.int16), v[M - 1].view(torch.int16))
 
 
 def test_repeat_runs_are_bit_stable(card):

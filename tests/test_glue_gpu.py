@@ -1,0 +1,125 @@
+"""The decode step's kernels between the matvecs, each against its numpy restatement in oracle/decode.py.
+
+Elementwise kernels round to bf16 where the reference's card kernels do; their f32 intermediates (rsqrt, exp) may
+differ from numpy's in the last bit, which can flip a bf16 rounding: outputs are held to one bf16 ulp (2^-7 relative,
+elementwise, plus an absolute floor of one ulp of the row's largest value). Attention is held to the reference's own
+yardstick, the worst relative error against f64 (native/tests/common/refs.rs:202-211), at the full 4096-key context."""
+
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import codecs
+from oracle import decode as od
+
+from .helpers import acts_bf16, bits16, gen, weights_bf16
+
+pytestmark = pytest.mark.gpu
+
+
+def ulp_close(got: torch.Tensor, want: np.ndarray, ulps: float = 1.0) -> None:
+    g = got.float().cpu().numpy().reshape(want.shape)
+    tol = ulps * 2.0**-7 * (np.abs(want) + np.abs(want).max() * 2.0**-7)
+    bad = np.abs(g - want) > tol
+    assert not bad.any(), (int(bad.sum()), float(np.abs(g - want).max()))
+
+
+@pytest.mark.parametrize("T,H", [(1, 2560), (3, 2048), (2, 100)])
+@pytest.mark.parametrize("with_y", [True, False])
+def test_add_rmsnorm(card, T, H, with_y):
+    h = acts_bf16(T, H, seed=600)
+    y = acts_bf16(T, H, seed=601) if with_y else None
+    w = (1.0 + 0.1 * torch.randn(H, generator=gen(602))).to(torch.bfloat16)
+    hg, x = h.clone().cuda(), torch.empty(T, H, dtype=torch.bfloat16, device="cuda")
+    card.add_rmsnorm(hg, None if y is None else y.cuda(), w.cuda(), 1e-6, x)
+    h2, want = od.add_rmsnorm(h.float().numpy(), None if y is None else y.float().numpy(), bits16(w), 1e-6)
+    assert np.array_equal(hg.float().cpu().numpy(), h2)          # the residual add is exact bf16 arithmetic
+    ulp_close(x, want)
+
+
+@pytest.mark.parametrize("T", [1, 3])
+def test_norm_rope_kv(card, T):
+    Hq, Hk, D, cap, n0 = 8, 2, 128, 64, 37
+    qkv = acts_bf16(T, (Hq + 2 * Hk) * D, seed=610)
+    wq = (1.0 + 0.1 * torch.randn(D, generator=gen(611))).to(torch.bfloat16)
+    wk = (1.0 + 0.1 * torch.randn(D, generator=gen(612))).to(torch.bfloat16)
+    from btb_amd.decode import StackConfig, rope_tables
+
+    cfg = StackConfig(layers=1, hidden=256, q_heads=Hq, kv_heads=Hk, head_dim=D, intermediate=256, vocab=256)
+    cos, sin = rope_tables(cfg, cap, "cuda")
+    ocos, osin = od.rope_tables(D, cfg.rope_theta, cap)
+    ulp_close(cos, ocos)   # the two tables agree to a rounding of cos / sin
+    K = torch.zeros(Hk, cap, D, dtype=torch.bfloat16, device="cuda")
+    V = torch.zeros_like(K)
+    q = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    card.norm_rope_kv(qkv.cuda(), wq.cuda(), wk.cuda(), 1e-6, cos, sin, n0t, K, V, q, Hq, Hk, D)
+    cosn, sinn = cos.float().cpu().numpy(), sin.float().cpu().numpy()
+    for t in range(T):
+        row = qkv[t].float().numpy()
+        wantq = od.norm_rope(row[: Hq * D].reshape(Hq, D), bits16(wq), 1e-6, cosn[n0 + t], sinn[n0 + t])
+        wantk = od.norm_rope(row[Hq * D : (Hq + Hk) * D].reshape(Hk, D), bits16(wk), 1e-6, cosn[n0 + t], sinn[n0 + t])
+        ulp_close(q[t], wantq, 2.0)
+        ulp_close(K[:, n0 + t], wantk, 2.0)
+        assert np.array_equal(V[:, n0 + t].float().cpu().numpy().reshape(-1), row[(Hq + Hk) * D :])  # v rows copied
+    assert torch.all(K[:, :n0] == 0) and torch.all(K[:, n0 + T :] == 0)                              # nothing else written
+
+
+@pytest.mark.parametrize("n0,T,Hq,Hk,S", [(4096, 1, 32, 8, 64), (100, 1, 32, 8, 4), (0, 1, 8, 8, 1), (63, 3, 16, 2, 7),
+                                           (500, 1, 8, 1, 16)])
+def test_attn_decode_against_f64(card, n0, T, Hq, Hk, S):
+    D = 128
+    cap = n0 + T + 5
+    g = gen(620 + n0)
+    K = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    V = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    q = torch.randn(T, Hq * D, generator=g).to(torch.bfloat16)
+    att = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+    scratch, cnt = card.attn_scratch(T, Hq, Hk, D, S)
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    scale = 1.0 / np.sqrt(D)
+    for rep in range(2):  # the arrival counts are left zero: a second launch gives the same bits
+        card.attn_decode(q.cuda(), K.cuda(), V.cuda(), att, n0t, Hq, Hk, D, scale, S, scratch, cnt)
+        got = att.clone()
+        if rep:
+            assert torch.equal(got, first)
+        first = got
+    assert torch.all(cnt == 0)
+    for t in range(T):
+        want = od.attention(q[t].float().numpy().reshape(Hq, D), K[:, : n0 + t + 1].float().numpy(),
+                            V[:, : n0 + t + 1].float().numpy(), scale)
+        g_ = got[t].float().cpu().numpy().reshape(Hq, D)
+        worst = np.abs(g_ - want).max() / np.abs(want).max()
+        assert worst <= 2.0**-7, worst
+
+
+def test_silu_mul_and_argmax_and_embed(card):
+    gu = acts_bf16(3, 2 * 768, seed=630)
+    m = torch.empty(3, 768, dtype=torch.bfloat16, device="cuda")
+    card.silu_mul(gu.cuda(), m)
+    ulp_close(m, od.silu_mul(gu.float().numpy()), 2.0)
+    logits = acts_bf16(2, 151936, seed=631)
+    logits[0, 777] = logits[0, 99999] = 30.0   # a tie: the lower index wins
+    logits[1, 151935] = 31.0
+    out = torch.zeros(2, dtype=torch.int32, device="cuda")
+    card.argmax(logits.cuda(), out)
+    assert out.tolist() == [777, 151935]
+    table = weights_bf16(1000, 64, seed=632).cuda()
+    ids = torch.tensor([5, 999, 0], dtype=torch.int32, device="cuda")
+    h = torch.zeros(3, 64, dtype=torch.bfloat16, device="cuda")
+    card.embed(table, ids, h)
+    assert torch.equal(h, table[ids.long()])
+
+
+def test_publish(card):
+    n0 = torch.tensor([41], dtype=torch.int32, device="cuda")
+    picked = torch.tensor([1234], dtype=torch.int32, device="cuda")
+    nxt = torch.zeros(1, dtype=torch.int32, device="cuda")
+    tok = torch.zeros(1, dtype=torch.int32).pin_memory()
+    ln = torch.zeros(1, dtype=torch.int32).pin_memory()
+    ts = torch.zeros(1, dtype=torch.int64).pin_memory()
+    card.publish(n0, picked, nxt, tok, ln, ts)
+    torch.cuda.synchronize()
+    assert int(tok[0]) == 1234 and int(ln[0]) == 42 and int(n0[0]) == 42 and int(nxt[0]) == 1234 and int(ts[0]) != 0
