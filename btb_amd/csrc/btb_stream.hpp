@@ -8,10 +8,23 @@
 namespace btb {
 
 // ------------------------------------------------------------------------------------------------------------
-// x staging: [M, C] bf16 into LDS as packed pairs, plain or through the SwiGLU fold
+// x staging: the M rows of x into LDS as packed bf16 pairs - copied as they are, made by the SwiGLU fold from a
+// [M, 2C] gate/up block, or made by the residual add + RMSNorm from the residual stream
 // ------------------------------------------------------------------------------------------------------------
 
-enum XMode { X_PLAIN = 0, X_SILU = 1 };
+enum XMode { X_PLAIN = 0, X_SILU = 1, X_ADDNORM = 2 };
+
+// where x comes from. X_PLAIN: x [M, C]. X_SILU: x is gu [M, 2C]. X_ADDNORM: x is the residual h [M, C]; y the block
+// output added to it (or null), norm_w the norm's weight, h_out where the new residual is written (not h itself:
+// other workgroups are still reading it).
+struct XArgs {
+    const uint16_t* x;
+    const uint16_t* y;
+    const uint16_t* norm_w;
+    uint16_t* h_out;
+    float eps;
+    int centered;
+};
 
 // the fold the reference's btb_gemv_silu_bf16 makes in its x load (native/cuda/btb_kernels.cu:168-209):
 // x = bf16(bf16(silu(g)) * u), g and u the two halves of a [M, 2C] row
@@ -23,22 +36,60 @@ __device__ __forceinline__ uint32_t silu_pair(uint32_t g2, uint32_t u2) {
     return lo | (hi << 16);
 }
 
+// sum over a 256-thread block in a fixed order: each wave's DPP tree, then waves 0..3 in order
+__device__ __forceinline__ float block_sum256(float v, float* red) {
+    v = group_sum<64>(v);
+    const int wv = threadIdx.x >> 6;
+    if ((threadIdx.x & 63) == 0) red[wv] = v;
+    __syncthreads();
+    const float s = ((red[0] + red[1]) + red[2]) + red[3];
+    __syncthreads();
+    return s;
+}
+
+// Leaves the rows in xs (a barrier included). 256 threads.
 template <int XMODE>
-__device__ __forceinline__ void stage_x(uint32_t* xs, const uint16_t* x, int M, int C) {
+__device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C) {
     const int tid = threadIdx.x, nt = blockDim.x;
     if (XMODE == X_PLAIN) {
-        const uint4* src = reinterpret_cast<const uint4*>(x);
+        const uint4* src = reinterpret_cast<const uint4*>(a.x);
         uint4* dst = reinterpret_cast<uint4*>(xs);
         const int n = M * C / 8;
         for (int i = tid; i < n; i += nt) dst[i] = src[i];
-    } else {
+    } else if (XMODE == X_SILU) {
         const int half = C / 2;  // pairs per row
-        const uint32_t* src = reinterpret_cast<const uint32_t*>(x);
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(a.x);
         for (int i = tid; i < M * half; i += nt) {
             const int m = i / half, c = i - m * half;
             xs[i] = silu_pair(src[(size_t)m * 2 * half + c], src[(size_t)m * 2 * half + half + c]);
         }
+    } else {
+        // h' = bf16(h + y); x = bf16(h' * rsqrt(mean(h'^2) + eps) * w): the arithmetic and the summation order of the
+        // stand-alone add_rmsnorm kernel (thread i takes elements i, i + 256, ...), so the bits are its bits. Every
+        // workgroup makes the whole row for itself; the first also writes the new residual out.
+        __shared__ float red[4];
+        uint16_t* xs16 = reinterpret_cast<uint16_t*>(xs);
+        for (int m = 0; m < M; ++m) {
+            const uint16_t* hr = a.x + (size_t)m * C;
+            const uint16_t* yr = a.y == nullptr ? nullptr : a.y + (size_t)m * C;
+            uint16_t* row = xs16 + (size_t)m * C;
+            float ss = 0.f;
+            for (int i = tid; i < C; i += 256) {
+                float hv = bf16_f32(hr[i]);
+                if (yr != nullptr) hv = bfround(hv + bf16_f32(yr[i]));
+                row[i] = f32_bf16(hv);
+                ss = fmaf(hv, hv, ss);
+            }
+            const float rstd = rsqrtf(block_sum256(ss, red) / (float)C + a.eps);
+            for (int i = tid; i < C; i += 256) {
+                const uint16_t hb = row[i];
+                if (blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr) a.h_out[(size_t)m * C + i] = hb;
+                const float wv = bf16_f32(a.norm_w[i]);
+                row[i] = f32_bf16(bf16_f32(hb) * rstd * (a.centered ? 1.f + wv : wv));
+            }
+        }
     }
+    __syncthreads();
 }
 
 // ------------------------------------------------------------------------------------------------------------

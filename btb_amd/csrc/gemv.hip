@@ -23,37 +23,44 @@ namespace btb {
 // the kernel
 // ------------------------------------------------------------------------------------------------------------
 
-template <class F, int M, int LPR, int RPW, int U, int XMODE, int XSRC>
-__global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, const uint16_t* __restrict__ x,
-                                                   uint16_t* __restrict__ y, int R, int C) {
+// what a finished pair of row sums becomes. E_PLAIN: y[m][r] = bf16(sum). E_GLU: the matrix is [2I, C], gate rows then
+// up rows; a wave works on gate row r and up row I + r together and writes m[m][r] = bf16(bf16(silu(g)) * u) with
+// g, u the two sums rounded to bf16 first - the values the gate_up matvec followed by btb_silu_mul would have
+// written (the reference's btb_gemv_mma_glu_silu does the same fold: native/cuda/btb_gemv_mma.cuh:216-315).
+enum Epilogue { E_PLAIN = 0, E_GLU = 1 };
+
+template <class F, int M, int LPR, int RPW, int U, int XMODE, int EPI>
+__global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs xa, uint16_t* __restrict__ y, int R, int C) {
     extern __shared__ __align__(16) uint32_t xs[];  // [M][C / 2] packed bf16 pairs
+    static_assert(EPI == E_PLAIN || RPW == 2, "the GLU form pairs a gate row with an up row");
     constexpr int UW = F::UW;
-    constexpr int G = WAVE / LPR;        // rows a wave covers per set
-    constexpr int ROWS = G * RPW;        // rows a wave covers per tile
+    constexpr int G = WAVE / LPR;                      // rows a wave covers per set
+    constexpr int ROWS = EPI == E_GLU ? G : G * RPW;   // output rows a wave covers per tile
+    const int Rout = EPI == E_GLU ? R / 2 : R;
     const int units = C / UW;            // units per row
     const int lane = threadIdx.x & (WAVE - 1);
     const int sl = lane % LPR;           // the lane's place among its row's lanes
     const int wave = blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
     const int nwaves = gridDim.x * (blockDim.x / WAVE);
-    const int ntiles = (R + ROWS - 1) / ROWS;
+    const int ntiles = (Rout + ROWS - 1) / ROWS;
     const int span = U * LPR;
     const int xrow4 = C / 8;  // uint4 per row of x
 
-    const uint4* xs4;
-    if (XSRC == XS_LDS) {
-        stage_x<XMODE>(xs, x, M, C);
-        __syncthreads();
-        xs4 = reinterpret_cast<const uint4*>(xs);
-    } else {
-        xs4 = reinterpret_cast<const uint4*>(x);
-    }
+    stage_x<XMODE>(xs, xa, M, C);
+    const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
 
     for (int tile = wave; tile < ntiles; tile += nwaves) {
         typename F::RowCtx ctx[RPW];
-        int rows[RPW];
+        int rows[RPW];   // weight rows
+        int out_row;     // E_GLU: the output row of the pair
 #pragma unroll
         for (int j = 0; j < RPW; ++j) {
-            rows[j] = tile * ROWS + j * G + lane / LPR;
+            if (EPI == E_GLU) {
+                out_row = tile * ROWS + lane / LPR;
+                rows[j] = min(out_row, Rout - 1) + j * Rout;
+            } else {
+                rows[j] = tile * ROWS + j * G + lane / LPR;
+            }
             // a row past the end reads the last row again (no divergence in the stream) and is not written
             ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
         }
@@ -77,13 +84,23 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, const u
         for (int j = 0; j < RPW; ++j)
             F::template tail<M>(p, ctx[j], (size_t)min(rows[j], R - 1), sl, LPR, C,
                                 reinterpret_cast<const uint32_t*>(xs4), acc[j]);
-#pragma unroll
-        for (int j = 0; j < RPW; ++j)
+        if (EPI == E_GLU) {
 #pragma unroll
             for (int m = 0; m < M; ++m) {
-                const float s = group_sum<LPR>(acc[j][m]);
-                if (sl == 0 && rows[j] < R) y[(size_t)m * R + rows[j]] = f32_bf16(s);
+                const float g = bfround(group_sum<LPR>(acc[0][m]));
+                const float u = bfround(group_sum<LPR>(acc[RPW - 1][m]));
+                const float sg = bfround(g / (1.f + expf(-g)));
+                if (sl == 0 && out_row < Rout) y[(size_t)m * Rout + out_row] = f32_bf16(sg * u);
             }
+        } else {
+#pragma unroll
+            for (int j = 0; j < RPW; ++j)
+#pragma unroll
+                for (int m = 0; m < M; ++m) {
+                    const float s = group_sum<LPR>(acc[j][m]);
+                    if (sl == 0 && rows[j] < R) y[(size_t)m * R + rows[j]] = f32_bf16(s);
+                }
+        }
     }
 }
 
@@ -98,101 +115,134 @@ static int lanes_per_row(int units) {
     return 16;
 }
 
-template <class F, int M, int LPR, int RPW, int U, int XMODE, int XSRC>
-static int32_t launch_variant(const typename F::Params& p, const void* x, void* y, int R, int C, hipStream_t st) {
+template <class F, int M, int LPR, int RPW, int U, int XMODE, int EPI>
+static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void* y, int R, int C, hipStream_t st) {
     constexpr int G = WAVE / LPR;
+    constexpr int ROWS = EPI == E_GLU ? G : G * RPW;
     const DeviceInfo& dev = device_info();
-    const size_t lds = XSRC == XS_LDS ? (size_t)M * C * 2 : 0;
+    const size_t lds = (size_t)M * C * 2;
     if (lds > (size_t)dev.lds_bytes) {
         set_error("gemv: the x rows do not fit LDS");
         return ERR_DOMAIN;
     }
     // Every workgroup stages x once, so the grid is kept to a few workgroups a CU and each wave walks a whole number
     // of tiles (the last wave of the grid may walk fewer): tiles_per_wave is the smallest count that fits the cap.
-    const int ntiles = (R + G * RPW - 1) / (G * RPW);
+    const int Rout = EPI == E_GLU ? R / 2 : R;
+    const int ntiles = (Rout + ROWS - 1) / ROWS;
     int per_cu = tuning("gemv_wgs_per_cu");
-    if (per_cu <= 0) per_cu = 3;
+    if (per_cu <= 0) per_cu = 6;
     const int cap_waves = dev.cus * per_cu * 4;
     const int tiles_per_wave = (ntiles + cap_waves - 1) / cap_waves;
     const int waves = (ntiles + tiles_per_wave - 1) / tiles_per_wave;
     int grid = (waves + 3) / 4;
     if (grid < 1) grid = 1;
-    auto kern = gemv_stream<F, M, LPR, RPW, U, XMODE, XSRC>;
+    auto kern = gemv_stream<F, M, LPR, RPW, U, XMODE, EPI>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
     }
-    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, p, static_cast<const uint16_t*>(x),
-                       static_cast<uint16_t*>(y), R, C);
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, p, xa, static_cast<uint16_t*>(y), R, C);
     return hip_status(hipGetLastError(), "gemv launch");
 }
 
-template <class F, int M, int LPR, int XMODE>
-static int32_t launch_stream(const typename F::Params& p, const void* x, void* y, int R, int C, hipStream_t st) {
+template <class F, int M, int LPR, int XMODE, int EPI>
+static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void* y, int R, int C, hipStream_t st) {
+    if (EPI == E_GLU) return launch_variant<F, M, LPR, 2, (M <= 2 ? 4 : 2), XMODE, E_GLU>(p, xa, y, R, C, st);
     // Rows per wave tile (RPW) and units in flight per row (U), measured on MI355X at the Qwen3-4B shapes: two rows
     // by four units where the matrix has rows enough to give every SIMD several waves that way, else one row by
     // eight units. Neither changes a result bit (a lane's units stay in ascending order).
     const int v = tuning("gemv_variant");
     const bool tall = v >= 0 ? (v == 1) : (R >= 4096 * (WAVE / LPR));
     if (M <= 2) {
-        if (tall) return launch_variant<F, M, LPR, 2, 4, XMODE, XS_LDS>(p, x, y, R, C, st);
-        return launch_variant<F, M, LPR, 1, 8, XMODE, XS_LDS>(p, x, y, R, C, st);
+        if (tall) return launch_variant<F, M, LPR, 2, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+        return launch_variant<F, M, LPR, 1, 8, XMODE, E_PLAIN>(p, xa, y, R, C, st);
     }
-    if (tall) return launch_variant<F, M, LPR, 2, 2, XMODE, XS_LDS>(p, x, y, R, C, st);
-    return launch_variant<F, M, LPR, 1, 4, XMODE, XS_LDS>(p, x, y, R, C, st);
+    if (tall) return launch_variant<F, M, LPR, 2, 2, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+    return launch_variant<F, M, LPR, 1, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
 }
 
-template <class F, int M, int XMODE>
-static int32_t launch_by_lanes(const typename F::Params& p, const void* x, void* y, int R, int C, hipStream_t st) {
+template <class F, int M, int XMODE, int EPI>
+static int32_t launch_by_lanes(const typename F::Params& p, const XArgs& xa, void* y, int R, int C, hipStream_t st) {
     switch (lanes_per_row(C / F::UW)) {
         case 64:
-            return launch_stream<F, M, 64, XMODE>(p, x, y, R, C, st);
+            return launch_stream<F, M, 64, XMODE, EPI>(p, xa, y, R, C, st);
         case 32:
-            return launch_stream<F, M, 32, XMODE>(p, x, y, R, C, st);
+            return launch_stream<F, M, 32, XMODE, EPI>(p, xa, y, R, C, st);
         default:
-            return launch_stream<F, M, 16, XMODE>(p, x, y, R, C, st);
+            return launch_stream<F, M, 16, XMODE, EPI>(p, xa, y, R, C, st);
     }
 }
 
-template <class F, int XMODE>
-static int32_t launch_by_m(const typename F::Params& p, const void* x, void* y, int R, int C, int M, hipStream_t st) {
+template <class F, int XMODE, int EPI>
+static int32_t launch_by_m(const typename F::Params& p, const XArgs& xa, void* y, int R, int C, int M, hipStream_t st) {
     switch (M) {
         case 1:
-            return launch_by_lanes<F, 1, XMODE>(p, x, y, R, C, st);
+            return launch_by_lanes<F, 1, XMODE, EPI>(p, xa, y, R, C, st);
         case 2:
-            return launch_by_lanes<F, 2, XMODE>(p, x, y, R, C, st);
+            return launch_by_lanes<F, 2, XMODE, EPI>(p, xa, y, R, C, st);
         case 3:
-            return launch_by_lanes<F, 3, XMODE>(p, x, y, R, C, st);
+            return launch_by_lanes<F, 3, XMODE, EPI>(p, xa, y, R, C, st);
         case 4:
-            return launch_by_lanes<F, 4, XMODE>(p, x, y, R, C, st);
+            return launch_by_lanes<F, 4, XMODE, EPI>(p, xa, y, R, C, st);
         default:
             return ERR_DOMAIN;
     }
 }
 
 // wider passes run as passes of at most four rows: each row's bits are those of its own one-row pass
-template <class F, int XMODE>
-static int32_t run_rows(const typename F::Params& p, const void* x, void* y, size_t R, size_t C, size_t M,
-                        size_t x_row_elems, hipStream_t st) {
-    const uint16_t* xp = static_cast<const uint16_t*>(x);
+template <class F, int XMODE, int EPI>
+static int32_t run_rows(const typename F::Params& p, XArgs xa, void* y, size_t R, size_t C, size_t M, hipStream_t st) {
+    const size_t x_row = XMODE == X_SILU ? 2 * C : C;
+    const size_t y_row = EPI == E_GLU ? R / 2 : R;
     uint16_t* yp = static_cast<uint16_t*>(y);
     for (size_t m0 = 0; m0 < M; m0 += 4) {
         const int mm = (int)(M - m0 < 4 ? M - m0 : 4);
-        int32_t rc = launch_by_m<F, XMODE>(p, xp + m0 * x_row_elems, yp + m0 * R, (int)R, (int)C, mm, st);
+        int32_t rc = launch_by_m<F, XMODE, EPI>(p, xa, yp + m0 * y_row, (int)R, (int)C, mm, st);
         if (rc != OK) return rc;
+        xa.x += 4 * x_row;
+        if (xa.y != nullptr) xa.y += 4 * C;
+        if (xa.h_out != nullptr) xa.h_out += 4 * C;
     }
     return OK;
 }
+
+static XArgs plain_x(const void* x) { return XArgs{static_cast<const uint16_t*>(x), nullptr, nullptr, nullptr, 0.f, 0}; }
 
 // the matrix-core form of the bf16 matvec (gemv_mfma.hip)
 int32_t gemv_mfma_bf16(const void* w, const void* x, void* y, int R, int C, int M, hipStream_t st);
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+static bool aligned2(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 1u) == 0; }
 
 static int32_t check_dims(size_t R, size_t C, size_t M, size_t uw) {
     if (R == 0 || C == 0 || M == 0) return ERR_DOMAIN;
     if (R > 0x7FFFFFFFu / 4 || C > (1u << 24) || M > 1024 || C % uw != 0) return ERR_DOMAIN;
+    return OK;
+}
+
+// the residual-and-norm arguments of the fused entry points, checked
+static int32_t norm_args(const void* h_in, const void* y, const void* norm_w, float eps, int32_t centered, void* h_out,
+                         XArgs* xa) {
+    if (h_in == nullptr || norm_w == nullptr) return ERR_NULL;
+    if (!(eps >= 0.f) || h_out == h_in) return ERR_DOMAIN;
+    if (!aligned2(h_in) || !aligned2(y) || !aligned2(norm_w) || !aligned2(h_out)) return ERR_DOMAIN;
+    *xa = XArgs{static_cast<const uint16_t*>(h_in), static_cast<const uint16_t*>(y),
+                static_cast<const uint16_t*>(norm_w), static_cast<uint16_t*>(h_out), eps, centered ? 1 : 0};
+    return OK;
+}
+
+static int32_t p12_params(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
+                          size_t n_esc, const void* row_ptr, size_t R, size_t C, FmtP12::Params* p) {
+    if (lo == nullptr || hi4 == nullptr || table == nullptr || row_ptr == nullptr) return ERR_NULL;
+    if (n_esc > 0 && (esc_idx == nullptr || esc_val == nullptr)) return ERR_NULL;
+    if (R * C > 0x7FFFFFFFull) return ERR_DOMAIN;  // the escape indices are int32
+    if (!aligned16(lo) || (reinterpret_cast<uintptr_t>(hi4) & 7u) || (reinterpret_cast<uintptr_t>(row_ptr) & 3u) ||
+        (reinterpret_cast<uintptr_t>(esc_idx) & 3u))
+        return ERR_DOMAIN;
+    *p = FmtP12::Params{static_cast<const uint8_t*>(lo),      static_cast<const uint8_t*>(hi4),
+                        static_cast<const uint8_t*>(table),   static_cast<const int32_t*>(esc_idx),
+                        static_cast<const uint8_t*>(esc_val), static_cast<const int32_t*>(row_ptr)};
     return OK;
 }
 
@@ -206,7 +256,7 @@ int32_t btb_hip_gemv_bf16(const void* w, const void* x, void* y, size_t R, size_
     if (w == nullptr || x == nullptr || y == nullptr) return ERR_NULL;
     int32_t rc = check_dims(R, C, M, FmtBf16::UW);
     if (rc != OK) return rc;
-    if (!aligned16(w) || !aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 1u)) return ERR_DOMAIN;
+    if (!aligned16(w) || !aligned16(x) || !aligned2(y)) return ERR_DOMAIN;
     // the verify widths go to the matrix cores, 32 rows of x a pass; narrower passes stay on the vector ALUs
     if (M >= 8 && C % 32 == 0 && tuning("gemv_no_mfma") <= 0) {
         const uint16_t* xp = static_cast<const uint16_t*>(x);
@@ -219,35 +269,77 @@ int32_t btb_hip_gemv_bf16(const void* w, const void* x, void* y, size_t R, size_
         return OK;
     }
     FmtBf16::Params p{static_cast<const uint4*>(w)};
-    return run_rows<FmtBf16, X_PLAIN>(p, x, y, R, C, M, C, static_cast<hipStream_t>(stream));
+    return run_rows<FmtBf16, X_PLAIN, E_PLAIN>(p, plain_x(x), y, R, C, M, static_cast<hipStream_t>(stream));
 }
 
 int32_t btb_hip_gemv_silu_bf16(const void* w, const void* gu, void* y, size_t R, size_t C, size_t M, void* stream) {
     if (w == nullptr || gu == nullptr || y == nullptr) return ERR_NULL;
     int32_t rc = check_dims(R, C, M, FmtBf16::UW);
     if (rc != OK) return rc;
-    if (!aligned16(w) || !aligned16(gu) || (reinterpret_cast<uintptr_t>(y) & 1u)) return ERR_DOMAIN;
+    if (!aligned16(w) || !aligned16(gu) || !aligned2(y)) return ERR_DOMAIN;
     FmtBf16::Params p{static_cast<const uint4*>(w)};
-    return run_rows<FmtBf16, X_SILU>(p, gu, y, R, C, M, 2 * C, static_cast<hipStream_t>(stream));
+    return run_rows<FmtBf16, X_SILU, E_PLAIN>(p, plain_x(gu), y, R, C, M, static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_gemv_glu_silu_bf16(const void* w, const void* x, void* m, size_t I, size_t C, size_t M, void* stream) {
+    if (w == nullptr || x == nullptr || m == nullptr) return ERR_NULL;
+    int32_t rc = check_dims(2 * I, C, M, FmtBf16::UW);
+    if (rc != OK) return rc;
+    if (!aligned16(w) || !aligned16(x) || !aligned2(m)) return ERR_DOMAIN;
+    FmtBf16::Params p{static_cast<const uint4*>(w)};
+    return run_rows<FmtBf16, X_PLAIN, E_GLU>(p, plain_x(x), m, 2 * I, C, M, static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_gemv_bf16_norm(const void* w, const void* h_in, const void* y, const void* norm_w, float eps,
+                               int32_t centered, void* h_out, void* out, size_t R, size_t C, size_t M, int32_t glu,
+                               void* stream) {
+    if (w == nullptr || out == nullptr) return ERR_NULL;
+    XArgs xa;
+    int32_t rc = norm_args(h_in, y, norm_w, eps, centered, h_out, &xa);
+    if (rc != OK) return rc;
+    rc = check_dims(R, C, M, FmtBf16::UW);
+    if (rc != OK) return rc;
+    if (!aligned16(w) || !aligned2(out) || (glu && R % 2 != 0)) return ERR_DOMAIN;
+    FmtBf16::Params p{static_cast<const uint4*>(w)};
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return glu ? run_rows<FmtBf16, X_ADDNORM, E_GLU>(p, xa, out, R, C, M, st)
+               : run_rows<FmtBf16, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, st);
 }
 
 int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
                          size_t n_esc, const void* row_ptr, const void* x, void* y, size_t R, size_t C, size_t M,
                          void* stream) {
-    if (lo == nullptr || hi4 == nullptr || table == nullptr || row_ptr == nullptr || x == nullptr || y == nullptr)
+    if (x == nullptr || y == nullptr || lo == nullptr || hi4 == nullptr || table == nullptr || row_ptr == nullptr)
         return ERR_NULL;
     if (n_esc > 0 && (esc_idx == nullptr || esc_val == nullptr)) return ERR_NULL;
     int32_t rc = check_dims(R, C, M, FmtP12::UW);
     if (rc != OK) return rc;
-    if (R * C > 0x7FFFFFFFull) return ERR_DOMAIN;  // the escape indices are int32
-    if (!aligned16(lo) || (reinterpret_cast<uintptr_t>(hi4) & 7u) || !aligned16(x) ||
-        (reinterpret_cast<uintptr_t>(row_ptr) & 3u) || (reinterpret_cast<uintptr_t>(esc_idx) & 3u) ||
-        (reinterpret_cast<uintptr_t>(y) & 1u))
-        return ERR_DOMAIN;
-    FmtP12::Params p{static_cast<const uint8_t*>(lo),       static_cast<const uint8_t*>(hi4),
-                     static_cast<const uint8_t*>(table),    static_cast<const int32_t*>(esc_idx),
-                     static_cast<const uint8_t*>(esc_val),  static_cast<const int32_t*>(row_ptr)};
-    return run_rows<FmtP12, X_PLAIN>(p, x, y, R, C, M, C, static_cast<hipStream_t>(stream));
+    FmtP12::Params p;
+    rc = p12_params(lo, hi4, table, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
+    if (rc != OK) return rc;
+    if (!aligned16(x) || !aligned2(y)) return ERR_DOMAIN;
+    return run_rows<FmtP12, X_PLAIN, E_PLAIN>(p, plain_x(x), y, R, C, M, static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table, const void* esc_idx,
+                              const void* esc_val, size_t n_esc, const void* row_ptr, const void* h_in, const void* y,
+                              const void* norm_w, float eps, int32_t centered, void* h_out, void* out, size_t R,
+                              size_t C, size_t M, int32_t glu, void* stream) {
+    if (out == nullptr) return ERR_NULL;
+    FmtP12::Params p;
+    XArgs xa;
+    int32_t rc = norm_args(h_in, y, norm_w, eps, centered, h_out, &xa);
+    if (rc == ERR_NULL) return rc;
+    const int32_t rp = p12_params(lo, hi4, table, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
+    if (rp == ERR_NULL) return rp;
+    if (rc != OK) return rc;
+    if (rp != OK) return rp;
+    rc = check_dims(R, C, M, FmtP12::UW);
+    if (rc != OK) return rc;
+    if (!aligned2(out) || (glu && R % 2 != 0)) return ERR_DOMAIN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    return glu ? run_rows<FmtP12, X_ADDNORM, E_GLU>(p, xa, out, R, C, M, st)
+               : run_rows<FmtP12, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, st);
 }
 
 int32_t btb_hip_gemv_fp8(const void* w, const void* scales, size_t sr, size_t sc, const void* x, void* y, size_t R,
@@ -257,13 +349,11 @@ int32_t btb_hip_gemv_fp8(const void* w, const void* scales, size_t sr, size_t sc
     int32_t rc = check_dims(R, C, M, FmtF8::UW);
     if (rc != OK) return rc;
     if (R % sr != 0 || C % sc != 0 || (C / sc) % FmtF8::UW != 0) return ERR_DOMAIN;
-    if (!aligned16(w) || !aligned16(x) || (reinterpret_cast<uintptr_t>(scales) & 3u) ||
-        (reinterpret_cast<uintptr_t>(y) & 1u))
-        return ERR_DOMAIN;
+    if (!aligned16(w) || !aligned16(x) || (reinterpret_cast<uintptr_t>(scales) & 3u) || !aligned2(y)) return ERR_DOMAIN;
     const uint32_t upb = (uint32_t)(C / sc / FmtF8::UW);
     FmtF8::Params p{static_cast<const uint8_t*>(w), static_cast<const float*>(scales), (int)sc, (int)(R / sr),
                     (int)upb, upb > 1 ? (uint32_t)(0x100000000ull / upb + 1) : 0u};
-    return run_rows<FmtF8, X_PLAIN>(p, x, y, R, C, M, C, static_cast<hipStream_t>(stream));
+    return run_rows<FmtF8, X_PLAIN, E_PLAIN>(p, plain_x(x), y, R, C, M, static_cast<hipStream_t>(stream));
 }
 
 int32_t btb_hip_gemv_mxfp4(const void* blocks, const void* scales, const void* x, void* y, size_t R, size_t C, size_t M,
@@ -271,9 +361,9 @@ int32_t btb_hip_gemv_mxfp4(const void* blocks, const void* scales, const void* x
     if (blocks == nullptr || scales == nullptr || x == nullptr || y == nullptr) return ERR_NULL;
     int32_t rc = check_dims(R, C, M, FmtMx4::UW);
     if (rc != OK) return rc;
-    if (!aligned16(blocks) || !aligned16(x) || (reinterpret_cast<uintptr_t>(y) & 1u)) return ERR_DOMAIN;
+    if (!aligned16(blocks) || !aligned16(x) || !aligned2(y)) return ERR_DOMAIN;
     FmtMx4::Params p{static_cast<const uint8_t*>(blocks), static_cast<const uint8_t*>(scales)};
-    return run_rows<FmtMx4, X_PLAIN>(p, x, y, R, C, M, C, static_cast<hipStream_t>(stream));
+    return run_rows<FmtMx4, X_PLAIN, E_PLAIN>(p, plain_x(x), y, R, C, M, static_cast<hipStream_t>(stream));
 }
 
 }  // extern "C"

@@ -13,22 +13,12 @@
 // Every reduction runs in an order fixed by the element's index alone, so a replayed graph repeats its bits.
 
 #include "btb_common.hpp"
+#include "btb_stream.hpp"
 #include "btb_tuning.hpp"
 
 #include "../../include/btb_hip.h"
 
 namespace btb {
-
-// sum over a 256-thread block in a fixed order: each wave's DPP tree, then waves 0..3 in order
-__device__ __forceinline__ float block_sum256(float v, float* red) {
-    v = group_sum<64>(v);
-    const int wv = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) red[wv] = v;
-    __syncthreads();
-    const float s = ((red[0] + red[1]) + red[2]) + red[3];
-    __syncthreads();
-    return s;
-}
 
 __global__ void __launch_bounds__(256) embed_kernel(const uint4* __restrict__ table, const int32_t* __restrict__ ids,
                                                     uint4* __restrict__ h, int H8, int vocab) {
@@ -126,18 +116,12 @@ __global__ void __launch_bounds__(64) norm_rope_kv_kernel(const uint16_t* __rest
 constexpr int ATT_D = 128;
 constexpr int ATT_MAXG = 8;
 
-// a value another workgroup wrote in this launch: read at device scope, past this CU's vector cache
-__device__ __forceinline__ float peek(const float* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
 template <int G>
 __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ K,
                                                           const uint16_t* __restrict__ V, uint16_t* __restrict__ att,
                                                           const int32_t* __restrict__ n0p, int Hq, int Hk, long long hs,
-                                                          long long rs, float scale_log2, float* __restrict__ part_m,
-                                                          float* __restrict__ part_l, float* __restrict__ part_acc,
-                                                          unsigned* __restrict__ cnt, int span) {
+                                                          long long rs, float scale_log2, float* part_m, float* part_l,
+                                                          float* part_acc, unsigned* __restrict__ cnt, int span) {
     constexpr int D = ATT_D;
     __shared__ float s_m[16][G], s_l[16][G];
     __shared__ float s_acc[16][G][D];
@@ -173,26 +157,36 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     }
     const uint16_t* Kh = K + (size_t)g * hs + dl * 8;
     const uint16_t* Vh = V + (size_t)g * hs + dl * 8;
-    for (int key = k_begin + grp; key < k_end; key += 16) {
-        const uint4 kr = *reinterpret_cast<const uint4*>(Kh + (size_t)key * rs);
-        const uint4 vr = *reinterpret_cast<const uint4*>(Vh + (size_t)key * rs);
-        const float kf[8] = {bf16lo_f32(kr.x), bf16hi_f32(kr.x), bf16lo_f32(kr.y), bf16hi_f32(kr.y),
-                             bf16lo_f32(kr.z), bf16hi_f32(kr.z), bf16lo_f32(kr.w), bf16hi_f32(kr.w)};
-        const float vf[8] = {bf16lo_f32(vr.x), bf16hi_f32(vr.x), bf16lo_f32(vr.y), bf16hi_f32(vr.y),
-                             bf16lo_f32(vr.z), bf16hi_f32(vr.z), bf16lo_f32(vr.w), bf16hi_f32(vr.w)};
+    // four keys of the stream a batch: their eight loads are issued together, then the keys are taken in order
+    for (int key0 = k_begin + grp; key0 < k_end; key0 += 64) {
+        uint4 kr[4], vr[4];
 #pragma unroll
-        for (int j = 0; j < G; ++j) {
-            float s = 0.f;
+        for (int b = 0; b < 4; ++b) {
+            const int key = min(key0 + 16 * b, k_end - 1);  // a key past the span's end is loaded again, not used
+            kr[b] = *reinterpret_cast<const uint4*>(Kh + (size_t)key * rs);
+            vr[b] = *reinterpret_cast<const uint4*>(Vh + (size_t)key * rs);
+        }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) s = fmaf(qv[j][e], kf[e], s);
-            s = group_sum<16>(s);
-            const float mn = fmaxf(m[j], s);
-            const float corr = exp2f(m[j] - mn);   // 0 on the stream's first key (m = -inf)
-            const float p = exp2f(s - mn);
-            l[j] = fmaf(l[j], corr, p);
+        for (int b = 0; b < 4; ++b) {
+            if (key0 + 16 * b >= k_end) break;
+            const float kf[8] = {bf16lo_f32(kr[b].x), bf16hi_f32(kr[b].x), bf16lo_f32(kr[b].y), bf16hi_f32(kr[b].y),
+                                 bf16lo_f32(kr[b].z), bf16hi_f32(kr[b].z), bf16lo_f32(kr[b].w), bf16hi_f32(kr[b].w)};
+            const float vf[8] = {bf16lo_f32(vr[b].x), bf16hi_f32(vr[b].x), bf16lo_f32(vr[b].y), bf16hi_f32(vr[b].y),
+                                 bf16lo_f32(vr[b].z), bf16hi_f32(vr[b].z), bf16lo_f32(vr[b].w), bf16hi_f32(vr[b].w)};
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[j][e] = fmaf(p, vf[e], acc[j][e] * corr);
-            m[j] = mn;
+            for (int j = 0; j < G; ++j) {
+                float s = 0.f;
+#pragma unroll
+                for (int e = 0; e < 8; ++e) s = fmaf(qv[j][e], kf[e], s);
+                s = group_sum<16>(s);
+                const float mn = fmaxf(m[j], s);
+                const float corr = exp2f(m[j] - mn);   // 0 on the stream's first key (m = -inf)
+                const float p = exp2f(s - mn);
+                l[j] = fmaf(l[j], corr, p);
+#pragma unroll
+                for (int e = 0; e < 8; ++e) acc[j][e] = fmaf(p, vf[e], acc[j][e] * corr);
+                m[j] = mn;
+            }
         }
     }
     // the 16 streams' states into LDS
@@ -231,17 +225,19 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     __syncthreads();
     if (s_last != (unsigned)(S - 1)) return;
     __threadfence();
+    // (the fence above is the acquire: the other workgroups' states are read with plain loads, several in flight)
     const size_t base = ((size_t)t * Hk + g) * S;
     for (int o = threadIdx.x; o < G * D; o += 256) {
         const int j = o / D, d = o - j * D;
         float M = bits_f32(0xff800000u);
-        for (int s2 = 0; s2 < S; ++s2) M = fmaxf(M, peek(&part_m[(base + s2) * G + j]));
+        for (int s2 = 0; s2 < S; ++s2) M = fmaxf(M, part_m[(base + s2) * G + j]);
         float L = 0.f, A = 0.f;
+#pragma unroll 8
         for (int s2 = 0; s2 < S; ++s2) {
-            const float pm = peek(&part_m[(base + s2) * G + j]);
+            const float pm = part_m[(base + s2) * G + j];
             const float f = pm == bits_f32(0xff800000u) ? 0.f : exp2f(pm - M);
-            L = fmaf(peek(&part_l[(base + s2) * G + j]), f, L);
-            A = fmaf(peek(&part_acc[((base + s2) * G + j) * D + d]), f, A);
+            L = fmaf(part_l[(base + s2) * G + j], f, L);
+            A = fmaf(part_acc[((base + s2) * G + j) * D + d], f, A);
         }
         att[((size_t)t * Hq + (size_t)g * G + j) * D + d] = f32_bf16(A * (1.f / L));
     }

@@ -131,8 +131,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
     F::Params p{stack + (size_t)expert * R * units};
     uint16_t* y = gu + (size_t)pair * R;
 
-    stage_x<X_PLAIN>(xs, x + (size_t)token * C, 1, C);
-    __syncthreads();
+    stage_x<X_PLAIN>(xs, XArgs{x + (size_t)token * C, nullptr, nullptr, nullptr, 0.f, 0}, 1, C);
     const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
     for (int tile = wave; tile < ntiles; tile += nwaves) {
         F::RowCtx ctx[RPW];
@@ -202,9 +201,9 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__
     __syncthreads();
     for (int q = 0; q < k; ++q) {
         const int j = s_expert[q] >> 20;
-        stage_x<X_SILU>(hs + (size_t)q * (C / 2), gu + ((size_t)token * k + j) * 2 * C, 1, C);
+        stage_x<X_SILU>(hs + (size_t)q * (C / 2), XArgs{gu + ((size_t)token * k + j) * 2 * C, nullptr, nullptr, nullptr, 0.f, 0},
+                        1, C);
     }
-    __syncthreads();
     const uint4* hs4 = reinterpret_cast<const uint4*>(hs);
 
     for (int tile = wave; tile < ntiles; tile += nwaves) {

@@ -3,8 +3,10 @@
 for a Qwen3-shaped stack with every weight resident in VRAM, in bf16 or in the 12-bit packed form.
 
 Per layer, as the reference sequences it: add_rmsnorm -> qkv matvec -> q/k norm + rope + cache write -> decode
-attention -> o matvec -> add_rmsnorm -> gate_up matvec -> down matvec with the SwiGLU fold in its x load; then the
-final norm, the head matvec, the greedy pick and the publish. `DecodeStep.capture()` records the whole step with
+attention -> o matvec -> add_rmsnorm -> gate_up matvec -> activation -> down matvec; then the final norm, the head
+matvec, the greedy pick and the publish. The default (`fused`) form issues the same arithmetic in six launches a
+layer instead of eight: every add_rmsnorm rides in the following matvec's x load and gate / up / activation are one
+kernel. `DecodeStep.capture()` records the whole step with
 torch's graph capture (a hipGraph on ROCm); afterwards the host only replays it and reads the token from pinned
 memory.
 """
@@ -88,12 +90,13 @@ class DecodeStep:
     (`Linear`), `embed` (bf16 [V, H]), `norm` and `head` (`Linear`)."""
 
     def __init__(self, card: Any, cfg: StackConfig, weights: dict[str, Any], cap: int, T: int = 1,
-                 attn_spans: int | None = None, fold_silu: bool = True) -> None:
+                 attn_spans: int | None = None, fold_silu: bool = True, fused: bool = True) -> None:
         dev = torch.device("cuda")
         self.card, self.cfg, self.w, self.cap, self.T = card, cfg, weights, int(cap), int(T)
         H, D, Hq, Hk, I = cfg.hidden, cfg.head_dim, cfg.q_heads, cfg.kv_heads, cfg.intermediate
         bf = dict(dtype=torch.bfloat16, device=dev)
         self.h = torch.zeros(T, H, **bf)
+        self.h2 = torch.zeros(T, H, **bf)
         self.x = torch.zeros(T, H, **bf)
         self.y = torch.zeros(T, H, **bf)
         self.qkv = torch.zeros(T, cfg.qkv_rows, **bf)
@@ -109,12 +112,13 @@ class DecodeStep:
         self.kv = torch.zeros(cfg.layers, 2, Hk, self.cap, D, **bf)
         self.cos, self.sin = rope_tables(cfg, self.cap, dev)
         self.scale = 1.0 / math.sqrt(D)
-        # key spans: enough workgroups (kv heads x spans) to cover the CUs about twice, a span at least 64 keys
+        # key spans: enough workgroups (kv heads x spans) to cover the CUs once, a span at least 64 keys
         if attn_spans is None:
-            attn_spans = max(1, min(self.cap // 64, (2 * card.sms + Hk - 1) // Hk))
+            attn_spans = max(1, min(self.cap // 64, (card.sms + Hk - 1) // Hk))
         self.S = int(attn_spans)
         self.scratch, self.cnt = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
         self.fold_silu = bool(fold_silu)
+        self.fused = bool(fused)
         # the handoff to the host: token, cache length and the GPU's clock in pinned memory
         self.host_tok = torch.zeros(1, dtype=torch.int32).pin_memory()
         self.host_n0 = torch.zeros(1, dtype=torch.int32).pin_memory()
@@ -142,6 +146,13 @@ class DecodeStep:
     # -- the kernel sequence ---------------------------------------------------------------------------------------
 
     def body(self) -> None:
+        if self.fused:
+            self._body_fused()
+        else:
+            self._body_plain()
+
+    def _body_plain(self) -> None:
+        """one launch per operator, in the reference's order (btb/engine/cuda.py:1722-1834)"""
         k, cfg, w = self.card, self.cfg, self.w
         Hq, Hk, D = cfg.q_heads, cfg.kv_heads, cfg.head_dim
         k.embed(w["embed"], self.ids, self.h)
@@ -166,6 +177,30 @@ class DecodeStep:
             y_prev = self.y
         k.add_rmsnorm(self.h, y_prev, w["norm"], cfg.eps, self.x)
         w["head"].matvec(self.x, self.logits)
+        k.argmax(self.logits, self.picked)
+        k.publish(self.n0, self.picked, self.ids, self.host_tok, self.host_n0, self.host_ts)
+
+    def _body_fused(self) -> None:
+        """the same arithmetic in fewer launches: each residual add + norm rides in the x load of the matvec that
+        follows it (the residual ping-pongs between two buffers), gate / up / activation are one kernel. Bit for bit
+        the plain sequence's result."""
+        k, cfg, w = self.card, self.cfg, self.w
+        Hq, Hk, D = cfg.q_heads, cfg.kv_heads, cfg.head_dim
+        ha, hb = self.h, self.h2
+        k.embed(w["embed"], self.ids, ha)
+        y_prev = None
+        for i in range(cfg.layers):
+            L = f"layers.{i}."
+            K, V = self.kv[i, 0], self.kv[i, 1]
+            k.gemv_norm(w[L + "qkv"].w, ha, y_prev, w[L + "ln1"], cfg.eps, hb, self.qkv)
+            k.norm_rope_kv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K, V,
+                           self.q, Hq, Hk, D)
+            k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch, self.cnt)
+            w[L + "o"].matvec(self.att, self.y)
+            k.gemv_norm(w[L + "gu"].w, hb, self.y, w[L + "ln2"], cfg.eps, ha, self.m, glu=True)
+            w[L + "down"].matvec(self.m, self.y)
+            y_prev = self.y
+        k.gemv_norm(w["head"].w, ha, y_prev, w["norm"], cfg.eps, None, self.logits)
         k.argmax(self.logits, self.picked)
         k.publish(self.n0, self.picked, self.ids, self.host_tok, self.host_n0, self.host_ts)
 

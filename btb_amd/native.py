@@ -34,6 +34,10 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_set_tuning": (_i32, [ctypes.c_char_p, _i32]),
     "btb_hip_gemv_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_gemv_silu_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_gemv_glu_silu_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_gemv_bf16_norm": (_i32, [_vp, _vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp, _sz, _sz, _sz, _i32, _vp]),
+    "btb_hip_gemv_p12_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp,
+                                     _sz, _sz, _sz, _i32, _vp]),
     "btb_hip_gemv_p12": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_p12_row_ptr": (_i32, [_vp, _sz, _sz, _sz, _vp, _vp]),
     "btb_hip_p12_widen": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _vp, _vp]),
@@ -155,6 +159,48 @@ class HipCard:
         self._call("btb_hip_gemv_silu_bf16", self.ptr(w), self.ptr(g2), self.ptr(y), R, C, M, _stream())
         return y
 
+
+    def gemv_glu_silu(self, w: torch.Tensor, x: torch.Tensor, m: torch.Tensor | None = None) -> torch.Tensor:
+        """m [M, I] = bf16(bf16(silu(g)) * u) with [g, u] = x @ w^T, w [2I, C]: gate, up and the activation in one
+        kernel (`btb_gemv_mma_glu_silu`)"""
+        self._need(w, torch.bfloat16, "w")
+        self._need(x, torch.bfloat16, "x")
+        R, C = (int(s) for s in w.shape)
+        x2 = x.reshape(-1, C)
+        M = int(x2.shape[0])
+        m = self._out(m, M, R // 2, x.device, "gemv_glu_silu")
+        self._call("btb_hip_gemv_glu_silu_bf16", self.ptr(w), self.ptr(x2), self.ptr(m), R // 2, C, M, _stream())
+        return m
+
+    def gemv_norm(self, w: Any, h_in: torch.Tensor, y: torch.Tensor | None, norm_w: torch.Tensor, eps: float,
+                  h_out: torch.Tensor | None, out: torch.Tensor, glu: bool = False, centered: bool = False) -> torch.Tensor:
+        """out = W . rmsnorm(h_in + y) with the add and the norm folded into the matvec's x load; the new residual
+        goes to `h_out` (a different tensor than `h_in`). `w` is a bf16 matrix or a `P12Weight`; `glu` folds the
+        SwiGLU activation into the epilogue (out is then [M, R / 2])."""
+        for t, what in ((h_in, "h_in"), (norm_w, "norm_w"), (out, "out")):
+            self._need(t, torch.bfloat16, what)
+        for t, what in ((y, "y"), (h_out, "h_out")):
+            if t is not None:
+                self._need(t, torch.bfloat16, what)
+        R, C = (int(s) for s in w.shape)
+        M = int(h_in.numel()) // C
+        if h_in.numel() != M * C or norm_w.numel() != C or out.numel() != M * (R // 2 if glu else R) \
+                or (y is not None and y.numel() != M * C) or (h_out is not None and h_out.numel() != M * C):
+            raise ValueError("[hip] gemv_norm: the rows, the norm weight and the output do not fit the matrix")
+        if h_out is not None and h_out.data_ptr() == h_in.data_ptr():
+            raise ValueError("[hip] gemv_norm: the new residual cannot be written over the one being read")
+        p = lambda t: None if t is None else self.ptr(t)
+        if isinstance(w, torch.Tensor):
+            self._need(w, torch.bfloat16, "w")
+            self._call("btb_hip_gemv_bf16_norm", self.ptr(w), self.ptr(h_in), p(y), self.ptr(norm_w), float(eps),
+                       int(centered), p(h_out), self.ptr(out), R, C, M, int(glu), _stream())
+        else:
+            ne = int(w.esc_idx.numel())
+            self._call("btb_hip_gemv_p12_norm", self.ptr(w.lo), self.ptr(w.hi4), self.ptr(w.table),
+                       self.ptr(w.esc_idx) if ne else None, self.ptr(w.esc_val) if ne else None, ne, self.ptr(w.row_ptr),
+                       self.ptr(h_in), p(y), self.ptr(norm_w), float(eps), int(centered), p(h_out), self.ptr(out), R, C,
+                       M, int(glu), _stream())
+        return out
 
     # -- the stored forms ---------------------------------------------------------------------------------------
 

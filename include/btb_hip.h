@@ -64,6 +64,20 @@ int32_t btb_hip_gemv_bf16(const void* w, const void* x, void* y, size_t R, size_
  * x[m][c] = bf16(bf16(silu(g)) * u). Replaces btb_gemv_silu_bf16_m{M} (native/cuda/btb_kernels.cu:168-227). */
 int32_t btb_hip_gemv_silu_bf16(const void* w, const void* gu, void* y, size_t R, size_t C, size_t M, void* stream);
 
+/* Gate, up and the activation in one kernel: w [2I, C] bf16 (gate rows, then up rows), x [M, C], m [M, I] =
+ * bf16(bf16(silu(g)) * u) with g = bf16(w[i] . x), u = bf16(w[I + i] . x): the bits of btb_hip_gemv_bf16 followed by
+ * btb_hip_silu_mul. Replaces btb_gemv_mma_glu_silu (native/cuda/btb_gemv_mma.cuh:216-315). */
+int32_t btb_hip_gemv_glu_silu_bf16(const void* w, const void* x, void* m, size_t I, size_t C, size_t M, void* stream);
+
+/* The matvec with the residual add and the RMSNorm folded into its x load: h' = bf16(h_in + y) (y NULL: h' = h_in),
+ * x = bf16(h' * rsqrt(mean(h'^2) + eps) * norm_w) (or * (1 + norm_w) when centered), out = W x; h' is written to
+ * h_out (NULL: not kept; never h_in itself). With glu != 0, W is [R = 2I, C] and out is the gate/up fold m [M, I] of
+ * btb_hip_gemv_glu_silu_bf16. The bits are those of btb_hip_add_rmsnorm followed by the matvec; it replaces that
+ * pair of launches of the reference's step (btb/engine/cuda.py:1730-1733, 1770-1793). */
+int32_t btb_hip_gemv_bf16_norm(const void* w, const void* h_in, const void* y, const void* norm_w, float eps,
+                               int32_t centered, void* h_out, void* out, size_t R, size_t C, size_t M, int32_t glu,
+                               void* stream);
+
 /* ---- the stored weight forms, widened in registers inside the matvec ------------------------------------ */
 
 /* The matvec over a pack12 matrix (n = R * C weights): lo u8[n], hi4 u8[(n + 1) / 2] (weight 2k in the low nibble
@@ -74,6 +88,12 @@ int32_t btb_hip_gemv_silu_bf16(const void* w, const void* gu, void* y, size_t R,
 int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
                          size_t n_esc, const void* row_ptr, const void* x, void* y, size_t R, size_t C, size_t M,
                          void* stream);
+
+/* btb_hip_gemv_bf16_norm over a pack12 matrix (the arrays of btb_hip_gemv_p12). */
+int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table, const void* esc_idx,
+                              const void* esc_val, size_t n_esc, const void* row_ptr, const void* h_in, const void* y,
+                              const void* norm_w, float eps, int32_t centered, void* h_out, void* out, size_t R,
+                              size_t C, size_t M, int32_t glu, void* stream);
 
 /* row_ptr[r] = how many escapes lie below weight r * cols, r = 0..rows: the per-row slices of the escape list the
  * matvec reads. Run once when a packed matrix is uploaded; replaces the per-call search of p12_cursors

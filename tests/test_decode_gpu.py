@@ -56,8 +56,8 @@ def make_weights(card, packed: bool):
     return W, dev, kv
 
 
-def run_gpu(card, dev, kv, graph: bool, fold: bool = True):
-    step = DecodeStep(card, CFG, dev, CAP, fold_silu=fold)
+def run_gpu(card, dev, kv, graph: bool, fold: bool = True, fused: bool = True):
+    step = DecodeStep(card, CFG, dev, CAP, fold_silu=fold, fused=fused)
     step.kv.copy_(kv.cuda())
     step.reset(N0, TOKEN)
     if graph:
@@ -97,6 +97,17 @@ def test_packed_stack_tracks_the_bf16_stack(card):
     assert (a - b).abs().max() <= 3e-2 * a.abs().max()
     c = run_gpu(card, dev_b, kv, graph=False, fold=True).logits.float()
     assert (a - c).abs().max() <= 3e-2 * a.abs().max()   # the SwiGLU fold and the two-kernel form agree
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_fused_launches_change_no_bit(card, packed):
+    """the six-launch layer (norms folded into the matvecs' x loads, gate / up / activation in one kernel) against the
+    one-launch-per-operator sequence: the same bits in the logits, the residual stream and the cache row"""
+    _, dev, kv = make_weights(card, packed)
+    a = run_gpu(card, dev, kv, graph=False, fold=False, fused=False)
+    b = run_gpu(card, dev, kv, graph=False, fused=True)
+    assert torch.equal(a.logits, b.logits) and a.token() == b.token()
+    assert torch.equal(a.kv[:, :, :, N0], b.kv[:, :, :, N0])
 
 
 def test_graph_replays_equal_the_eager_step(card):

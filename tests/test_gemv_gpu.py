@@ -108,6 +108,37 @@ def test_silu_fold_equals_two_steps(card, M):
     assert frac < 0.02, frac
 
 
+@pytest.mark.parametrize("M", [1, 3])
+def test_glu_kernel_equals_matvec_then_silu_mul(card, M):
+    I, C = 9728, 2560
+    w = weights_bf16(2 * I, C, seed=150).cuda()
+    x = acts_bf16(M, C, seed=151).cuda()
+    gu = card.gemv(w, x)
+    want = torch.empty(M, I, dtype=torch.bfloat16, device="cuda")
+    card.silu_mul(gu, want)
+    got = card.gemv_glu_silu(w, x)
+    assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+
+
+@pytest.mark.parametrize("M,with_y,glu", [(1, True, False), (1, False, False), (2, True, True), (1, True, True)])
+def test_norm_folded_into_the_x_load_changes_no_bit(card, M, with_y, glu):
+    R, C = 6144, 2560
+    w = weights_bf16(R, C, seed=160).cuda()
+    h = acts_bf16(M, C, seed=161).cuda()
+    y = acts_bf16(M, C, seed=162).cuda() if with_y else None
+    nw = (1.0 + 0.1 * torch.randn(C, generator=torch.Generator().manual_seed(163))).to(torch.bfloat16).cuda()
+    h1, x1 = h.clone(), torch.empty_like(h)
+    card.add_rmsnorm(h1, y, nw, 1e-6, x1)
+    want = card.gemv_glu_silu(w, x1) if glu else card.gemv(w, x1)
+    h2 = torch.empty_like(h)
+    out = torch.empty(M, R // 2 if glu else R, dtype=torch.bfloat16, device="cuda")
+    card.gemv_norm(w, h, y, nw, 1e-6, h2, out, glu=glu)
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(h2.view(torch.int16), h1.view(torch.int16))
+    with pytest.raises(ValueError):
+        card.gemv_norm(w, h, y, nw, 1e-6, h, out, glu=glu)
+
+
 def test_refusals_launch_nothing(card):
     w = weights_bf16(16, 64, seed=140).cuda()
     x = acts_bf16(1, 64, seed=141).cuda()
