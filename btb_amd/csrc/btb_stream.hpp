@@ -67,25 +67,56 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
         // h' = bf16(h + y); x = bf16(h' * rsqrt(mean(h'^2) + eps) * w): the arithmetic and the summation order of the
         // stand-alone add_rmsnorm kernel (thread i takes elements i, i + 256, ...), so the bits are its bits. Every
         // workgroup makes the whole row for itself; the first also writes the new residual out.
+        // The row's three inputs are requested together, ahead of any arithmetic: one round trip to memory, not three.
         __shared__ float red[4];
         uint16_t* xs16 = reinterpret_cast<uint16_t*>(xs);
+        constexpr int PER = 16;  // elements a thread holds at once: rows up to 4096 wide take one pass
         for (int m = 0; m < M; ++m) {
             const uint16_t* hr = a.x + (size_t)m * C;
             const uint16_t* yr = a.y == nullptr ? nullptr : a.y + (size_t)m * C;
             uint16_t* row = xs16 + (size_t)m * C;
             float ss = 0.f;
-            for (int i = tid; i < C; i += 256) {
-                float hv = bf16_f32(hr[i]);
-                if (yr != nullptr) hv = bfround(hv + bf16_f32(yr[i]));
-                row[i] = f32_bf16(hv);
-                ss = fmaf(hv, hv, ss);
-            }
-            const float rstd = rsqrtf(block_sum256(ss, red) / (float)C + a.eps);
-            for (int i = tid; i < C; i += 256) {
-                const uint16_t hb = row[i];
-                if (blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr) a.h_out[(size_t)m * C + i] = hb;
-                const float wv = bf16_f32(a.norm_w[i]);
-                row[i] = f32_bf16(bf16_f32(hb) * rstd * (a.centered ? 1.f + wv : wv));
+            if (C <= PER * 256) {
+                uint16_t hv16[PER], yv16[PER], wv16[PER];
+#pragma unroll
+                for (int q = 0; q < PER; ++q) {
+                    const int i = tid + q * 256;
+                    hv16[q] = i < C ? hr[i] : (uint16_t)0;
+                    yv16[q] = (i < C && yr != nullptr) ? yr[i] : (uint16_t)0;
+                    wv16[q] = i < C ? a.norm_w[i] : (uint16_t)0;
+                }
+                float hv[PER];
+#pragma unroll
+                for (int q = 0; q < PER; ++q) {
+                    hv[q] = bf16_f32(hv16[q]);
+                    if (yr != nullptr) hv[q] = bfround(hv[q] + bf16_f32(yv16[q]));
+                    if (tid + q * 256 < C) ss = fmaf(hv[q], hv[q], ss);
+                }
+                const float rstd = rsqrtf(block_sum256(ss, red) / (float)C + a.eps);
+#pragma unroll
+                for (int q = 0; q < PER; ++q) {
+                    const int i = tid + q * 256;
+                    if (i < C) {
+                        if (blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr)
+                            a.h_out[(size_t)m * C + i] = f32_bf16(hv[q]);
+                        const float wv = bf16_f32(wv16[q]);
+                        row[i] = f32_bf16(hv[q] * rstd * (a.centered ? 1.f + wv : wv));
+                    }
+                }
+            } else {
+                for (int i = tid; i < C; i += 256) {
+                    float hv = bf16_f32(hr[i]);
+                    if (yr != nullptr) hv = bfround(hv + bf16_f32(yr[i]));
+                    row[i] = f32_bf16(hv);
+                    ss = fmaf(hv, hv, ss);
+                }
+                const float rstd = rsqrtf(block_sum256(ss, red) / (float)C + a.eps);
+                for (int i = tid; i < C; i += 256) {
+                    const uint16_t hb = row[i];
+                    if (blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr) a.h_out[(size_t)m * C + i] = hb;
+                    const float wv = bf16_f32(a.norm_w[i]);
+                    row[i] = f32_bf16(bf16_f32(hb) * rstd * (a.centered ? 1.f + wv : wv));
+                }
             }
         }
     }

@@ -110,22 +110,23 @@ __global__ void __launch_bounds__(64) norm_rope_kv_kernel(const uint16_t* __rest
 // keys four at a time (16 lanes a key, 8 dims a lane: a wave's load covers four whole 256-byte rows). Each 16-lane
 // group keeps an online-softmax state (max, sum, 8 output dims) for each of the G query heads over its own keys, in
 // log2 units (the scale carries log2 e, exp is exp2). The groups' states fold through LDS in a fixed order, the
-// spans' through memory: every workgroup writes its state, and the last to arrive for a (row, kv head) folds the
-// spans in span order, writes bf16(O / L) and resets the arrival count, so the graph replays. G <= 8.
+// spans' through memory: every workgroup writes its state, and a second small kernel folds the spans in span order and
+// writes bf16(O / L). (A last-arriver fold inside one kernel needs a device-scope fence per workgroup; on this GPU the
+// fences of a die's workgroups queue behind one another and cost more than the second launch.) G <= 8.
 // ------------------------------------------------------------------------------------------------------------
 constexpr int ATT_D = 128;
 constexpr int ATT_MAXG = 8;
 
 template <int G>
 __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ K,
-                                                          const uint16_t* __restrict__ V, uint16_t* __restrict__ att,
+                                                          const uint16_t* __restrict__ V,
                                                           const int32_t* __restrict__ n0p, int Hq, int Hk, long long hs,
-                                                          long long rs, float scale_log2, float* part_m, float* part_l,
-                                                          float* part_acc, unsigned* __restrict__ cnt, int span) {
+                                                          long long rs, float scale_log2, float* __restrict__ part_m,
+                                                          float* __restrict__ part_l, float* __restrict__ part_acc,
+                                                          int span) {
     constexpr int D = ATT_D;
     __shared__ float s_m[16][G], s_l[16][G];
     __shared__ float s_acc[16][G][D];
-    __shared__ unsigned s_last;
     const int g = blockIdx.x, sp = blockIdx.y, t = blockIdx.z, S = gridDim.y;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int sub = lane >> 4, dl = lane & 15;   // the lane's key within a quad of keys, its 8 dims
@@ -157,17 +158,18 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     }
     const uint16_t* Kh = K + (size_t)g * hs + dl * 8;
     const uint16_t* Vh = V + (size_t)g * hs + dl * 8;
-    // four keys of the stream a batch: their eight loads are issued together, then the keys are taken in order
-    for (int key0 = k_begin + grp; key0 < k_end; key0 += 64) {
-        uint4 kr[4], vr[4];
+    // eight keys of the stream a batch: their sixteen loads are issued together, then the keys are taken in order
+    constexpr int KB = 8;
+    for (int key0 = k_begin + grp; key0 < k_end; key0 += 16 * KB) {
+        uint4 kr[KB], vr[KB];
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
+        for (int b = 0; b < KB; ++b) {
             const int key = min(key0 + 16 * b, k_end - 1);  // a key past the span's end is loaded again, not used
             kr[b] = *reinterpret_cast<const uint4*>(Kh + (size_t)key * rs);
             vr[b] = *reinterpret_cast<const uint4*>(Vh + (size_t)key * rs);
         }
 #pragma unroll
-        for (int b = 0; b < 4; ++b) {
+        for (int b = 0; b < KB; ++b) {
             if (key0 + 16 * b >= k_end) break;
             const float kf[8] = {bf16lo_f32(kr[b].x), bf16hi_f32(kr[b].x), bf16lo_f32(kr[b].y), bf16hi_f32(kr[b].y),
                                  bf16lo_f32(kr[b].z), bf16hi_f32(kr[b].z), bf16lo_f32(kr[b].w), bf16hi_f32(kr[b].w)};
@@ -218,30 +220,47 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
             part_l[prow * G + j] = L;
         }
     }
-    // the last workgroup in for this (row, kv head) folds the spans
-    __threadfence();
-    __syncthreads();
-    if (threadIdx.x == 0) s_last = atomicAdd(&cnt[(size_t)t * Hk + g], 1u);
-    __syncthreads();
-    if (s_last != (unsigned)(S - 1)) return;
-    __threadfence();
-    // (the fence above is the acquire: the other workgroups' states are read with plain loads, several in flight)
+}
+
+// the spans' states folded in span order: one workgroup per (row, kv head). Launched right after attn_decode_kernel,
+// it reads what that kernel wrote across a kernel boundary, so no fence or arrival count is needed.
+template <int G>
+__global__ void __launch_bounds__(256) attn_merge_kernel(uint16_t* __restrict__ att, int Hq, int Hk, int S,
+                                                         const float* __restrict__ part_m,
+                                                         const float* __restrict__ part_l,
+                                                         const float* __restrict__ part_acc) {
+    constexpr int D = ATT_D;
+    extern __shared__ float f_m[];  // [S][G] maxima, then the factors exp2(m_s - M); then [S][G] sums
+    __shared__ float s_L[G];
+    float* f_l = f_m + S * G;
+    const int g = blockIdx.x, t = blockIdx.y;
     const size_t base = ((size_t)t * Hk + g) * S;
+    for (int o = threadIdx.x; o < S * G; o += 256) {
+        f_m[o] = part_m[base * G + o];
+        f_l[o] = part_l[base * G + o];
+    }
+    __syncthreads();
+    if (threadIdx.x < G) {
+        const int j = threadIdx.x;
+        float M = bits_f32(0xff800000u);
+        for (int s2 = 0; s2 < S; ++s2) M = fmaxf(M, f_m[s2 * G + j]);
+        float L = 0.f;
+        for (int s2 = 0; s2 < S; ++s2) {
+            const float pm = f_m[s2 * G + j];
+            const float f = pm == bits_f32(0xff800000u) ? 0.f : exp2f(pm - M);
+            L = fmaf(f_l[s2 * G + j], f, L);
+            f_m[s2 * G + j] = f;
+        }
+        s_L[j] = L;
+    }
+    __syncthreads();
     for (int o = threadIdx.x; o < G * D; o += 256) {
         const int j = o / D, d = o - j * D;
-        float M = bits_f32(0xff800000u);
-        for (int s2 = 0; s2 < S; ++s2) M = fmaxf(M, part_m[(base + s2) * G + j]);
-        float L = 0.f, A = 0.f;
+        float A = 0.f;
 #pragma unroll 8
-        for (int s2 = 0; s2 < S; ++s2) {
-            const float pm = part_m[(base + s2) * G + j];
-            const float f = pm == bits_f32(0xff800000u) ? 0.f : exp2f(pm - M);
-            L = fmaf(part_l[(base + s2) * G + j], f, L);
-            A = fmaf(part_acc[((base + s2) * G + j) * D + d], f, A);
-        }
-        att[((size_t)t * Hq + (size_t)g * G + j) * D + d] = f32_bf16(A * (1.f / L));
+        for (int s2 = 0; s2 < S; ++s2) A = fmaf(part_acc[((base + s2) * G + j) * D + d], f_m[s2 * G + j], A);
+        att[((size_t)t * Hq + (size_t)g * G + j) * D + d] = f32_bf16(A * (1.f / s_L[j]));
     }
-    if (threadIdx.x == 0) cnt[(size_t)t * Hk + g] = 0u;
 }
 
 __global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ m,
@@ -378,11 +397,10 @@ size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, siz
 
 int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0, size_t T,
                             size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap, size_t S,
-                            float* scratch, uint32_t* cnt, void* stream) {
-    if (q == nullptr || K == nullptr || V == nullptr || att == nullptr || n0 == nullptr || scratch == nullptr ||
-        cnt == nullptr)
+                            float* scratch, void* stream) {
+    if (q == nullptr || K == nullptr || V == nullptr || att == nullptr || n0 == nullptr || scratch == nullptr)
         return ERR_NULL;
-    if (T == 0 || Hq == 0 || Hk == 0 || S == 0 || cap == 0 || T > 65535 || S > 65535 || Hq % Hk != 0 || hs <= 0 ||
+    if (T == 0 || Hq == 0 || Hk == 0 || S == 0 || cap == 0 || T > 65535 || S > 1024 || Hq % Hk != 0 || hs <= 0 ||
         rs <= 0 || !(scale == scale))
         return ERR_DOMAIN;
     const size_t G = Hq / Hk;
@@ -398,11 +416,14 @@ int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* a
     const float scale_log2 = scale * 1.4426950408889634f;
     const dim3 grid((unsigned)Hk, (unsigned)S, (unsigned)T);
     hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 mgrid((unsigned)Hk, (unsigned)T);
+    const size_t mlds = 2 * S * G * sizeof(float);
 #define ATT(GG)                                                                                                      \
     hipLaunchKernelGGL(attn_decode_kernel<GG>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(q),              \
-                       static_cast<const uint16_t*>(K), static_cast<const uint16_t*>(V), static_cast<uint16_t*>(att), \
-                       n0, (int)Hq, (int)Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, cnt,   \
-                       span)
+                       static_cast<const uint16_t*>(K), static_cast<const uint16_t*>(V), n0, (int)Hq, (int)Hk,        \
+                       (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, span);                     \
+    hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,       \
+                       (int)Hk, (int)S, part_m, part_l, part_acc)
     switch (G) {
         case 1: ATT(1); break;
         case 2: ATT(2); break;

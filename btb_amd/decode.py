@@ -116,7 +116,7 @@ class DecodeStep:
         if attn_spans is None:
             attn_spans = max(1, min(self.cap // 64, (card.sms + Hk - 1) // Hk))
         self.S = int(attn_spans)
-        self.scratch, self.cnt = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
+        self.scratch = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
         self.fold_silu = bool(fold_silu)
         self.fused = bool(fused)
         # the handoff to the host: token, cache length and the GPU's clock in pinned memory
@@ -164,7 +164,7 @@ class DecodeStep:
             w[L + "qkv"].matvec(self.x, self.qkv)
             k.norm_rope_kv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K, V,
                            self.q, Hq, Hk, D)
-            k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch, self.cnt)
+            k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch)
             w[L + "o"].matvec(self.att, self.y)
             k.add_rmsnorm(self.h, self.y, w[L + "ln2"], cfg.eps, self.x)
             w[L + "gu"].matvec(self.x, self.gu)
@@ -195,7 +195,7 @@ class DecodeStep:
             k.gemv_norm(w[L + "qkv"].w, ha, y_prev, w[L + "ln1"], cfg.eps, hb, self.qkv)
             k.norm_rope_kv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K, V,
                            self.q, Hq, Hk, D)
-            k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch, self.cnt)
+            k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch)
             w[L + "o"].matvec(self.att, self.y)
             k.gemv_norm(w[L + "gu"].w, hb, self.y, w[L + "ln2"], cfg.eps, ha, self.m, glu=True)
             w[L + "down"].matvec(self.m, self.y)

@@ -60,7 +60,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
                                     _sz, ctypes.c_int64, ctypes.c_int64, _i32, _vp]),
     "btb_hip_attn_scratch_floats": (_sz, [_sz, _sz, _sz, _sz, _sz]),
     "btb_hip_attn_decode": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
-                                   ctypes.c_float, _sz, _sz, _vp, _vp, _vp]),
+                                   ctypes.c_float, _sz, _sz, _vp, _vp]),
     "btb_hip_silu_mul": (_i32, [_vp, _vp, _sz, _sz, _vp]),
     "btb_hip_argmax": (_i32, [_vp, _vp, _sz, _sz, _vp]),
     "btb_hip_publish": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
@@ -441,27 +441,26 @@ class HipCard:
                    None if depth is None else self.ptr(depth), self.ptr(K), self.ptr(V), self.ptr(q), T, Hq, Hk, D,
                    int(K.stride(0)), int(K.stride(1)), int(bool(centered)), _stream())
 
-    def attn_scratch(self, T: int, Hq: int, Hk: int, D: int, S: int, device: Any = "cuda"):
-        """(scratch f32, arrival counts u32) for `attn_decode` at these sizes; the counts start, and stay, zero"""
+    def attn_scratch(self, T: int, Hq: int, Hk: int, D: int, S: int, device: Any = "cuda") -> torch.Tensor:
+        """the f32 scratch `attn_decode` leaves its spans' states in, at these sizes"""
         n = int(self.lib.btb_hip_attn_scratch_floats(T, Hq, Hk, D, S))
-        return (torch.empty(n, dtype=torch.float32, device=device),
-                torch.zeros(T * Hk, dtype=torch.int32, device=device))
+        return torch.empty(n, dtype=torch.float32, device=device)
 
     def attn_decode(self, q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, att: torch.Tensor, n0: torch.Tensor,
-                    Hq: int, Hk: int, D: int, scale: float, S: int, scratch: torch.Tensor, cnt: torch.Tensor) -> None:
+                    Hq: int, Hk: int, D: int, scale: float, S: int, scratch: torch.Tensor) -> None:
         """att [T, Hq * D] = the rows' attention over the cache (row t sees keys 0 .. n0 + t)"""
         self._need(q, torch.bfloat16, "q")
         self._need(att, torch.bfloat16, "att")
         self._need(n0, torch.int32, "n0")
+        self._need(scratch, torch.float32, "scratch")
         if K.dtype != torch.bfloat16 or V.dtype != torch.bfloat16 or K.stride(2) != 1 or K.stride() != V.stride():
             raise ValueError("[hip] attn_decode: K and V are bf16 [Hk, cap, D] views with the same strides")
         T = int(q.numel()) // (Hq * D)
         need = int(self.lib.btb_hip_attn_scratch_floats(T, Hq, Hk, D, S))
-        if scratch.numel() < need or cnt.numel() < T * Hk:
+        if scratch.numel() < need:
             raise ValueError(f"[hip] attn_decode: scratch holds {scratch.numel()} floats, {need} are needed")
         self._call("btb_hip_attn_decode", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0), T, Hq, Hk,
-                   D, int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S, self.ptr(scratch),
-                   self.ptr(cnt), _stream())
+                   D, int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S, self.ptr(scratch), _stream())
 
     def silu_mul(self, gu: torch.Tensor, m: torch.Tensor) -> torch.Tensor:
         self._need(gu, torch.bfloat16, "gu")

@@ -206,14 +206,13 @@ int32_t btb_hip_norm_rope_kv(const void* qkv, const void* wq, const void* wk, fl
 size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, size_t S);
 
 /* Decode attention: att [T, Hq * D] = softmax(q K^T * scale) V, row t over the keys 0 .. *n0 + t, f32 throughout,
- * bf16 out. The keys (capacity `cap`) are cut into S spans, a workgroup per (kv head, span, row); `scratch`
- * (btb_hip_attn_scratch_floats) and cnt u32 [T * Hk] (zero before the first launch; every launch leaves it zero)
- * carry the spans' partial states to the last arriver, which folds them in span order. head_dim 128, Hq / Hk in
- * {1, 2, 4, 8}. Replaces btb_attn_flash_d128's decode form (native/cuda/btb_attn_flash.cuh:277-675) for a chain of
- * rows. */
+ * bf16 out. The keys (capacity `cap`) are cut into S spans, a workgroup per (kv head, span, row) leaving its
+ * online-softmax state in `scratch` (btb_hip_attn_scratch_floats floats); a second small launch folds the spans in
+ * span order. head_dim 128, Hq / Hk in {1, 2, 4, 8}, S <= 1024. Replaces btb_attn_flash_d128's decode form
+ * (native/cuda/btb_attn_flash.cuh:277-675) for a chain of rows. */
 int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0, size_t T,
                             size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap, size_t S,
-                            float* scratch, uint32_t* cnt, void* stream);
+                            float* scratch, void* stream);
 
 /* m [T, I] = bf16(bf16(silu(g)) * u) over gu [T, 2I] (gate then up). Replaces btb_silu_mul
  * (native/cuda/btb_kernels.cu:467-484); the matvec btb_hip_gemv_silu_bf16 folds the same values into its x load. */

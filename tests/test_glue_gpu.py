@@ -77,16 +77,15 @@ def test_attn_decode_against_f64(card, n0, T, Hq, Hk, S):
     V = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
     q = torch.randn(T, Hq * D, generator=g).to(torch.bfloat16)
     att = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
-    scratch, cnt = card.attn_scratch(T, Hq, Hk, D, S)
+    scratch = card.attn_scratch(T, Hq, Hk, D, S)
     n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
     scale = 1.0 / np.sqrt(D)
-    for rep in range(2):  # the arrival counts are left zero: a second launch gives the same bits
-        card.attn_decode(q.cuda(), K.cuda(), V.cuda(), att, n0t, Hq, Hk, D, scale, S, scratch, cnt)
+    for rep in range(2):  # a second launch over the same scratch gives the same bits
+        card.attn_decode(q.cuda(), K.cuda(), V.cuda(), att, n0t, Hq, Hk, D, scale, S, scratch)
         got = att.clone()
         if rep:
             assert torch.equal(got, first)
         first = got
-    assert torch.all(cnt == 0)
     for t in range(T):
         want = od.attention(q[t].float().numpy().reshape(Hq, D), K[:, : n0 + t + 1].float().numpy(),
                             V[:, : n0 + t + 1].float().numpy(), scale)
