@@ -143,7 +143,8 @@ def main() -> int:
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
     if os.path.exists(tpath):
         with open(tpath) as f:
-            traffic = json.load(f).get(args.workload)
+            entry = json.load(f).get(args.workload)
+            traffic = None if entry is None else entry.get("bytes_per_launch")
 
     line = {
         "metric": METRIC,
