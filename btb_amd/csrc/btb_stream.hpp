@@ -162,6 +162,12 @@ __device__ __forceinline__ void fma_unit(const typename F::RowCtx (&ctx)[RPW], c
     }
 }
 
+// what a finished pair of row sums becomes. E_PLAIN: y[m][r] = bf16(sum). E_GLU: the matrix is [2I, C], gate rows then
+// up rows; a wave works on gate row r and up row I + r together and writes m[m][r] = bf16(bf16(silu(g)) * u) with
+// g, u the two sums rounded to bf16 first - the values the gate_up matvec followed by btb_silu_mul would have
+// written (the reference's btb_gemv_mma_glu_silu does the same fold: native/cuda/btb_gemv_mma.cuh:216-315).
+enum Epilogue { E_PLAIN = 0, E_GLU = 1 };
+
 // where the kernel reads x from: LDS (staged once per workgroup) or straight from global memory through the caches
 enum XSrc { XS_LDS = 0, XS_GLOBAL = 1 };
 

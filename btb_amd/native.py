@@ -64,7 +64,31 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_silu_mul": (_i32, [_vp, _vp, _sz, _sz, _vp]),
     "btb_hip_argmax": (_i32, [_vp, _vp, _sz, _sz, _vp]),
     "btb_hip_publish": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "btb_hip_step_sync_bytes": (_sz, []),
+    "btb_hip_decode_step": (_i32, [_vp, _i32, _i32, _vp]),
 }
+
+
+class StepMat(ctypes.Structure):
+    """btb_hip_step_mat: one matrix of the persistent step in its stored form"""
+    _fields_ = [(n, _vp) for n in ("w", "hi4", "table", "esc_idx", "esc_val", "row_ptr")]
+
+
+class StepLayer(ctypes.Structure):
+    """btb_hip_step_layer"""
+    _fields_ = [("qkv", StepMat), ("o", StepMat), ("gu", StepMat), ("down", StepMat)] + \
+               [(n, _vp) for n in ("ln1", "ln2", "wq", "wk", "K", "V")]
+
+
+class StepArgs(ctypes.Structure):
+    """btb_hip_step_args"""
+    _fields_ = [("layers", _vp)] + [(n, _i32) for n in ("nlayers", "H", "Hq", "Hk", "I", "vocab", "S", "span")] + \
+               [("hs", ctypes.c_int64), ("rs", ctypes.c_int64), ("eps", ctypes.c_float),
+                ("scale_log2", ctypes.c_float), ("centered", _i32), ("embed", _vp), ("norm_w", _vp),
+                ("head", StepMat)] + \
+               [(n, _vp) for n in ("cos_t", "sin_t", "ids", "picked", "n0", "h_a", "h_b", "qkv", "att", "y", "m",
+                                   "logits", "part", "cand_v", "cand_i", "sync", "host_tok", "host_n0", "host_ts",
+                                   "trace")]
 
 
 class HipError(RuntimeError):
@@ -483,6 +507,17 @@ class HipCard:
         p = lambda t: None if t is None else self.ptr(t)
         self._call("btb_hip_publish", self.ptr(n0), self.ptr(picked), p(next_ids), p(out_tok), p(out_n0), p(out_ts),
                    _stream())
+
+    # -- the step as one persistent launch ------------------------------------------------------------------------
+
+    def step_sync(self, device: Any = "cuda") -> torch.Tensor:
+        """the zeroed barrier words `decode_step` needs (one tensor per step object, reused by every step)"""
+        n = int(self.lib.btb_hip_step_sync_bytes())
+        return torch.zeros(n // 4, dtype=torch.int32, device=device)
+
+    def decode_step(self, args: StepArgs, packed: bool, workgroups: int) -> None:
+        """one decode step as one launch of `workgroups` resident workgroups (see btb_hip_decode_step)"""
+        self._call("btb_hip_decode_step", ctypes.byref(args), 1 if packed else 0, int(workgroups), _stream())
 
 
 class Native:

@@ -228,6 +228,83 @@ int32_t btb_hip_argmax(const void* logits, int32_t* out, size_t T, size_t V, voi
 int32_t btb_hip_publish(int32_t* n0, const int32_t* picked, int32_t* next_ids, int32_t* out_tok, int32_t* out_n0,
                         int64_t* out_ts, void* stream);
 
+/* ---- the whole decode step as one persistent launch ---------------------------------------------------------- */
+
+/* One matrix of the step in its stored form. bf16: w [R, C], the other fields NULL. pack12: the arguments of
+ * btb_hip_gemv_p12 (w is `lo`). */
+typedef struct btb_hip_step_mat {
+    const void* w;
+    const void* hi4;
+    const void* table;
+    const void* esc_idx;
+    const void* esc_val;
+    const void* row_ptr;
+} btb_hip_step_mat;
+
+/* One layer: qkv [(Hq + 2 Hk) D, H], o [H, Hq D], gu [2 I, H] (gate rows then up rows), down [H, I]; the norm
+ * weights ln1 / ln2 [H] and wq / wk [D] (NULL: no q/k norm) in bf16; the layer's caches (head g's slot j at
+ * g * hs + j * rs elements). */
+typedef struct btb_hip_step_layer {
+    btb_hip_step_mat qkv, o, gu, down;
+    const void* ln1;
+    const void* ln2;
+    const void* wq;
+    const void* wk;
+    void* K;
+    void* V;
+} btb_hip_step_layer;
+
+/* Everything one step touches; every pointer is device memory except host_* (pinned host memory or NULL).
+ * `layers` is a device array of nlayers btb_hip_step_layer. S key spans of `span` keys each cover the cache.
+ * Buffers the step owns between its phases: h_a / h_b [H] (the residual, ping-pong), qkv [(Hq + 2 Hk) D], att
+ * [Hq D], y [H], m [I], logits [vocab] in bf16; part: 2 Hq S + Hq S D floats; cand_v / cand_i: 4 * workgroups
+ * floats / ints; sync: btb_hip_step_sync_bytes() bytes, zeroed once by the caller before the first step. */
+typedef struct btb_hip_step_args {
+    const btb_hip_step_layer* layers;
+    int32_t nlayers, H, Hq, Hk, I, vocab, S, span;
+    int64_t hs, rs;
+    float eps, scale_log2; /* scale_log2 = softmax scale * log2(e) */
+    int32_t centered;
+    const void* embed;     /* [vocab, H] bf16 */
+    const void* norm_w;    /* the final norm [H] */
+    btb_hip_step_mat head; /* [vocab, H] */
+    const void* cos_t;     /* rope tables [positions, D] bf16 */
+    const void* sin_t;
+    int32_t* ids;          /* in: the step's token; out: the picked one (the next step's input) */
+    int32_t* picked;
+    int32_t* n0;           /* in: rows the caches hold; out: + 1 */
+    void* h_a;
+    void* h_b;
+    void* qkv;
+    void* att;
+    void* y;
+    void* m;
+    void* logits;
+    float* part;
+    float* cand_v;
+    int32_t* cand_i;
+    uint32_t* sync;
+    int32_t* host_tok;
+    int32_t* host_n0;
+    int64_t* host_ts;
+    int64_t* trace;        /* NULL, or 2 * (5 nlayers + 1) device words: workgroup 0's clock (100 MHz) before and after
+                              every grid barrier, in order - the step's timeline by phase */
+} btb_hip_step_args;
+
+size_t btb_hip_step_sync_bytes(void);
+
+/* One decode step (M = 1, greedy pick) of a dense stack with 4 query heads per kv head of 128 dims, as ONE launch of
+ * `workgroups` resident workgroups that walk the step's phases and meet at grid barriers: the arithmetic, rounding
+ * points and summation orders of btb_hip_embed, btb_hip_gemv_bf16_norm (or _p12_norm, `packed` != 0),
+ * btb_hip_norm_rope_kv, btb_hip_attn_decode, btb_hip_gemv_bf16, btb_hip_argmax and btb_hip_publish in the order
+ * of the reference's _card_body (btb/engine/cuda.py:1722-1834), so logits and token are theirs bit for bit. The
+ * reference replays those launches as a CUDA graph; this entry is that graph collapsed into one kernel. DOMAIN when
+ * the grid would not be resident at once (the barriers need every workgroup running). A barrier that does not
+ * complete within its bounded wait sets word 64 of `sync` and the step runs to its end with wrong results: read
+ * that word after the step where a hang elsewhere on the GPU is possible, and zero `sync` before the next step. The
+ * barrier words carry over from step to step: zero them as well before a step with a different `workgroups`. */
+int32_t btb_hip_decode_step(const btb_hip_step_args* args, int32_t packed, int32_t workgroups, void* stream);
+
 #ifdef __cplusplus
 }
 #endif
