@@ -47,16 +47,29 @@ __device__ __forceinline__ float block_sum256(float v, float* red) {
     return s;
 }
 
-// Leaves the rows in xs (a barrier included). 256 threads.
-template <int XMODE>
-__device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C) {
+// LDS the staging needs for M rows of C values: the rows themselves, and for X_ADDNORM three raw rows (h, y and the
+// norm's weight) behind them
+__host__ __device__ constexpr size_t stage_lds_bytes(int xmode, int M, int C) {
+    return (size_t)(M + (xmode == X_ADDNORM ? 3 : 0)) * (size_t)C * 2;
+}
+
+// Leaves the rows in xs (a barrier included). 256 threads. `after_issue` is called once, right after the first loads
+// of the staging have been issued and before anything waits for them: the caller requests its first weights there,
+// so they travel while the staging's own (short) round trip and arithmetic run.
+template <int XMODE, class AfterIssue>
+__device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C, AfterIssue after_issue) {
     const int tid = threadIdx.x, nt = blockDim.x;
     if (XMODE == X_PLAIN) {
         const uint4* src = reinterpret_cast<const uint4*>(a.x);
         uint4* dst = reinterpret_cast<uint4*>(xs);
         const int n = M * C / 8;
-        for (int i = tid; i < n; i += nt) dst[i] = src[i];
+        uint4 v0 = make_uint4(0, 0, 0, 0);
+        if (tid < n) v0 = src[tid];
+        after_issue();
+        if (tid < n) dst[tid] = v0;
+        for (int i = tid + nt; i < n; i += nt) dst[i] = src[i];
     } else if (XMODE == X_SILU) {
+        after_issue();
         const int half = C / 2;  // pairs per row
         const uint32_t* src = reinterpret_cast<const uint32_t*>(a.x);
         for (int i = tid; i < M * half; i += nt) {
@@ -66,61 +79,68 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
     } else {
         // h' = bf16(h + y); x = bf16(h' * rsqrt(mean(h'^2) + eps) * w): the arithmetic and the summation order of the
         // stand-alone add_rmsnorm kernel (thread i takes elements i, i + 256, ...), so the bits are its bits. Every
-        // workgroup makes the whole row for itself; the first also writes the new residual out.
-        // The row's three inputs are requested together, ahead of any arithmetic: one round trip to memory, not three.
+        // workgroup makes the whole row for itself; the first also writes the new residual out. The row's inputs
+        // come in with 8-byte loads, all issued together, into raw rows in LDS; the arithmetic then reads LDS in its
+        // own element order.
         __shared__ float red[4];
         uint16_t* xs16 = reinterpret_cast<uint16_t*>(xs);
-        constexpr int PER = 16;  // elements a thread holds at once: rows up to 4096 wide take one pass
+        uint16_t* hraw = xs16 + (size_t)M * C;
+        uint16_t* yraw = hraw + C;
+        uint16_t* wraw = yraw + C;
+        const int n4 = C / 4;  // 8-byte words per row (C is a multiple of the format's unit, at least 8)
+        constexpr int PER = 3;  // words a thread holds at once: rows up to 3072 wide take one pass
         for (int m = 0; m < M; ++m) {
-            const uint16_t* hr = a.x + (size_t)m * C;
-            const uint16_t* yr = a.y == nullptr ? nullptr : a.y + (size_t)m * C;
-            uint16_t* row = xs16 + (size_t)m * C;
-            float ss = 0.f;
-            if (C <= PER * 256) {
-                uint16_t hv16[PER], yv16[PER], wv16[PER];
+            const uint2* hs = reinterpret_cast<const uint2*>(a.x + (size_t)m * C);
+            const uint2* ys = a.y == nullptr ? nullptr : reinterpret_cast<const uint2*>(a.y + (size_t)m * C);
+            const uint2* ws = reinterpret_cast<const uint2*>(a.norm_w);
+            for (int base = 0; base < n4; base += PER * 256) {
+                uint2 hv[PER], yv[PER], wv[PER];
 #pragma unroll
                 for (int q = 0; q < PER; ++q) {
-                    const int i = tid + q * 256;
-                    hv16[q] = i < C ? hr[i] : (uint16_t)0;
-                    yv16[q] = (i < C && yr != nullptr) ? yr[i] : (uint16_t)0;
-                    wv16[q] = i < C ? a.norm_w[i] : (uint16_t)0;
-                }
-                float hv[PER];
-#pragma unroll
-                for (int q = 0; q < PER; ++q) {
-                    hv[q] = bf16_f32(hv16[q]);
-                    if (yr != nullptr) hv[q] = bfround(hv[q] + bf16_f32(yv16[q]));
-                    if (tid + q * 256 < C) ss = fmaf(hv[q], hv[q], ss);
-                }
-                const float rstd = rsqrtf(block_sum256(ss, red) / (float)C + a.eps);
-#pragma unroll
-                for (int q = 0; q < PER; ++q) {
-                    const int i = tid + q * 256;
-                    if (i < C) {
-                        if (blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr)
-                            a.h_out[(size_t)m * C + i] = f32_bf16(hv[q]);
-                        const float wv = bf16_f32(wv16[q]);
-                        row[i] = f32_bf16(hv[q] * rstd * (a.centered ? 1.f + wv : wv));
+                    const int i = base + q * 256 + tid;
+                    hv[q] = yv[q] = wv[q] = make_uint2(0, 0);
+                    if (i < n4) {
+                        hv[q] = hs[i];
+                        if (ys != nullptr) yv[q] = ys[i];
+                        if (m == 0) wv[q] = ws[i];
                     }
                 }
-            } else {
-                for (int i = tid; i < C; i += 256) {
-                    float hv = bf16_f32(hr[i]);
-                    if (yr != nullptr) hv = bfround(hv + bf16_f32(yr[i]));
-                    row[i] = f32_bf16(hv);
-                    ss = fmaf(hv, hv, ss);
-                }
-                const float rstd = rsqrtf(block_sum256(ss, red) / (float)C + a.eps);
-                for (int i = tid; i < C; i += 256) {
-                    const uint16_t hb = row[i];
-                    if (blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr) a.h_out[(size_t)m * C + i] = hb;
-                    const float wv = bf16_f32(a.norm_w[i]);
-                    row[i] = f32_bf16(bf16_f32(hb) * rstd * (a.centered ? 1.f + wv : wv));
+                if (m == 0 && base == 0) after_issue();
+#pragma unroll
+                for (int q = 0; q < PER; ++q) {
+                    const int i = base + q * 256 + tid;
+                    if (i < n4) {
+                        reinterpret_cast<uint2*>(hraw)[i] = hv[q];
+                        reinterpret_cast<uint2*>(yraw)[i] = yv[q];
+                        if (m == 0) reinterpret_cast<uint2*>(wraw)[i] = wv[q];
+                    }
                 }
             }
+            __syncthreads();
+            uint16_t* row = xs16 + (size_t)m * C;
+            float ss = 0.f;
+            for (int i = tid; i < C; i += 256) {
+                float hv = bf16_f32(hraw[i]);
+                if (ys != nullptr) hv = bfround(hv + bf16_f32(yraw[i]));
+                row[i] = f32_bf16(hv);
+                ss = fmaf(hv, hv, ss);
+            }
+            const float rstd = rsqrtf(block_sum256(ss, red) / (float)C + a.eps);
+            for (int i = tid; i < C; i += 256) {
+                const uint16_t hb = row[i];
+                if (blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr) a.h_out[(size_t)m * C + i] = hb;
+                const float wv = bf16_f32(wraw[i]);
+                row[i] = f32_bf16(bf16_f32(hb) * rstd * (a.centered ? 1.f + wv : wv));
+            }
+            __syncthreads();  // the raw rows are free for the next row
         }
     }
     __syncthreads();
+}
+
+template <int XMODE>
+__device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C) {
+    stage_x<XMODE>(xs, a, M, C, [] {});
 }
 
 // ------------------------------------------------------------------------------------------------------------

@@ -24,79 +24,111 @@ namespace btb {
 // ------------------------------------------------------------------------------------------------------------
 
 
+// one tile of gemv_stream: its RPW rows' sums over the M rows of x, written out. PRIMED: the tile's first span is
+// already in `first` (requested before x was staged).
+template <class F, int M, int LPR, int RPW, int U, int EPI, bool PRIMED>
+__device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typename F::Raw (&first)[U][RPW], int tile,
+                                          const uint4* xs4, uint16_t* __restrict__ y, int R, int C, int lane) {
+    constexpr int G = WAVE / LPR;                      // rows a wave covers per set
+    constexpr int ROWS = EPI == E_GLU ? G : G * RPW;   // output rows a wave covers per tile
+    const int Rout = EPI == E_GLU ? R / 2 : R;
+    const int units = C / F::UW;         // units per row
+    const int sl = lane % LPR;           // the lane's place among its row's lanes
+    const int span = U * LPR;
+    const int xrow4 = C / 8;             // uint4 per row of x
+    typename F::RowCtx ctx[RPW];
+    int rows[RPW];   // weight rows
+    int out_row;     // E_GLU: the output row of the pair
+#pragma unroll
+    for (int j = 0; j < RPW; ++j) {
+        if (EPI == E_GLU) {
+            out_row = tile * ROWS + lane / LPR;
+            rows[j] = min(out_row, Rout - 1) + j * Rout;
+        } else {
+            rows[j] = tile * ROWS + j * G + lane / LPR;
+        }
+        // a row past the end reads the last row again (no divergence in the stream) and is not written
+        ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
+    }
+    float acc[RPW][M];
+#pragma unroll
+    for (int j = 0; j < RPW; ++j)
+#pragma unroll
+        for (int m = 0; m < M; ++m) acc[j][m] = 0.f;
+
+    int k0 = 0;
+    if (PRIMED) {
+        fma_span<F, M, LPR, RPW, U, true>(first, ctx, 0, sl, units, xs4, xrow4, acc);
+        k0 = span;
+    }
+    for (; k0 < units; k0 += span) {
+        typename F::Raw raw[U][RPW];
+        if (k0 + span <= units) {
+            load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
+            fma_span<F, M, LPR, RPW, U, false>(raw, ctx, k0, sl, units, xs4, xrow4, acc);
+        } else {
+            load_span<F, LPR, RPW, U, true>(raw, ctx, k0, sl, units);
+            fma_span<F, M, LPR, RPW, U, true>(raw, ctx, k0, sl, units, xs4, xrow4, acc);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < RPW; ++j)
+        F::template tail<M>(p, ctx[j], (size_t)min(rows[j], R - 1), sl, LPR, C, reinterpret_cast<const uint32_t*>(xs4),
+                            acc[j]);
+    if (EPI == E_GLU) {
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const float g = bfround(group_sum<LPR>(acc[0][m]));
+            const float u = bfround(group_sum<LPR>(acc[RPW - 1][m]));
+            const float sg = bfround(g / (1.f + expf(-g)));
+            if (sl == 0 && out_row < Rout) y[(size_t)m * Rout + out_row] = f32_bf16(sg * u);
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < RPW; ++j)
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                const float s = group_sum<LPR>(acc[j][m]);
+                if (sl == 0 && rows[j] < R) y[(size_t)m * R + rows[j]] = f32_bf16(s);
+            }
+    }
+}
+
+// The wave's first span of weights is requested while x is being staged - right after the staging's own loads have
+// been issued, so those (served by L2) are not queued behind the weights: the weights do not depend on x, and their
+// round trip to HBM overlaps the staging (for the add + norm form a block-wide sum and a second pass) instead of
+// following it.
 template <class F, int M, int LPR, int RPW, int U, int XMODE, int EPI>
 __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs xa, uint16_t* __restrict__ y, int R, int C) {
     extern __shared__ __align__(16) uint32_t xs[];  // [M][C / 2] packed bf16 pairs
     static_assert(EPI == E_PLAIN || RPW == 2, "the GLU form pairs a gate row with an up row");
-    constexpr int UW = F::UW;
-    constexpr int G = WAVE / LPR;                      // rows a wave covers per set
-    constexpr int ROWS = EPI == E_GLU ? G : G * RPW;   // output rows a wave covers per tile
+    constexpr int G = WAVE / LPR;
+    constexpr int ROWS = EPI == E_GLU ? G : G * RPW;
     const int Rout = EPI == E_GLU ? R / 2 : R;
-    const int units = C / UW;            // units per row
+    const int units = C / F::UW;
     const int lane = threadIdx.x & (WAVE - 1);
-    const int sl = lane % LPR;           // the lane's place among its row's lanes
     const int wave = blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
     const int nwaves = gridDim.x * (blockDim.x / WAVE);
     const int ntiles = (Rout + ROWS - 1) / ROWS;
-    const int span = U * LPR;
-    const int xrow4 = C / 8;  // uint4 per row of x
 
-    stage_x<XMODE>(xs, xa, M, C);
+    typename F::Raw first[U][RPW] = {};
+    stage_x<XMODE>(xs, xa, M, C, [&] {
+        if (wave < ntiles) {
+            typename F::RowCtx ctx[RPW];
+#pragma unroll
+            for (int j = 0; j < RPW; ++j) {
+                const int row = EPI == E_GLU ? min(wave * ROWS + lane / LPR, Rout - 1) + j * Rout
+                                             : min(wave * ROWS + j * G + lane / LPR, R - 1);
+                ctx[j] = F::row_ctx(p, (size_t)row, units);
+            }
+            load_span<F, LPR, RPW, U, true>(first, ctx, 0, lane % LPR, units);
+        }
+    });
     const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
-
-    for (int tile = wave; tile < ntiles; tile += nwaves) {
-        typename F::RowCtx ctx[RPW];
-        int rows[RPW];   // weight rows
-        int out_row;     // E_GLU: the output row of the pair
-#pragma unroll
-        for (int j = 0; j < RPW; ++j) {
-            if (EPI == E_GLU) {
-                out_row = tile * ROWS + lane / LPR;
-                rows[j] = min(out_row, Rout - 1) + j * Rout;
-            } else {
-                rows[j] = tile * ROWS + j * G + lane / LPR;
-            }
-            // a row past the end reads the last row again (no divergence in the stream) and is not written
-            ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
-        }
-        float acc[RPW][M];
-#pragma unroll
-        for (int j = 0; j < RPW; ++j)
-#pragma unroll
-            for (int m = 0; m < M; ++m) acc[j][m] = 0.f;
-
-        for (int k0 = 0; k0 < units; k0 += span) {
-            typename F::Raw raw[U][RPW];
-            if (k0 + span <= units) {
-                load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
-                fma_span<F, M, LPR, RPW, U, false>(raw, ctx, k0, sl, units, xs4, xrow4, acc);
-            } else {
-                load_span<F, LPR, RPW, U, true>(raw, ctx, k0, sl, units);
-                fma_span<F, M, LPR, RPW, U, true>(raw, ctx, k0, sl, units, xs4, xrow4, acc);
-            }
-        }
-#pragma unroll
-        for (int j = 0; j < RPW; ++j)
-            F::template tail<M>(p, ctx[j], (size_t)min(rows[j], R - 1), sl, LPR, C,
-                                reinterpret_cast<const uint32_t*>(xs4), acc[j]);
-        if (EPI == E_GLU) {
-#pragma unroll
-            for (int m = 0; m < M; ++m) {
-                const float g = bfround(group_sum<LPR>(acc[0][m]));
-                const float u = bfround(group_sum<LPR>(acc[RPW - 1][m]));
-                const float sg = bfround(g / (1.f + expf(-g)));
-                if (sl == 0 && out_row < Rout) y[(size_t)m * Rout + out_row] = f32_bf16(sg * u);
-            }
-        } else {
-#pragma unroll
-            for (int j = 0; j < RPW; ++j)
-#pragma unroll
-                for (int m = 0; m < M; ++m) {
-                    const float s = group_sum<LPR>(acc[j][m]);
-                    if (sl == 0 && rows[j] < R) y[(size_t)m * R + rows[j]] = f32_bf16(s);
-                }
-        }
-    }
+    if (wave >= ntiles) return;
+    gemv_tile<F, M, LPR, RPW, U, EPI, true>(p, first, wave, xs4, y, R, C, lane);
+    for (int tile = wave + nwaves; tile < ntiles; tile += nwaves)
+        gemv_tile<F, M, LPR, RPW, U, EPI, false>(p, first, tile, xs4, y, R, C, lane);
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -115,7 +147,7 @@ static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void
     constexpr int G = WAVE / LPR;
     constexpr int ROWS = EPI == E_GLU ? G : G * RPW;
     const DeviceInfo& dev = device_info();
-    const size_t lds = (size_t)M * C * 2;
+    const size_t lds = stage_lds_bytes(XMODE, M, C);
     if (lds > (size_t)dev.lds_bytes) {
         set_error("gemv: the x rows do not fit LDS");
         return ERR_DOMAIN;
