@@ -12,6 +12,7 @@
 //
 // Every reduction runs in an order fixed by the element's index alone, so a replayed graph repeats its bits.
 
+#include "btb_attn.hpp"
 #include "btb_common.hpp"
 #include "btb_stream.hpp"
 #include "btb_tuning.hpp"
@@ -204,6 +205,103 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     __syncthreads();
     // fold them in stream order: thread (j, d) for d < D; G * D <= 1024 values over 256 threads
     const size_t prow = ((size_t)t * Hk + g) * S + sp;  // this workgroup's slot among the partial states
+    for (int o = threadIdx.x; o < G * D; o += 256) {
+        const int j = o / D, d = o - j * D;
+        float M = bits_f32(0xff800000u);
+        for (int s2 = 0; s2 < 16; ++s2) M = fmaxf(M, s_m[s2][j]);
+        float L = 0.f, A = 0.f;
+        for (int s2 = 0; s2 < 16; ++s2) {
+            const float f = s_m[s2][j] == bits_f32(0xff800000u) ? 0.f : exp2f(s_m[s2][j] - M);
+            L = fmaf(s_l[s2][j], f, L);
+            A = fmaf(s_acc[s2][j][d], f, A);
+        }
+        part_acc[(prow * G + j) * D + d] = A;
+        if (d == 0) {
+            part_m[prow * G + j] = M;
+            part_l[prow * G + j] = L;
+        }
+    }
+}
+
+// The step's own form (one row): the kernel reads the fused qkv row itself. Each workgroup norms and ropes the G query
+// heads of its kv head (a wave a head; the result never leaves LDS), and the workgroup whose span holds slot *n0 also
+// norms and ropes the new key, copies the new value, writes both into the cache and takes them from LDS where its
+// stream reaches that slot. One launch (norm_rope_kv) less, and the stream's first keys are requested before q is
+// touched. The arithmetic is norm_rope_kv_kernel's followed by attn_decode_kernel's: the states it leaves are theirs.
+template <int G>
+__global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __restrict__ qkv, const uint16_t* __restrict__ wq,
+                                                              const uint16_t* __restrict__ wk, float eps, int centered,
+                                                              const uint16_t* __restrict__ cos_t,
+                                                              const uint16_t* __restrict__ sin_t,
+                                                              const int32_t* __restrict__ n0p, uint16_t* __restrict__ K,
+                                                              uint16_t* __restrict__ V, int Hq, int Hk, long long hs,
+                                                              long long rs, float scale_log2, float* __restrict__ part_m,
+                                                              float* __restrict__ part_l, float* __restrict__ part_acc,
+                                                              int span) {
+    constexpr int D = ATT_D;
+    __shared__ float s_q[G][D];
+    __shared__ __align__(16) uint16_t s_k[D], s_v[D];
+    __shared__ float s_m[16][G], s_l[16][G];
+    __shared__ float s_acc[16][G][D];
+    const int g = blockIdx.x, sp = blockIdx.y, S = gridDim.y;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int sub = lane >> 4, dl = lane & 15, grp = wv * 4 + sub;
+    const int n0 = *n0p;
+    const int k_begin = sp * span, k_end = min(n0 + 1, k_begin + span);
+    const uint16_t* Kh = K + (size_t)g * hs + dl * 8;
+    const uint16_t* Vh = V + (size_t)g * hs + dl * 8;
+    KeyBatch kb = {};
+    const int key_first = k_begin + grp;
+    if (key_first < k_end) load_keys(kb, Kh, Vh, rs, key_first, k_end, n0);
+
+    for (int j = wv; j < G; j += 4) {
+        uint16_t o[2];
+        head_norm_rope<false>(qkv + (size_t)(g * G + j) * D, wq, eps, centered, cos_t, sin_t, n0, lane, o);
+        s_q[j][lane * 2 + 0] = bf16_f32(o[0]) * scale_log2;
+        s_q[j][lane * 2 + 1] = bf16_f32(o[1]) * scale_log2;
+    }
+    if (wv == 3 && n0 >= k_begin && n0 < k_begin + span) {
+        uint16_t o[2];
+        head_norm_rope<false>(qkv + (size_t)(Hq + g) * D, wk, eps, centered, cos_t, sin_t, n0, lane, o);
+        const uint32_t vraw = reinterpret_cast<const uint32_t*>(qkv + (size_t)(Hq + Hk + g) * D)[lane];
+        s_k[lane * 2] = o[0];
+        s_k[lane * 2 + 1] = o[1];
+        s_v[lane * 2] = (uint16_t)(vraw & 0xFFFFu);
+        s_v[lane * 2 + 1] = (uint16_t)(vraw >> 16);
+        reinterpret_cast<uint32_t*>(K + (size_t)g * hs + (size_t)n0 * rs)[lane] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+        reinterpret_cast<uint32_t*>(V + (size_t)g * hs + (size_t)n0 * rs)[lane] = vraw;
+    }
+    __syncthreads();
+
+    float qv[G][8];
+#pragma unroll
+    for (int j = 0; j < G; ++j)
+#pragma unroll
+        for (int e = 0; e < 8; ++e) qv[j][e] = s_q[j][dl * 8 + e];
+    float m[G], l[G], acc[G][8];
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+        m[j] = bits_f32(0xff800000u);
+        l[j] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
+    }
+    for (int key0 = key_first; key0 < k_end;) {
+        use_keys<G>(kb, key0, k_end, n0, s_k, s_v, dl, qv, m, l, acc);
+        key0 += 16 * KB;
+        if (key0 < k_end) load_keys(kb, Kh, Vh, rs, key0, k_end, n0);
+    }
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+        if (dl == 0) {
+            s_m[grp][j] = m[j];
+            s_l[grp][j] = l[j];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s_acc[grp][j][dl * 8 + e] = acc[j][e];
+    }
+    __syncthreads();
+    const size_t prow = (size_t)g * S + sp;
     for (int o = threadIdx.x; o < G * D; o += 256) {
         const int j = o / D, d = o - j * D;
         float M = bits_f32(0xff800000u);
@@ -435,6 +533,52 @@ int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* a
     }
 #undef ATT
     return hip_status(hipGetLastError(), "attn_decode launch");
+}
+
+int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk, float eps, int32_t centered,
+                                const void* cos_t, const void* sin_t, const int32_t* n0, void* K, void* V, void* att,
+                                size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap,
+                                size_t S, float* scratch, void* stream) {
+    if (qkv == nullptr || cos_t == nullptr || sin_t == nullptr || n0 == nullptr || K == nullptr || V == nullptr ||
+        att == nullptr || scratch == nullptr)
+        return ERR_NULL;
+    if (Hq == 0 || Hk == 0 || S == 0 || cap == 0 || S > 1024 || Hq % Hk != 0 || hs <= 0 || rs <= 0 ||
+        !(scale == scale) || !(eps >= 0.f))
+        return ERR_DOMAIN;
+    const size_t G = Hq / Hk;
+    if (D != (size_t)ATT_D || G > (size_t)ATT_MAXG) {
+        set_error("attn_decode_qkv: head_dim 128 and at most 8 query heads per kv head");
+        return ERR_DOMAIN;
+    }
+    if (!al(qkv, 4) || !al(K, 16) || !al(V, 16) || (rs % 8) != 0 || (hs % 8) != 0) return ERR_DOMAIN;
+    const int span = (int)((cap + S - 1) / S);
+    float* part_m = scratch;
+    float* part_l = scratch + Hq * S;
+    float* part_acc = scratch + 2 * Hq * S;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    const dim3 grid((unsigned)Hk, (unsigned)S);
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const dim3 mgrid((unsigned)Hk, 1);
+    const size_t mlds = 2 * S * G * sizeof(float);
+#define ATT(GG)                                                                                                      \
+    hipLaunchKernelGGL(attn_decode_qkv_kernel<GG>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(qkv),        \
+                       static_cast<const uint16_t*>(wq), static_cast<const uint16_t*>(wk), eps, centered ? 1 : 0,    \
+                       static_cast<const uint16_t*>(cos_t), static_cast<const uint16_t*>(sin_t), n0,                 \
+                       static_cast<uint16_t*>(K), static_cast<uint16_t*>(V), (int)Hq, (int)Hk, (long long)hs,        \
+                       (long long)rs, scale_log2, part_m, part_l, part_acc, span);                                   \
+    hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,       \
+                       (int)Hk, (int)S, part_m, part_l, part_acc)
+    switch (G) {
+        case 1: ATT(1); break;
+        case 2: ATT(2); break;
+        case 4: ATT(4); break;
+        case 8: ATT(8); break;
+        default:
+            set_error("attn_decode_qkv: 1, 2, 4 or 8 query heads per kv head");
+            return ERR_DOMAIN;
+    }
+#undef ATT
+    return hip_status(hipGetLastError(), "attn_decode_qkv launch");
 }
 
 int32_t btb_hip_silu_mul(const void* gu, void* m, size_t T, size_t I, void* stream) {

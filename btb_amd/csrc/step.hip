@@ -24,6 +24,7 @@
 
 #include <cstring>
 
+#include "btb_attn.hpp"
 #include "btb_common.hpp"
 #include "btb_formats.hpp"
 #include "btb_stream.hpp"
@@ -36,15 +37,6 @@ namespace btb {
 // ------------------------------------------------------------------------------------------------------------
 // device-scope access, the barrier
 // ------------------------------------------------------------------------------------------------------------
-
-template <class T>
-__device__ __forceinline__ T ld_dev(const T* p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-template <class T>
-__device__ __forceinline__ void st_dev(T* p, T v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 
 // The thread's index as a value the compiler cannot see through: address arithmetic built on it inside a phase stays in
 // that phase instead of being hoisted out of the layer loop, where a dozen phases' worth of it would sit in registers
@@ -371,87 +363,6 @@ __device__ __forceinline__ void matvec_phase(PRE_T& pre, const StepMat& mat, con
 // fold (attn_merge). head_dim 128, G = Hq / Hk = 4.
 // ------------------------------------------------------------------------------------------------------------
 
-constexpr int AD = 128;
-
-// one head's 128 values: RMSNorm (weight wn or none), rope at `pos`; lane holds dims 2 * lane, 2 * lane + 1
-__device__ __forceinline__ void head_norm_rope(const uint16_t* src, const uint16_t* wn, float eps, int centered,
-                                               const uint16_t* cos_t, const uint16_t* sin_t, int pos, int lane,
-                                               uint16_t (&out)[2]) {
-    const uint32_t raw = ld_dev(reinterpret_cast<const uint32_t*>(src) + lane);
-    float v[2] = {bf16lo_f32(raw), bf16hi_f32(raw)};
-    if (wn != nullptr) {
-        float ss = fmaf(v[1], v[1], fmaf(v[0], v[0], 0.f));
-        ss = group_sum<64>(ss);
-        const float rstd = rsqrtf(ss / (float)AD + eps);
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const float wv = bf16_f32(wn[lane * 2 + e]);
-            v[e] = bfround(v[e] * rstd * (centered ? 1.f + wv : wv));
-        }
-    }
-    const float sgn = lane < 32 ? -1.f : 1.f;
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-        const float rot = __shfl_xor(v[e], 32, WAVE);
-        const float qc = bfround(v[e] * bf16_f32(cos_t[(size_t)pos * AD + lane * 2 + e]));
-        out[e] = f32_bf16(fmaf(sgn * rot, bf16_f32(sin_t[(size_t)pos * AD + lane * 2 + e]), qc));
-    }
-}
-
-// one batch of a key stream: eight keys sixteen apart, their K and V rows (this lane's 8 dims) requested together
-constexpr int KB = 8;
-struct KeyBatch {
-    uint4 k[KB], v[KB];
-};
-__device__ __forceinline__ void load_keys(KeyBatch& kb, const uint16_t* Kh, const uint16_t* Vh, long long rs, int key0,
-                                          int k_end, int n0) {
-#pragma unroll
-    for (int b = 0; b < KB; ++b) {
-        const int key = min(key0 + 16 * b, k_end - 1);  // a key past the span's end is loaded again, not used
-        // slot n0 is this step's own row: it is taken from LDS, the cache's copy may not have landed yet
-        const int safe = key == n0 ? max(n0 - 1, 0) : key;
-        kb.k[b] = *reinterpret_cast<const uint4*>(Kh + (size_t)safe * rs);
-        kb.v[b] = *reinterpret_cast<const uint4*>(Vh + (size_t)safe * rs);
-    }
-}
-
-// the batch's keys, in ascending order, folded into the G query heads' online-softmax states (attn_decode_kernel's
-// arithmetic). A key's rows are widened once and meet all G heads before the next key is touched.
-template <int G>
-__device__ __forceinline__ void use_keys(const KeyBatch& kb, int key0, int k_end, int n0, const uint16_t* s_k,
-                                         const uint16_t* s_v, int dl, const float (&qv)[G][8], float (&m)[G],
-                                         float (&l)[G], float (&acc)[G][8]) {
-#pragma unroll
-    for (int b = 0; b < KB; ++b) {
-        if (key0 + 16 * b < k_end) {
-            uint4 kr = kb.k[b], vr = kb.v[b];
-            if (key0 + 16 * b == n0) {  // the step's own row, from LDS
-                kr = *reinterpret_cast<const uint4*>(s_k + dl * 8);
-                vr = *reinterpret_cast<const uint4*>(s_v + dl * 8);
-            }
-            const float kf[8] = {bf16lo_f32(kr.x), bf16hi_f32(kr.x), bf16lo_f32(kr.y), bf16hi_f32(kr.y),
-                                 bf16lo_f32(kr.z), bf16hi_f32(kr.z), bf16lo_f32(kr.w), bf16hi_f32(kr.w)};
-            const float vf[8] = {bf16lo_f32(vr.x), bf16hi_f32(vr.x), bf16lo_f32(vr.y), bf16hi_f32(vr.y),
-                                 bf16lo_f32(vr.z), bf16hi_f32(vr.z), bf16lo_f32(vr.w), bf16hi_f32(vr.w)};
-#pragma unroll
-            for (int j = 0; j < G; ++j) {
-                float sc = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) sc = fmaf(qv[j][e], kf[e], sc);
-                sc = group_sum<16>(sc);
-                const float mn = fmaxf(m[j], sc);
-                const float corr = exp2f(m[j] - mn);  // 0 on the stream's first key (m = -inf)
-                const float pp = exp2f(sc - mn);
-                l[j] = fmaf(l[j], corr, pp);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc[j][e] = fmaf(pp, vf[e], acc[j][e] * corr);
-                m[j] = mn;
-            }
-        }
-        __builtin_amdgcn_sched_barrier(0);  // a key at a time: widening every key's rows ahead costs the registers
-    }
-}
-
 // the spans of kv head g folded in span order (attn_merge_kernel's arithmetic) by the workgroup that finished the
 // head's last span. Thread (j, d) makes two output values; the states' loads are all requested before any is used.
 template <int G>
@@ -564,7 +475,7 @@ __device__ __forceinline__ void attention_item(const StepArgs& a, const StepLaye
     const uint16_t* qkv = a.qkv;
     {
         uint16_t o[2];
-        head_norm_rope(qkv + (size_t)(g * G + wv) * AD, L.wq, a.eps, a.centered, a.cos_t, a.sin_t, n0, lane, o);
+        head_norm_rope<true>(qkv + (size_t)(g * G + wv) * AD, L.wq, a.eps, a.centered, a.cos_t, a.sin_t, n0, lane, o);
         s_q[wv * AD + lane * 2 + 0] = bf16_f32(o[0]) * a.scale_log2;
         s_q[wv * AD + lane * 2 + 1] = bf16_f32(o[1]) * a.scale_log2;
     }
@@ -572,7 +483,7 @@ __device__ __forceinline__ void attention_item(const StepArgs& a, const StepLaye
     // slot n0 uses them (from LDS) and writes them into the cache
     if (wv == 3 && n0 >= k_begin && n0 < k_begin + a.span) {
         uint16_t o[2];
-        head_norm_rope(qkv + (size_t)(Hq + g) * AD, L.wk, a.eps, a.centered, a.cos_t, a.sin_t, n0, lane, o);
+        head_norm_rope<true>(qkv + (size_t)(Hq + g) * AD, L.wk, a.eps, a.centered, a.cos_t, a.sin_t, n0, lane, o);
         const uint32_t vraw = ld_dev(reinterpret_cast<const uint32_t*>(qkv + (size_t)(Hq + Hk + g) * AD) + lane);
         s_k[lane * 2] = o[0];
         s_k[lane * 2 + 1] = o[1];

@@ -251,7 +251,8 @@ class DecodeStep:
 
     def _body_fused(self) -> None:
         """the same arithmetic in fewer launches: each residual add + norm rides in the x load of the matvec that
-        follows it (the residual ping-pongs between two buffers), gate / up / activation are one kernel. Bit for bit
+        follows it (the residual ping-pongs between two buffers), gate / up / activation are one kernel, the q / k norm
+        and rope ride in the attention kernel. Bit for bit
         the plain sequence's result."""
         k, cfg, w = self.card, self.cfg, self.w
         Hq, Hk, D = cfg.q_heads, cfg.kv_heads, cfg.head_dim
@@ -262,9 +263,13 @@ class DecodeStep:
             L = f"layers.{i}."
             K, V = self.kv[i, 0], self.kv[i, 1]
             k.gemv_norm(w[L + "qkv"].w, ha, y_prev, w[L + "ln1"], cfg.eps, hb, self.qkv)
-            k.norm_rope_kv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K, V,
-                           self.q, Hq, Hk, D)
-            k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch)
+            if self.T == 1 and D == 128:
+                k.attn_decode_qkv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K,
+                                  V, self.att, Hq, Hk, D, self.scale, self.S, self.scratch)
+            else:
+                k.norm_rope_kv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K, V,
+                               self.q, Hq, Hk, D)
+                k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch)
             w[L + "o"].matvec(self.att, self.y)
             k.gemv_norm(w[L + "gu"].w, hb, self.y, w[L + "ln2"], cfg.eps, ha, self.m, glu=True)
             w[L + "down"].matvec(self.m, self.y)

@@ -61,6 +61,8 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_attn_scratch_floats": (_sz, [_sz, _sz, _sz, _sz, _sz]),
     "btb_hip_attn_decode": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
                                    ctypes.c_float, _sz, _sz, _vp, _vp]),
+    "btb_hip_attn_decode_qkv": (_i32, [_vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
+                                       ctypes.c_int64, ctypes.c_int64, ctypes.c_float, _sz, _sz, _vp, _vp]),
     "btb_hip_silu_mul": (_i32, [_vp, _vp, _sz, _sz, _vp]),
     "btb_hip_argmax": (_i32, [_vp, _vp, _sz, _sz, _vp]),
     "btb_hip_publish": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
@@ -485,6 +487,35 @@ class HipCard:
             raise ValueError(f"[hip] attn_decode: scratch holds {scratch.numel()} floats, {need} are needed")
         self._call("btb_hip_attn_decode", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0), T, Hq, Hk,
                    D, int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S, self.ptr(scratch), _stream())
+
+    def attn_decode_qkv(self, qkv: torch.Tensor, wq: torch.Tensor | None, wk: torch.Tensor | None, eps: float,
+                        cos_t: torch.Tensor, sin_t: torch.Tensor, n0: torch.Tensor, K: torch.Tensor, V: torch.Tensor,
+                        att: torch.Tensor, Hq: int, Hk: int, D: int, scale: float, S: int, scratch: torch.Tensor,
+                        centered: bool = False) -> None:
+        """the step's own attention straight from the fused qkv row: `norm_rope_kv` + `attn_decode` at one row, one
+        launch less (q stays on the chip; the new K / V row is written by the workgroup whose span holds slot n0)"""
+        for t, what in ((qkv, "qkv"), (att, "att"), (cos_t, "cos"), (sin_t, "sin")):
+            self._need(t, torch.bfloat16, what)
+        for t, what in ((wq, "wq"), (wk, "wk")):
+            if t is not None:
+                self._need(t, torch.bfloat16, what)
+                if t.numel() != D:
+                    raise ValueError(f"[hip] attn_decode_qkv: {what} holds {t.numel()} values, head_dim is {D}")
+        self._need(n0, torch.int32, "n0")
+        self._need(scratch, torch.float32, "scratch")
+        if K.dtype != torch.bfloat16 or V.dtype != torch.bfloat16 or K.stride(2) != 1 or K.stride() != V.stride():
+            raise ValueError("[hip] attn_decode_qkv: K and V are bf16 [Hk, cap, D] views with the same strides")
+        if qkv.numel() != (Hq + 2 * Hk) * D or att.numel() != Hq * D:
+            raise ValueError("[hip] attn_decode_qkv: one row of qkv [(Hq + 2 Hk) D] and of att [Hq D]")
+        if cos_t.shape[-1] != D or cos_t.shape != sin_t.shape or cos_t.shape[0] < K.shape[1]:
+            raise ValueError("[hip] attn_decode_qkv: rope tables are [positions >= cap, D]")
+        need = int(self.lib.btb_hip_attn_scratch_floats(1, Hq, Hk, D, S))
+        if scratch.numel() < need:
+            raise ValueError(f"[hip] attn_decode_qkv: scratch holds {scratch.numel()} floats, {need} are needed")
+        p = lambda t: None if t is None else self.ptr(t)
+        self._call("btb_hip_attn_decode_qkv", self.ptr(qkv), p(wq), p(wk), float(eps), 1 if centered else 0,
+                   self.ptr(cos_t), self.ptr(sin_t), self.ptr(n0), self.ptr(K), self.ptr(V), self.ptr(att), Hq, Hk, D,
+                   int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S, self.ptr(scratch), _stream())
 
     def silu_mul(self, gu: torch.Tensor, m: torch.Tensor) -> torch.Tensor:
         self._need(gu, torch.bfloat16, "gu")

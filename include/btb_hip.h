@@ -214,6 +214,16 @@ int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* a
                             size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap, size_t S,
                             float* scratch, void* stream);
 
+/* The decode step's own attention (one row), straight from the fused qkv row [(Hq + 2 Hk) D] bf16: what
+ * btb_hip_norm_rope_kv followed by btb_hip_attn_decode compute at T = 1, bit for bit, in one launch less - the
+ * q / k norm and rope happen inside the attention workgroups (q never reaches memory), the workgroup whose key span
+ * holds slot *n0 writes the new K / V row. Same scratch, spans and limits as btb_hip_attn_decode. Replaces the pair
+ * btb_norm_rope_kv_d128 + btb_attn_flash_d128 of the reference's card step (btb/engine/cuda.py:1756-1790). */
+int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk, float eps, int32_t centered,
+                                const void* cos_t, const void* sin_t, const int32_t* n0, void* K, void* V, void* att,
+                                size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap,
+                                size_t S, float* scratch, void* stream);
+
 /* m [T, I] = bf16(bf16(silu(g)) * u) over gu [T, 2I] (gate then up). Replaces btb_silu_mul
  * (native/cuda/btb_kernels.cu:467-484); the matvec btb_hip_gemv_silu_bf16 folds the same values into its x load. */
 int32_t btb_hip_silu_mul(const void* gu, void* m, size_t T, size_t I, void* stream);

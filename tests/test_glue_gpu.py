@@ -94,6 +94,42 @@ def test_attn_decode_against_f64(card, n0, T, Hq, Hk, S):
         assert worst <= 2.0**-7, worst
 
 
+@pytest.mark.parametrize("n0,Hq,Hk,S", [(4096, 32, 8, 36), (100, 32, 8, 4), (0, 8, 8, 1), (63, 16, 2, 7), (64, 16, 2, 2),
+                                         (500, 8, 1, 16), (31, 4, 2, 3)])
+@pytest.mark.parametrize("with_norm", [True, False])
+def test_attn_decode_qkv_is_the_two_kernels_in_one(card, n0, Hq, Hk, S, with_norm):
+    """the step's own attention from the fused qkv row against norm_rope_kv followed by attn_decode: the same output
+    bits, the same cache row, nothing else in the cache touched - with slot n0 first, last and inside its span"""
+    from btb_amd.decode import StackConfig, rope_tables
+
+    D = 128
+    cap = n0 + 6
+    g = gen(640 + n0 + Hq)
+    K0 = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda()
+    V0 = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda()
+    qkv = torch.randn(1, (Hq + 2 * Hk) * D, generator=g).to(torch.bfloat16).cuda()
+    wq = (1.0 + 0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).cuda() if with_norm else None
+    wk = (1.0 + 0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).cuda() if with_norm else None
+    cfg = StackConfig(layers=1, hidden=256, q_heads=Hq, kv_heads=Hk, head_dim=D, intermediate=256, vocab=256)
+    cos, sin = rope_tables(cfg, cap, "cuda")
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    scale = 1.0 / np.sqrt(D)
+    scratch = card.attn_scratch(1, Hq, Hk, D, S)
+    Ka, Va = K0.clone(), V0.clone()
+    q = torch.zeros(1, Hq * D, dtype=torch.bfloat16, device="cuda")
+    want = torch.zeros(1, Hq * D, dtype=torch.bfloat16, device="cuda")
+    card.norm_rope_kv(qkv, wq, wk, 1e-6, cos, sin, n0t, Ka, Va, q, Hq, Hk, D)
+    card.attn_decode(q, Ka, Va, want, n0t, Hq, Hk, D, scale, S, scratch)
+    Kb, Vb = K0.clone(), V0.clone()
+    got = torch.zeros_like(want)
+    scratch.fill_(float("nan"))
+    card.attn_decode_qkv(qkv, wq, wk, 1e-6, cos, sin, n0t, Kb, Vb, got, Hq, Hk, D, scale, S, scratch)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    assert torch.equal(Ka, Kb) and torch.equal(Va, Vb)
+    assert not torch.equal(Kb[:, n0], K0[:, n0])  # the row was written
+
+
 def test_silu_mul_and_argmax_and_embed(card):
     gu = acts_bf16(3, 2 * 768, seed=630)
     m = torch.empty(3, 768, dtype=torch.bfloat16, device="cuda")
