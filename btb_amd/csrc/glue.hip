@@ -373,8 +373,10 @@ __global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restric
     }
 }
 
-// one workgroup of 1024 per row: each thread its own strided elements in ascending order (a tie keeps the earlier),
-// then the (value, index) maximum over the block in the total order value descending, index ascending
+// one workgroup of 1024 per row: each thread its own strided elements in ascending order, taking an element only when
+// it is strictly larger than its best so far (a tie keeps the earlier; a NaN never wins; the scan starts from -inf as
+// native/src/sample.rs:53-67 does), then the (value, index) maximum over the block in the total order value descending,
+// index ascending
 __global__ void __launch_bounds__(1024) argmax_kernel(const uint16_t* __restrict__ logits, int32_t* __restrict__ out,
                                                       int V) {
     __shared__ float s_v[16];
@@ -383,11 +385,37 @@ __global__ void __launch_bounds__(1024) argmax_kernel(const uint16_t* __restrict
     const uint16_t* row = logits + (size_t)t * V;
     float bv = bits_f32(0xff800000u);
     int bi = 0x7fffffff;
-    for (int i = tid; i < V; i += 1024) {
-        const float v = bf16_f32(row[i]);
-        if (v > bv || bi == 0x7fffffff) {
-            bv = v;
-            bi = i;
+    if ((V & 7) == 0 && (reinterpret_cast<uintptr_t>(row) & 15u) == 0) {
+        // eight logits a load, four loads in flight: a thread meets its elements in ascending index order
+        const uint4* row8 = reinterpret_cast<const uint4*>(row);
+        const int n8 = V / 8;
+        for (int base = tid; base < n8; base += 4 * 1024) {
+            uint4 v[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = row8[min(base + q * 1024, n8 - 1)];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int i8 = base + q * 1024;
+                if (i8 < n8) {
+                    const uint32_t w[4] = {v[q].x, v[q].y, v[q].z, v[q].w};
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        const float x = (e & 1) ? bf16hi_f32(w[e >> 1]) : bf16lo_f32(w[e >> 1]);
+                        if (x > bv) {
+                            bv = x;
+                            bi = i8 * 8 + e;
+                        }
+                    }
+                }
+            }
+        }
+    } else {
+        for (int i = tid; i < V; i += 1024) {
+            const float v = bf16_f32(row[i]);
+            if (v > bv) {
+                bv = v;
+                bi = i;
+            }
         }
     }
 #pragma unroll
@@ -410,7 +438,7 @@ __global__ void __launch_bounds__(1024) argmax_kernel(const uint16_t* __restrict
                 bv = s_v[k];
                 bi = s_i[k];
             }
-        out[t] = bi;
+        out[t] = bi == 0x7fffffff ? 0 : bi;  // nothing above -inf (or only NaNs): index 0, as the reference's scan
     }
 }
 

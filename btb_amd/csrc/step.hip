@@ -308,7 +308,7 @@ __device__ __forceinline__ void tile_out(float (&acc)[RPW][1], const int (&outs)
                 st_dev(&y[outs[j]], b);
                 if (HEAD) {
                     const float v = bf16_f32(b);
-                    if (v > best_v || best_i == 0x7fffffff) {  // rows ascend within the lane: a tie keeps the earlier
+                    if (v > best_v) {  // rows ascend within the lane: a tie keeps the earlier; a NaN never wins
                         best_v = v;
                         best_i = outs[j];
                     }
@@ -636,7 +636,7 @@ __global__ void __launch_bounds__(256, 3) decode_step_kernel(StepArgs a) {
     for (int s = 32; s > 0; s >>= 1) {
         const float ov = __shfl_xor(best_v, s, WAVE);
         const int oi = __shfl_xor(best_i, s, WAVE);
-        if (oi != 0x7fffffff && (best_i == 0x7fffffff || ov > best_v || (ov == best_v && oi < best_i))) {
+        if (ov > best_v || (ov == best_v && oi < best_i)) {
             best_v = ov;
             best_i = oi;
         }
@@ -653,7 +653,7 @@ __global__ void __launch_bounds__(256, 3) decode_step_kernel(StepArgs a) {
     for (int w = threadIdx.x; w < nwaves; w += 256) {
         const float v = ld_dev(&a.cand_v[w]);
         const int i = ld_dev(&a.cand_i[w]);
-        if (i != 0x7fffffff && (bi == 0x7fffffff || v > bv || (v == bv && i < bi))) {
+        if (v > bv || (v == bv && i < bi)) {
             bv = v;
             bi = i;
         }
@@ -665,10 +665,11 @@ __global__ void __launch_bounds__(256, 3) decode_step_kernel(StepArgs a) {
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int k = 1; k < 256; ++k)
-            if (s_bi[k] != 0x7fffffff && (bi == 0x7fffffff || s_bv[k] > bv || (s_bv[k] == bv && s_bi[k] < bi))) {
+            if (s_bv[k] > bv || (s_bv[k] == bv && s_bi[k] < bi)) {
                 bv = s_bv[k];
                 bi = s_bi[k];
             }
+        if (bi == 0x7fffffff) bi = 0;  // nothing above -inf: index 0, as the reference's scan
         a.picked[0] = bi;
         a.ids[0] = bi;
         a.n0[0] = n0 + 1;

@@ -141,6 +141,25 @@ def test_silu_mul_and_argmax_and_embed(card):
     out = torch.zeros(2, dtype=torch.int32, device="cuda")
     card.argmax(logits.cuda(), out)
     assert out.tolist() == [777, 151935]
+    # the reference's scan (native/src/sample.rs:53-67): a NaN never wins, a row with nothing above -inf gives 0,
+    # and a width that is no multiple of 8 takes the element-wise path
+    odd = acts_bf16(4, 1003, seed=633)
+    odd[0, 0] = float("nan")
+    odd[0, 500] = odd[0, 1002] = 9.0
+    odd[1, :] = float("-inf")
+    odd[2, :] = float("nan")
+    odd[3, 1002] = 50.0
+    out4 = torch.zeros(4, dtype=torch.int32, device="cuda")
+    card.argmax(odd.cuda(), out4)
+    assert out4.tolist() == [500, 0, 0, 1002]
+    wide = acts_bf16(2, 4096, seed=634)
+    wide[0, 8] = float("nan")
+    wide[0, 4095] = wide[0, 9] = 12.0
+    wide[1, :] = float("-inf")
+    wide[1, 3000] = -1e30
+    out2 = torch.zeros(2, dtype=torch.int32, device="cuda")
+    card.argmax(wide.cuda(), out2)
+    assert out2.tolist() == [9, 3000]
     table = weights_bf16(1000, 64, seed=632).cuda()
     ids = torch.tensor([5, 999, 0], dtype=torch.int32, device="cuda")
     h = torch.zeros(3, 64, dtype=torch.bfloat16, device="cuda")
