@@ -16,6 +16,7 @@ namespace btb {
 // ------------------------------------------------------------------------------------------------------------
 struct FmtBf16 {
     static constexpr int UW = 8;
+    static constexpr bool TWO_ROWS = false;  // the tile shape the streaming matvec prefers for this form (gemv.hip)
     struct Params {
         const uint4* w;
     };
@@ -25,6 +26,7 @@ struct FmtBf16 {
     struct RowCtx {
         const uint4* row;
     };
+    __device__ static __forceinline__ void prepare(Params&) {}
     __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
         return RowCtx{p.w + r * (size_t)units};
     }
@@ -51,6 +53,7 @@ struct FmtBf16 {
 // ------------------------------------------------------------------------------------------------------------
 struct FmtP12 {
     static constexpr int UW = 16;
+    static constexpr bool TWO_ROWS = false;
     struct Params {
         const uint8_t* lo;
         const uint8_t* hi4;
@@ -58,6 +61,7 @@ struct FmtP12 {
         const int32_t* esc_idx;
         const uint8_t* esc_val;
         const int32_t* row_ptr;  // [rows + 1] first escape at or past each row's start
+        uint4 tbl;               // the table in registers: filled by prepare() on the device, not by the host
     };
     struct Raw {
         uint4 lo;
@@ -78,11 +82,13 @@ struct FmtP12 {
                    ((uint32_t)t[4 * k + 3] << 24);
         return make_uint4(d[0], d[1], d[2], d[3]);
     }
+    // once per kernel (or phase), before any row_ctx: the table's 16 bytes are read here and only here
+    __device__ static __forceinline__ void prepare(Params& p) { p.tbl = load_table(p.table); }
     __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
         RowCtx c;
         c.lo = reinterpret_cast<const uint4*>(p.lo) + r * (size_t)units;
         c.hi4 = reinterpret_cast<const uint2*>(p.hi4) + r * (size_t)units;
-        c.table = load_table(p.table);
+        c.table = p.tbl;
         c.e0 = p.row_ptr[r];
         c.e1 = p.row_ptr[r + 1];
         return c;
@@ -90,13 +96,15 @@ struct FmtP12 {
     __device__ static __forceinline__ Raw load(const RowCtx& c, int unit) {
         return Raw{load_stream16(c.lo + unit), load_stream8(c.hi4 + unit)};
     }
-    // four codes (one per byte of v) to their four table bytes
+    // four codes (one per byte of v) to their four table bytes: two byte-permutes look the code's low three bits up
+    // in entries 0..7 and in entries 8..15, a third picks per byte between the two by the code's top bit (selector
+    // i takes byte i of the first lookup, 4 + i of the second)
     __device__ static __forceinline__ uint32_t lut16(const uint4& t, uint32_t v) {
         const uint32_t sel = v & 0x07070707u;
         const uint32_t a = __builtin_amdgcn_perm(t.y, t.x, sel);  // entries 0..7
         const uint32_t b = __builtin_amdgcn_perm(t.w, t.z, sel);  // entries 8..15
-        const uint32_t m = ((v >> 3) & 0x01010101u) * 0xFFu;      // 0xFF in the bytes whose code is 8..15
-        return (b & m) | (a & ~m);
+        const uint32_t pick = 0x03020100u | ((v & 0x08080808u) >> 1);
+        return __builtin_amdgcn_perm(b, a, pick);
     }
     // eight weights as four bf16 pairs: codes c (weight k in nibble k), their low bytes l0 (weights 0..3), l1 (4..7).
     // A byte-permute's selector 0..3 takes a byte of its second operand, 4..7 of its first.
@@ -145,6 +153,7 @@ struct FmtP12 {
 // ------------------------------------------------------------------------------------------------------------
 struct FmtF8 {
     static constexpr int UW = 16;
+    static constexpr bool TWO_ROWS = true;
     struct Params {
         const uint8_t* w;
         const float* scales;
@@ -163,6 +172,7 @@ struct FmtF8 {
         int upb;
         uint32_t magic;
     };
+    __device__ static __forceinline__ void prepare(Params&) {}
     __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
         return RowCtx{reinterpret_cast<const uint4*>(p.w) + r * (size_t)units, p.scales + (r / p.bm) * (size_t)p.sc,
                       p.upb, p.magic};
@@ -199,6 +209,7 @@ struct FmtF8 {
 // ------------------------------------------------------------------------------------------------------------
 struct FmtMx4 {
     static constexpr int UW = 32;
+    static constexpr bool TWO_ROWS = false;
     struct Params {
         const uint8_t* blocks;
         const uint8_t* scales;
@@ -211,6 +222,7 @@ struct FmtMx4 {
         const uint4* row;
         const uint8_t* srow;
     };
+    __device__ static __forceinline__ void prepare(Params&) {}
     __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
         return RowCtx{reinterpret_cast<const uint4*>(p.blocks) + r * (size_t)units, p.scales + r * (size_t)units};
     }

@@ -110,6 +110,7 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs x
     const int wave = blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
     const int nwaves = gridDim.x * (blockDim.x / WAVE);
     const int ntiles = (Rout + ROWS - 1) / ROWS;
+    F::prepare(p);
 
     typename F::Raw first[U][RPW] = {};
     stage_x<XMODE>(xs, xa, M, C, [&] {
@@ -175,13 +176,17 @@ static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void
 
 template <class F, int M, int LPR, int XMODE, int EPI>
 static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void* y, int R, int C, hipStream_t st) {
-    if (EPI == E_GLU) return launch_variant<F, M, LPR, 2, (M <= 2 ? 4 : 2), XMODE, E_GLU>(p, xa, y, R, C, st);
-    // Rows per wave tile (RPW) and units in flight per row (U), measured on MI355X at the Qwen3-4B shapes: two rows
-    // by four units where the matrix has rows enough to give every SIMD several waves that way, else one row by
-    // eight units. Neither changes a result bit (a lane's units stay in ascending order).
+    // Rows per wave tile (RPW) and units in flight per row (U), measured on MI355X. bf16 at M <= 2: two rows by four
+    // units where the matrix has rows enough to give every SIMD several waves that way, else one row by eight. The
+    // forms that widen in registers spend those registers on the widening, and run best with half the span and more
+    // waves resident: one row by four (pack12, MXFP4), two rows by two (FP8, whose two rows share a scale fetch
+    // pattern). Neither choice changes a result bit (a lane's units stay in ascending order).
+    constexpr bool WIDENS = sizeof(typename F::Raw) != 16;  // everything but plain bf16
+    if (EPI == E_GLU) return launch_variant<F, M, LPR, 2, (M <= 2 && !WIDENS ? 4 : 2), XMODE, E_GLU>(p, xa, y, R, C, st);
     const int v = tuning("gemv_variant");
-    const bool tall = v >= 0 ? (v == 1) : (R >= 4096 * (WAVE / LPR));
-    if (M <= 2) {
+    const int shorter = tuning("gemv_short_span");
+    const bool tall = v >= 0 ? (v == 1) : (WIDENS ? F::TWO_ROWS : R >= 4096 * (WAVE / LPR));
+    if (M <= 2 && (shorter >= 0 ? shorter == 0 : !WIDENS)) {
         if (tall) return launch_variant<F, M, LPR, 2, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
         return launch_variant<F, M, LPR, 1, 8, XMODE, E_PLAIN>(p, xa, y, R, C, st);
     }

@@ -154,7 +154,8 @@ template <>
 __device__ __forceinline__ FmtP12::Params mat_params<FmtP12>(const StepMat& m) {
     return FmtP12::Params{static_cast<const uint8_t*>(m.w),       static_cast<const uint8_t*>(m.hi4),
                           static_cast<const uint8_t*>(m.table),   static_cast<const int32_t*>(m.esc_idx),
-                          static_cast<const uint8_t*>(m.esc_val), static_cast<const int32_t*>(m.row_ptr)};
+                          static_cast<const uint8_t*>(m.esc_val), static_cast<const int32_t*>(m.row_ptr),
+                          make_uint4(0, 0, 0, 0)};
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -281,7 +282,8 @@ __device__ __forceinline__ void prefetch_span(PRE_T& pre, const StepMat& mat, in
     constexpr int RPW = PRE_T::RPW, U = PRE_T::U;
     const Deal d = deal_tiles<LPR, EPI, RPW>(R, wave, nwaves);
     if (d.first >= d.last) return;
-    const typename F::Params p = mat_params<F>(mat);
+    typename F::Params p = mat_params<F>(mat);
+    F::prepare(p);
     const int units = C / F::UW;
     const int lane = phase_tid() & 63;
     typename F::RowCtx ctx[RPW];
@@ -350,7 +352,8 @@ template <bool HEAD, PRE_ARGS>
 __device__ __forceinline__ void matvec_phase(PRE_T& pre, const StepMat& mat, const uint32_t* xs, uint16_t* y, int R,
                                              int C, int wave, int nwaves, float& best_v, int& best_i) {
     const Deal d = deal_tiles<LPR, EPI, PRE_T::RPW>(R, wave, nwaves);
-    const typename F::Params p = mat_params<F>(mat);
+    typename F::Params p = mat_params<F>(mat);
+    F::prepare(p);
     const int lane = phase_tid() & 63;
     if (d.first >= d.last) return;
     tile_body<HEAD, true>(pre, p, d.first, xs, y, R, C, lane, best_v, best_i);
