@@ -63,8 +63,7 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
         const uint4* src = reinterpret_cast<const uint4*>(a.x);
         uint4* dst = reinterpret_cast<uint4*>(xs);
         const int n = M * C / 8;
-        uint4 v0 = make_uint4(0, 0, 0, 0);
-        if (tid < n) v0 = src[tid];
+        const uint4 v0 = src[min(tid, n - 1)];
         after_issue();
         if (tid < n) dst[tid] = v0;
         for (int i = tid + nt; i < n; i += nt) dst[i] = src[i];
@@ -97,13 +96,12 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
                 uint2 hv[PER], yv[PER], wv[PER];
 #pragma unroll
                 for (int q = 0; q < PER; ++q) {
-                    const int i = base + q * 256 + tid;
-                    hv[q] = yv[q] = wv[q] = make_uint2(0, 0);
-                    if (i < n4) {
-                        hv[q] = hs[i];
-                        if (ys != nullptr) yv[q] = ys[i];
-                        if (m == 0) wv[q] = ws[i];
-                    }
+                    // a word past the row's end reads the last word again: the loads stay unconditional, and the
+                    // wait for them is then counted exactly (they are not held up behind the weights requested next)
+                    const int i = min(base + q * 256 + tid, n4 - 1);
+                    hv[q] = hs[i];
+                    yv[q] = ys != nullptr ? ys[i] : make_uint2(0, 0);
+                    wv[q] = ws[i];
                 }
                 if (m == 0 && base == 0) after_issue();
 #pragma unroll
@@ -186,7 +184,31 @@ __device__ __forceinline__ void fma_unit(const typename F::RowCtx (&ctx)[RPW], c
 // up rows; a wave works on gate row r and up row I + r together and writes m[m][r] = bf16(bf16(silu(g)) * u) with
 // g, u the two sums rounded to bf16 first - the values the gate_up matvec followed by btb_silu_mul would have
 // written (the reference's btb_gemv_mma_glu_silu does the same fold: native/cuda/btb_gemv_mma.cuh:216-315).
-enum Epilogue { E_PLAIN = 0, E_GLU = 1 };
+// E_GLU_SPLIT: the same fold with the gate row and the up row side by side in one wave - even row groups of the
+// wave take gate rows, the odd group next to each its up row (rows of at most 32 lanes) - and the two sums meeting by
+// one cross-lane exchange: the tile shape of a one-row-per-lane pass, which the register-hungry packed forms prefer.
+enum Epilogue { E_PLAIN = 0, E_GLU = 1, E_GLU_SPLIT = 2 };
+
+// output rows a wave's tile covers, and the weight row of the lane's row group (set j) with the row its sum goes to
+template <int LPR, int RPW, int EPI>
+__host__ __device__ constexpr int tile_outputs() {
+    return EPI == E_GLU ? WAVE / LPR : EPI == E_GLU_SPLIT ? WAVE / LPR / 2 : (WAVE / LPR) * RPW;
+}
+template <int LPR, int RPW, int EPI>
+__device__ __forceinline__ int tile_row(int tile, int j, int lane, int R, int& out_row) {
+    constexpr int G = WAVE / LPR;
+    const int grp = lane / LPR;
+    if (EPI == E_GLU) {
+        out_row = tile * G + grp;
+        return min(out_row, R / 2 - 1) + j * (R / 2);
+    }
+    if (EPI == E_GLU_SPLIT) {
+        out_row = tile * (G / 2) + grp / 2;
+        return min(out_row, R / 2 - 1) + (grp & 1) * (R / 2);
+    }
+    out_row = tile * G * RPW + j * G + grp;
+    return min(out_row, R - 1);  // a row past the end reads the last row again (no divergence) and is not written
+}
 
 // where the kernel reads x from: LDS (staged once per workgroup) or straight from global memory through the caches
 enum XSrc { XS_LDS = 0, XS_GLOBAL = 1 };

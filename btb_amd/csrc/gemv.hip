@@ -29,26 +29,18 @@ namespace btb {
 template <class F, int M, int LPR, int RPW, int U, int EPI, bool PRIMED>
 __device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typename F::Raw (&first)[U][RPW], int tile,
                                           const uint4* xs4, uint16_t* __restrict__ y, int R, int C, int lane) {
-    constexpr int G = WAVE / LPR;                      // rows a wave covers per set
-    constexpr int ROWS = EPI == E_GLU ? G : G * RPW;   // output rows a wave covers per tile
-    const int Rout = EPI == E_GLU ? R / 2 : R;
+    const int Rout = EPI == E_PLAIN ? R : R / 2;
     const int units = C / F::UW;         // units per row
     const int sl = lane % LPR;           // the lane's place among its row's lanes
     const int span = U * LPR;
     const int xrow4 = C / 8;             // uint4 per row of x
     typename F::RowCtx ctx[RPW];
     int rows[RPW];   // weight rows
-    int out_row;     // E_GLU: the output row of the pair
+    int outs[RPW];   // the rows their sums are written to (the GLU forms: the output row of the pair)
 #pragma unroll
     for (int j = 0; j < RPW; ++j) {
-        if (EPI == E_GLU) {
-            out_row = tile * ROWS + lane / LPR;
-            rows[j] = min(out_row, Rout - 1) + j * Rout;
-        } else {
-            rows[j] = tile * ROWS + j * G + lane / LPR;
-        }
-        // a row past the end reads the last row again (no divergence in the stream) and is not written
-        ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
+        rows[j] = tile_row<LPR, RPW, EPI>(tile, j, lane, R, outs[j]);
+        ctx[j] = F::row_ctx(p, (size_t)rows[j], units);
     }
     float acc[RPW][M];
 #pragma unroll
@@ -73,15 +65,23 @@ __device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typ
     }
 #pragma unroll
     for (int j = 0; j < RPW; ++j)
-        F::template tail<M>(p, ctx[j], (size_t)min(rows[j], R - 1), sl, LPR, C, reinterpret_cast<const uint32_t*>(xs4),
-                            acc[j]);
-    if (EPI == E_GLU) {
+        F::template tail<M>(p, ctx[j], (size_t)rows[j], sl, LPR, C, reinterpret_cast<const uint32_t*>(xs4), acc[j]);
+    if constexpr (EPI == E_GLU) {
 #pragma unroll
         for (int m = 0; m < M; ++m) {
             const float g = bfround(group_sum<LPR>(acc[0][m]));
             const float u = bfround(group_sum<LPR>(acc[RPW - 1][m]));
             const float sg = bfround(g / (1.f + expf(-g)));
-            if (sl == 0 && out_row < Rout) y[(size_t)m * Rout + out_row] = f32_bf16(sg * u);
+            if (sl == 0 && outs[0] < Rout) y[(size_t)m * Rout + outs[0]] = f32_bf16(sg * u);
+        }
+    } else if (EPI == E_GLU_SPLIT) {
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const float mine = group_sum<LPR>(acc[0][m]);
+            const float other = __shfl_xor(mine, LPR, WAVE);  // the neighbouring row group's sum: the up row's
+            const float g = bfround(mine), u = bfround(other);
+            const float sg = bfround(g / (1.f + expf(-g)));
+            if (sl == 0 && ((lane / LPR) & 1) == 0 && outs[0] < Rout) y[(size_t)m * Rout + outs[0]] = f32_bf16(sg * u);
         }
     } else {
 #pragma unroll
@@ -89,7 +89,7 @@ __device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typ
 #pragma unroll
             for (int m = 0; m < M; ++m) {
                 const float s = group_sum<LPR>(acc[j][m]);
-                if (sl == 0 && rows[j] < R) y[(size_t)m * R + rows[j]] = f32_bf16(s);
+                if (sl == 0 && outs[j] < R) y[(size_t)m * R + outs[j]] = f32_bf16(s);
             }
     }
 }
@@ -101,10 +101,10 @@ __device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typ
 template <class F, int M, int LPR, int RPW, int U, int XMODE, int EPI>
 __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs xa, uint16_t* __restrict__ y, int R, int C) {
     extern __shared__ __align__(16) uint32_t xs[];  // [M][C / 2] packed bf16 pairs
-    static_assert(EPI == E_PLAIN || RPW == 2, "the GLU form pairs a gate row with an up row");
-    constexpr int G = WAVE / LPR;
-    constexpr int ROWS = EPI == E_GLU ? G : G * RPW;
-    const int Rout = EPI == E_GLU ? R / 2 : R;
+    static_assert(EPI != E_GLU || RPW == 2, "the GLU form pairs a gate row with an up row");
+    static_assert(EPI != E_GLU_SPLIT || (RPW == 1 && LPR <= 32), "the split GLU form: gate and up in neighbouring row groups");
+    constexpr int ROWS = tile_outputs<LPR, RPW, EPI>();
+    const int Rout = EPI == E_PLAIN ? R : R / 2;
     const int units = C / F::UW;
     const int lane = threadIdx.x & (WAVE - 1);
     const int wave = blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
@@ -118,9 +118,8 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs x
             typename F::RowCtx ctx[RPW];
 #pragma unroll
             for (int j = 0; j < RPW; ++j) {
-                const int row = EPI == E_GLU ? min(wave * ROWS + lane / LPR, Rout - 1) + j * Rout
-                                             : min(wave * ROWS + j * G + lane / LPR, R - 1);
-                ctx[j] = F::row_ctx(p, (size_t)row, units);
+                int out_row;
+                ctx[j] = F::row_ctx(p, (size_t)tile_row<LPR, RPW, EPI>(wave, j, lane, R, out_row), units);
             }
             load_span<F, LPR, RPW, U, true>(first, ctx, 0, lane % LPR, units);
         }
@@ -145,8 +144,7 @@ static int lanes_per_row(int units) {
 
 template <class F, int M, int LPR, int RPW, int U, int XMODE, int EPI>
 static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void* y, int R, int C, hipStream_t st) {
-    constexpr int G = WAVE / LPR;
-    constexpr int ROWS = EPI == E_GLU ? G : G * RPW;
+    constexpr int ROWS = tile_outputs<LPR, RPW, EPI>();
     const DeviceInfo& dev = device_info();
     const size_t lds = stage_lds_bytes(XMODE, M, C);
     if (lds > (size_t)dev.lds_bytes) {
@@ -155,7 +153,7 @@ static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void
     }
     // Every workgroup stages x once, so the grid is kept to a few workgroups a CU and each wave walks a whole number
     // of tiles (the last wave of the grid may walk fewer): tiles_per_wave is the smallest count that fits the cap.
-    const int Rout = EPI == E_GLU ? R / 2 : R;
+    const int Rout = EPI == E_PLAIN ? R : R / 2;
     const int ntiles = (Rout + ROWS - 1) / ROWS;
     int per_cu = tuning("gemv_wgs_per_cu");
     if (per_cu <= 0) per_cu = 6;
@@ -182,7 +180,13 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
     // waves resident: one row by four (pack12, MXFP4), two rows by two (FP8, whose two rows share a scale fetch
     // pattern). Neither choice changes a result bit (a lane's units stay in ascending order).
     constexpr bool WIDENS = sizeof(typename F::Raw) != 16;  // everything but plain bf16
-    if (EPI == E_GLU) return launch_variant<F, M, LPR, 2, (M <= 2 && !WIDENS ? 4 : 2), XMODE, E_GLU>(p, xa, y, R, C, st);
+    if constexpr (EPI == E_GLU) {
+        // a widening form whose rows take at most 32 lanes: gate and up side by side, one row a lane
+        if constexpr (WIDENS && LPR <= 32) {
+            if (tuning("gemv_glu_split") != 0) return launch_variant<F, M, LPR, 1, 4, XMODE, E_GLU_SPLIT>(p, xa, y, R, C, st);
+        }
+        return launch_variant<F, M, LPR, 2, (M <= 2 && !WIDENS ? 4 : 2), XMODE, E_GLU>(p, xa, y, R, C, st);
+    }
     const int v = tuning("gemv_variant");
     const int shorter = tuning("gemv_short_span");
     const bool tall = v >= 0 ? (v == 1) : (WIDENS ? F::TWO_ROWS : R >= 4096 * (WAVE / LPR));
