@@ -19,6 +19,8 @@ from typing import Any
 
 import torch
 
+from .fp8 import F8Weight
+from .mxfp4 import MxWeight
 from .pack12 import P12Weight
 
 
@@ -75,11 +77,20 @@ class Linear:
 
     @property
     def nbytes(self) -> int:
-        return int(self.w.nbytes) if isinstance(self.w, P12Weight) else int(self.w.numel()) * 2
+        return int(self.w.numel()) * 2 if isinstance(self.w, torch.Tensor) else int(self.w.nbytes)
+
+    @property
+    def fusable(self) -> bool:
+        """whether the residual add + norm and the gate/up activation can ride in this matrix's matvec (bf16, pack12)"""
+        return isinstance(self.w, (torch.Tensor, P12Weight))
 
     def matvec(self, x: torch.Tensor, y: torch.Tensor) -> None:
         if isinstance(self.w, P12Weight):
             self.card.gemv_p12(self.w, x, y)
+        elif isinstance(self.w, F8Weight):
+            self.card.gemv_fp8(self.w, x, y)
+        elif isinstance(self.w, MxWeight):
+            self.card.gemv_mx4(self.w, x, y)
         else:
             self.card.gemv(self.w, x, y)
 
@@ -119,7 +130,9 @@ class DecodeStep:
         self.S = int(attn_spans)
         self.scratch = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
         self.fold_silu = bool(fold_silu)
-        self.fused = bool(fused)
+        # the fused launches exist for bf16 and 12-bit matrices; any other stored form takes one launch per operator
+        lins = [weights[f"layers.{i}.{k}"] for i in range(cfg.layers) for k in ("qkv", "o", "gu", "down")] + [weights["head"]]
+        self.fused = bool(fused) and all(getattr(m, "fusable", False) for m in lins)
         # the handoff to the host: token, cache length and the GPU's clock in pinned memory
         self.host_tok = torch.zeros(1, dtype=torch.int32).pin_memory()
         self.host_n0 = torch.zeros(1, dtype=torch.int32).pin_memory()

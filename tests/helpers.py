@@ -85,3 +85,39 @@ def conditioned_err(y: np.ndarray, w64: np.ndarray, x64: np.ndarray) -> float:
     ref = x64 @ w64.T
     scale = np.abs(x64) @ np.abs(w64).T
     return float(np.max(np.abs(y.astype(np.float64) - ref) / np.maximum(scale, 1e-300)))
+
+
+def reference_logits(cfg, get, prompt):
+    """the last position's logits of a Qwen3-style dense stack in f32 torch: the textbook forward pass"""
+    H, D, Hq, Hk = cfg.hidden, cfg.head_dim, cfg.q_heads, cfg.kv_heads
+    x = get("model.embed_tokens.weight")[torch.tensor(prompt)]
+    T = x.shape[0]
+    pos = torch.arange(T, dtype=torch.float32)
+    inv = 1.0 / (cfg.rope_theta ** (torch.arange(0, D // 2, dtype=torch.float32) * 2.0 / D))
+    ang = torch.cat([pos[:, None] * inv[None, :]] * 2, dim=-1)
+    cos, sin = ang.cos()[:, None, :], ang.sin()[:, None, :]
+
+    def norm(v, wname):
+        return v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + cfg.eps) * get(wname)
+
+    def rope(v):
+        rot = torch.cat([-v[..., D // 2 :], v[..., : D // 2]], dim=-1)
+        return v * cos + rot * sin
+
+    for i in range(cfg.layers):
+        L = f"model.layers.{i}."
+        h = norm(x, L + "input_layernorm.weight")
+        q = (h @ get(L + "self_attn.q_proj.weight").T).reshape(T, Hq, D)
+        k = (h @ get(L + "self_attn.k_proj.weight").T).reshape(T, Hk, D)
+        v = (h @ get(L + "self_attn.v_proj.weight").T).reshape(T, Hk, D)
+        q, k = rope(norm(q, L + "self_attn.q_norm.weight")), rope(norm(k, L + "self_attn.k_norm.weight"))
+        k, v = k.repeat_interleave(Hq // Hk, dim=1), v.repeat_interleave(Hq // Hk, dim=1)
+        s = torch.einsum("thd,shd->hts", q, k) / D**0.5
+        s = s.masked_fill(torch.triu(torch.ones(T, T, dtype=torch.bool), 1), float("-inf"))
+        a = torch.einsum("hts,shd->thd", s.softmax(-1), v).reshape(T, Hq * D)
+        x = x + a @ get(L + "self_attn.o_proj.weight").T
+        h = norm(x, L + "post_attention_layernorm.weight")
+        g, u = h @ get(L + "mlp.gate_proj.weight").T, h @ get(L + "mlp.up_proj.weight").T
+        x = x + (torch.nn.functional.silu(g) * u) @ get(L + "mlp.down_proj.weight").T
+    x = norm(x, "model.norm.weight")
+    return (x[-1] @ get("model.embed_tokens.weight").T).numpy()
