@@ -1,6 +1,7 @@
 """Benchmark of the decode hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode|decode_p12] [--no-cpu]
+    python bench.py --workload gemv_bf16|gemv_p12|gemv_fp8|gemv_mxfp4|moe [--m M]      (the other configs, one kernel each)
 
 A step is one decode step of a random-init Qwen3-4B-shaped dense stack (36 layers, hidden 2560, 32 query / 8 kv heads
 of 128, SwiGLU 9728, vocab 151936; weights ~N(0, 0.02) in bf16, seeded N(0, 1) K/V for a 4096-token context), M = 1
@@ -54,17 +55,135 @@ def cpu_baseline(budget_s: float = 12.0) -> dict:
                       f"f32 x and y, all {cores} host threads, {dt:.1f} s"}
 
 
+def kernel_workload(args: argparse.Namespace) -> int:
+    """The single-operator configs: one JSON line each, `value` the operator's HBM stream in GB/s. A step is one call
+    over the next operand set of a pool larger than the last-level cache (256 MB), so nothing repeats from cache; the
+    calls of one pass are replayed as a hipGraph and timed with device events.
+
+      gemv_bf16   configs[0] (C1): W bf16 [9728, 2560], M rows of x
+      gemv_p12    the same matrix packed to 12 bits a weight
+      gemv_fp8    C5a: fp8.quantize(N(0, 0.02) [18432, 7168], (128, 128))
+      gemv_mxfp4  C5b: the same source through the MXFP4 encoder
+      moe         C4: router [128, 2048] + top-8 of 128 experts (gate_up [1536, 2048], down [2048, 768]), M tokens
+    """
+    import torch
+
+    from btb_amd import fp8, mxfp4
+    from btb_amd.moe import Experts, Router
+    from btb_amd.native import Native
+    from btb_amd.pack12 import P12Weight
+
+    card = Native.card_kernels()
+    dev, M = torch.device("cuda"), int(args.m)
+    g = torch.Generator(device=dev).manual_seed(0x0B7B0500)
+    bf = dict(dtype=torch.bfloat16, device=dev)
+
+    def normal(*shape: int) -> torch.Tensor:
+        return torch.randn(*shape, generator=g, device=dev, dtype=torch.float32) * 0.02
+
+    name = args.workload
+    if name == "moe":
+        E, k, H, I, pool = 128, 8, 2048, 768, 2
+        sets = [(Router(card, normal(E, H).to(torch.bfloat16), k), Experts(card, normal(E, 2 * I, H).to(torch.bfloat16),
+                                                                           normal(E, H, I).to(torch.bfloat16)))
+                for _ in range(pool)]
+        x = torch.randn(M, H, generator=g, device=dev).to(torch.bfloat16)
+        distinct = []
+
+        def call(i: int) -> None:
+            router, experts = sets[i]
+            _, w, idx = router(x)
+            experts(x, idx, w)
+
+        for i in range(pool):  # the bytes a call streams: the router and every DISTINCT expert its picks name
+            _, _, idx = sets[i][0](x)
+            distinct.append(int(torch.unique(idx).numel()))
+        per_expert = (2 * I * H + H * I) * 2
+        nbytes = [E * H * 2 + d * per_expert for d in distinct]
+        what = f"C4: top-{k} of {E} experts, gate_up [{2 * I}, {H}] + down [{H}, {I}] bf16, M={M} tokens"
+        extra = {"distinct_experts": distinct}
+        dtype = "bf16 weights and activations, f32 accumulate"
+    else:
+        R, C = (9728, 2560) if name in ("gemv_bf16", "gemv_p12") else (18432, 7168)
+        pool = 8 if R == 9728 else 4
+        mats = []
+        for _ in range(pool):
+            t = normal(R, C)
+            if name == "gemv_bf16":
+                mats.append(t.to(torch.bfloat16))
+            elif name == "gemv_p12":
+                mats.append(P12Weight.pack(t.to(torch.bfloat16), card))
+            elif name == "gemv_fp8":
+                q, sc = fp8.quantize(t, (128, 128))
+                mats.append(fp8.F8Weight(q, sc, R, C))
+            else:
+                b, sc = mxfp4.quantize(t)
+                mats.append(mxfp4.MxWeight(b.reshape(-1), sc.reshape(-1), R, C))
+            del t
+        x = torch.randn(M, C, generator=g, device=dev).to(torch.bfloat16)
+        y = torch.empty(M, R, **bf)
+        op = {"gemv_bf16": card.gemv, "gemv_p12": card.gemv_p12, "gemv_fp8": card.gemv_fp8, "gemv_mxfp4": card.gemv_mx4}[name]
+
+        def call(i: int) -> None:
+            op(mats[i], x, y)
+
+        stored = [m.numel() * 2 if isinstance(m, torch.Tensor) else m.nbytes for m in mats]
+        nbytes = [b + 2 * M * C + 2 * M * R for b in stored]
+        what = f"{name} [{R}, {C}], M={M}"
+        extra = {"weight_bytes": stored[0]}
+        dtype = {"gemv_bf16": "bf16", "gemv_p12": "pack12 widened to bf16 in registers",
+                 "gemv_fp8": "fp8 e4m3 x f32 block scale -> bf16 in registers",
+                 "gemv_mxfp4": "mxfp4 -> bf16 in registers"}[name] + ", f32 accumulate"
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        for i in range(pool):
+            call(i)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for i in range(pool):
+            call(i)
+    passes = max(1, (args.steps + pool - 1) // pool)
+    for _ in range(max(1, args.warmup // pool)):
+        graph.replay()
+    torch.cuda.synchronize()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(passes):
+        graph.replay()
+    e1.record()
+    torch.cuda.synchronize()
+    us = e0.elapsed_time(e1) * 1e3 / (passes * pool)
+    mean_bytes = sum(nbytes) / len(nbytes)
+    gbs = mean_bytes / (us * 1e-6) / 1e9
+    print(json.dumps({
+        "metric": "decode matvec HBM GB/s (% of peak), one operator", "value": round(gbs, 1), "unit": "GB/s",
+        "n_gpus": 1, "steps": passes * pool, "warmup": args.warmup, "ms_per_step": round(us * 1e-3, 5),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
+        "data": "synthetic: N(0, 0.02) weights, N(0, 1) x, seeded", "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
+        "config": {"workload": what, "pool": pool, "algorithmic_bytes_per_step": int(mean_bytes), **extra},
+        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
+        "cpu_baseline": None,
+    }))
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
-    ap.add_argument("--workload", default="decode", choices=["decode", "decode_p12"])
+    ap.add_argument("--workload", default="decode",
+                    choices=["decode", "decode_p12", "gemv_bf16", "gemv_p12", "gemv_fp8", "gemv_mxfp4", "moe"])
+    ap.add_argument("--m", type=int, default=1, help="rows of x (tokens) for the single-operator workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         return 2
+    if args.workload not in ("decode", "decode_p12"):
+        return kernel_workload(args)
     if args.steps < 1 or args.warmup < 0 or args.steps + args.warmup > 480:
         print("bench.py: steps + warmup must stay within the cache's 480 spare rows", file=sys.stderr)
         return 2
@@ -168,7 +287,7 @@ def main() -> int:
                          "configs[2]: the same stack with every linear in pack12, widened in registers"),
             "layers": cfg.layers, "hidden": cfg.hidden, "q_heads": cfg.q_heads, "kv_heads": cfg.kv_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate, "vocab": cfg.vocab, "context": CTX,
-            "weight_bytes_per_step": wbytes, "kv_bytes_per_step": kvbytes, "kernels_per_step": 2 + 8 * cfg.layers + 4,
+            "weight_bytes_per_step": wbytes, "kv_bytes_per_step": kvbytes, "kernels_per_step": 4 + 6 * cfg.layers,
             "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
         },
         "roofline": {

@@ -64,6 +64,7 @@ static Knob g_knobs[] = {
     {"gemv_glu_split", {-1}},
     {"mfma_wgs_per_cu", {-1}},
     {"mfma_classic", {-1}},
+    {"mfma_lds", {-1}},
     {"moe_wgs_per_cu", {-1}},
     {"attn_split", {-1}},
 };

@@ -245,8 +245,21 @@ static int32_t run_rows(const typename F::Params& p, XArgs xa, void* y, size_t R
 
 static XArgs plain_x(const void* x) { return XArgs{static_cast<const uint16_t*>(x), nullptr, nullptr, nullptr, 0.f, 0}; }
 
-// the matrix-core form of the bf16 matvec (gemv_mfma.hip)
+// the matrix-core forms of the matvec for the verify widths (gemv_mfma.hip, gemv_mfma_lds.hip)
 int32_t gemv_mfma_bf16(const void* w, const void* x, void* y, int R, int C, int M, hipStream_t st);
+bool mfma_lds_fits_bf16(int R, int C);
+bool mfma_lds_fits_packed(int R, int C);
+int32_t gemv_mfma_lds_bf16(const void* w, const void* x, void* y, int R, int C, int M, hipStream_t st);
+int32_t gemv_mfma_lds_fp8(const void* w, const float* scales, int sc, int bm, int bn, const void* x, void* y, int R,
+                          int C, int M, hipStream_t st);
+int32_t gemv_mfma_lds_mxfp4(const void* blocks, const void* scales, const void* x, void* y, int R, int C, int M,
+                            hipStream_t st);
+
+// whether a pass of M rows goes to the matrix cores through the LDS-staged kernel
+static bool wide_pass(size_t M, size_t R, size_t C, bool packed) {
+    return M >= 8 && (packed ? mfma_lds_fits_packed((int)R, (int)C) : mfma_lds_fits_bf16((int)R, (int)C)) &&
+           tuning("gemv_no_mfma") <= 0 && tuning("mfma_lds") != 0;
+}
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static bool aligned2(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 1u) == 0; }
@@ -299,7 +312,10 @@ int32_t btb_hip_gemv_bf16(const void* w, const void* x, void* y, size_t R, size_
         uint16_t* yp = static_cast<uint16_t*>(y);
         for (size_t m0 = 0; m0 < M; m0 += 32) {
             const int mm = (int)(M - m0 < 32 ? M - m0 : 32);
-            rc = gemv_mfma_bf16(w, xp + m0 * C, yp + m0 * R, (int)R, (int)C, mm, static_cast<hipStream_t>(stream));
+            rc = wide_pass(M, R, C, false) ? gemv_mfma_lds_bf16(w, xp + m0 * C, yp + m0 * R, (int)R, (int)C, mm,
+                                                      static_cast<hipStream_t>(stream))
+                                 : gemv_mfma_bf16(w, xp + m0 * C, yp + m0 * R, (int)R, (int)C, mm,
+                                                  static_cast<hipStream_t>(stream));
             if (rc != OK) return rc;
         }
         return OK;
@@ -386,6 +402,17 @@ int32_t btb_hip_gemv_fp8(const void* w, const void* scales, size_t sr, size_t sc
     if (rc != OK) return rc;
     if (R % sr != 0 || C % sc != 0 || (C / sc) % FmtF8::UW != 0) return ERR_DOMAIN;
     if (!aligned16(w) || !aligned16(x) || (reinterpret_cast<uintptr_t>(scales) & 3u) || !aligned2(y)) return ERR_DOMAIN;
+    if (wide_pass(M, R, C, true)) {  // the verify widths: the matrix cores, 32 rows of x a pass
+        const uint16_t* xp = static_cast<const uint16_t*>(x);
+        uint16_t* yp = static_cast<uint16_t*>(y);
+        for (size_t m0 = 0; m0 < M; m0 += 32) {
+            const int mm = (int)(M - m0 < 32 ? M - m0 : 32);
+            rc = gemv_mfma_lds_fp8(w, static_cast<const float*>(scales), (int)sc, (int)(R / sr), (int)(C / sc),
+                                   xp + m0 * C, yp + m0 * R, (int)R, (int)C, mm, static_cast<hipStream_t>(stream));
+            if (rc != OK) return rc;
+        }
+        return OK;
+    }
     const uint32_t upb = (uint32_t)(C / sc / FmtF8::UW);
     FmtF8::Params p{static_cast<const uint8_t*>(w), static_cast<const float*>(scales), (int)sc, (int)(R / sr),
                     (int)upb, upb > 1 ? (uint32_t)(0x100000000ull / upb + 1) : 0u};
@@ -398,6 +425,17 @@ int32_t btb_hip_gemv_mxfp4(const void* blocks, const void* scales, const void* x
     int32_t rc = check_dims(R, C, M, FmtMx4::UW);
     if (rc != OK) return rc;
     if (!aligned16(blocks) || !aligned16(x) || !aligned2(y)) return ERR_DOMAIN;
+    if (wide_pass(M, R, C, true)) {
+        const uint16_t* xp = static_cast<const uint16_t*>(x);
+        uint16_t* yp = static_cast<uint16_t*>(y);
+        for (size_t m0 = 0; m0 < M; m0 += 32) {
+            const int mm = (int)(M - m0 < 32 ? M - m0 : 32);
+            rc = gemv_mfma_lds_mxfp4(blocks, scales, xp + m0 * C, yp + m0 * R, (int)R, (int)C, mm,
+                                     static_cast<hipStream_t>(stream));
+            if (rc != OK) return rc;
+        }
+        return OK;
+    }
     FmtMx4::Params p{static_cast<const uint8_t*>(blocks), static_cast<const uint8_t*>(scales)};
     return run_rows<FmtMx4, X_PLAIN, E_PLAIN>(p, plain_x(x), y, R, C, M, static_cast<hipStream_t>(stream));
 }

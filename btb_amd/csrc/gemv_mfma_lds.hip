@@ -1,0 +1,295 @@
+// The verify widths (M = 8..32 rows of x) on the matrix cores, with the weights brought in the way memory likes them.
+//
+// A v_mfma_f32_16x16x32_bf16 wants its A operand as "lane l: row l % 16, eight columns"; loading it that way straight
+// from memory makes every load instruction touch sixteen rows, 64 bytes of each, and HBM then runs at half speed
+// (measured: 3.1 TB/s against 4.5 for the same bytes read in long runs). So here a wave reads its share of the 16-row
+// tile in long contiguous runs per row (one 16-byte load per lane, a load instruction covering one or a few whole row
+// segments), parks the bytes in a private slab of LDS - still in their stored form - and reads them back in the MFMA's
+// layout, widening the packed forms to bf16 in registers on the way (FP8: v_cvt_pk_f32_fp8, one multiply by the block
+// scale, v_cvt_pk_bf16_f32; MXFP4: v_cvt_scalef32_pk_bf16_fp4). Nothing is synchronised between waves inside a tile:
+// a wave's LDS traffic is its own and executes in order.
+//
+// Decomposition. A workgroup of KS waves owns 16 rows of W at a time; wave k owns a fixed slice of the columns -
+// `spw` consecutive 32-column MFMA steps - and keeps the x fragments of that slice (operand B of every step, for one or
+// two 16-row tiles of x) in registers for the whole kernel, so x is read once per wave instead of once per row tile. The workgroup walks row
+// tiles (blockIdx.x, + gridDim.x, ...); the next sub-block's loads - also across a tile's end - are in flight while the
+// current one is multiplied. The KS partial tiles fold through LDS in wave order. KS and the slices come from C alone,
+// so a row's bits depend on neither M nor R nor the launch.
+// The reference's counterpart is btb_gemv_mma_bf16 (native/cuda/btb_gemv_mma.cuh:1-214); it has no packed forms.
+
+#include "btb_common.hpp"
+#include "btb_formats.hpp"
+#include "btb_tuning.hpp"
+
+#include "../../include/btb_hip.h"
+
+namespace btb {
+
+
+// ---- the stored forms: bytes a row contributes to a 32-column step, and the step's A fragment out of LDS ----------
+
+struct MfBf16 {
+    static constexpr int STEPB = 64;
+    struct Mat {
+        const uint8_t* w;
+    };
+    struct RowInfo {};
+    __device__ static __forceinline__ RowInfo row_info(const Mat&, int, int) { return RowInfo{}; }
+    // p: the lane's row in the slab, at the step's first byte; g: the lane's 8-column group of the step
+    // the step's scale for this lane (none here), requested a sub-block ahead of its use
+    __device__ static __forceinline__ uint32_t scale(const Mat&, const RowInfo&, int /*g*/, int /*step*/) { return 0u; }
+    __device__ static __forceinline__ bf16x8 frag(const uint8_t* p, int g, uint32_t /*scale*/) {
+        return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p + g * 16));
+    }
+};
+
+struct MfF8 {
+    static constexpr int STEPB = 32;
+    struct Mat {
+        const uint8_t* w;
+        const float* scales;
+        int sc;  // scales per grid row
+        int bm;  // rows per block
+        int bn;  // columns per block (a multiple of 16)
+    };
+    struct RowInfo {
+        const float* srow;
+    };
+    __device__ static __forceinline__ RowInfo row_info(const Mat& m, int row, int) {
+        return RowInfo{m.scales + (size_t)(row / m.bm) * m.sc};
+    }
+    __device__ static __forceinline__ uint32_t scale(const Mat& m, const RowInfo& ri, int g, int step) {
+        return f32_bits(ri.srow[(step * 32 + g * 8) / m.bn]);
+    }
+    __device__ static __forceinline__ bf16x8 frag(const uint8_t* p, int g, uint32_t scale) {
+        const uint2 q = *reinterpret_cast<const uint2*>(p + g * 8);
+        const float s = bits_f32(scale);
+        uint32_t w[4];
+        FmtF8::widen4(q.x, s, w);
+        FmtF8::widen4(q.y, s, w + 2);
+        return __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
+    }
+};
+
+struct MfMx4 {
+    static constexpr int STEPB = 16;
+    struct Mat {
+        const uint8_t* w;
+        const uint8_t* scales;
+    };
+    struct RowInfo {
+        const uint8_t* srow;
+    };
+    __device__ static __forceinline__ RowInfo row_info(const Mat& m, int row, int nsteps) {
+        return RowInfo{m.scales + (size_t)row * nsteps};
+    }
+    __device__ static __forceinline__ uint32_t scale(const Mat&, const RowInfo& ri, int /*g*/, int step) {
+        return (uint32_t)ri.srow[step];
+    }
+    __device__ static __forceinline__ bf16x8 frag(const uint8_t* p, int g, uint32_t scale) {
+        const uint32_t q = *reinterpret_cast<const uint32_t*>(p + g * 4);
+        const float s = bits_f32(scale << 23);
+        uint32_t w[4];
+        FmtMx4::widen8(q, s, w);
+        return __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
+    }
+};
+
+// ---- the kernel -----------------------------------------------------------------------------------------------------
+
+// KS waves a workgroup; MT 16-row tiles of x; SPW the steps a wave holds x fragments for (MT * SPW fragments in
+// registers); SB steps per sub-block (a slab holds 16 rows x SB steps)
+template <class MF, int KS, int MT, int SPW, int SB>
+__global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, const uint4* __restrict__ x,
+                                                         uint16_t* __restrict__ y, int R, int C, int M) {
+    constexpr int ROWB = SB * MF::STEPB;      // bytes a row contributes to a sub-block
+    constexpr int STRIDE = ROWB + 16;         // the slab's row stride: 4 banks past a multiple of 64, so the sixteen
+                                              // rows a fragment read touches fall in sixteen different bank groups
+    constexpr int SLAB = 16 * STRIDE;
+    constexpr int NLD = 16 * ROWB / 1024;     // 16-byte-per-lane loads a sub-block takes
+    constexpr int MAXSB = (SPW + SB - 1) / SB;
+    static_assert((16 * ROWB) % 1024 == 0 && NLD >= 1, "a sub-block is a whole number of wave loads");
+    extern __shared__ __align__(16) uint8_t lds[];  // KS slabs, then two sets of KS * MT partial tiles
+    const int lane = threadIdx.x & (WAVE - 1);
+    const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
+    const int li = lane & 15, lg = lane >> 4;
+    uint8_t* slab = lds + wv * SLAB;
+    f32x4* part = reinterpret_cast<f32x4*>(lds + KS * SLAB);
+
+    const int chunk4 = C / 8;  // uint4 per row of x
+    const int nsteps = C / 32;
+    const int spw = (nsteps + KS - 1) / KS;
+    const int s0 = wv * spw;
+    const int n = max(min(s0 + spw, nsteps) - s0, 0);  // this wave's steps: s0 .. s0 + n - 1
+    const size_t rowbytes = (size_t)nsteps * MF::STEPB;
+
+    uint4 xb[MT][SPW];
+#pragma unroll
+    for (int t = 0; t < MT; ++t) {
+        const uint4* xr = x + (size_t)min(t * 16 + li, M - 1) * chunk4 + lg + (size_t)s0 * 4;
+#pragma unroll
+        for (int i = 0; i < SPW; ++i) xb[t][i] = i < n ? xr[i * 4] : make_uint4(0, 0, 0, 0);
+    }
+
+    // A load instruction covers RPI whole rows of the sub-block (ROWB bytes each); the lane's place in it - row and
+    // byte within the row - is the same for every load of the kernel, so every address is a uniform base (tile, load,
+    // sub-block) plus one per-lane offset
+    constexpr int RPI = 1024 / ROWB;
+    static_assert(ROWB <= 1024 && 1024 % ROWB == 0, "a load instruction covers whole rows of a sub-block");
+    const uint32_t lane_row = (uint32_t)(lane * 16) / ROWB, lane_byte = (uint32_t)(lane * 16) % ROWB;
+    const uint32_t goff = lane_row * (uint32_t)rowbytes + lane_byte;
+    const uint32_t loff = lane_row * STRIDE + lane_byte;
+    uint4 raw[NLD] = {};
+    uint32_t scl[SB] = {};  // the scales of the sub-block in flight, one per step, for this lane's row and column group
+    auto request = [&](int tile, int sb) {  // the loads of sub-block sb of the tile (R is a multiple of 16)
+        const uint32_t valid = (uint32_t)(min(SB, n - sb * SB) * MF::STEPB);
+        const typename MF::RowInfo rn = MF::row_info(mat, tile * 16 + li, nsteps);
+#pragma unroll
+        for (int t = 0; t < SB; ++t)
+            if (sb * SB + t < n) scl[t] = MF::scale(mat, rn, lg, s0 + sb * SB + t);
+#pragma unroll
+        for (int q = 0; q < NLD; ++q) {
+            const uint8_t* base = mat.w + (size_t)(tile * 16 + q * RPI) * rowbytes + (size_t)(s0 + sb * SB) * MF::STEPB;
+            if (lane_byte < valid) raw[q] = load_stream16(reinterpret_cast<const uint4*>(base + goff));
+        }
+    };
+
+    const int ntiles = R / 16;
+    const int nsb = (n + SB - 1) / SB;
+    int tile = blockIdx.x;
+    if (tile < ntiles && nsb > 0) request(tile, 0);
+    for (int turn = 0; tile < ntiles; tile += gridDim.x, ++turn) {
+        f32x4 acc[MT];
+#pragma unroll
+        for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
+        const bool more = tile + (int)gridDim.x < ntiles;
+#pragma unroll
+        for (int sb = 0; sb < MAXSB; ++sb) {
+            if (sb < nsb) {
+                // the sub-block's bytes into the slab, as stored
+#pragma unroll
+                for (int q = 0; q < NLD; ++q) *reinterpret_cast<uint4*>(slab + q * RPI * STRIDE + loff) = raw[q];
+                uint32_t sc[SB];
+#pragma unroll
+                for (int t = 0; t < SB; ++t) sc[t] = scl[t];
+                // the next sub-block - of this tile, or the first of the workgroup's next tile - on its way
+                if (sb + 1 < nsb)
+                    request(tile, sb + 1);
+                else if (more)
+                    request(tile + (int)gridDim.x, 0);
+#pragma unroll
+                for (int t = 0; t < SB; ++t) {
+                    const int i = sb * SB + t;  // the wave's step (a compile-time index into xb)
+                    if (i < SPW && i < n) {
+                        const bf16x8 a = MF::frag(slab + li * STRIDE + t * MF::STEPB, lg, sc[t]);
+#pragma unroll
+                        for (int m = 0; m < MT; ++m)
+                            acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
+                                a, __builtin_bit_cast(bf16x8, xb[m][i < SPW ? i : 0]), acc[m], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        // the KS partial tiles, folded in wave order; two sets of partials alternate so one barrier a tile suffices
+        f32x4* mine = part + (size_t)(turn & 1) * KS * MT * WAVE;
+#pragma unroll
+        for (int t = 0; t < MT; ++t) mine[(wv * MT + t) * WAVE + lane] = acc[t];
+        __syncthreads();
+        if (wv < MT) {
+            f32x4 s = mine[(0 * MT + wv) * WAVE + lane];
+            for (int q = 1; q < KS; ++q) {
+                const f32x4 o = mine[(q * MT + wv) * WAVE + lane];
+                s.x += o.x;
+                s.y += o.y;
+                s.z += o.z;
+                s.w += o.w;
+            }
+            const int m = wv * 16 + li;
+            const int row = tile * 16 + lg * 4;
+            if (m < M) {
+                uint16_t* o = y + (size_t)m * R + row;
+                if (row + 0 < R) o[0] = f32_bf16(s.x);
+                if (row + 1 < R) o[1] = f32_bf16(s.y);
+                if (row + 2 < R) o[2] = f32_bf16(s.z);
+                if (row + 3 < R) o[3] = f32_bf16(s.w);
+            }
+        }
+    }
+}
+
+template <class MF, int KS, int MT, int SPW, int SB>
+static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st) {
+    constexpr int SLAB = 16 * (SB * MF::STEPB + 16);
+    const size_t lds = (size_t)KS * SLAB + 2 * (size_t)KS * MT * WAVE * sizeof(f32x4);
+    const int ntiles = R / 16;
+    int per_cu = tuning("mfma_wgs_per_cu");
+    if (per_cu <= 0) per_cu = 12 / KS;  // twelve waves a CU: what the kernel's registers leave resident
+    const int cap = device_info().cus * per_cu;
+    // whole turns of the grid over the tiles: the smallest grid that walks them in ceil(ntiles / cap) turns
+    const int turns = (ntiles + cap - 1) / cap;
+    const int grid = (ntiles + turns - 1) / turns;
+    auto kern = gemv_mfma_lds<MF, KS, MT, SPW, SB>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
+    }
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(KS * 64), lds, st, mat, static_cast<const uint4*>(x),
+                       static_cast<uint16_t*>(y), R, C, M);
+    return hip_status(hipGetLastError(), "gemv_mfma launch");
+}
+
+// The split of the columns over a workgroup's waves comes from the row length alone: at most eight waves (a workgroup
+// of sixteen would leave each wave 128 registers, less than the x fragments and a sub-block in flight need), each
+// holding x for 10, 16 or 28 steps. Up to 16 steps a wave there is room for two tiles of x rows; at 28 for one, and a
+// pass of more than 16 rows runs as two. Rows up to 7168 wide fit; wider ones stay with the column-interleaved kernel
+// (bf16) or the vector-ALU passes (packed forms).
+template <class MF>
+static bool lds_fits(int R, int C) {
+    return R % 16 == 0 && C % 32 == 0 && C / 32 <= 8 * 28;
+}
+bool mfma_lds_fits_bf16(int R, int C) { return lds_fits<MfBf16>(R, C); }
+bool mfma_lds_fits_packed(int R, int C) { return lds_fits<MfF8>(R, C); }
+
+template <class MF, int MT>
+static int32_t run_narrow(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st) {
+    constexpr int SB = MF::STEPB == 64 ? 8 : 16;  // eight (bf16, FP8) or four (MXFP4) loads of a sub-block in flight
+    const int nsteps = C / 32;
+    if (nsteps <= 20) return launch_lds<MF, 2, MT, 10, 8>(mat, x, y, R, C, M, st);
+    if (nsteps <= 40) return launch_lds<MF, 4, MT, 10, 8>(mat, x, y, R, C, M, st);
+    if (nsteps <= 80) return launch_lds<MF, 8, MT, 10, 8>(mat, x, y, R, C, M, st);
+    return launch_lds<MF, 8, MT, 16, SB>(mat, x, y, R, C, M, st);
+}
+
+template <class MF>
+static int32_t run_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st) {
+    constexpr int SB = MF::STEPB == 64 ? 8 : 16;
+    const int nsteps = C / 32;
+    if (nsteps <= 128) return M <= 16 ? run_narrow<MF, 1>(mat, x, y, R, C, M, st) : run_narrow<MF, 2>(mat, x, y, R, C, M, st);
+    const uint16_t* xp = static_cast<const uint16_t*>(x);
+    uint16_t* yp = static_cast<uint16_t*>(y);
+    constexpr int SBW = MF::STEPB == 16 ? 16 : 8;  // the wide rows' x fragments leave room for four loads in flight
+    for (int m0 = 0; m0 < M; m0 += 16) {
+        int32_t rc = launch_lds<MF, 8, 1, 28, SBW>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * R, R, C,
+                                                  M - m0 < 16 ? M - m0 : 16, st);
+        if (rc != OK) return rc;
+    }
+    return OK;
+}
+
+// M = 5..32 and a shape the fits() above take (whole 16-row tiles among them): the callers (gemv.hip) check before
+// they come here
+int32_t gemv_mfma_lds_bf16(const void* w, const void* x, void* y, int R, int C, int M, hipStream_t st) {
+    return run_lds<MfBf16>(MfBf16::Mat{static_cast<const uint8_t*>(w)}, x, y, R, C, M, st);
+}
+int32_t gemv_mfma_lds_fp8(const void* w, const float* scales, int sc, int bm, int bn, const void* x, void* y, int R,
+                          int C, int M, hipStream_t st) {
+    return run_lds<MfF8>(MfF8::Mat{static_cast<const uint8_t*>(w), scales, sc, bm, bn}, x, y, R, C, M, st);
+}
+int32_t gemv_mfma_lds_mxfp4(const void* blocks, const void* scales, const void* x, void* y, int R, int C, int M,
+                            hipStream_t st) {
+    return run_lds<MfMx4>(MfMx4::Mat{static_cast<const uint8_t*>(blocks), static_cast<const uint8_t*>(scales)}, x, y, R,
+                          C, M, st);
+}
+
+}  // namespace btb
