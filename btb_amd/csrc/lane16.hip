@@ -80,7 +80,24 @@ __global__ void __launch_bounds__(256) lane16_kernel(W w, const float* __restric
     float acc[B];
 #pragma unroll
     for (int i = 0; i < B; ++i) acc[i] = 0.f;
-    for (size_t c = (size_t)j; c < cols; c += 16) {
+    // eight of the lane's columns a batch: their loads are issued together, the products then taken in column order
+    constexpr int UB = 8;
+    size_t c = (size_t)j;
+    for (; c + 16 * (UB - 1) < cols; c += 16 * UB) {
+        float wv[UB], xv[UB][B];
+#pragma unroll
+        for (int u = 0; u < UB; ++u) {
+            wv[u] = w.at(rr, c + 16 * u, cols);
+#pragma unroll
+            for (int i = 0; i < B; ++i) xv[u][i] = b0 + i < btotal ? x[(b0 + i) * cols + c + 16 * u] : 0.f;
+        }
+#pragma unroll
+        for (int u = 0; u < UB; ++u)
+#pragma unroll
+            for (int i = 0; i < B; ++i)
+                if (b0 + i < btotal) acc[i] = fmaf(wv[u], xv[u][i], acc[i]);
+    }
+    for (; c < cols; c += 16) {
         const float wv = w.at(rr, c, cols);
 #pragma unroll
         for (int i = 0; i < B; ++i) {

@@ -166,7 +166,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
 // down + weighted sum: blockIdx.y is the token; the k experts of a row are walked in ascending expert id
 // ------------------------------------------------------------------------------------------------------------
 
-template <int LPR, int RPW, int U>
+template <int LPR, int RPW, int U, int KB>
 __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__ stack, const uint16_t* __restrict__ gu,
                                                        const int32_t* __restrict__ idx, const uint16_t* __restrict__ wts,
                                                        uint16_t* __restrict__ y, int R, int C, int k, int E) {
@@ -199,11 +199,47 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__
         s_expert[place] |= j << 20;
     }
     __syncthreads();
-    for (int q = 0; q < k; ++q) {
-        const int j = s_expert[q] >> 20;
-        stage_x<X_SILU>(hs + (size_t)q * (C / 2), XArgs{gu + ((size_t)token * k + j) * 2 * C, nullptr, nullptr, nullptr, 0.f, 0},
-                        1, C);
+    // The first KB experts' rows of the wave's first tile are requested now - they need the picks only - so their trip
+    // to memory (long: a layer's experts lie megabytes apart) runs while the h rows are being made.
+    F::RowCtx ctx[KB][RPW];
+    F::Raw first[KB][U][RPW] = {};
+    auto request = [&](int tile, int q0) {
+#pragma unroll
+        for (int b = 0; b < KB; ++b) {
+            const int expert = s_expert[min(q0 + b, k - 1)] & 0xFFFFF;
+            F::Params p{stack + (size_t)expert * R * units};
+#pragma unroll
+            for (int j = 0; j < RPW; ++j)
+                ctx[b][j] = F::row_ctx(p, (size_t)min(tile * ROWS + j * G + lane / LPR, R - 1), units);
+            if (q0 + b < k) load_span<F, LPR, RPW, U, true>(first[b], ctx[b], 0, sl, units);
+        }
+    };
+    if (wave < ntiles) request(wave, 0);
+
+    // the k picks' h rows = bf16(bf16(silu(g)) * u), each at its place in ascending expert order: one pass over all of
+    // them, four pairs a thread in flight, one barrier
+    {
+        const int half = C / 2;  // bf16 pairs per row
+        const uint32_t* src = reinterpret_cast<const uint32_t*>(gu);
+        const int n = k * half;
+        for (int i0 = threadIdx.x; i0 < n; i0 += 4 * (int)blockDim.x) {
+            uint32_t g2[4], u2[4];
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int i = min(i0 + v * (int)blockDim.x, n - 1);
+                const int q = i / half, c = i - q * half;
+                const size_t row = ((size_t)token * k + (s_expert[q] >> 20)) * 2 * half;
+                g2[v] = src[row + c];
+                u2[v] = src[row + half + c];
+            }
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const int i = i0 + v * (int)blockDim.x;
+                if (i < n) hs[i] = silu_pair(g2[v], u2[v]);
+            }
+        }
     }
+    __syncthreads();
     const uint4* hs4 = reinterpret_cast<const uint4*>(hs);
 
     for (int tile = wave; tile < ntiles; tile += nwaves) {
@@ -213,31 +249,29 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__
         float out[RPW];
 #pragma unroll
         for (int j = 0; j < RPW; ++j) out[j] = 0.f;
-        for (int q = 0; q < k; ++q) {
-            const int expert = s_expert[q] & 0xFFFFF;
-            F::Params p{stack + (size_t)expert * R * units};
-            F::RowCtx ctx[RPW];
+        for (int q0 = 0; q0 < k; q0 += KB) {
+            if (tile != wave || q0 != 0) request(tile, q0);
 #pragma unroll
-            for (int j = 0; j < RPW; ++j) ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
-            float acc[RPW][1];
+            for (int b = 0; b < KB; ++b) {
+                const int q = q0 + b;
+                if (q < k) {
+                    float acc[RPW][1];
 #pragma unroll
-            for (int j = 0; j < RPW; ++j) acc[j][0] = 0.f;
-            const uint4* xq = hs4 + (size_t)q * (C / 8);
-            for (int k0 = 0; k0 < units; k0 += span) {
-                F::Raw raw[U][RPW];
-                if (k0 + span <= units) {
-                    load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
-                    fma_span<F, 1, LPR, RPW, U, false>(raw, ctx, k0, sl, units, xq, C / 8, acc);
-                } else {
-                    load_span<F, LPR, RPW, U, true>(raw, ctx, k0, sl, units);
-                    fma_span<F, 1, LPR, RPW, U, true>(raw, ctx, k0, sl, units, xq, C / 8, acc);
+                    for (int j = 0; j < RPW; ++j) acc[j][0] = 0.f;
+                    const uint4* xq = hs4 + (size_t)q * (C / 8);
+                    fma_span<F, 1, LPR, RPW, U, true>(first[b], ctx[b], 0, sl, units, xq, C / 8, acc);
+                    for (int k0 = span; k0 < units; k0 += span) {
+                        F::Raw raw[U][RPW];
+                        load_span<F, LPR, RPW, U, true>(raw, ctx[b], k0, sl, units);
+                        fma_span<F, 1, LPR, RPW, U, true>(raw, ctx[b], k0, sl, units, xq, C / 8, acc);
+                    }
+                    const float wq = s_weight[q];
+#pragma unroll
+                    for (int j = 0; j < RPW; ++j) {
+                        const float d = bfround(group_sum<LPR>(acc[j][0]));  // the expert's down product, as the row's dtype
+                        out[j] = bfround(out[j] + bfround(d * wq));          // times its weight, added in bf16
+                    }
                 }
-            }
-            const float wq = s_weight[q];
-#pragma unroll
-            for (int j = 0; j < RPW; ++j) {
-                const float d = bfround(group_sum<LPR>(acc[j][0]));  // the expert's down product, as the row's dtype
-                out[j] = bfround(out[j] + bfround(d * wq));          // times its weight, added in bf16
             }
         }
 #pragma unroll
@@ -269,11 +303,13 @@ static int32_t launch_gate_up(const void* stack, const void* x, const int32_t* i
 template <int LPR>
 static int32_t launch_down(const void* stack, const void* gu, const int32_t* idx, const void* w, void* y, int R, int C,
                            int k, int E, int T, hipStream_t st) {
-    constexpr int RPW = 1, U = 4, G = WAVE / LPR;
+    constexpr int RPW = 1, G = WAVE / LPR;
     const int ntiles = (R + G * RPW - 1) / (G * RPW);
     const int grid = (ntiles + 3) / 4;
     const size_t lds = (size_t)k * C * 2;
-    auto kern = moe_down_kernel<LPR, RPW, U>;
+    // a row of at most three units a lane (the 768-wide experts of the C4 shape): all eight picks' rows in one request
+    const bool shallow = C / FmtBf16::UW <= 3 * LPR;
+    auto kern = shallow ? moe_down_kernel<LPR, RPW, 3, 8> : moe_down_kernel<LPR, RPW, 4, 4>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
