@@ -8,6 +8,8 @@
 // definition of btb_widen.hpp. These are the parity and routing kernels (the router's logits must be the CPU's, bit
 // for bit, for the top-k picks to be); the bandwidth path is gemv.hip.
 
+#include <type_traits>
+
 #include "btb_common.hpp"
 #include "btb_tuning.hpp"
 #include "btb_widen.hpp"
@@ -69,9 +71,13 @@ struct W16F8 {
     }
 };
 
+// x is f32, or bf16 widened on the way in (exact, so the sums are those of the widened copy)
+__device__ __forceinline__ float x_at(const float* x, size_t i) { return x[i]; }
+__device__ __forceinline__ float x_at(const uint16_t* x, size_t i) { return bf16_f32(x[i]); }
+
 // B rows of x per pass (the host walks up to 8 at a time; the order within one (row, vector) pair is the same)
-template <class W, int B>
-__global__ void __launch_bounds__(256) lane16_kernel(W w, const float* __restrict__ x, float* __restrict__ y, size_t rows,
+template <class W, int B, class XT>
+__global__ void __launch_bounds__(256) lane16_kernel(W w, const XT* __restrict__ x, float* __restrict__ y, size_t rows,
                                                      size_t cols, size_t b0, size_t btotal) {
     const int j = threadIdx.x & 15;
     const size_t r = (size_t)blockIdx.x * (blockDim.x >> 4) + (threadIdx.x >> 4);
@@ -80,8 +86,8 @@ __global__ void __launch_bounds__(256) lane16_kernel(W w, const float* __restric
     float acc[B];
 #pragma unroll
     for (int i = 0; i < B; ++i) acc[i] = 0.f;
-    // eight of the lane's columns a batch: their loads are issued together, the products then taken in column order
-    constexpr int UB = 8;
+    // a batch of the lane's columns: their loads are issued together, the products then taken in column order
+    constexpr int UB = B == 1 ? 32 : 8;
     size_t c = (size_t)j;
     for (; c + 16 * (UB - 1) < cols; c += 16 * UB) {
         float wv[UB], xv[UB][B];
@@ -89,7 +95,7 @@ __global__ void __launch_bounds__(256) lane16_kernel(W w, const float* __restric
         for (int u = 0; u < UB; ++u) {
             wv[u] = w.at(rr, c + 16 * u, cols);
 #pragma unroll
-            for (int i = 0; i < B; ++i) xv[u][i] = b0 + i < btotal ? x[(b0 + i) * cols + c + 16 * u] : 0.f;
+            for (int i = 0; i < B; ++i) xv[u][i] = b0 + i < btotal ? x_at(x, (b0 + i) * cols + c + 16 * u) : 0.f;
         }
 #pragma unroll
         for (int u = 0; u < UB; ++u)
@@ -101,7 +107,7 @@ __global__ void __launch_bounds__(256) lane16_kernel(W w, const float* __restric
         const float wv = w.at(rr, c, cols);
 #pragma unroll
         for (int i = 0; i < B; ++i) {
-            if (b0 + i < btotal) acc[i] = fmaf(wv, x[(b0 + i) * cols + c], acc[i]);
+            if (b0 + i < btotal) acc[i] = fmaf(wv, x_at(x, (b0 + i) * cols + c), acc[i]);
         }
     }
 #pragma unroll
@@ -111,17 +117,103 @@ __global__ void __launch_bounds__(256) lane16_kernel(W w, const float* __restric
     }
 }
 
-template <class W>
-static int32_t launch_lane16(const W& w, const float* x, float* y, size_t rows, size_t cols, size_t b, hipStream_t st) {
+// bf16 rows 128 columns wide a step: the group's sixteen lanes bring 256 contiguous bytes in with one 16-byte load each
+// and hand them round through a slab of LDS the group owns, where lane j then finds its columns j, j + 16, ... - one
+// request a lane for eight of its columns instead of eight. x is staged once a workgroup, as f32. The sums are the same
+// chain of fused multiply-adds in the same column order. Writes and reads of a slab are one wave's, which LDS serves in
+// program order: no barrier between them.
+template <int B, int NB, class XT>
+__global__ void __launch_bounds__(256) lane16_bf16_wide_kernel(const uint16_t* __restrict__ w, const XT* __restrict__ x,
+                                                               float* __restrict__ y, size_t rows, size_t cols, size_t b0,
+                                                               size_t btotal) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float* xs = reinterpret_cast<float*>(smem);         // [B][cols]
+    unsigned char* slabs = smem + (size_t)B * cols * 4;  // [16 groups][NB][256]
+    const int tid = threadIdx.x, j = tid & 15, grp = tid >> 4;
+    const size_t r = (size_t)blockIdx.x * 16 + grp;
+    const bool live = r < rows;
+    const uint4* wrow = reinterpret_cast<const uint4*>(w + (live ? r : rows - 1) * cols);
+    const int nchunks = (int)(cols / 128);
+    uint4 raw[NB];
+    auto request = [&](int n0) {
+#pragma unroll
+        for (int n = 0; n < NB; ++n) raw[n] = wrow[(size_t)min(n0 + n, nchunks - 1) * 16 + j];
+    };
+    request(0);
+    const size_t nx = (size_t)B * cols;
+    for (size_t i = tid; i < nx; i += 256) {
+        const size_t b = i / cols, c = i - b * cols;
+        xs[i] = b0 + b < btotal ? x_at(x, (b0 + b) * cols + c) : 0.f;
+    }
+    __syncthreads();
+    unsigned char* mine = slabs + (size_t)grp * (NB * 256);
+    float acc[B];
+#pragma unroll
+    for (int i = 0; i < B; ++i) acc[i] = 0.f;
+    for (int n0 = 0; n0 < nchunks; n0 += NB) {
+#pragma unroll
+        for (int n = 0; n < NB; ++n) *reinterpret_cast<uint4*>(mine + n * 256 + 16 * j) = raw[n];
+        if (n0 + NB < nchunks) request(n0 + NB);
+#pragma unroll
+        for (int n = 0; n < NB; ++n) {
+            if (n0 + n < nchunks) {
+#pragma unroll
+                for (int u = 0; u < 8; ++u) {
+                    const float wv = bf16_f32(*reinterpret_cast<const uint16_t*>(mine + n * 256 + 2 * (j + 16 * u)));
+                    const size_t c = (size_t)(n0 + n) * 128 + j + 16 * u;
+#pragma unroll
+                    for (int i = 0; i < B; ++i) acc[i] = fmaf(wv, xs[(size_t)i * cols + c], acc[i]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < B; ++i) {
+        const float s = group_sum<16>(acc[i]);
+        if (j == 0 && live && b0 + i < btotal) y[(b0 + i) * rows + r] = s;
+    }
+}
+
+template <int B, int NB, class XT>
+static bool launch_wide(const uint16_t* w, const XT* x, float* y, size_t rows, size_t cols, size_t b0, size_t b,
+                        hipStream_t st) {
+    const size_t lds = (size_t)B * cols * 4 + 16 * NB * 256;
+    if (lds > (size_t)device_info().lds_bytes) return false;
+    auto kern = lane16_bf16_wide_kernel<B, NB, XT>;
+    static bool raised = false;  // per instance; the attribute is the function's, set before its first large launch
+    if (lds > 64 * 1024 && !raised) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                device_info().lds_bytes) != hipSuccess)
+            return false;
+        raised = true;
+    }
+    hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 15) / 16)), dim3(256), lds, st, w, x, y, rows, cols, b0, b);
+    return true;
+}
+
+template <class W, class XT>
+static int32_t launch_lane16(const W& w, const XT* x, float* y, size_t rows, size_t cols, size_t b, hipStream_t st) {
     const unsigned grid = (unsigned)((rows + 15) / 16);
     for (size_t b0 = 0; b0 < b; b0 += 4) {
         const size_t left = b - b0;
+        if constexpr (std::is_same<W, W16Bf16>::value) {
+            if (cols % 128 == 0 && (reinterpret_cast<uintptr_t>(w.w) & 15) == 0) {
+                const bool done = left >= 4   ? launch_wide<4, 4>(w.w, x, y, rows, cols, b0, b, st)
+                                  : left >= 2 ? launch_wide<3, 4>(w.w, x, y, rows, cols, b0, b, st)
+                                              : launch_wide<1, 8>(w.w, x, y, rows, cols, b0, b, st);
+                if (done) {
+                    int32_t rc = hip_status(hipGetLastError(), "lane16 launch");
+                    if (rc != OK) return rc;
+                    continue;
+                }
+            }
+        }
         if (left >= 4)
-            hipLaunchKernelGGL((lane16_kernel<W, 4>), dim3(grid), dim3(256), 0, st, w, x, y, rows, cols, b0, b);
+            hipLaunchKernelGGL((lane16_kernel<W, 4, XT>), dim3(grid), dim3(256), 0, st, w, x, y, rows, cols, b0, b);
         else if (left >= 2)
-            hipLaunchKernelGGL((lane16_kernel<W, 3>), dim3(grid), dim3(256), 0, st, w, x, y, rows, cols, b0, b);
+            hipLaunchKernelGGL((lane16_kernel<W, 3, XT>), dim3(grid), dim3(256), 0, st, w, x, y, rows, cols, b0, b);
         else
-            hipLaunchKernelGGL((lane16_kernel<W, 1>), dim3(grid), dim3(256), 0, st, w, x, y, rows, cols, b0, b);
+            hipLaunchKernelGGL((lane16_kernel<W, 1, XT>), dim3(grid), dim3(256), 0, st, w, x, y, rows, cols, b0, b);
         int32_t rc = hip_status(hipGetLastError(), "lane16 launch");
         if (rc != OK) return rc;
     }
@@ -138,6 +230,14 @@ static bool shape_ok(size_t rows, size_t cols, size_t b) {
     if (__builtin_mul_overflow(b, cols, &n) || n > cap) return false;
     if (__builtin_mul_overflow(b, rows, &n) || n > cap) return false;
     return rows / 16 < 0x7FFFFFFFull;
+}
+
+// the router's logits from the rows as they are held (bf16): the f32 copy the host path makes first is the widening
+// done in the load
+int32_t lane16_bf16_rows16(const uint16_t* w, size_t rows, size_t cols, const uint16_t* x, size_t b, float* y,
+                           hipStream_t st) {
+    if (!shape_ok(rows, cols, b)) return ERR_DOMAIN;
+    return launch_lane16(W16Bf16{w}, x, y, rows, cols, b, st);
 }
 
 }  // namespace btb

@@ -11,6 +11,8 @@
 //
 // Nothing goes back to the host between the steps, so the layer records into a hipGraph.
 
+#include <type_traits>
+
 #include "btb_common.hpp"
 #include "btb_formats.hpp"
 #include "btb_stream.hpp"
@@ -19,6 +21,9 @@
 #include "../../include/btb_hip.h"
 
 namespace btb {
+
+int32_t lane16_bf16_rows16(const uint16_t* w, size_t rows, size_t cols, const uint16_t* x, size_t b, float* y,
+                           hipStream_t st);  // lane16.hip
 
 constexpr int ROUTE_MAX_K = 32;  // the reference's ROUTE_MAX_K (native/cuda/btb_kernels.cu:859)
 
@@ -105,6 +110,130 @@ __global__ void __launch_bounds__(64) moe_route_kernel(const void* __restrict__ 
         w[o] = f32_bf16(wv);
         if (w32 != nullptr) w32[o] = wv;
     }
+}
+
+// Up to 256 experts: the row's probabilities stay in registers, P a lane, and a pick is the maximum of 64-bit keys
+// (the probability's bits above the complement of the index: p >= 0, so the bits order as p does, and of equal p the
+// lower index has the greater key). A taken key is 0, below every live one. The same arithmetic in the same order as
+// the kernel above, so the same picks and weights; a row of NaN probabilities takes the experts 0..k-1.
+__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
+    auto step = [&](auto ctrl) {
+        constexpr int C = decltype(ctrl)::value;
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, C, 0xF, 0xF, true);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), C, 0xF, 0xF, true);
+        const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+        v = o > v ? o : v;
+    };
+    step(std::integral_constant<int, 0xB1>{});
+    step(std::integral_constant<int, 0x4E>{});
+    step(std::integral_constant<int, 0x141>{});
+    step(std::integral_constant<int, 0x140>{});
+    unsigned long long best = 0;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 16 * r);
+        const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 16 * r);
+        const unsigned long long o = ((unsigned long long)hi << 32) | lo;
+        best = o > best ? o : best;
+    }
+    return best;
+}
+
+template <bool F32, int P>
+__global__ void __launch_bounds__(64) moe_route_reg_kernel(const void* __restrict__ logits, size_t ls, int E, int k,
+                                                           int32_t* __restrict__ idx, uint16_t* __restrict__ w,
+                                                           float* __restrict__ w32, uint16_t* __restrict__ logits16) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const size_t base = (size_t)t * ls;
+    float lv[P];
+#pragma unroll
+    for (int s = 0; s < P; ++s) {
+        const int e = lane + WAVE * s;
+        lv[s] = e < E ? logit_at<F32>(logits, base + e) : bits_f32(0xff800000u);
+    }
+    if (logits16 != nullptr) {
+#pragma unroll
+        for (int s = 0; s < P; ++s) {
+            const int e = lane + WAVE * s;
+            if (e < E) logits16[(size_t)t * E + e] = f32_bf16(lv[s]);
+        }
+    }
+    float m = bits_f32(0xff800000u);
+#pragma unroll
+    for (int s = 0; s < P; ++s) m = fmaxf(m, lv[s]);
+    m = wave_max(m);
+    float pr[P], sum_p = 0.f;
+#pragma unroll
+    for (int s = 0; s < P; ++s) {
+        const int e = lane + WAVE * s;
+        pr[s] = e < E ? expf(lv[s] - m) : 0.f;
+        if (e < E) sum_p += pr[s];
+    }
+    sum_p = group_sum<64>(sum_p);
+    sum_p = __shfl(sum_p, 0, WAVE);
+    unsigned long long key[P];
+#pragma unroll
+    for (int s = 0; s < P; ++s) {
+        const int e = lane + WAVE * s;
+        const float p = pr[s] / sum_p;
+        const uint32_t bits = p != p ? 0x7fc00000u : f32_bits(p);
+        key[s] = e < E ? (((unsigned long long)bits << 32) | (0xFFFFFFFFu - (uint32_t)e)) : 0ull;
+    }
+    float topv = 0.f;  // lane j keeps pick j
+    int topi = 0;
+    for (int j = 0; j < k; ++j) {
+        unsigned long long best = key[0];
+#pragma unroll
+        for (int s = 1; s < P; ++s) best = key[s] > best ? key[s] : best;
+        best = wave_max_u64(best);
+        const int e = (int)(0xFFFFFFFFu - (uint32_t)best);
+        if (lane == j) {
+            topv = bits_f32((uint32_t)(best >> 32));
+            topi = e;
+        }
+#pragma unroll
+        for (int s = 0; s < P; ++s)
+            if (lane + WAVE * s == e) key[s] = 0ull;
+    }
+    float sum = 0.f;
+    for (int j = 0; j < k; ++j) sum += __shfl(topv, j, WAVE);
+    if (lane < k) {
+        const float wv = topv / sum;
+        const size_t o = (size_t)t * k + lane;
+        idx[o] = topi;
+        w[o] = f32_bf16(wv);
+        if (w32 != nullptr) w32[o] = wv;
+    }
+}
+
+// a row's logits rounded to bf16, for the wide rows the kernel above does not take
+__global__ void __launch_bounds__(256) round_rows_kernel(const float* __restrict__ src, size_t ls, int E,
+                                                         uint16_t* __restrict__ dst) {
+    const int t = blockIdx.y, e = blockIdx.x * 256 + threadIdx.x;
+    if (e < E) dst[(size_t)t * E + e] = f32_bf16(src[(size_t)t * ls + e]);
+}
+
+template <bool F32>
+static int32_t launch_route(const void* logits, size_t ls, int E, int k, int T, int32_t* idx, uint16_t* w, float* w32,
+                            uint16_t* logits16, hipStream_t st) {
+    const int P = (E + WAVE - 1) / WAVE;
+#define BTB_ROUTE_REG(P_)                                                                                            \
+    hipLaunchKernelGGL((moe_route_reg_kernel<F32, P_>), dim3((unsigned)T), dim3(64), 0, st, logits, ls, E, k, idx, w, \
+                       w32, logits16)
+    if (P == 1)
+        BTB_ROUTE_REG(1);
+    else if (P == 2)
+        BTB_ROUTE_REG(2);
+    else if (P <= 4)
+        BTB_ROUTE_REG(4);
+    else {
+        hipLaunchKernelGGL(moe_route_kernel<F32>, dim3((unsigned)T), dim3(64), E * 4, st, logits, ls, E, k, idx, w, w32);
+        if (logits16 != nullptr && F32)
+            hipLaunchKernelGGL(round_rows_kernel, dim3((E + 255) / 256, T), dim3(256), 0, st,
+                               static_cast<const float*>(logits), ls, E, logits16);
+    }
+#undef BTB_ROUTE_REG
+    return hip_status(hipGetLastError(), "moe_route launch");
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -335,12 +464,23 @@ int32_t btb_hip_moe_route(const void* logits, int32_t logits_f32, size_t ls, siz
     if (!al(logits, logits_f32 ? 4 : 2) || !al(idx, 4) || !al(w, 2) || !al(w32, 4)) return ERR_DOMAIN;
     hipStream_t st = static_cast<hipStream_t>(stream);
     if (logits_f32)
-        hipLaunchKernelGGL(moe_route_kernel<true>, dim3((unsigned)T), dim3(64), E * 4, st, logits, ls, (int)E, (int)k, idx,
-                           static_cast<uint16_t*>(w), w32);
-    else
-        hipLaunchKernelGGL(moe_route_kernel<false>, dim3((unsigned)T), dim3(64), E * 4, st, logits, ls, (int)E, (int)k, idx,
-                           static_cast<uint16_t*>(w), w32);
-    return hip_status(hipGetLastError(), "moe_route launch");
+        return launch_route<true>(logits, ls, (int)E, (int)k, (int)T, idx, static_cast<uint16_t*>(w), w32, nullptr, st);
+    return launch_route<false>(logits, ls, (int)E, (int)k, (int)T, idx, static_cast<uint16_t*>(w), w32, nullptr, st);
+}
+
+int32_t btb_hip_moe_router_bf16(const void* router, const void* x, size_t T, size_t E, size_t H, size_t k, float* logits,
+                                void* logits16, int32_t* idx, void* w, float* w32, void* stream) {
+    if (router == nullptr || x == nullptr || logits == nullptr || idx == nullptr || w == nullptr) return ERR_NULL;
+    if (E == 0 || k == 0 || T == 0 || H == 0 || k > E || k > (size_t)ROUTE_MAX_K || E > 8192 || T > 65535)
+        return ERR_DOMAIN;
+    if (!al(router, 2) || !al(x, 2) || !al(logits, 4) || !al(logits16, 2) || !al(idx, 4) || !al(w, 2) || !al(w32, 4))
+        return ERR_DOMAIN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    int32_t rc = lane16_bf16_rows16(static_cast<const uint16_t*>(router), E, H, static_cast<const uint16_t*>(x), T,
+                                    logits, st);
+    if (rc != OK) return rc;
+    return launch_route<true>(logits, E, (int)E, (int)k, (int)T, idx, static_cast<uint16_t*>(w), w32,
+                              static_cast<uint16_t*>(logits16), st);
 }
 
 int32_t btb_hip_moe_experts_bf16(const void* gate_up, const void* down, const void* x, const int32_t* idx, const void* w,

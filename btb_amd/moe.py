@@ -31,6 +31,9 @@ class Router:
 
     def __call__(self, hidden_states: torch.Tensor):
         x = hidden_states.reshape(-1, self.hidden_dim)
+        if x.dtype == torch.bfloat16:  # the rows as held: logits and routing in two launches, nothing between them
+            _, logits16, picks, weights, _ = self.card.moe_router(self.weight, x.contiguous(), self.top_k)
+            return logits16, weights, picks
         logits = self.card.gemv_lane16(self.weight, x.float().contiguous())
         picks, weights, _ = self.card.moe_route(logits, self.top_k)
         return logits.to(hidden_states.dtype), weights.to(hidden_states.dtype), picks

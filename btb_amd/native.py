@@ -53,6 +53,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_gemv_fp8_rows": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _vp]),
     "btb_hip_gemv_fp8_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_moe_route": (_i32, [_vp, _i32, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp]),
+    "btb_hip_moe_router_bf16": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_moe_experts_bf16": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _vp]),
     "btb_hip_embed": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_add_rmsnorm": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _sz, _sz, _i32, _vp]),
@@ -403,6 +404,25 @@ class HipCard:
         self._call("btb_hip_moe_route", self.ptr(logits), int(logits.dtype == torch.float32), ls, E, k, T, self.ptr(idx),
                    self.ptr(w), self.ptr(w32), _stream())
         return idx, w, w32
+
+    def moe_router(self, router: torch.Tensor, x: torch.Tensor, k: int):
+        """(logits f32 [T, E], logits bf16 [T, E], idx int32 [T, k], weights bf16 [T, k], weights f32 [T, k]) of bf16
+        rows x [T, H] against the bf16 router matrix [E, H]: the host-order logits and their routing, two launches"""
+        self._need(router, torch.bfloat16, "router")
+        self._need(x, torch.bfloat16, "x")
+        E, H = (int(s) for s in router.shape)
+        if x.dim() != 2 or int(x.shape[1]) != H:
+            raise ValueError(f"[hip] moe_router: x {tuple(x.shape)} is not [T, {H}]")
+        T = int(x.shape[0])
+        dev = x.device
+        logits = torch.empty(T, E, dtype=torch.float32, device=dev)
+        logits16 = torch.empty(T, E, dtype=torch.bfloat16, device=dev)
+        idx = torch.empty(T, k, dtype=torch.int32, device=dev)
+        w = torch.empty(T, k, dtype=torch.bfloat16, device=dev)
+        w32 = torch.empty(T, k, dtype=torch.float32, device=dev)
+        self._call("btb_hip_moe_router_bf16", self.ptr(router), self.ptr(x), T, E, H, k, self.ptr(logits),
+                   self.ptr(logits16), self.ptr(idx), self.ptr(w), self.ptr(w32), _stream())
+        return logits, logits16, idx, w, w32
 
     def moe_experts(self, gate_up: torch.Tensor, down: torch.Tensor, x: torch.Tensor, idx: torch.Tensor,
                     w: torch.Tensor, y: torch.Tensor | None = None, gu: torch.Tensor | None = None) -> torch.Tensor:

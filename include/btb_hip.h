@@ -174,6 +174,13 @@ int32_t btb_hip_gemv_fp8_group(size_t n, const uint8_t* const* w, const float* c
 int32_t btb_hip_moe_route(const void* logits, int32_t logits_f32, size_t ls, size_t E, size_t k, size_t T, int32_t* idx,
                           void* w, float* w32, void* stream);
 
+/* Qwen4Router.forward for bf16 rows in two launches (btb/engine/families/qwen4/router.py:43-51): the f32 logits of
+ * x [T, H] bf16 against router [E, H] bf16 in the host matvec's order (btb_hip_gemv_bf16_rows of the rows widened to
+ * f32, to the bit) into logits f32 [T, E], then btb_hip_moe_route over them. logits16, when not NULL, receives the
+ * logits rounded to bf16 [T, E] (the reference hands them back in the rows' dtype). k <= 32, E <= 8192, T <= 65535. */
+int32_t btb_hip_moe_router_bf16(const void* router, const void* x, size_t T, size_t E, size_t H, size_t k, float* logits,
+                                void* logits16, int32_t* idx, void* w, float* w32, void* stream);
+
 /* The routed experts of T rows: gate_up [E, 2I, H] and down [E, H, I] bf16 stacks (gate rows then up rows), x [T, H]
  * bf16, the picks idx [T, k] and weights w bf16 [T, k] of btb_hip_moe_route, gu [T, k, 2I] bf16 scratch the caller
  * owns, y [T, H] bf16. Per pick: gu = bf16(W_gu x), h = bf16(bf16(silu(g)) * u), d = bf16(W_dn h); per row

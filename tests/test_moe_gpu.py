@@ -88,3 +88,50 @@ def test_route_tie_rule_and_bf16_logits(card):
     assert torch.allclose(w32.cpu(), top / top.sum(-1, keepdim=True), rtol=1e-5, atol=0)
     with pytest.raises(Exception):
         card.moe_route(g.cuda(), 33)
+
+
+def test_route_in_registers_and_through_lds_agree(card):
+    """up to 256 experts the row stays in registers, beyond that it goes through LDS: a 300-wide row whose upper
+    experts are far below the rest must route as its first 128, 200 and 256 do, ties, zeros of probability and a row
+    of NaN included"""
+    g = torch.randn(9, 300, generator=gen(531))
+    g[:, 128:] -= 200.0                       # exp underflows to +0: live, never picked before a real one
+    g[1, :128] = g[1, :128].round()           # many exact ties
+    g[2, 5] = float("nan")                    # every probability NaN: the first k experts
+    g[3, :128] = 1.5                          # all equal: index order
+    g[4, 17] = float("inf")                   # inf - inf: NaN again
+    wide = card.moe_route(g.cuda(), 8)
+    for E in (64, 100, 128, 200, 256):
+        head = card.moe_route(g.cuda(), 8, E=E)
+        if E >= 128:
+            assert torch.equal(head[0], wide[0]), E
+            ok = ~torch.isnan(wide[2])
+            assert torch.equal(head[2][ok], wide[2][ok]) and torch.equal(torch.isnan(head[2]), ~ok), E
+        ref = torch.softmax(g[:, :E], dim=-1)
+        top, ids = torch.topk(ref[[0, 5, 6, 7, 8]], 8, dim=-1)
+        assert torch.equal(head[0].cpu().long()[[0, 5, 6, 7, 8]], ids), E
+    assert wide[0][2].tolist() == list(range(8)) and wide[0][4].tolist() == list(range(8))
+    # k = 32 of 40: the zero-probability tail is taken in index order
+    z = torch.full((1, 40), -300.0)
+    z[0, [9, 4, 30]] = torch.tensor([3.0, 2.0, 1.0])
+    idx, _, _ = card.moe_route(z.cuda(), 32)
+    assert idx[0].tolist() == [9, 4, 30] + [i for i in range(40) if i not in (9, 4, 30)][:29]
+
+
+@pytest.mark.parametrize("T,E,H", [(1, 128, 2048), (5, 128, 2048), (3, 60, 520), (2, 384, 256)])
+def test_router_in_two_launches_is_the_three_step_form(card, T, E, H):
+    """bf16 rows straight into the host-order matvec, the logits rounded inside the routing kernel: the same bits as
+    widening the rows first, routing the f32 logits and rounding them afterwards"""
+    g = gen(540 + T)
+    wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).cuda()
+    x = acts_bf16(T, H, seed=545 + T).cuda()
+    logits, logits16, idx, w, w32 = card.moe_router(wr, x, 8)
+    raw = card.gemv_lane16(wr, x.float())
+    ridx, rw, rw32 = card.moe_route(raw, 8)
+    assert torch.equal(logits.view(torch.int32), raw.view(torch.int32))
+    assert torch.equal(logits16.view(torch.int16), raw.to(torch.bfloat16).view(torch.int16))
+    assert torch.equal(idx, ridx) and torch.equal(w.view(torch.int16), rw.view(torch.int16))
+    assert torch.equal(w32.view(torch.int32), rw32.view(torch.int32))
+    want, ow, opicks = omoe.router(bits16(wr.cpu()), x.float().cpu().numpy(), 8, "bf16")
+    assert np.array_equal(f32_bits(logits.cpu().numpy()), f32_bits(want))
+    assert np.array_equal(idx.cpu().numpy().astype(np.int64), opicks)
