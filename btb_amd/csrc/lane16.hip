@@ -8,6 +8,7 @@
 // definition of btb_widen.hpp. These are the parity and routing kernels (the router's logits must be the CPU's, bit
 // for bit, for the top-k picks to be); the bandwidth path is gemv.hip.
 
+#include <algorithm>
 #include <type_traits>
 
 #include "btb_common.hpp"
@@ -127,8 +128,10 @@ __global__ void __launch_bounds__(256) lane16_bf16_wide_kernel(const uint16_t* _
                                                                float* __restrict__ y, size_t rows, size_t cols, size_t b0,
                                                                size_t btotal) {
     extern __shared__ __align__(16) unsigned char smem[];
-    float* xs = reinterpret_cast<float*>(smem);         // [B][cols]
-    unsigned char* slabs = smem + (size_t)B * cols * 4;  // [16 groups][NB][256]
+    constexpr int BP = B == 3 ? 4 : B;  // a column's B values of x side by side, one LDS read
+    float* xs = reinterpret_cast<float*>(smem);           // [cols][BP]
+    unsigned char* slabs = smem + (size_t)BP * cols * 4;  // [16 groups][NB][256]
+    b0 += (size_t)blockIdx.y * B;
     const int tid = threadIdx.x, j = tid & 15, grp = tid >> 4;
     const size_t r = (size_t)blockIdx.x * 16 + grp;
     const bool live = r < rows;
@@ -140,11 +143,8 @@ __global__ void __launch_bounds__(256) lane16_bf16_wide_kernel(const uint16_t* _
         for (int n = 0; n < NB; ++n) raw[n] = wrow[(size_t)min(n0 + n, nchunks - 1) * 16 + j];
     };
     request(0);
-    const size_t nx = (size_t)B * cols;
-    for (size_t i = tid; i < nx; i += 256) {
-        const size_t b = i / cols, c = i - b * cols;
-        xs[i] = b0 + b < btotal ? x_at(x, (b0 + b) * cols + c) : 0.f;
-    }
+    for (int b = 0; b < B; ++b)
+        for (size_t c = tid; c < cols; c += 256) xs[c * BP + b] = b0 + b < btotal ? x_at(x, (b0 + b) * cols + c) : 0.f;
     __syncthreads();
     unsigned char* mine = slabs + (size_t)grp * (NB * 256);
     float acc[B];
@@ -162,7 +162,7 @@ __global__ void __launch_bounds__(256) lane16_bf16_wide_kernel(const uint16_t* _
                     const float wv = bf16_f32(*reinterpret_cast<const uint16_t*>(mine + n * 256 + 2 * (j + 16 * u)));
                     const size_t c = (size_t)(n0 + n) * 128 + j + 16 * u;
 #pragma unroll
-                    for (int i = 0; i < B; ++i) acc[i] = fmaf(wv, xs[(size_t)i * cols + c], acc[i]);
+                    for (int i = 0; i < B; ++i) acc[i] = fmaf(wv, xs[c * BP + i], acc[i]);
                 }
             }
         }
@@ -176,8 +176,8 @@ __global__ void __launch_bounds__(256) lane16_bf16_wide_kernel(const uint16_t* _
 
 template <int B, int NB, class XT>
 static bool launch_wide(const uint16_t* w, const XT* x, float* y, size_t rows, size_t cols, size_t b0, size_t b,
-                        hipStream_t st) {
-    const size_t lds = (size_t)B * cols * 4 + 16 * NB * 256;
+                        unsigned passes, hipStream_t st) {
+    const size_t lds = (size_t)(B == 3 ? 4 : B) * cols * 4 + 16 * NB * 256;
     if (lds > (size_t)device_info().lds_bytes) return false;
     auto kern = lane16_bf16_wide_kernel<B, NB, XT>;
     static bool raised = false;  // per instance; the attribute is the function's, set before its first large launch
@@ -187,27 +187,40 @@ static bool launch_wide(const uint16_t* w, const XT* x, float* y, size_t rows, s
             return false;
         raised = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 15) / 16)), dim3(256), lds, st, w, x, y, rows, cols, b0, b);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 15) / 16), passes), dim3(256), lds, st, w, x, y, rows, cols, b0, b);
     return true;
 }
 
 template <class W, class XT>
 static int32_t launch_lane16(const W& w, const XT* x, float* y, size_t rows, size_t cols, size_t b, hipStream_t st) {
     const unsigned grid = (unsigned)((rows + 15) / 16);
-    for (size_t b0 = 0; b0 < b; b0 += 4) {
-        const size_t left = b - b0;
-        if constexpr (std::is_same<W, W16Bf16>::value) {
-            if (cols % 128 == 0 && (reinterpret_cast<uintptr_t>(w.w) & 15) == 0) {
-                const bool done = left >= 4   ? launch_wide<4, 4>(w.w, x, y, rows, cols, b0, b, st)
-                                  : left >= 2 ? launch_wide<3, 4>(w.w, x, y, rows, cols, b0, b, st)
-                                              : launch_wide<1, 8>(w.w, x, y, rows, cols, b0, b, st);
-                if (done) {
-                    int32_t rc = hip_status(hipGetLastError(), "lane16 launch");
-                    if (rc != OK) return rc;
-                    continue;
+    size_t b0 = 0;
+    if constexpr (std::is_same<W, W16Bf16>::value) {
+        if (cols % 128 == 0 && (reinterpret_cast<uintptr_t>(w.w) & 15) == 0) {
+            // every pass of four rows of x in one launch (the pass is the grid's second dimension), then the rest
+            bool done = true;
+            const size_t fours = std::min<size_t>(b / 4, 65535);
+            if (fours > 0) {
+                done = launch_wide<4, 4>(w.w, x, y, rows, cols, 0, b, (unsigned)fours, st);
+                if (done) b0 = 4 * fours;
+            }
+            while (done && b0 < b) {
+                const size_t left = b - b0;
+                if (left >= 4) {
+                    done = launch_wide<4, 4>(w.w, x, y, rows, cols, b0, b, 1, st);
+                    if (done) b0 += 4;
+                } else {
+                    done = left >= 2 ? launch_wide<3, 4>(w.w, x, y, rows, cols, b0, b, 1, st)
+                                     : launch_wide<1, 8>(w.w, x, y, rows, cols, b0, b, 1, st);
+                    if (done) b0 = b;
                 }
             }
+            int32_t rc = hip_status(hipGetLastError(), "lane16 launch");
+            if (rc != OK) return rc;
         }
+    }
+    for (; b0 < b; b0 += 4) {
+        const size_t left = b - b0;
         if (left >= 4)
             hipLaunchKernelGGL((lane16_kernel<W, 4, XT>), dim3(grid), dim3(256), 0, st, w, x, y, rows, cols, b0, b);
         else if (left >= 2)

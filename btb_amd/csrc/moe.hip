@@ -3,11 +3,12 @@
 //   route      per token: f32 softmax over the E logits, the top k in the total order (p descending, index ascending),
 //              weights p / sum(top k) summed in rank order, rounded to bf16 - the reference's btb_moe_route
 //              (native/cuda/btb_kernels.cu:845-948) and Qwen4Router.forward (btb/engine/families/qwen4/router.py:43-51)
-//   gate_up    for every (token, pick): gu = W_gu[expert] . x[token], f32 accumulate, bf16 out; the experts' matrices
-//              are streamed once per pick with the dense matvec's loop (btb_stream.hpp)
-//   down       for every token and output row: the k experts in ASCENDING expert id, each d = bf16(W_dn[e] . h_e) with
-//              h_e = bf16(bf16(silu(g)) * u) folded into the x staging, then y = bf16(y + bf16(d * w_e)) - the dtype
-//              chain and the summation order of _Experts._one_row / _loop (btb/engine/host.py:508-569, 906-967)
+//   gate_up    for every (token, pick): g, u = bf16(W_gu[expert] . x[token]) (f32 accumulate), a wave holding gate row
+//              r and up row I + r together and writing h[r] = bf16(bf16(silu(g)) * u); the experts' matrices are
+//              streamed once per pick with the dense matvec's loop (btb_stream.hpp)
+//   down       for every token and output row: the k experts in ASCENDING expert id, each d = bf16(W_dn[e] . h_e), then
+//              y = bf16(y + bf16(d * w_e)) - the dtype chain and the summation order of _Experts._one_row / _loop
+//              (btb/engine/host.py:508-569, 906-967)
 //
 // Nothing goes back to the host between the steps, so the layer records into a hipGraph.
 
@@ -240,13 +241,16 @@ static int32_t launch_route(const void* logits, size_t ls, int E, int k, int T, 
 // gate_up: the dense loop over (token, pick) pairs; blockIdx.y is the pair
 // ------------------------------------------------------------------------------------------------------------
 
+// A wave takes gate row r and up row I + r together (RPW = 2) and writes h[r] = bf16(bf16(silu(bf16(g))) * bf16(u)): the
+// pair's gu row is never stored, the down kernel finds its x ready.
 template <int LPR, int RPW, int U>
 __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restrict__ stack, const uint16_t* __restrict__ x,
-                                                          const int32_t* __restrict__ idx, uint16_t* __restrict__ gu,
+                                                          const int32_t* __restrict__ idx, uint16_t* __restrict__ h,
                                                           int R, int C, int k, int E) {
+    static_assert(RPW == 2, "gate and up");
     extern __shared__ __align__(16) uint32_t xs[];
     using F = FmtBf16;
-    constexpr int G = WAVE / LPR, ROWS = G * RPW;
+    constexpr int G = WAVE / LPR, ROWS = G;
     const int pair = blockIdx.y;
     const int token = pair / k;
     int expert = idx[pair];
@@ -255,10 +259,11 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
     const int lane = threadIdx.x & (WAVE - 1), sl = lane % LPR;
     const int wave = blockIdx.x * (blockDim.x / WAVE) + (threadIdx.x / WAVE);
     const int nwaves = gridDim.x * (blockDim.x / WAVE);
-    const int ntiles = (R + ROWS - 1) / ROWS;
+    const int I = R / 2;
+    const int ntiles = (I + ROWS - 1) / ROWS;
     const int span = U * LPR;
     F::Params p{stack + (size_t)expert * R * units};
-    uint16_t* y = gu + (size_t)pair * R;
+    uint16_t* y = h + (size_t)pair * I;
 
     stage_x<X_PLAIN>(xs, XArgs{x + (size_t)token * C, nullptr, nullptr, nullptr, 0.f, 0}, 1, C);
     const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
@@ -267,8 +272,8 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
         int rows[RPW];
 #pragma unroll
         for (int j = 0; j < RPW; ++j) {
-            rows[j] = tile * ROWS + j * G + lane / LPR;
-            ctx[j] = F::row_ctx(p, (size_t)min(rows[j], R - 1), units);
+            rows[j] = tile * ROWS + lane / LPR;
+            ctx[j] = F::row_ctx(p, (size_t)(min(rows[j], I - 1) + j * I), units);
         }
         float acc[RPW][1];
 #pragma unroll
@@ -283,11 +288,9 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
                 fma_span<F, 1, LPR, RPW, U, true>(raw, ctx, k0, sl, units, xs4, C / 8, acc);
             }
         }
-#pragma unroll
-        for (int j = 0; j < RPW; ++j) {
-            const float s = group_sum<LPR>(acc[j][0]);
-            if (sl == 0 && rows[j] < R) y[rows[j]] = f32_bf16(s);
-        }
+        const float g = bfround(group_sum<LPR>(acc[0][0]));
+        const float u = bfround(group_sum<LPR>(acc[1][0]));
+        if (sl == 0 && rows[0] < I) y[rows[0]] = f32_bf16(bfround(g / (1.f + expf(-g))) * u);
     }
 }
 
@@ -296,7 +299,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
 // ------------------------------------------------------------------------------------------------------------
 
 template <int LPR, int RPW, int U, int KB>
-__global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__ stack, const uint16_t* __restrict__ gu,
+__global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__ stack, const uint16_t* __restrict__ h,
                                                        const int32_t* __restrict__ idx, const uint16_t* __restrict__ wts,
                                                        uint16_t* __restrict__ y, int R, int C, int k, int E) {
     extern __shared__ __align__(16) uint32_t hs[];  // [k][C / 2] the k experts' h rows, in ascending expert order
@@ -345,26 +348,24 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__
     };
     if (wave < ntiles) request(wave, 0);
 
-    // the k picks' h rows = bf16(bf16(silu(g)) * u), each at its place in ascending expert order: one pass over all of
-    // them, four pairs a thread in flight, one barrier
+    // the k picks' h rows, each to its place in ascending expert order: 16 bytes a load, four a thread in flight
     {
-        const int half = C / 2;  // bf16 pairs per row
-        const uint32_t* src = reinterpret_cast<const uint32_t*>(gu);
-        const int n = k * half;
+        const int per = C / 8;  // 16-byte pieces a row
+        const uint4* src = reinterpret_cast<const uint4*>(h);
+        uint4* dst = reinterpret_cast<uint4*>(hs);
+        const int n = k * per;
         for (int i0 = threadIdx.x; i0 < n; i0 += 4 * (int)blockDim.x) {
-            uint32_t g2[4], u2[4];
+            uint4 v[4];
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int i = min(i0 + v * (int)blockDim.x, n - 1);
-                const int q = i / half, c = i - q * half;
-                const size_t row = ((size_t)token * k + (s_expert[q] >> 20)) * 2 * half;
-                g2[v] = src[row + c];
-                u2[v] = src[row + half + c];
+            for (int t = 0; t < 4; ++t) {
+                const int i = min(i0 + t * (int)blockDim.x, n - 1);
+                const int q = i / per, c = i - q * per;
+                v[t] = src[((size_t)token * k + (s_expert[q] >> 20)) * per + c];
             }
 #pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const int i = i0 + v * (int)blockDim.x;
-                if (i < n) hs[i] = silu_pair(g2[v], u2[v]);
+            for (int t = 0; t < 4; ++t) {
+                const int i = i0 + t * (int)blockDim.x;
+                if (i < n) dst[i] = v[t];
             }
         }
     }
@@ -421,7 +422,7 @@ template <int LPR>
 static int32_t launch_gate_up(const void* stack, const void* x, const int32_t* idx, void* gu, int R, int C, int k, int E,
                               int pairs, hipStream_t st) {
     constexpr int RPW = 2, U = 4, G = WAVE / LPR;
-    const int ntiles = (R + G * RPW - 1) / (G * RPW);
+    const int ntiles = (R / 2 + G - 1) / G;
     const int grid = (ntiles + 3) / 4;
     hipLaunchKernelGGL((moe_gate_up_kernel<LPR, RPW, U>), dim3(grid, pairs), dim3(256), (size_t)C * 2, st,
                        static_cast<const uint4*>(stack), static_cast<const uint16_t*>(x), idx,

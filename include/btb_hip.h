@@ -183,7 +183,7 @@ int32_t btb_hip_moe_router_bf16(const void* router, const void* x, size_t T, siz
 
 /* The routed experts of T rows: gate_up [E, 2I, H] and down [E, H, I] bf16 stacks (gate rows then up rows), x [T, H]
  * bf16, the picks idx [T, k] and weights w bf16 [T, k] of btb_hip_moe_route, gu [T, k, 2I] bf16 scratch the caller
- * owns, y [T, H] bf16. Per pick: gu = bf16(W_gu x), h = bf16(bf16(silu(g)) * u), d = bf16(W_dn h); per row
+ * owns (the kernels keep the picks' h rows in it), y [T, H] bf16. Per pick: gu = bf16(W_gu x), h = bf16(bf16(silu(g)) * u), d = bf16(W_dn h); per row
  * y = sum over the picks in ASCENDING expert id of bf16(d * w), each addition rounded to bf16: the arithmetic of
  * _Experts._one_row / _loop (btb/engine/host.py:508-569, 906-967). T * k <= 65535. */
 int32_t btb_hip_moe_experts_bf16(const void* gate_up, const void* down, const void* x, const int32_t* idx, const void* w,
