@@ -143,8 +143,29 @@ __global__ void __launch_bounds__(256) lane16_bf16_wide_kernel(const uint16_t* _
         for (int n = 0; n < NB; ++n) raw[n] = wrow[(size_t)min(n0 + n, nchunks - 1) * 16 + j];
     };
     request(0);
-    for (int b = 0; b < B; ++b)
-        for (size_t c = tid; c < cols; c += 256) xs[c * BP + b] = b0 + b < btotal ? x_at(x, (b0 + b) * cols + c) : 0.f;
+    // x in 16-byte pieces (rows are 16-byte aligned: cols is a multiple of 128), every piece of every row requested
+    // before the first is spread out
+    constexpr int PER = 16 / (int)sizeof(XT);  // values a piece
+    const size_t pieces = cols / PER;
+#pragma unroll
+    for (int b = 0; b < B; ++b) {
+        const bool have = b0 + b < btotal;
+        const uint4* src = reinterpret_cast<const uint4*>(x + (have ? b0 + b : b0) * cols);
+        for (size_t i = tid; i < pieces; i += 256) {
+            const uint4 v = src[i];
+            const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+            float* dst = xs + i * PER * BP + b;
+#pragma unroll
+            for (int e = 0; e < PER; ++e) {
+                float f;
+                if (sizeof(XT) == 4)
+                    f = bits_f32(d[e]);
+                else
+                    f = (e & 1) ? bf16hi_f32(d[e >> 1]) : bf16lo_f32(d[e >> 1]);
+                dst[e * BP] = have ? f : 0.f;
+            }
+        }
+    }
     __syncthreads();
     unsigned char* mine = slabs + (size_t)grp * (NB * 256);
     float acc[B];
@@ -196,7 +217,7 @@ static int32_t launch_lane16(const W& w, const XT* x, float* y, size_t rows, siz
     const unsigned grid = (unsigned)((rows + 15) / 16);
     size_t b0 = 0;
     if constexpr (std::is_same<W, W16Bf16>::value) {
-        if (cols % 128 == 0 && (reinterpret_cast<uintptr_t>(w.w) & 15) == 0) {
+        if (cols % 128 == 0 && ((reinterpret_cast<uintptr_t>(w.w) | reinterpret_cast<uintptr_t>(x)) & 15) == 0) {
             // every pass of four rows of x in one launch (the pass is the grid's second dimension), then the rest
             bool done = true;
             const size_t fours = std::min<size_t>(b / 4, 65535);
@@ -211,7 +232,7 @@ static int32_t launch_lane16(const W& w, const XT* x, float* y, size_t rows, siz
                     if (done) b0 += 4;
                 } else {
                     done = left >= 2 ? launch_wide<3, 4>(w.w, x, y, rows, cols, b0, b, 1, st)
-                                     : launch_wide<1, 8>(w.w, x, y, rows, cols, b0, b, 1, st);
+                                     : launch_wide<1, 16>(w.w, x, y, rows, cols, b0, b, 1, st);
                     if (done) b0 = b;
                 }
             }
