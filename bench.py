@@ -83,20 +83,22 @@ def kernel_workload(args: argparse.Namespace) -> int:
 
     name = args.workload
     if name == "moe":
-        E, k, H, I, pool = 128, 8, 2048, 768, 2
+        # two layers' stacks (3.6 GB) and eight sets of rows: every call routes to other experts, so a pass streams
+        # 0.6 GB (one token) to 3 GB of distinct expert matrices - nothing comes back out of the 256 MB cache
+        E, k, H, I, pool = 128, 8, 2048, 768, 8
         sets = [(Router(card, normal(E, H).to(torch.bfloat16), k), Experts(card, normal(E, 2 * I, H).to(torch.bfloat16),
                                                                            normal(E, H, I).to(torch.bfloat16)))
-                for _ in range(pool)]
-        x = torch.randn(M, H, generator=g, device=dev).to(torch.bfloat16)
+                for _ in range(2)]
+        xs = [torch.randn(M, H, generator=g, device=dev).to(torch.bfloat16) for _ in range(pool)]
         distinct = []
 
         def call(i: int) -> None:
-            router, experts = sets[i]
-            _, w, idx = router(x)
-            experts(x, idx, w)
+            router, experts = sets[i % 2]
+            _, w, idx = router(xs[i])
+            experts(xs[i], idx, w)
 
         for i in range(pool):  # the bytes a call streams: the router and every DISTINCT expert its picks name
-            _, _, idx = sets[i][0](x)
+            _, _, idx = sets[i % 2][0](xs[i])
             distinct.append(int(torch.unique(idx).numel()))
         per_expert = (2 * I * H + H * I) * 2
         nbytes = [E * H * 2 + d * per_expert for d in distinct]
@@ -105,7 +107,9 @@ def kernel_workload(args: argparse.Namespace) -> int:
         dtype = "bf16 weights and activations, f32 accumulate"
     else:
         R, C = (9728, 2560) if name in ("gemv_bf16", "gemv_p12") else (18432, 7168)
-        pool = 8 if R == 9728 else 4
+        # operands of a pass: at least 600 MB of stored weights, well past the 256 MB last-level cache
+        per = {"gemv_bf16": 2.0, "gemv_p12": 1.5, "gemv_fp8": 1.0, "gemv_mxfp4": 17 / 32}[name] * R * C
+        pool = max(4, -(-600_000_000 // int(per)))
         mats = []
         for _ in range(pool):
             t = normal(R, C)
