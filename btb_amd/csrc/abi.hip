@@ -62,6 +62,7 @@ static Knob g_knobs[] = {
     {"gemv_no_mfma", {-1}},
     {"gemv_short_span", {-1}},
     {"gemv_glu_split", {-1}},
+    {"gemv_stretch", {-1}},
     {"mfma_wgs_per_cu", {-1}},
     {"mfma_classic", {-1}},
     {"mfma_lds", {-1}},

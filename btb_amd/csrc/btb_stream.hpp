@@ -50,7 +50,7 @@ __device__ __forceinline__ float block_sum256(float v, float* red) {
 // LDS the staging needs for M rows of C values: the rows themselves, and for X_ADDNORM three raw rows (h, y and the
 // norm's weight) behind them
 __host__ __device__ constexpr size_t stage_lds_bytes(int xmode, int M, int C) {
-    return (size_t)(M + (xmode == X_ADDNORM ? 3 : 0)) * (size_t)C * 2;
+    return (size_t)(M + (xmode == X_ADDNORM ? 1 : 0)) * (size_t)C * 2;
 }
 
 // Leaves the rows in xs (a barrier included). 256 threads. `after_issue` is called once, right after the first loads
@@ -60,13 +60,22 @@ template <int XMODE, class AfterIssue>
 __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C, AfterIssue after_issue) {
     const int tid = threadIdx.x, nt = blockDim.x;
     if (XMODE == X_PLAIN) {
+        // the first five 16-byte pieces a thread copies (rows up to 10240 values) are requested together and
+        // unconditionally - a piece past the end reads the last piece again - so that the wait for them is counted
+        // exactly and does not take in the weights requested behind them. The stores are unconditional as well (a
+        // load whose only use sits in a branch is moved into it, behind the weights): the repeated piece is written
+        // to its own place again
         const uint4* src = reinterpret_cast<const uint4*>(a.x);
         uint4* dst = reinterpret_cast<uint4*>(xs);
         const int n = M * C / 8;
-        const uint4 v0 = src[min(tid, n - 1)];
+        constexpr int PER = 5;
+        uint4 v[PER];
+#pragma unroll
+        for (int q = 0; q < PER; ++q) v[q] = src[min(tid + q * 256, n - 1)];
         after_issue();
-        if (tid < n) dst[tid] = v0;
-        for (int i = tid + nt; i < n; i += nt) dst[i] = src[i];
+#pragma unroll
+        for (int q = 0; q < PER; ++q) dst[min(tid + q * 256, n - 1)] = v[q];
+        for (int i = tid + PER * 256; i < n; i += 256) dst[i] = src[i];
     } else if (XMODE == X_SILU) {
         after_issue();
         const int half = C / 2;  // pairs per row
@@ -77,21 +86,23 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
         }
     } else {
         // h' = bf16(h + y); x = bf16(h' * rsqrt(mean(h'^2) + eps) * w): the arithmetic and the summation order of the
-        // stand-alone add_rmsnorm kernel (thread i takes elements i, i + 256, ...), so the bits are its bits. Every
-        // workgroup makes the whole row for itself; the first also writes the new residual out. The row's inputs
-        // come in with 8-byte loads, all issued together, into raw rows in LDS; the arithmetic then reads LDS in its
-        // own element order.
+        // stand-alone add_rmsnorm kernel (thread i takes the 4-element words i, i + 256, ..., a word's elements in
+        // order), so the bits are its bits. Every workgroup makes the whole row for itself; the first also writes the
+        // new residual out. A thread's words come in with 8-byte loads, all issued together, and it works on them in
+        // registers: h' and the norm weight wait in the thread's own LDS slots while the block sums the squares, so
+        // no barrier is needed besides the sum's own.
         __shared__ float red[4];
-        uint16_t* xs16 = reinterpret_cast<uint16_t*>(xs);
-        uint16_t* hraw = xs16 + (size_t)M * C;
-        uint16_t* yraw = hraw + C;
-        uint16_t* wraw = yraw + C;
+        uint2* rows4 = reinterpret_cast<uint2*>(xs);
         const int n4 = C / 4;  // 8-byte words per row (C is a multiple of the format's unit, at least 8)
+        uint2* wkeep = rows4 + (size_t)M * n4;
         constexpr int PER = 3;  // words a thread holds at once: rows up to 3072 wide take one pass
+        const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr;
         for (int m = 0; m < M; ++m) {
             const uint2* hs = reinterpret_cast<const uint2*>(a.x + (size_t)m * C);
-            const uint2* ys = a.y == nullptr ? nullptr : reinterpret_cast<const uint2*>(a.y + (size_t)m * C);
+            const uint2* ys = a.y == nullptr ? hs : reinterpret_cast<const uint2*>(a.y + (size_t)m * C);
             const uint2* ws = reinterpret_cast<const uint2*>(a.norm_w);
+            uint2* row = rows4 + (size_t)m * n4;
+            float ss = 0.f;
             for (int base = 0; base < n4; base += PER * 256) {
                 uint2 hv[PER], yv[PER], wv[PER];
 #pragma unroll
@@ -100,37 +111,45 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
                     // wait for them is then counted exactly (they are not held up behind the weights requested next)
                     const int i = min(base + q * 256 + tid, n4 - 1);
                     hv[q] = hs[i];
-                    yv[q] = ys != nullptr ? ys[i] : make_uint2(0, 0);
+                    yv[q] = ys[i];  // no y: h again, unused
                     wv[q] = ws[i];
                 }
                 if (m == 0 && base == 0) after_issue();
+                // the arithmetic and the stores are unconditional too (selects, not branches: a load whose only use
+                // sits in a branch is moved into it, behind the weights); a word past the end is the last word
+                // again, and is written to the last word's place again
+                const bool has_y = a.y != nullptr;
 #pragma unroll
                 for (int q = 0; q < PER; ++q) {
                     const int i = base + q * 256 + tid;
-                    if (i < n4) {
-                        reinterpret_cast<uint2*>(hraw)[i] = hv[q];
-                        reinterpret_cast<uint2*>(yraw)[i] = yv[q];
-                        if (m == 0) reinterpret_cast<uint2*>(wraw)[i] = wv[q];
+                    const bool live = i < n4;
+                    float f[4] = {bf16lo_f32(hv[q].x), bf16hi_f32(hv[q].x), bf16lo_f32(hv[q].y), bf16hi_f32(hv[q].y)};
+                    const float g[4] = {bf16lo_f32(yv[q].x), bf16hi_f32(yv[q].x), bf16lo_f32(yv[q].y), bf16hi_f32(yv[q].y)};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float sum = bfround(f[e] + g[e]);
+                        f[e] = has_y ? sum : f[e];
+                        const float sq = fmaf(f[e], f[e], ss);
+                        ss = live ? sq : ss;
                     }
+                    const uint2 hb = make_uint2(f32_bf16(f[0]) | ((uint32_t)f32_bf16(f[1]) << 16),
+                                                f32_bf16(f[2]) | ((uint32_t)f32_bf16(f[3]) << 16));
+                    const int ic = min(i, n4 - 1);
+                    row[ic] = hb;
+                    wkeep[ic] = wv[q];
+                    if (writer) reinterpret_cast<uint2*>(a.h_out + (size_t)m * C)[ic] = hb;
                 }
             }
-            __syncthreads();
-            uint16_t* row = xs16 + (size_t)m * C;
-            float ss = 0.f;
-            for (int i = tid; i < C; i += 256) {
-                float hv = bf16_f32(hraw[i]);
-                if (ys != nullptr) hv = bfround(hv + bf16_f32(yraw[i]));
-                row[i] = f32_bf16(hv);
-                ss = fmaf(hv, hv, ss);
-            }
             const float rstd = rsqrtf(block_sum256(ss, red) / (float)C + a.eps);
-            for (int i = tid; i < C; i += 256) {
-                const uint16_t hb = row[i];
-                if (blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr) a.h_out[(size_t)m * C + i] = hb;
-                const float wv = bf16_f32(wraw[i]);
-                row[i] = f32_bf16(bf16_f32(hb) * rstd * (a.centered ? 1.f + wv : wv));
+            for (int i = tid; i < n4; i += 256) {
+                const uint2 hb = row[i], wb = wkeep[i];
+                const float f[4] = {bf16lo_f32(hb.x), bf16hi_f32(hb.x), bf16lo_f32(hb.y), bf16hi_f32(hb.y)};
+                const float g[4] = {bf16lo_f32(wb.x), bf16hi_f32(wb.x), bf16lo_f32(wb.y), bf16hi_f32(wb.y)};
+                uint32_t o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = f32_bf16(f[e] * rstd * (a.centered ? 1.f + g[e] : g[e]));
+                row[i] = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
             }
-            __syncthreads();  // the raw rows are free for the next row
         }
     }
     __syncthreads();
@@ -224,6 +243,20 @@ __device__ __forceinline__ void load_span(typename F::Raw (&raw)[U][RPW], const 
 #pragma unroll
             for (int j = 0; j < RPW; ++j) raw[u][j] = F::load(ctx[j], unit);
         }
+    }
+}
+
+// the same loads with nothing conditional about them: a unit past the row's end reads the row's last unit again (and
+// is not used). Requested ahead of a wait for earlier loads, every one of these is certain to have been issued, so that
+// wait is counted exactly and does not hold out for these as well.
+template <class F, int LPR, int RPW, int U>
+__device__ __forceinline__ void load_span_always(typename F::Raw (&raw)[U][RPW], const typename F::RowCtx (&ctx)[RPW],
+                                                 int k0, int sl, int units) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+        const int unit = min(k0 + u * LPR + sl, units - 1);
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) raw[u][j] = F::load(ctx[j], unit);
     }
 }
 

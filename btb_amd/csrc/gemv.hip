@@ -114,15 +114,15 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs x
 
     typename F::Raw first[U][RPW] = {};
     stage_x<XMODE>(xs, xa, M, C, [&] {
-        if (wave < ntiles) {
-            typename F::RowCtx ctx[RPW];
+        // a wave with no tile requests the last tile's span and drops it: nothing here is conditional (see
+        // load_span_always)
+        typename F::RowCtx ctx[RPW];
 #pragma unroll
-            for (int j = 0; j < RPW; ++j) {
-                int out_row;
-                ctx[j] = F::row_ctx(p, (size_t)tile_row<LPR, RPW, EPI>(wave, j, lane, R, out_row), units);
-            }
-            load_span<F, LPR, RPW, U, true>(first, ctx, 0, lane % LPR, units);
+        for (int j = 0; j < RPW; ++j) {
+            int out_row;
+            ctx[j] = F::row_ctx(p, (size_t)tile_row<LPR, RPW, EPI>(min(wave, ntiles - 1), j, lane, R, out_row), units);
         }
+        load_span_always<F, LPR, RPW, U>(first, ctx, 0, lane % LPR, units);
     });
     const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
     if (wave >= ntiles) return;
@@ -180,10 +180,25 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
     // waves resident: one row by four (pack12, MXFP4), two rows by two (FP8, whose two rows share a scale fetch
     // pattern). Neither choice changes a result bit (a lane's units stay in ascending order).
     constexpr bool WIDENS = sizeof(typename F::Raw) != 16;  // everything but plain bf16
+    // One row of x (the decode step proper): where a slightly longer span saves a whole round trip to memory - a row of
+    // 5 units a lane read as 5, not 4 + 1; 19 as 10 + 9, not 8 + 8 + 3 - the span is stretched to 5 (10 for one bf16
+    // row a wave). A lane's units stay in ascending order, so no result bit changes.
+    const int per_lane = (C / F::UW + LPR - 1) / LPR;
+    auto fewer = [per_lane](int u_new, int u_base) { return (per_lane + u_new - 1) / u_new < (per_lane + u_base - 1) / u_base; };
+    const int stretch_knob = tuning("gemv_stretch");  // measured: a gain for bf16, a loss for the forms that widen
+    const bool stretch = M == 1 && (stretch_knob >= 0 ? stretch_knob == 1 : !WIDENS);
     if constexpr (EPI == E_GLU) {
         // a widening form whose rows take at most 32 lanes: gate and up side by side, one row a lane
         if constexpr (WIDENS && LPR <= 32) {
-            if (tuning("gemv_glu_split") != 0) return launch_variant<F, M, LPR, 1, 4, XMODE, E_GLU_SPLIT>(p, xa, y, R, C, st);
+            if (tuning("gemv_glu_split") != 0) {
+                if constexpr (M == 1 && F::TWO_ROWS == false) {
+                    if (stretch && fewer(5, 4)) return launch_variant<F, M, LPR, 1, 5, XMODE, E_GLU_SPLIT>(p, xa, y, R, C, st);
+                }
+                return launch_variant<F, M, LPR, 1, 4, XMODE, E_GLU_SPLIT>(p, xa, y, R, C, st);
+            }
+        }
+        if constexpr (M == 1 && !WIDENS) {
+            if (stretch && fewer(5, 4)) return launch_variant<F, M, LPR, 2, 5, XMODE, E_GLU>(p, xa, y, R, C, st);
         }
         return launch_variant<F, M, LPR, 2, (M <= 2 && !WIDENS ? 4 : 2), XMODE, E_GLU>(p, xa, y, R, C, st);
     }
@@ -191,8 +206,15 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
     const int shorter = tuning("gemv_short_span");
     const bool tall = v >= 0 ? (v == 1) : (WIDENS ? F::TWO_ROWS : R >= 4096 * (WAVE / LPR));
     if (M <= 2 && (shorter >= 0 ? shorter == 0 : !WIDENS)) {
+        if constexpr (M == 1 && !WIDENS) {
+            if (stretch && tall && fewer(5, 4)) return launch_variant<F, M, LPR, 2, 5, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+            if (stretch && !tall && fewer(10, 8)) return launch_variant<F, M, LPR, 1, 10, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+        }
         if (tall) return launch_variant<F, M, LPR, 2, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
         return launch_variant<F, M, LPR, 1, 8, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+    }
+    if constexpr (M == 1 && WIDENS && F::TWO_ROWS == false) {
+        if (stretch && !tall && fewer(5, 4)) return launch_variant<F, M, LPR, 1, 5, XMODE, E_PLAIN>(p, xa, y, R, C, st);
     }
     if (tall) return launch_variant<F, M, LPR, 2, 2, XMODE, E_PLAIN>(p, xa, y, R, C, st);
     return launch_variant<F, M, LPR, 1, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);

@@ -37,14 +37,18 @@ __global__ void __launch_bounds__(256) add_rmsnorm_kernel(uint16_t* __restrict__
     uint16_t* hr = h + (size_t)t * H;
     const uint16_t* yr = y == nullptr ? nullptr : y + (size_t)t * H;
     uint16_t* xr = x + (size_t)t * H;
+    // thread i takes the 4-element words i, i + 256, ... of the row, a word's elements in order (the order the matvec's
+    // fused staging sums in, where a word is one 8-byte load)
     float ss = 0.f;
-    for (int i = tid; i < H; i += 256) {
-        float hv = bf16_f32(hr[i]);
-        if (yr != nullptr) {
-            hv = bfround(hv + bf16_f32(yr[i]));
-            hr[i] = f32_bf16(hv);
+    for (int wd = tid; 4 * wd < H; wd += 256) {
+        for (int i = 4 * wd; i < min(4 * wd + 4, H); ++i) {
+            float hv = bf16_f32(hr[i]);
+            if (yr != nullptr) {
+                hv = bfround(hv + bf16_f32(yr[i]));
+                hr[i] = f32_bf16(hv);
+            }
+            ss = fmaf(hv, hv, ss);
         }
-        ss = fmaf(hv, hv, ss);
     }
     const float rstd = rsqrtf(block_sum256(ss, red) / (float)H + eps);
     for (int i = tid; i < H; i += 256) {

@@ -186,7 +186,7 @@ __device__ __forceinline__ void stage_rows(uint32_t* xs, const uint16_t* x, int 
 }
 
 // h' = bf16(h + y), x = bf16(h' * rsqrt(mean(h'^2) + eps) * w): stage_x<X_ADDNORM>'s arithmetic and order (thread i
-// takes elements i, i + 256, ...). The two rows come into LDS first, in wide loads all in flight at once (one round
+// takes the 4-element words i, i + 256, ...). The two rows come into LDS first, in wide loads all in flight at once (one round
 // trip to memory), behind the x row: LDS holds 3 * C values here. `fresh` is false where h is read-only data (the
 // embedding row).
 __device__ __forceinline__ void stage_addnorm(uint32_t* xs, const uint16_t* h, bool fresh, const uint16_t* y,
@@ -207,11 +207,15 @@ __device__ __forceinline__ void stage_addnorm(uint32_t* xs, const uint16_t* h, b
         copy_dev8(reinterpret_cast<unsigned long long*>(yraw), reinterpret_cast<const unsigned long long*>(y), C / 4);
     __syncthreads();
     float ss = 0.f;
-    for (int i = tid; i < C; i += 256) {
-        float hv = bf16_f32(hraw[i]);
-        if (y != nullptr) hv = bfround(hv + bf16_f32(yraw[i]));
-        row[i] = f32_bf16(hv);
-        ss = fmaf(hv, hv, ss);
+    for (int wd = tid; wd < C / 4; wd += 256) {  // 4-element words, a word's elements in order
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int i = 4 * wd + e;
+            float hv = bf16_f32(hraw[i]);
+            if (y != nullptr) hv = bfround(hv + bf16_f32(yraw[i]));
+            row[i] = f32_bf16(hv);
+            ss = fmaf(hv, hv, ss);
+        }
     }
     const float rstd = rsqrtf(block_sum256(ss, red) / (float)C + eps);
     for (int i = tid; i < C; i += 256) {
