@@ -21,31 +21,48 @@ __device__ __forceinline__ void st_dev(T* p, T v) {
 
 constexpr int AD = 128;
 
-// one head's 128 values: RMSNorm (weight wn or none), rope at `pos`; lane holds dims 2 * lane, 2 * lane + 1
+// one head's 128 values: RMSNorm (weight wn or none), rope at `pos`; lane holds dims 2 * lane, 2 * lane + 1. In two
+// steps, so that a caller can request the head's inputs, then other data, and only then wait for the inputs.
+struct HeadIn {
+    uint32_t raw, wn, cs, sn;  // the lane's pair of values, of norm weights, of cosines and of sines
+};
+template <bool DEV>
+__device__ __forceinline__ HeadIn head_request(const uint16_t* src, const uint16_t* wn, const uint16_t* cos_t,
+                                               const uint16_t* sin_t, int pos, int lane) {
+    HeadIn in;
+    const uint32_t* src2 = reinterpret_cast<const uint32_t*>(src) + lane;
+    in.raw = DEV ? ld_dev(src2) : *src2;
+    in.wn = reinterpret_cast<const uint32_t*>(wn != nullptr ? wn : cos_t)[lane];  // no weight: any word, unused
+    in.cs = reinterpret_cast<const uint32_t*>(cos_t + (size_t)pos * AD)[lane];
+    in.sn = reinterpret_cast<const uint32_t*>(sin_t + (size_t)pos * AD)[lane];
+    return in;
+}
+__device__ __forceinline__ void head_finish(const HeadIn& in, bool has_wn, float eps, int centered, int lane,
+                                            uint16_t (&out)[2]) {
+    float v[2] = {bf16lo_f32(in.raw), bf16hi_f32(in.raw)};
+    if (has_wn) {
+        float ss = fmaf(v[1], v[1], fmaf(v[0], v[0], 0.f));
+        ss = group_sum<64>(ss);
+        const float rstd = rsqrtf(ss / (float)AD + eps);
+        const float w2[2] = {bf16lo_f32(in.wn), bf16hi_f32(in.wn)};
+#pragma unroll
+        for (int e = 0; e < 2; ++e) v[e] = bfround(v[e] * rstd * (centered ? 1.f + w2[e] : w2[e]));
+    }
+    const float sgn = lane < 32 ? -1.f : 1.f;
+    const float c2[2] = {bf16lo_f32(in.cs), bf16hi_f32(in.cs)}, s2[2] = {bf16lo_f32(in.sn), bf16hi_f32(in.sn)};
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {
+        const float rot = __shfl_xor(v[e], 32, WAVE);
+        const float qc = bfround(v[e] * c2[e]);
+        out[e] = f32_bf16(fmaf(sgn * rot, s2[e], qc));
+    }
+}
 template <bool DEV>
 __device__ __forceinline__ void head_norm_rope(const uint16_t* src, const uint16_t* wn, float eps, int centered,
                                                const uint16_t* cos_t, const uint16_t* sin_t, int pos, int lane,
                                                uint16_t (&out)[2]) {
-    const uint32_t* src2 = reinterpret_cast<const uint32_t*>(src) + lane;
-    const uint32_t raw = DEV ? ld_dev(src2) : *src2;
-    float v[2] = {bf16lo_f32(raw), bf16hi_f32(raw)};
-    if (wn != nullptr) {
-        float ss = fmaf(v[1], v[1], fmaf(v[0], v[0], 0.f));
-        ss = group_sum<64>(ss);
-        const float rstd = rsqrtf(ss / (float)AD + eps);
-#pragma unroll
-        for (int e = 0; e < 2; ++e) {
-            const float wv = bf16_f32(wn[lane * 2 + e]);
-            v[e] = bfround(v[e] * rstd * (centered ? 1.f + wv : wv));
-        }
-    }
-    const float sgn = lane < 32 ? -1.f : 1.f;
-#pragma unroll
-    for (int e = 0; e < 2; ++e) {
-        const float rot = __shfl_xor(v[e], 32, WAVE);
-        const float qc = bfround(v[e] * bf16_f32(cos_t[(size_t)pos * AD + lane * 2 + e]));
-        out[e] = f32_bf16(fmaf(sgn * rot, bf16_f32(sin_t[(size_t)pos * AD + lane * 2 + e]), qc));
-    }
+    const HeadIn in = head_request<DEV>(src, wn, cos_t, sin_t, pos, lane);
+    head_finish(in, wn != nullptr, eps, centered, lane, out);
 }
 
 // one batch of a key stream: eight keys sixteen apart, their K and V rows (this lane's 8 dims) requested together

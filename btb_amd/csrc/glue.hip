@@ -254,20 +254,33 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
     const int k_begin = sp * span, k_end = min(n0 + 1, k_begin + span);
     const uint16_t* Kh = K + (size_t)g * hs + dl * 8;
     const uint16_t* Vh = V + (size_t)g * hs + dl * 8;
+    // requests in the order their answers are needed (loads come back in order): the heads' inputs - a few words out
+    // of L2 - then the stream's first keys; the norm and rope then run while the keys travel
+    constexpr int NQ = (G + 3) / 4;  // query heads a wave prepares
+    HeadIn qin[NQ];
+#pragma unroll
+    for (int i = 0; i < NQ; ++i)
+        qin[i] = head_request<false>(qkv + (size_t)(g * G + min(wv + 4 * i, G - 1)) * D, wq, cos_t, sin_t, n0, lane);
+    const bool owner = wv == 3 && n0 >= k_begin && n0 < k_begin + span;  // this workgroup's span holds the new slot
+    const HeadIn kin = head_request<false>(qkv + (size_t)(Hq + g) * D, wk, cos_t, sin_t, n0, lane);
+    const uint32_t vraw = reinterpret_cast<const uint32_t*>(qkv + (size_t)(Hq + Hk + g) * D)[lane];
     KeyBatch kb = {};
     const int key_first = k_begin + grp;
-    if (key_first < k_end) load_keys(kb, Kh, Vh, rs, key_first, k_end, n0);
+    load_keys(kb, Kh, Vh, rs, min(key_first, max(k_end - 1, 0)), max(k_end, 1), n0);
 
-    for (int j = wv; j < G; j += 4) {
+#pragma unroll
+    for (int i = 0; i < NQ; ++i) {
+        const int j = wv + 4 * i;
         uint16_t o[2];
-        head_norm_rope<false>(qkv + (size_t)(g * G + j) * D, wq, eps, centered, cos_t, sin_t, n0, lane, o);
-        s_q[j][lane * 2 + 0] = bf16_f32(o[0]) * scale_log2;
-        s_q[j][lane * 2 + 1] = bf16_f32(o[1]) * scale_log2;
+        head_finish(qin[i], wq != nullptr, eps, centered, lane, o);
+        if (j < G) {
+            s_q[j][lane * 2 + 0] = bf16_f32(o[0]) * scale_log2;
+            s_q[j][lane * 2 + 1] = bf16_f32(o[1]) * scale_log2;
+        }
     }
-    if (wv == 3 && n0 >= k_begin && n0 < k_begin + span) {
+    if (owner) {
         uint16_t o[2];
-        head_norm_rope<false>(qkv + (size_t)(Hq + g) * D, wk, eps, centered, cos_t, sin_t, n0, lane, o);
-        const uint32_t vraw = reinterpret_cast<const uint32_t*>(qkv + (size_t)(Hq + Hk + g) * D)[lane];
+        head_finish(kin, wk != nullptr, eps, centered, lane, o);
         s_k[lane * 2] = o[0];
         s_k[lane * 2 + 1] = o[1];
         s_v[lane * 2] = (uint16_t)(vraw & 0xFFFFu);
