@@ -82,40 +82,66 @@ __device__ __forceinline__ void load_keys(KeyBatch& kb, const uint16_t* Kh, cons
     }
 }
 
-// the batch's keys, in ascending order, folded into the G query heads' online-softmax states (attn_decode_kernel's
-// arithmetic). A key's rows are widened once and meet all G heads before the next key is touched.
+// The batch's keys folded into the G query heads' online-softmax states, a batch at a time: the 8 x G scores first
+// (q and the key row meet as bf16 pairs in v_dot2_f32_bf16 - products exact, f32 sums - then the 16 lanes' sums are
+// folded and scaled into log2 units), then per head one new maximum, one correction of the running sum and output for
+// the whole batch, and the batch's weights; then each value row, widened once, meets all G heads. A key past the
+// span's end scores -inf and weighs 0. qp: the heads' q, this lane's 8 dims as 4 bf16 pairs. own >= 0: the step's
+// own row is key `own` and is taken from LDS (s_k, s_v) - the cache's copy may not have landed yet.
 template <int G>
-__device__ __forceinline__ void use_keys(const KeyBatch& kb, int key0, int k_end, int n0, const uint16_t* s_k,
-                                         const uint16_t* s_v, int dl, const float (&qv)[G][8], float (&m)[G],
-                                         float (&l)[G], float (&acc)[G][8]) {
+__device__ __forceinline__ void use_keys(KeyBatch& kb, int key0, int k_end, int own, const uint16_t* s_k,
+                                         const uint16_t* s_v, int dl, const uint32_t (&qp)[G][4], float scale_log2,
+                                         float (&m)[G], float (&l)[G], float (&acc)[G][8]) {
+    const float ninf = bits_f32(0xff800000u);
+    if (own >= 0) {  // uniform: only the workgroup whose span holds the slot gets here with own set
+#pragma unroll
+        for (int b = 0; b < KB; ++b)
+            if (key0 + 16 * b == own) {
+                kb.k[b] = *reinterpret_cast<const uint4*>(s_k + dl * 8);
+                kb.v[b] = *reinterpret_cast<const uint4*>(s_v + dl * 8);
+            }
+    }
+    float w[KB][G];  // scores, then weights
 #pragma unroll
     for (int b = 0; b < KB; ++b) {
-        if (key0 + 16 * b < k_end) {
-            uint4 kr = kb.k[b], vr = kb.v[b];
-            if (key0 + 16 * b == n0) {  // the step's own row, from LDS
-                kr = *reinterpret_cast<const uint4*>(s_k + dl * 8);
-                vr = *reinterpret_cast<const uint4*>(s_v + dl * 8);
-            }
-            const float kf[8] = {bf16lo_f32(kr.x), bf16hi_f32(kr.x), bf16lo_f32(kr.y), bf16hi_f32(kr.y),
-                                 bf16lo_f32(kr.z), bf16hi_f32(kr.z), bf16lo_f32(kr.w), bf16hi_f32(kr.w)};
-            const float vf[8] = {bf16lo_f32(vr.x), bf16hi_f32(vr.x), bf16lo_f32(vr.y), bf16hi_f32(vr.y),
-                                 bf16lo_f32(vr.z), bf16hi_f32(vr.z), bf16lo_f32(vr.w), bf16hi_f32(vr.w)};
+        const uint4 kr = kb.k[b];
+        const bool live = key0 + 16 * b < k_end;
 #pragma unroll
-            for (int j = 0; j < G; ++j) {
-                float sc = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) sc = fmaf(qv[j][e], kf[e], sc);
-                sc = group_sum<16>(sc);
-                const float mn = fmaxf(m[j], sc);
-                const float corr = exp2f(m[j] - mn);  // 0 on the stream's first key (m = -inf)
-                const float pp = exp2f(sc - mn);
-                l[j] = fmaf(l[j], corr, pp);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc[j][e] = fmaf(pp, vf[e], acc[j][e] * corr);
-                m[j] = mn;
-            }
+        for (int j = 0; j < G; ++j) {
+            float sc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr.x), __builtin_bit_cast(bf16x2, qp[j][0]), 0.f, false);
+            sc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr.y), __builtin_bit_cast(bf16x2, qp[j][1]), sc, false);
+            sc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr.z), __builtin_bit_cast(bf16x2, qp[j][2]), sc, false);
+            sc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr.w), __builtin_bit_cast(bf16x2, qp[j][3]), sc, false);
+            sc = group_sum<16>(sc) * scale_log2;
+            w[b][j] = live ? sc : ninf;
         }
-        __builtin_amdgcn_sched_barrier(0);  // a key at a time: widening every key's rows ahead costs the registers
+    }
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+        float mn = m[j];
+#pragma unroll
+        for (int b = 0; b < KB; ++b) mn = fmaxf(mn, w[b][j]);
+        const float corr = __builtin_amdgcn_exp2f(m[j] - mn);  // 0 on the stream's first batch (m = -inf)
+        float lj = l[j] * corr;
+#pragma unroll
+        for (int b = 0; b < KB; ++b) {
+            w[b][j] = __builtin_amdgcn_exp2f(w[b][j] - mn);
+            lj += w[b][j];
+        }
+        l[j] = lj;
+        m[j] = mn;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[j][e] *= corr;
+    }
+#pragma unroll
+    for (int b = 0; b < KB; ++b) {
+        const uint4 vr = kb.v[b];
+        const float vf[8] = {bf16lo_f32(vr.x), bf16hi_f32(vr.x), bf16lo_f32(vr.y), bf16hi_f32(vr.y),
+                             bf16lo_f32(vr.z), bf16hi_f32(vr.z), bf16lo_f32(vr.w), bf16hi_f32(vr.w)};
+#pragma unroll
+        for (int j = 0; j < G; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[j][e] = fmaf(w[b][j], vf[e], acc[j][e]);
     }
 }
 

@@ -139,19 +139,15 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     const int n = *n0p + t + 1;                  // row t sees the cache's keys and the pass's rows up to itself
     const int k_begin = sp * span, k_end = min(n, k_begin + span);
 
-    // the row's G query heads, scaled into log2 units, the lane's 8 dims of each
-    float qv[G][8];
+    // the row's G query heads, the lane's 8 dims of each as bf16 pairs (the scale meets the folded score)
+    uint32_t qp[G][4];
 #pragma unroll
     for (int j = 0; j < G; ++j) {
         const uint4 raw = *reinterpret_cast<const uint4*>(q + ((size_t)t * Hq + (size_t)g * G + j) * D + dl * 8);
-        qv[j][0] = bf16lo_f32(raw.x) * scale_log2;
-        qv[j][1] = bf16hi_f32(raw.x) * scale_log2;
-        qv[j][2] = bf16lo_f32(raw.y) * scale_log2;
-        qv[j][3] = bf16hi_f32(raw.y) * scale_log2;
-        qv[j][4] = bf16lo_f32(raw.z) * scale_log2;
-        qv[j][5] = bf16hi_f32(raw.z) * scale_log2;
-        qv[j][6] = bf16lo_f32(raw.w) * scale_log2;
-        qv[j][7] = bf16hi_f32(raw.w) * scale_log2;
+        qp[j][0] = raw.x;
+        qp[j][1] = raw.y;
+        qp[j][2] = raw.z;
+        qp[j][3] = raw.w;
     }
     float m[G], l[G], acc[G][8];
 #pragma unroll
@@ -163,38 +159,11 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     }
     const uint16_t* Kh = K + (size_t)g * hs + dl * 8;
     const uint16_t* Vh = V + (size_t)g * hs + dl * 8;
-    // eight keys of the stream a batch: their sixteen loads are issued together, then the keys are taken in order
-    constexpr int KB = 8;
+    // eight keys of the stream a batch: their sixteen loads are issued together, then the batch is folded in
     for (int key0 = k_begin + grp; key0 < k_end; key0 += 16 * KB) {
-        uint4 kr[KB], vr[KB];
-#pragma unroll
-        for (int b = 0; b < KB; ++b) {
-            const int key = min(key0 + 16 * b, k_end - 1);  // a key past the span's end is loaded again, not used
-            kr[b] = *reinterpret_cast<const uint4*>(Kh + (size_t)key * rs);
-            vr[b] = *reinterpret_cast<const uint4*>(Vh + (size_t)key * rs);
-        }
-#pragma unroll
-        for (int b = 0; b < KB; ++b) {
-            if (key0 + 16 * b >= k_end) break;
-            const float kf[8] = {bf16lo_f32(kr[b].x), bf16hi_f32(kr[b].x), bf16lo_f32(kr[b].y), bf16hi_f32(kr[b].y),
-                                 bf16lo_f32(kr[b].z), bf16hi_f32(kr[b].z), bf16lo_f32(kr[b].w), bf16hi_f32(kr[b].w)};
-            const float vf[8] = {bf16lo_f32(vr[b].x), bf16hi_f32(vr[b].x), bf16lo_f32(vr[b].y), bf16hi_f32(vr[b].y),
-                                 bf16lo_f32(vr[b].z), bf16hi_f32(vr[b].z), bf16lo_f32(vr[b].w), bf16hi_f32(vr[b].w)};
-#pragma unroll
-            for (int j = 0; j < G; ++j) {
-                float s = 0.f;
-#pragma unroll
-                for (int e = 0; e < 8; ++e) s = fmaf(qv[j][e], kf[e], s);
-                s = group_sum<16>(s);
-                const float mn = fmaxf(m[j], s);
-                const float corr = exp2f(m[j] - mn);   // 0 on the stream's first key (m = -inf)
-                const float p = exp2f(s - mn);
-                l[j] = fmaf(l[j], corr, p);
-#pragma unroll
-                for (int e = 0; e < 8; ++e) acc[j][e] = fmaf(p, vf[e], acc[j][e] * corr);
-                m[j] = mn;
-            }
-        }
+        KeyBatch kb;
+        load_keys(kb, Kh, Vh, rs, key0, k_end, -1);
+        use_keys<G>(kb, key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, m, l, acc);
     }
     // the 16 streams' states into LDS
 #pragma unroll
@@ -243,7 +212,7 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
                                                               float* __restrict__ part_l, float* __restrict__ part_acc,
                                                               int span) {
     constexpr int D = ATT_D;
-    __shared__ float s_q[G][D];
+    __shared__ uint32_t s_q[G][D / 2];  // the heads' q after norm and rope, bf16 pairs
     __shared__ __align__(16) uint16_t s_k[D], s_v[D];
     __shared__ float s_m[16][G], s_l[16][G];
     __shared__ float s_acc[16][G][D];
@@ -261,7 +230,8 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
 #pragma unroll
     for (int i = 0; i < NQ; ++i)
         qin[i] = head_request<false>(qkv + (size_t)(g * G + min(wv + 4 * i, G - 1)) * D, wq, cos_t, sin_t, n0, lane);
-    const bool owner = wv == 3 && n0 >= k_begin && n0 < k_begin + span;  // this workgroup's span holds the new slot
+    const bool holds_own = n0 >= k_begin && n0 < k_begin + span;  // this workgroup's span holds the new slot
+    const bool owner = wv == 3 && holds_own;
     const HeadIn kin = head_request<false>(qkv + (size_t)(Hq + g) * D, wk, cos_t, sin_t, n0, lane);
     const uint32_t vraw = reinterpret_cast<const uint32_t*>(qkv + (size_t)(Hq + Hk + g) * D)[lane];
     KeyBatch kb = {};
@@ -273,10 +243,7 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
         const int j = wv + 4 * i;
         uint16_t o[2];
         head_finish(qin[i], wq != nullptr, eps, centered, lane, o);
-        if (j < G) {
-            s_q[j][lane * 2 + 0] = bf16_f32(o[0]) * scale_log2;
-            s_q[j][lane * 2 + 1] = bf16_f32(o[1]) * scale_log2;
-        }
+        if (j < G) s_q[j][lane] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
     }
     if (owner) {
         uint16_t o[2];
@@ -290,11 +257,11 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
     }
     __syncthreads();
 
-    float qv[G][8];
+    uint32_t qp[G][4];
 #pragma unroll
     for (int j = 0; j < G; ++j)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qv[j][e] = s_q[j][dl * 8 + e];
+        for (int e = 0; e < 4; ++e) qp[j][e] = s_q[j][dl * 4 + e];
     float m[G], l[G], acc[G][8];
 #pragma unroll
     for (int j = 0; j < G; ++j) {
@@ -304,7 +271,7 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
         for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
     }
     for (int key0 = key_first; key0 < k_end;) {
-        use_keys<G>(kb, key0, k_end, n0, s_k, s_v, dl, qv, m, l, acc);
+        use_keys<G>(kb, key0, k_end, holds_own ? n0 : -1, s_k, s_v, dl, qp, scale_log2, m, l, acc);
         key0 += 16 * KB;
         if (key0 < k_end) load_keys(kb, Kh, Vh, rs, key0, k_end, n0);
     }

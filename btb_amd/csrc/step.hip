@@ -483,8 +483,7 @@ __device__ __forceinline__ void attention_item(const StepArgs& a, const StepLaye
     {
         uint16_t o[2];
         head_norm_rope<true>(qkv + (size_t)(g * G + wv) * AD, L.wq, a.eps, a.centered, a.cos_t, a.sin_t, n0, lane, o);
-        s_q[wv * AD + lane * 2 + 0] = bf16_f32(o[0]) * a.scale_log2;
-        s_q[wv * AD + lane * 2 + 1] = bf16_f32(o[1]) * a.scale_log2;
+        reinterpret_cast<uint32_t*>(s_q)[wv * (AD / 2) + lane] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
     }
     // the step's own key and value of this kv head: every span's workgroup makes them, the one whose span holds
     // slot n0 uses them (from LDS) and writes them into the cache
@@ -503,11 +502,11 @@ __device__ __forceinline__ void attention_item(const StepArgs& a, const StepLaye
     }
     __syncthreads();
 
-    float qv[G][8];
+    uint32_t qp[G][4];
 #pragma unroll
     for (int j = 0; j < G; ++j)
 #pragma unroll
-        for (int e = 0; e < 8; ++e) qv[j][e] = s_q[j * AD + dl * 8 + e];
+        for (int e = 0; e < 4; ++e) qp[j][e] = reinterpret_cast<const uint32_t*>(s_q)[j * (AD / 2) + dl * 4 + e];
     float m[G], l[G], acc[G][8];
 #pragma unroll
     for (int j = 0; j < G; ++j) {
@@ -517,7 +516,7 @@ __device__ __forceinline__ void attention_item(const StepArgs& a, const StepLaye
         for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
     }
     for (int key0 = key_first; key0 < k_end;) {
-        use_keys<G>(kb, key0, k_end, n0, s_k, s_v, dl, qv, m, l, acc);
+        use_keys<G>(kb, key0, k_end, (n0 >= k_begin && n0 < k_begin + a.span) ? n0 : -1, s_k, s_v, dl, qp, a.scale_log2, m, l, acc);
         key0 += 16 * KB;
         if (key0 < k_end) load_keys(kb, Kh, Vh, a.rs, key0, k_end, n0);
     }
