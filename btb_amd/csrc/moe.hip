@@ -265,7 +265,17 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
     F::Params p{stack + (size_t)expert * R * units};
     uint16_t* y = h + (size_t)pair * I;
 
-    stage_x<X_PLAIN>(xs, XArgs{x + (size_t)token * C, nullptr, nullptr, nullptr, 0.f, 0}, 1, C);
+    // the wave's first span of weights is requested right behind x's own loads, before anything waits for x: the
+    // weights do not depend on x, and nothing about these loads is conditional (a wave past the last tile requests the
+    // last tile's and drops them)
+    F::Raw first[U][RPW] = {};
+    stage_x<X_PLAIN>(xs, XArgs{x + (size_t)token * C, nullptr, nullptr, nullptr, 0.f, 0}, 1, C, [&] {
+        F::RowCtx c0[RPW];
+#pragma unroll
+        for (int j = 0; j < RPW; ++j)
+            c0[j] = F::row_ctx(p, (size_t)(min(min(wave, ntiles - 1) * ROWS + lane / LPR, I - 1) + j * I), units);
+        load_span_always<F, LPR, RPW, U>(first, c0, 0, sl, units);
+    });
     const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
     for (int tile = wave; tile < ntiles; tile += nwaves) {
         F::RowCtx ctx[RPW];
@@ -278,7 +288,12 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
         float acc[RPW][1];
 #pragma unroll
         for (int j = 0; j < RPW; ++j) acc[j][0] = 0.f;
-        for (int k0 = 0; k0 < units; k0 += span) {
+        int k0 = 0;
+        if (tile == wave) {
+            fma_span<F, 1, LPR, RPW, U, true>(first, ctx, 0, sl, units, xs4, C / 8, acc);
+            k0 = span;
+        }
+        for (; k0 < units; k0 += span) {
             F::Raw raw[U][RPW];
             if (k0 + span <= units) {
                 load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
@@ -331,11 +346,26 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__
         s_expert[place] |= j << 20;
     }
     __syncthreads();
-    // The first KB experts' rows of the wave's first tile are requested now - they need the picks only - so their trip
-    // to memory (long: a layer's experts lie megabytes apart) runs while the h rows are being made.
+    // Requests in the order their answers are needed (loads come back in order), none of them conditional (a wait
+    // is counted exactly only over loads that are certain to have been issued): the first pieces of the k picks' h
+    // rows - out of L2, staged first - then the first KB experts' rows of the wave's first tile, which need the picks
+    // only and whose trip to memory (long: a layer's experts lie megabytes apart) runs while the h rows are staged.
+    const int per = C / 8;  // 16-byte pieces a row
+    const uint4* hsrc = reinterpret_cast<const uint4*>(h);
+    uint4* hdst = reinterpret_cast<uint4*>(hs);
+    const int n = k * per;
+    auto piece = [&](int i) {  // the i-th piece of the rows in ascending expert order
+        const int q = i / per, c = i - q * per;
+        return hsrc[((size_t)token * k + (s_expert[q] >> 20)) * per + c];
+    };
+    constexpr int PER = 4;
+    uint4 hv[PER];
+#pragma unroll
+    for (int t = 0; t < PER; ++t) hv[t] = piece(min((int)threadIdx.x + t * 256, n - 1));
+
     F::RowCtx ctx[KB][RPW];
     F::Raw first[KB][U][RPW] = {};
-    auto request = [&](int tile, int q0) {
+    auto request = [&](int tile, int q0, auto always) {
 #pragma unroll
         for (int b = 0; b < KB; ++b) {
             const int expert = s_expert[min(q0 + b, k - 1)] & 0xFFFFF;
@@ -343,32 +373,18 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__
 #pragma unroll
             for (int j = 0; j < RPW; ++j)
                 ctx[b][j] = F::row_ctx(p, (size_t)min(tile * ROWS + j * G + lane / LPR, R - 1), units);
-            if (q0 + b < k) load_span<F, LPR, RPW, U, true>(first[b], ctx[b], 0, sl, units);
+            if constexpr (decltype(always)::value)
+                load_span_always<F, LPR, RPW, U>(first[b], ctx[b], 0, sl, units);  // past the k-th: the k-th again
+            else if (q0 + b < k)
+                load_span<F, LPR, RPW, U, true>(first[b], ctx[b], 0, sl, units);
         }
     };
-    if (wave < ntiles) request(wave, 0);
+    request(min(wave, ntiles - 1), 0, std::true_type{});
 
-    // the k picks' h rows, each to its place in ascending expert order: 16 bytes a load, four a thread in flight
-    {
-        const int per = C / 8;  // 16-byte pieces a row
-        const uint4* src = reinterpret_cast<const uint4*>(h);
-        uint4* dst = reinterpret_cast<uint4*>(hs);
-        const int n = k * per;
-        for (int i0 = threadIdx.x; i0 < n; i0 += 4 * (int)blockDim.x) {
-            uint4 v[4];
+    // a piece past the end is the last piece again and is written to the last piece's place again
 #pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const int i = min(i0 + t * (int)blockDim.x, n - 1);
-                const int q = i / per, c = i - q * per;
-                v[t] = src[((size_t)token * k + (s_expert[q] >> 20)) * per + c];
-            }
-#pragma unroll
-            for (int t = 0; t < 4; ++t) {
-                const int i = i0 + t * (int)blockDim.x;
-                if (i < n) dst[i] = v[t];
-            }
-        }
-    }
+    for (int t = 0; t < PER; ++t) hdst[min((int)threadIdx.x + t * 256, n - 1)] = hv[t];
+    for (int i = threadIdx.x + PER * 256; i < n; i += 256) hdst[i] = piece(i);
     __syncthreads();
     const uint4* hs4 = reinterpret_cast<const uint4*>(hs);
 
@@ -380,7 +396,7 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__
 #pragma unroll
         for (int j = 0; j < RPW; ++j) out[j] = 0.f;
         for (int q0 = 0; q0 < k; q0 += KB) {
-            if (tile != wave || q0 != 0) request(tile, q0);
+            if (tile != wave || q0 != 0) request(tile, q0, std::false_type{});
 #pragma unroll
             for (int b = 0; b < KB; ++b) {
                 const int q = q0 + b;
