@@ -96,3 +96,104 @@ def test_format_refusals(card):
     assert L.btb_hip_gemv_fp8(p(z), p(s), 1, 8, p(x), p(y), 4, 64, 1, None) == -6       # 8-column blocks: not 16
     assert L.btb_hip_gemv_p12(p(z), p(z), p(z), None, None, 2, p(s), p(x), p(y), 4, 64, 1, None) == -1
     assert L.btb_hip_gemv_p12(p(z), p(z), p(z), None, None, 0, p(s), p(x), p(y), 4, 60, 1, None) == -6  # C % 16
+
+
+# ---- the verify widths (M >= 8): FP8 and MXFP4 widened into bf16 fragments for the matrix cores -------------------
+
+def _width_law(card, op, w, x, ref):
+    """the bar against the oracle at the full width; rows of an 8-row pass are the rows of the wide pass bit for bit
+    (native/cuda/btb_kernels.cu:84-88 for the family of tensor-core passes); the vector-ALU passes of the same rows
+    stay within the same bar of the matrix-core pass"""
+    y = op(w, x)
+    check(y, ref)
+    y8 = op(w, x[:8].contiguous())
+    assert torch.equal(y8.view(torch.int16), y[:8].view(torch.int16))
+    card.set_tuning("gemv_no_mfma", 1)
+    try:
+        v = op(w, x)
+    finally:
+        card.set_tuning("gemv_no_mfma", -1)
+    check(v, ref)
+    peak = float(y.float().abs().max())
+    assert float((v.float() - y.float()).abs().max()) <= peak * 2.0**-7
+
+
+@pytest.mark.parametrize("R,C,block", [(18432, 7168, (128, 128)), (2048, 7168, (128, 128)), (512, 1024, (128, 128)),
+                                       (1024, 2560, (128, 128)), (64, 256, (16, 16)), (50, 96, (50, 96))])
+@pytest.mark.parametrize("M", [8, 16, 12])
+def test_gemv_fp8_verify_widths(card, R, C, block, M):
+    """config C5a at its full shape and at shapes that take each of the matrix-core kernel's forms (rows of 2, 4, 8
+    waves; the wide form) and its fall-backs (rows not a multiple of 16)"""
+    src = weights_bf16(R, C, seed=330).float()
+    q, s = fp8.quantize(src, block)
+    x = acts_bf16(M, C, seed=331)
+    w = fp8.F8Weight(q.view(torch.uint8).cuda(), s.cuda(), R, C)
+    ref = oracle.gemv_fp8(q.view(torch.uint8).numpy(), s.numpy(), x.float().numpy(), threads=0)
+    _width_law(card, card.gemv_fp8, w, x.cuda(), ref)
+
+
+@pytest.mark.parametrize("R,C", [(18432, 7168), (2048, 7168), (1536, 2048), (2048, 768), (1024, 2560), (24, 64), (48, 32)])
+@pytest.mark.parametrize("M", [8, 16, 12])
+def test_gemv_mxfp4_verify_widths(card, R, C, M):
+    """config C5b at its full shape, the MoE expert shapes, and small shapes"""
+    src = weights_bf16(R, C, seed=340).float()
+    blocks, scales = mxfp4.quantize(src)
+    x = acts_bf16(M, C, seed=341)
+    w = mxfp4.MxWeight(blocks.reshape(-1).cuda(), scales.reshape(-1).cuda(), R, C)
+    ref = oracle.gemv_mxfp4(blocks.numpy(), scales.numpy(), R, C, x.float().numpy(), threads=0)
+    _width_law(card, card.gemv_mx4, w, x.cuda(), ref)
+
+
+@pytest.mark.parametrize("form", ["fp8", "mxfp4"])
+def test_full_shape_one_row_and_linearity(card, form):
+    """C5 at M = 1 on the full [18432, 7168] matrix against the oracle, and a size-independent property on top: the
+    matvec is linear in x up to the output's rounding - y(x1) + y(x2) against y over the f32 sum, each within the bar"""
+    R, C = 18432, 7168
+    src = weights_bf16(R, C, seed=350).float()
+    x = acts_bf16(2, C, seed=351)
+    if form == "fp8":
+        q, s = fp8.quantize(src, (128, 128))
+        w = fp8.F8Weight(q.view(torch.uint8).cuda(), s.cuda(), R, C)
+        op = card.gemv_fp8
+        ref = oracle.gemv_fp8(q.view(torch.uint8).numpy(), s.numpy(), x.float().numpy(), threads=0)
+    else:
+        blocks, scales = mxfp4.quantize(src)
+        w = mxfp4.MxWeight(blocks.reshape(-1).cuda(), scales.reshape(-1).cuda(), R, C)
+        op = card.gemv_mx4
+        ref = oracle.gemv_mxfp4(blocks.numpy(), scales.numpy(), R, C, x.float().numpy(), threads=0)
+    y1 = op(w, x[:1].contiguous().cuda())
+    check(y1, ref[:1])
+    both = op(w, x.cuda())
+    assert torch.equal(both[:1].view(torch.int16), y1.view(torch.int16))      # row 0 of the 2-row pass: the same bits
+    total = both.float().sum(dim=0).cpu().numpy()
+    want = ref.sum(axis=0)
+    assert np.abs(total - want).max() <= 1e-2 * np.abs(want).max()
+
+
+@pytest.mark.parametrize("M", [8, 16])
+def test_gemv_p12_verify_widths(card, M):
+    """12-bit matrices at the verify widths (passes of four rows of x): the oracle's bar, and row m's bits are those of
+    its one-row pass"""
+    R, C = 9728, 2560
+    w = weights_bf16(R, C, seed=360)
+    pw = P12Weight.pack(w.cuda(), card)
+    x = acts_bf16(M, C, seed=361)
+    y = card.gemv_p12(pw, x.cuda())
+    check(y, oracle.gemv_bf16(bits16(w), x.float().numpy()))
+    solo = card.gemv_p12(pw, x[M - 1 :].contiguous().cuda())
+    assert torch.equal(solo[0].view(torch.int16), y[M - 1].view(torch.int16))
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_the_head_shape(card, packed):
+    """the largest matrix of the step, the [151936, 2560] head (778 MB of bf16), stored as bf16 and as 12 bits a weight:
+    every logit against the oracle"""
+    R, C = 151936, 2560
+    w = weights_bf16(R, C, seed=370)
+    x = acts_bf16(1, C, seed=371)
+    ref = oracle.gemv_bf16(bits16(w), x.float().numpy())
+    if packed:
+        y = card.gemv_p12(P12Weight.pack(w.cuda(), card), x.cuda())
+    else:
+        y = card.gemv(w.cuda(), x.cuda())
+    check(y, ref)
