@@ -1,4 +1,4 @@
-"""Shared test helpers: seeded inputs in the shapes BASELINE names, an exact model of the f32 fused multiply-add for
+"""Shared test helpers: seeded inputs in the benchmark configurations' shapes, an exact model of the f32 fused multiply-add for
 brute-force checks, the f64 reference and the error measures the reference's own tests use."""
 
 from __future__ import annotations

@@ -1,6 +1,6 @@
 """The bf16 decode matvec on the GPU (through the C ABI) against the CPU oracle on the same seeded inputs.
 
-Bar (BASELINE.json north_star): max |y_gpu - y_ref| / max |y_ref| <= 1e-2 on the bf16 outputs, y_ref the oracle's f32
+Bar: max |y_gpu - y_ref| / max |y_ref| <= 1e-2 on the bf16 outputs, y_ref the oracle's f32
 result rounded to bf16. Both sides accumulate in f32 with one fused multiply-add per weight; they differ only in the
 order of the additions (<= ~sqrt(C) * 2^-24 relative to sum |w x|, far below a bf16 ulp), so what is seen is at most a
 bf16 rounding flip: 2^-8 relative to the output. The reference's own card bar, one bf16 ulp of the largest output

@@ -1,7 +1,7 @@
 """The routed MoE decode layer on the GPU (Qwen3-30B-A3B shape: hidden 2048, 128 experts, top-8, intermediate 768)
 against the CPU path restated in oracle/moe.py, on the same seeded inputs.
 
-Bars (BASELINE.json north_star): the top-k picks, as ordered lists, are bit-exact; the router's f32 logits are
+Bars: the top-k picks, as ordered lists, are bit-exact; the router's f32 logits are
 bit-exact (they are made in the CPU's order); the routing weights agree to one bf16 ulp (the two sides' expf may
 differ in the last bit); the layer output agrees within max relative error 1e-2 of the largest output (bf16 rows; the
 expert matvecs accumulate in f32 in a different order than the CPU's, which can flip a bf16 rounding of gu, h or d)."""
