@@ -37,7 +37,9 @@ struct MfBf16 {
     __device__ static __forceinline__ RowInfo row_info(const Mat&, int, int) { return RowInfo{}; }
     // p: the lane's row in the slab, at the step's first byte; g: the lane's 8-column group of the step
     // the step's scale for this lane (none here), requested a sub-block ahead of its use
-    __device__ static __forceinline__ uint32_t scale(const Mat&, const RowInfo&, int /*g*/, int /*step*/) { return 0u; }
+    template <int SB>
+    __device__ static __forceinline__ void scales(const Mat&, const RowInfo&, int /*g*/, int /*step0*/, int /*nsteps*/,
+                                                  uint32_t (&)[SB]) {}
     __device__ static __forceinline__ bf16x8 frag(const uint8_t* p, int g, uint32_t /*scale*/) {
         return __builtin_bit_cast(bf16x8, *reinterpret_cast<const uint4*>(p + g * 16));
     }
@@ -58,8 +60,42 @@ struct MfF8 {
     __device__ static __forceinline__ RowInfo row_info(const Mat& m, int row, int) {
         return RowInfo{m.scales + (size_t)(row / m.bm) * m.sc};
     }
-    __device__ static __forceinline__ uint32_t scale(const Mat& m, const RowInfo& ri, int g, int step) {
-        return f32_bits(ri.srow[(step * 32 + g * 8) / m.bn]);
+    // The scales of SB steps from step0 on, for the lane's row and its 8-column group g - every load unconditional (a
+    // step past the row's end takes the row's last scale, unused). Blocks a multiple of 128 columns wide, reached at
+    // a multiple of four steps: one scale serves four steps, a quarter of the loads. Otherwise one division finds
+    // the first block and the rest follow by stepping (a block is at least 16 columns, a step is 32).
+    template <int SB>
+    __device__ static __forceinline__ void scales(const Mat& m, const RowInfo& ri, int g, int step0, int nsteps,
+                                                  uint32_t (&scl)[SB]) {
+        const int last = (nsteps * 32 - 1) / m.bn;
+        if (m.bn % 128 == 0 && step0 % 4 == 0 && SB % 4 == 0) {
+            const int b0 = step0 * 32 / m.bn, per = m.bn / 128;  // `per` groups of four steps share a block
+            int left = per - (step0 / 4) % per, b = b0;
+#pragma unroll
+            for (int q = 0; q < SB / 4; ++q) {
+                const uint32_t v = f32_bits(ri.srow[min(b, last)]);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) scl[4 * q + t] = v;
+                if (--left == 0) {
+                    ++b;
+                    left = per;
+                }
+            }
+            return;
+        }
+        const int col0 = step0 * 32 + g * 8;
+        int b = col0 / m.bn, rem = col0 - b * m.bn;
+#pragma unroll
+        for (int t = 0; t < SB; ++t) {
+            scl[t] = f32_bits(ri.srow[min(b, last)]);
+            rem += 32;
+#pragma unroll
+            for (int k = 0; k < 2; ++k) {
+                const bool over = rem >= m.bn;
+                b += over ? 1 : 0;
+                rem -= over ? m.bn : 0;
+            }
+        }
     }
     __device__ static __forceinline__ bf16x8 frag(const uint8_t* p, int g, uint32_t scale) {
         const uint2 q = *reinterpret_cast<const uint2*>(p + g * 8);
@@ -83,8 +119,23 @@ struct MfMx4 {
     __device__ static __forceinline__ RowInfo row_info(const Mat& m, int row, int nsteps) {
         return RowInfo{m.scales + (size_t)row * nsteps};
     }
-    __device__ static __forceinline__ uint32_t scale(const Mat&, const RowInfo& ri, int /*g*/, int step) {
-        return (uint32_t)ri.srow[step];
+    // The e8m0 bytes of SB steps from step0 on (a step is one 32-weight block of the lane's row), unconditional: four
+    // bytes a load where the row's bytes are reached at a multiple of four (rows are a multiple of four blocks long
+    // then too, so the last word ends with the row), else a byte a load, a step past the end taking the last byte.
+    template <int SB>
+    __device__ static __forceinline__ void scales(const Mat& m, const RowInfo& ri, int /*g*/, int step0, int nsteps,
+                                                  uint32_t (&scl)[SB]) {
+        if (step0 % 4 == 0 && nsteps % 4 == 0 && SB % 4 == 0 && (reinterpret_cast<uintptr_t>(m.scales) & 3) == 0) {
+#pragma unroll
+            for (int q = 0; q < SB / 4; ++q) {
+                const uint32_t v = *reinterpret_cast<const uint32_t*>(ri.srow + min(step0 + 4 * q, nsteps - 4));
+#pragma unroll
+                for (int t = 0; t < 4; ++t) scl[4 * q + t] = (v >> (8 * t)) & 0xFFu;
+            }
+            return;
+        }
+#pragma unroll
+        for (int t = 0; t < SB; ++t) scl[t] = (uint32_t)ri.srow[min(step0 + t, nsteps - 1)];
     }
     __device__ static __forceinline__ bf16x8 frag(const uint8_t* p, int g, uint32_t scale) {
         const uint32_t q = *reinterpret_cast<const uint32_t*>(p + g * 4);
@@ -144,9 +195,7 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
     auto request = [&](int tile, int sb) {  // the loads of sub-block sb of the tile (R is a multiple of 16)
         const uint32_t valid = (uint32_t)(min(SB, n - sb * SB) * MF::STEPB);
         const typename MF::RowInfo rn = MF::row_info(mat, tile * 16 + li, nsteps);
-#pragma unroll
-        for (int t = 0; t < SB; ++t)
-            if (sb * SB + t < n) scl[t] = MF::scale(mat, rn, lg, s0 + sb * SB + t);
+        MF::template scales<SB>(mat, rn, lg, s0 + sb * SB, nsteps, scl);
 #pragma unroll
         for (int q = 0; q < NLD; ++q) {
             const uint8_t* base = mat.w + (size_t)(tile * 16 + q * RPI) * rowbytes + (size_t)(s0 + sb * SB) * MF::STEPB;
