@@ -145,4 +145,46 @@ __device__ __forceinline__ void use_keys(KeyBatch& kb, int key0, int k_end, int 
     }
 }
 
+// A workgroup's 16 key streams folded into one state per query head, in stream order. Each stream first brings its own
+// state to the workgroup's maximum (the 16 maxima meet in LDS; one exp2 per head and lane), then the scaled sums and
+// outputs are added up in stream order: thread (j, d) of 256 makes output d of head j, G * 128 / 256 of them a
+// thread, and hands it to `store(j, d, M, L, A)` (M and L are the head's; use them where d == 0). s_m and s_l hold
+// 16 * G floats, s_acc 16 * G * 128. 256 threads, all of them call.
+template <int G, class Store>
+__device__ __forceinline__ void fold_streams(float (&m)[G], float (&l)[G], float (&acc)[G][8], int grp, int dl,
+                                             float* s_m, float* s_l, float* s_acc, int tid, Store store) {
+    const float ninf = bits_f32(0xff800000u);
+    if (dl == 0) {
+#pragma unroll
+        for (int j = 0; j < G; ++j) s_m[grp * G + j] = m[j];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+        float M = ninf;
+#pragma unroll
+        for (int s2 = 0; s2 < 16; ++s2) M = fmaxf(M, s_m[s2 * G + j]);
+        const float f = m[j] == ninf ? 0.f : __builtin_amdgcn_exp2f(m[j] - M);
+        if (dl == 0) s_l[grp * G + j] = l[j] * f;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) s_acc[(grp * G + j) * AD + dl * 8 + e] = acc[j][e] * f;
+    }
+    __syncthreads();
+    for (int o = tid; o < G * AD; o += 256) {
+        const int j = o / AD, d = o - j * AD;
+        float A = 0.f;
+#pragma unroll
+        for (int s2 = 0; s2 < 16; ++s2) A += s_acc[(s2 * G + j) * AD + d];
+        float M = ninf, L = 0.f;
+        if (d == 0) {
+#pragma unroll
+            for (int s2 = 0; s2 < 16; ++s2) {
+                M = fmaxf(M, s_m[s2 * G + j]);
+                L += s_l[s2 * G + j];
+            }
+        }
+        store(j, d, M, L, A);
+    }
+}
+
 }  // namespace btb

@@ -165,35 +165,16 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
         load_keys(kb, Kh, Vh, rs, key0, k_end, -1);
         use_keys<G>(kb, key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, m, l, acc);
     }
-    // the 16 streams' states into LDS
-#pragma unroll
-    for (int j = 0; j < G; ++j) {
-        if (dl == 0) {
-            s_m[grp][j] = m[j];
-            s_l[grp][j] = l[j];
-        }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s_acc[grp][j][dl * 8 + e] = acc[j][e];
-    }
-    __syncthreads();
-    // fold them in stream order: thread (j, d) for d < D; G * D <= 1024 values over 256 threads
+    // the 16 streams folded in stream order, the workgroup's state out
     const size_t prow = ((size_t)t * Hk + g) * S + sp;  // this workgroup's slot among the partial states
-    for (int o = threadIdx.x; o < G * D; o += 256) {
-        const int j = o / D, d = o - j * D;
-        float M = bits_f32(0xff800000u);
-        for (int s2 = 0; s2 < 16; ++s2) M = fmaxf(M, s_m[s2][j]);
-        float L = 0.f, A = 0.f;
-        for (int s2 = 0; s2 < 16; ++s2) {
-            const float f = s_m[s2][j] == bits_f32(0xff800000u) ? 0.f : exp2f(s_m[s2][j] - M);
-            L = fmaf(s_l[s2][j], f, L);
-            A = fmaf(s_acc[s2][j][d], f, A);
-        }
-        part_acc[(prow * G + j) * D + d] = A;
-        if (d == 0) {
-            part_m[prow * G + j] = M;
-            part_l[prow * G + j] = L;
-        }
-    }
+    fold_streams<G>(m, l, acc, grp, dl, &s_m[0][0], &s_l[0][0], &s_acc[0][0][0], threadIdx.x,
+                    [&](int j, int d, float M, float L, float A) {
+                        part_acc[(prow * G + j) * D + d] = A;
+                        if (d == 0) {
+                            part_m[prow * G + j] = M;
+                            part_l[prow * G + j] = L;
+                        }
+                    });
 }
 
 // The step's own form (one row): the kernel reads the fused qkv row itself. Each workgroup norms and ropes the G query
@@ -275,33 +256,15 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
         key0 += 16 * KB;
         if (key0 < k_end) load_keys(kb, Kh, Vh, rs, key0, k_end, n0);
     }
-#pragma unroll
-    for (int j = 0; j < G; ++j) {
-        if (dl == 0) {
-            s_m[grp][j] = m[j];
-            s_l[grp][j] = l[j];
-        }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s_acc[grp][j][dl * 8 + e] = acc[j][e];
-    }
-    __syncthreads();
     const size_t prow = (size_t)g * S + sp;
-    for (int o = threadIdx.x; o < G * D; o += 256) {
-        const int j = o / D, d = o - j * D;
-        float M = bits_f32(0xff800000u);
-        for (int s2 = 0; s2 < 16; ++s2) M = fmaxf(M, s_m[s2][j]);
-        float L = 0.f, A = 0.f;
-        for (int s2 = 0; s2 < 16; ++s2) {
-            const float f = s_m[s2][j] == bits_f32(0xff800000u) ? 0.f : exp2f(s_m[s2][j] - M);
-            L = fmaf(s_l[s2][j], f, L);
-            A = fmaf(s_acc[s2][j][d], f, A);
-        }
-        part_acc[(prow * G + j) * D + d] = A;
-        if (d == 0) {
-            part_m[prow * G + j] = M;
-            part_l[prow * G + j] = L;
-        }
-    }
+    fold_streams<G>(m, l, acc, grp, dl, &s_m[0][0], &s_l[0][0], &s_acc[0][0][0], threadIdx.x,
+                    [&](int j, int d, float M, float L, float A) {
+                        part_acc[(prow * G + j) * D + d] = A;
+                        if (d == 0) {
+                            part_m[prow * G + j] = M;
+                            part_l[prow * G + j] = L;
+                        }
+                    });
 }
 
 // the spans' states folded in span order: one workgroup per (row, kv head). Launched right after attn_decode_kernel,

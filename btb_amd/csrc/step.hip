@@ -520,36 +520,17 @@ __device__ __forceinline__ void attention_item(const StepArgs& a, const StepLaye
         key0 += 16 * KB;
         if (key0 < k_end) load_keys(kb, Kh, Vh, a.rs, key0, k_end, n0);
     }
-#pragma unroll
-    for (int j = 0; j < G; ++j) {
-        if (dl == 0) {
-            s_m[grp * G + j] = m[j];
-            s_l[grp * G + j] = l[j];
-        }
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s_acc[(grp * G + j) * AD + dl * 8 + e] = acc[j][e];
-    }
-    __syncthreads();
     float* part_m = a.part;
     float* part_l = a.part + (size_t)Hq * a.S;
     float* part_acc = a.part + 2 * (size_t)Hq * a.S;
     const size_t prow = (size_t)g * a.S + sp;
-    for (int o = tid; o < G * AD; o += 256) {
-        const int j = o / AD, d = o - j * AD;
-        float M = bits_f32(0xff800000u);
-        for (int s2 = 0; s2 < 16; ++s2) M = fmaxf(M, s_m[s2 * G + j]);
-        float Lsum = 0.f, A = 0.f;
-        for (int s2 = 0; s2 < 16; ++s2) {
-            const float f = s_m[s2 * G + j] == bits_f32(0xff800000u) ? 0.f : exp2f(s_m[s2 * G + j] - M);
-            Lsum = fmaf(s_l[s2 * G + j], f, Lsum);
-            A = fmaf(s_acc[(s2 * G + j) * AD + d], f, A);
-        }
+    fold_streams<G>(m, l, acc, grp, dl, s_m, s_l, s_acc, tid, [&](int j, int d, float M, float Lsum, float A) {
         st_dev(&part_acc[(prow * G + j) * AD + d], A);
         if (d == 0) {
             st_dev(&part_m[prow * G + j], M);
             st_dev(&part_l[prow * G + j], Lsum);
         }
-    }
+    });
     // the head's arrival count only ever counts up (S arrivals a layer): the workgroup that brings it to a multiple of
     // S came last, every other span's state was complete before its own arrival, and it folds the head
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
