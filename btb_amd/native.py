@@ -13,7 +13,7 @@ from __future__ import annotations
 import ctypes
 import os
 from collections.abc import Sequence
-from typing import Any
+from typing import Any, Sequence
 
 import torch
 
@@ -114,6 +114,36 @@ def _stream() -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+
+def _launch_table() -> dict[str, tuple[int, Any]]:
+    """reference kernel name -> (its parameter count, parameters -> (entry point, its arguments less the stream))"""
+    t: dict[str, tuple[int, Any]] = {}
+    for M in (1, 2, 4, 8, 16, 32):
+        t[f"btb_gemv_bf16_m{M}"] = (5, lambda v, g, M=M: ("btb_hip_gemv_bf16", (v[0], v[1], v[2], v[3], v[4], M)))
+        t[f"btb_gemv_silu_bf16_m{M}"] = (5, lambda v, g, M=M: ("btb_hip_gemv_silu_bf16", (v[0], v[1], v[2], v[3], v[4], M)))
+        t[f"btb_gemv_lane16_f32_m{M}"] = (5, lambda v, g, M=M: ("btb_hip_gemv_bf16_rows", (v[0], v[3], v[4], v[1], M, v[2])))
+        t[f"btb_gemv_lane16_mx4_f32_m{M}"] = (
+            6, lambda v, g, M=M: ("btb_hip_gemv_mxfp4_rows", (v[0], v[1], v[4], v[5], v[2], M, v[3])))
+    for n in ("btb_gemv_mma_bf16", "btb_gemv_mma8_bf16"):
+        t[n] = (6, lambda v, g: ("btb_hip_gemv_bf16", (v[0], v[1], v[2], v[3], v[4], v[5])))
+    t["btb_gemv_mma_glu_silu"] = (6, lambda v, g: ("btb_hip_gemv_glu_silu_bf16", (v[0], v[1], v[2], v[3], v[4], v[5])))
+    t["btb_silu_mul"] = (4, lambda v, g: ("btb_hip_silu_mul", (v[0], v[1], v[2], v[3])))
+    # btb_add_rmsnorm(h, y, w, eps, x, H, centered), a block a row
+    t["btb_add_rmsnorm"] = (7, lambda v, g: ("btb_hip_add_rmsnorm", (v[0], v[1], v[2], v[3], v[4], g[0], v[5], v[6])))
+    for D in (64, 128, 256):
+        # (qkv, wq, wk, eps, cos, sin, n0, depth, K, V, q, T, Hq, Hk, hs, rs, centered)
+        t[f"btb_norm_rope_kv_d{D}"] = (17, lambda v, g, D=D: ("btb_hip_norm_rope_kv", (
+            v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], v[9], v[10], v[11], v[12], v[13], D, v[14], v[15], v[16])))
+    # btb_moe_route(logits bf16, ls, E, k, idx, w, hidx, hw, cnt, seq, hseq), a block a row; the host copies are the
+    # reference's way of fetching experts from the host tier and are not made here
+    t["btb_moe_route"] = (11, lambda v, g: ("btb_hip_moe_route", (v[0], 0, v[1], v[2], v[3], g[0], v[4], v[5], None)))
+    # btb_mx4_widen(blocks, scales, seats, groups, out), grid.y seats
+    t["btb_mx4_widen"] = (5, lambda v, g: ("btb_hip_mx4_widen", (v[0], v[1], v[2], g[1], v[3], v[4], 0)))
+    return t
+
+
+_LAUNCH = _launch_table()
+
 class HipCard:
     """The card's operators over torch tensors. `GEMV_ROWS` are the pass widths the reference's card graphs are
     captured at (btb/engine/native.py:1918); any M up to 1024 is taken here."""
@@ -151,6 +181,35 @@ class HipCard:
         if not isinstance(t, torch.Tensor) or t.dtype != dtype or not t.is_cuda or not t.is_contiguous():
             raise ValueError(f"[hip] {what} must be a contiguous {dtype} tensor on the GPU, got "
                              f"{getattr(t, 'dtype', type(t))} {getattr(t, 'device', '')}")
+
+    # -- the reference's launcher surface: kernels by name -------------------------------------------------------
+
+    def launch(self, name: str, grid: tuple[int, int, int], block: tuple[int, int, int], args: Sequence[Any],
+               stream: torch.cuda.Stream | None = None, shared: int = 0) -> None:
+        """The reference's `Launcher.launch` (btb/engine/card_launch.py:428-440) for the kernels of this path: `name`
+        is the reference kernel's name, `args` its parameters in its own order (native/cuda/btb_kernels.cu,
+        btb_gemv_mma.cuh), one ctypes value (or int / float) each. `block` and `shared` are the CUDA kernel's and
+        mean nothing here - the library picks its own wave64 geometry - and of `grid` only what carries a size is
+        read (rows in grid[0] for btb_add_rmsnorm and btb_moe_route, seats in grid[1] for btb_mx4_widen). The
+        parameter count is checked before anything is launched; an unknown name is a KeyError naming it."""
+        entry = _LAUNCH.get(name)
+        if entry is None:
+            raise KeyError(f"[hip] {name} is not a kernel of this path ({len(_LAUNCH)} are: see HipCard.fn)")
+        count, call = entry
+        if len(args) != count:
+            raise ValueError(f"[hip] {name} takes {count} parameters, got {len(args)}")
+        vals = [a.value if isinstance(a, ctypes._SimpleCData) else a for a in args]
+        st = ctypes.c_void_p((stream or torch.cuda.current_stream()).cuda_stream)
+        sym, cargs = call(vals, tuple(int(g) for g in grid))
+        self._call(sym, *cargs, st)
+
+    @property
+    def fn(self) -> dict[str, str]:
+        """kernel name -> the library entry point that serves it (the reference keeps its loaded kernels here)"""
+        return {n: call([0] * count, (1, 1, 1))[0] for n, (count, call) in _LAUNCH.items()}
+
+    def close(self) -> None:
+        """nothing to release (the library stays loaded for the process); may be called any number of times"""
 
     # -- bf16 matvec ------------------------------------------------------------------------------------------
 
