@@ -88,10 +88,13 @@ __device__ __forceinline__ void load_keys(KeyBatch& kb, const uint16_t* Kh, cons
 // the whole batch, and the batch's weights; then each value row, widened once, meets all G heads. A key past the
 // span's end scores -inf and weighs 0. qp: the heads' q, this lane's 8 dims as 4 bf16 pairs. own >= 0: the step's
 // own row is key `own` and is taken from LDS (s_k, s_v) - the cache's copy may not have landed yet.
+// tree_base >= 0: the keys from slot tree_base on are the pass's own rows, and of those the row sees the ones whose
+// bit is set in tree_mask (its ancestors and itself: a verify pass's tree).
 template <int G>
 __device__ __forceinline__ void use_keys(KeyBatch& kb, int key0, int k_end, int own, const uint16_t* s_k,
                                          const uint16_t* s_v, int dl, const uint32_t (&qp)[G][4], float scale_log2,
-                                         float (&m)[G], float (&l)[G], float (&acc)[G][8]) {
+                                         float (&m)[G], float (&l)[G], float (&acc)[G][8], int tree_base = -1,
+                                         uint32_t tree_mask = 0u) {
     const float ninf = bits_f32(0xff800000u);
     if (own >= 0) {  // uniform: only the workgroup whose span holds the slot gets here with own set
 #pragma unroll
@@ -105,7 +108,9 @@ __device__ __forceinline__ void use_keys(KeyBatch& kb, int key0, int k_end, int 
 #pragma unroll
     for (int b = 0; b < KB; ++b) {
         const uint4 kr = kb.k[b];
-        const bool live = key0 + 16 * b < k_end;
+        const int key = key0 + 16 * b;
+        bool live = key < k_end;
+        if (tree_base >= 0) live = live && (key < tree_base || ((tree_mask >> min(key - tree_base, 31)) & 1u) != 0u);
 #pragma unroll
         for (int j = 0; j < G; ++j) {
             float sc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr.x), __builtin_bit_cast(bf16x2, qp[j][0]), 0.f, false);
@@ -121,11 +126,14 @@ __device__ __forceinline__ void use_keys(KeyBatch& kb, int key0, int k_end, int 
         float mn = m[j];
 #pragma unroll
         for (int b = 0; b < KB; ++b) mn = fmaxf(mn, w[b][j]);
-        const float corr = __builtin_amdgcn_exp2f(m[j] - mn);  // 0 on the stream's first batch (m = -inf)
+        // a tree pass can hand a stream a batch none of whose keys the row sees while the stream has seen none yet:
+        // the maximum is still -inf then, and the batch must leave the state as it is (not -inf - -inf)
+        const bool none = tree_base >= 0 && mn == ninf;
+        const float corr = none ? 1.f : __builtin_amdgcn_exp2f(m[j] - mn);  // 0 on the stream's first keys (m = -inf)
         float lj = l[j] * corr;
 #pragma unroll
         for (int b = 0; b < KB; ++b) {
-            w[b][j] = __builtin_amdgcn_exp2f(w[b][j] - mn);
+            w[b][j] = none ? 0.f : __builtin_amdgcn_exp2f(w[b][j] - mn);
             lj += w[b][j];
         }
         l[j] = lj;

@@ -125,7 +125,8 @@ constexpr int ATT_MAXG = 8;
 template <int G>
 __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ K,
                                                           const uint16_t* __restrict__ V,
-                                                          const int32_t* __restrict__ n0p, int Hq, int Hk, long long hs,
+                                                          const int32_t* __restrict__ n0p,
+                                                          const int32_t* __restrict__ par, int T, int Hq, int Hk, long long hs,
                                                           long long rs, float scale_log2, float* __restrict__ part_m,
                                                           float* __restrict__ part_l, float* __restrict__ part_acc,
                                                           int span) {
@@ -136,7 +137,18 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int sub = lane >> 4, dl = lane & 15;   // the lane's key within a quad of keys, its 8 dims
     const int grp = wv * 4 + sub;                // one of the workgroup's 16 key streams
-    const int n = *n0p + t + 1;                  // row t sees the cache's keys and the pass's rows up to itself
+    // a chain of rows (par null): row t sees the cache's keys and the pass's rows up to itself. A tree (par[t] the
+    // row's parent among the pass's rows, -1 at a root; the reference's TREE form, native/cuda/btb_attn_flash.cuh:
+    // 284-286, 407-419): the cache's keys, and of the pass's rows - slots n0 .. n0 + T - 1 - its ancestors and itself
+    const int n0 = *n0p;
+    int tree_base = -1;
+    uint32_t tree_mask = 0u;
+    int n = n0 + t + 1;
+    if (par != nullptr) {
+        tree_base = n0;
+        n = n0 + T;
+        for (int p = t, hops = 0; p >= 0 && p < T && hops < 32; p = par[p], ++hops) tree_mask |= 1u << p;
+    }
     const int k_begin = sp * span, k_end = min(n, k_begin + span);
 
     // the row's G query heads, the lane's 8 dims of each as bf16 pairs (the scale meets the folded score)
@@ -163,7 +175,7 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     for (int key0 = k_begin + grp; key0 < k_end; key0 += 16 * KB) {
         KeyBatch kb;
         load_keys(kb, Kh, Vh, rs, key0, k_end, -1);
-        use_keys<G>(kb, key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, m, l, acc);
+        use_keys<G>(kb, key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, m, l, acc, tree_base, tree_mask);
     }
     // the 16 streams folded in stream order, the workgroup's state out
     const size_t prow = ((size_t)t * Hk + g) * S + sp;  // this workgroup's slot among the partial states
@@ -468,9 +480,9 @@ size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, siz
     return T * Hq * S * (2 + D);
 }
 
-int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0, size_t T,
-                            size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap, size_t S,
-                            float* scratch, void* stream) {
+int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
+                            const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
+                            float scale, size_t cap, size_t S, float* scratch, void* stream) {
     if (q == nullptr || K == nullptr || V == nullptr || att == nullptr || n0 == nullptr || scratch == nullptr)
         return ERR_NULL;
     if (T == 0 || Hq == 0 || Hk == 0 || S == 0 || cap == 0 || T > 65535 || S > 1024 || Hq % Hk != 0 || hs <= 0 ||
@@ -481,7 +493,11 @@ int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* a
         set_error("attn_decode: head_dim 128 and at most 8 query heads per kv head");
         return ERR_DOMAIN;
     }
-    if (!al(q, 16) || !al(K, 16) || !al(V, 16) || (rs % 8) != 0 || (hs % 8) != 0) return ERR_DOMAIN;
+    if (!al(q, 16) || !al(K, 16) || !al(V, 16) || !al(par, 4) || (rs % 8) != 0 || (hs % 8) != 0) return ERR_DOMAIN;
+    if (par != nullptr && T > 32) {
+        set_error("attn_decode: a tree pass holds at most 32 rows");
+        return ERR_DOMAIN;
+    }
     const int span = (int)((cap + S - 1) / S);
     float* part_m = scratch;
     float* part_l = scratch + T * Hq * S;
@@ -493,8 +509,8 @@ int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* a
     const size_t mlds = 2 * S * G * sizeof(float);
 #define ATT(GG)                                                                                                      \
     hipLaunchKernelGGL(attn_decode_kernel<GG>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(q),              \
-                       static_cast<const uint16_t*>(K), static_cast<const uint16_t*>(V), n0, (int)Hq, (int)Hk,        \
-                       (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, span);                     \
+                       static_cast<const uint16_t*>(K), static_cast<const uint16_t*>(V), n0, par, (int)T, (int)Hq,   \
+                       (int)Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, span);            \
     hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,       \
                        (int)Hk, (int)S, part_m, part_l, part_acc)
     switch (G) {

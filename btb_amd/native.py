@@ -60,7 +60,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_norm_rope_kv": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
                                     _sz, ctypes.c_int64, ctypes.c_int64, _i32, _vp]),
     "btb_hip_attn_scratch_floats": (_sz, [_sz, _sz, _sz, _sz, _sz]),
-    "btb_hip_attn_decode": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
+    "btb_hip_attn_decode": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
                                    ctypes.c_float, _sz, _sz, _vp, _vp]),
     "btb_hip_attn_decode_qkv": (_i32, [_vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
                                        ctypes.c_int64, ctypes.c_int64, ctypes.c_float, _sz, _sz, _vp, _vp]),
@@ -552,8 +552,11 @@ class HipCard:
         return torch.empty(n, dtype=torch.float32, device=device)
 
     def attn_decode(self, q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, att: torch.Tensor, n0: torch.Tensor,
-                    Hq: int, Hk: int, D: int, scale: float, S: int, scratch: torch.Tensor) -> None:
-        """att [T, Hq * D] = the rows' attention over the cache (row t sees keys 0 .. n0 + t)"""
+                    Hq: int, Hk: int, D: int, scale: float, S: int, scratch: torch.Tensor,
+                    par: torch.Tensor | None = None) -> None:
+        """att [T, Hq * D] = the rows' attention over the cache: row t sees keys 0 .. n0 + t, or with `par` (int32 [T],
+        a verify pass's tree: the row's parent among the pass's rows, -1 at a root) the cache's n0 keys and, of the
+        pass's rows, its ancestors and itself"""
         self._need(q, torch.bfloat16, "q")
         self._need(att, torch.bfloat16, "att")
         self._need(n0, torch.int32, "n0")
@@ -564,8 +567,13 @@ class HipCard:
         need = int(self.lib.btb_hip_attn_scratch_floats(T, Hq, Hk, D, S))
         if scratch.numel() < need:
             raise ValueError(f"[hip] attn_decode: scratch holds {scratch.numel()} floats, {need} are needed")
-        self._call("btb_hip_attn_decode", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0), T, Hq, Hk,
-                   D, int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S, self.ptr(scratch), _stream())
+        if par is not None:
+            self._need(par, torch.int32, "par")
+            if par.numel() != T:
+                raise ValueError(f"[hip] attn_decode: par names {par.numel()} rows, the pass has {T}")
+        self._call("btb_hip_attn_decode", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0),
+                   None if par is None else self.ptr(par), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)),
+                   float(scale), int(K.shape[1]), S, self.ptr(scratch), _stream())
 
     def attn_decode_qkv(self, qkv: torch.Tensor, wq: torch.Tensor | None, wk: torch.Tensor | None, eps: float,
                         cos_t: torch.Tensor, sin_t: torch.Tensor, n0: torch.Tensor, K: torch.Tensor, V: torch.Tensor,

@@ -212,14 +212,17 @@ int32_t btb_hip_norm_rope_kv(const void* qkv, const void* wq, const void* wk, fl
 /* floats of scratch btb_hip_attn_decode needs for T rows and S key spans */
 size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, size_t S);
 
-/* Decode attention: att [T, Hq * D] = softmax(q K^T * scale) V, row t over the keys 0 .. *n0 + t, f32 throughout,
- * bf16 out. The keys (capacity `cap`) are cut into S spans, a workgroup per (kv head, span, row) leaving its
+/* Decode attention: att [T, Hq * D] = softmax(q K^T * scale) V, f32 throughout, bf16 out. par NULL: a chain of rows,
+ * row t over the keys 0 .. *n0 + t. par given (a verify pass's tree, T <= 32: par[t] the row's parent among the
+ * pass's rows, -1 at a root): row t over the cache's keys 0 .. *n0 - 1 and, of the pass's own rows at slots
+ * *n0 .. *n0 + T - 1, its ancestors and itself - the reference's TREE form (native/cuda/btb_attn_flash.cuh:284-286,
+ * 407-419). The keys (capacity `cap`) are cut into S spans, a workgroup per (kv head, span, row) leaving its
  * online-softmax state in `scratch` (btb_hip_attn_scratch_floats floats); a second small launch folds the spans in
  * span order. head_dim 128, Hq / Hk in {1, 2, 4, 8}, S <= 1024. Replaces btb_attn_flash_d128's decode form
- * (native/cuda/btb_attn_flash.cuh:277-675) for a chain of rows. */
-int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0, size_t T,
-                            size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap, size_t S,
-                            float* scratch, void* stream);
+ * (native/cuda/btb_attn_flash.cuh:277-675); the cache's row map (`tbl`) and the window are not taken. */
+int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
+                            const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
+                            float scale, size_t cap, size_t S, float* scratch, void* stream);
 
 /* The decode step's own attention (one row), straight from the fused qkv row [(Hq + 2 Hk) D] bf16: what
  * btb_hip_norm_rope_kv followed by btb_hip_attn_decode compute at T = 1, bit for bit, in one launch less - the

@@ -94,6 +94,48 @@ def test_attn_decode_against_f64(card, n0, T, Hq, Hk, S):
         assert worst <= 2.0**-7, worst
 
 
+@pytest.mark.parametrize("n0,T,Hq,Hk,S,seed", [(300, 8, 32, 8, 5, 0), (0, 5, 8, 2, 1, 1), (63, 32, 16, 2, 7, 2),
+                                                (1000, 16, 8, 1, 16, 3)])
+def test_attn_decode_over_a_tree_of_rows(card, n0, T, Hq, Hk, S, seed):
+    """a verify pass's tree (the reference's TREE form, native/cuda/btb_attn_flash.cuh:284-286): row t sees the cache's
+    n0 keys and, of the pass's own rows, its ancestors and itself - against f64 attention over exactly those keys; a
+    tree that is a chain gives the chain form's bits"""
+    D = 128
+    cap = n0 + T + 3
+    g = gen(650 + seed)
+    K = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    V = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    q = torch.randn(T, Hq * D, generator=g).to(torch.bfloat16)
+    par = [-1] + [int(torch.randint(-1, t, (1,), generator=g)) for t in range(1, T)]   # any earlier row, or a new root
+    part = torch.tensor(par, dtype=torch.int32, device="cuda")
+    att = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+    scratch = card.attn_scratch(T, Hq, Hk, D, S)
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    scale = 1.0 / np.sqrt(D)
+    card.attn_decode(q.cuda(), K.cuda(), V.cuda(), att, n0t, Hq, Hk, D, scale, S, scratch, par=part)
+    got = att.float().cpu().numpy()
+    for t in range(T):
+        seen, p_ = [], t
+        while p_ >= 0:
+            seen.append(n0 + p_)
+            p_ = par[p_]
+        keys = list(range(n0)) + sorted(seen)
+        want = od.attention(q[t].float().numpy().reshape(Hq, D), K[:, keys].float().numpy(), V[:, keys].float().numpy(),
+                            scale)
+        worst = np.abs(got[t].reshape(Hq, D) - want).max() / np.abs(want).max()
+        assert worst <= 2.0**-7, (t, worst)
+    chain = torch.arange(-1, T - 1, dtype=torch.int32, device="cuda")
+    a = torch.zeros_like(att)
+    b = torch.zeros_like(att)
+    card.attn_decode(q.cuda(), K.cuda(), V.cuda(), a, n0t, Hq, Hk, D, scale, S, scratch, par=chain)
+    card.attn_decode(q.cuda(), K.cuda(), V.cuda(), b, n0t, Hq, Hk, D, scale, S, scratch)
+    assert torch.equal(a, b)
+    with pytest.raises(Exception):
+        card.attn_decode(torch.zeros(33, Hq * D, dtype=torch.bfloat16, device="cuda"), K.cuda(), V.cuda(),
+                         torch.zeros(33, Hq * D, dtype=torch.bfloat16, device="cuda"), n0t, Hq, Hk, D, scale, 1,
+                         card.attn_scratch(33, Hq, Hk, D, 1), par=torch.zeros(33, dtype=torch.int32, device="cuda"))
+
+
 @pytest.mark.parametrize("n0,Hq,Hk,S", [(4096, 32, 8, 36), (100, 32, 8, 4), (0, 8, 8, 1), (63, 16, 2, 7), (64, 16, 2, 2),
                                          (500, 8, 1, 16), (31, 4, 2, 3), (300, 8, 1, 40), (200, 4, 4, 5)])
 @pytest.mark.parametrize("with_norm", [True, False])
