@@ -138,6 +138,10 @@ class DecodeStep:
         self.host_n0 = torch.zeros(1, dtype=torch.int32).pin_memory()
         self.host_ts = torch.zeros(1, dtype=torch.int64).pin_memory()
         self.graph: torch.cuda.CUDAGraph | None = None
+        # a pass of several rows is a chain unless `set_tree` says otherwise: each row's parent among the pass's rows
+        # and its depth (the rope position past the cache), read by the kernels from these two device tensors
+        self.par = torch.arange(-1, self.T - 1, dtype=torch.int32, device=dev) if self.T > 1 else None
+        self.depth = torch.arange(self.T, dtype=torch.int32, device=dev) if self.T > 1 else None
         self.persistent = bool(persistent)
         if self.persistent:
             self._bind_persistent(workgroups, trace)
@@ -214,6 +218,23 @@ class DecodeStep:
         self.n0.fill_(int(n0))
         self.ids.fill_(int(token))
 
+    def set_tree(self, par: list[int] | None) -> None:
+        """the pass's rows as a tree (a speculative verify pass: the reference's `par` / `depth` arguments,
+        native/cuda/btb_attn_flash.cuh:284-286, btb_kernels.cu:330-335): par[t] is row t's parent among the pass's
+        rows, -1 for a root (a child of the cache's last row); a row attends to the cache, its ancestors and itself
+        and takes the rope position n0 + its depth. None: a chain. Written into the tensors a captured graph reads."""
+        if self.T == 1:
+            raise ValueError("[decode] a pass of one row has no tree")
+        if par is None:
+            par = list(range(-1, self.T - 1))
+        if len(par) != self.T or self.T > 32 or any(not -1 <= p < t for t, p in enumerate(par)):
+            raise ValueError("[decode] par names, for each of at most 32 rows, an earlier row of the pass or -1")
+        depth = []
+        for p in par:
+            depth.append(0 if p < 0 else depth[p] + 1)
+        self.par.copy_(torch.tensor(par, dtype=torch.int32))
+        self.depth.copy_(torch.tensor(depth, dtype=torch.int32))
+
     def weight_bytes(self) -> int:
         """bytes of linear weights one step streams"""
         n = sum(self.w[f"layers.{i}.{k}"].nbytes for i in range(self.cfg.layers) for k in ("qkv", "o", "gu", "down"))
@@ -245,8 +266,8 @@ class DecodeStep:
             k.add_rmsnorm(self.h, y_prev, w[L + "ln1"], cfg.eps, self.x)
             w[L + "qkv"].matvec(self.x, self.qkv)
             k.norm_rope_kv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K, V,
-                           self.q, Hq, Hk, D)
-            k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch)
+                           self.q, Hq, Hk, D, depth=self.depth)
+            k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch, par=self.par)
             w[L + "o"].matvec(self.att, self.y)
             k.add_rmsnorm(self.h, self.y, w[L + "ln2"], cfg.eps, self.x)
             w[L + "gu"].matvec(self.x, self.gu)
@@ -281,8 +302,9 @@ class DecodeStep:
                                   V, self.att, Hq, Hk, D, self.scale, self.S, self.scratch)
             else:
                 k.norm_rope_kv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K, V,
-                               self.q, Hq, Hk, D)
-                k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch)
+                               self.q, Hq, Hk, D, depth=self.depth)
+                k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch,
+                              par=self.par)
             w[L + "o"].matvec(self.att, self.y)
             k.gemv_norm(w[L + "gu"].w, hb, self.y, w[L + "ln2"], cfg.eps, ha, self.m, glu=True)
             w[L + "down"].matvec(self.m, self.y)

@@ -186,3 +186,33 @@ def test_persistent_step_replays_as_a_graph(card):
         junk = torch.randn(1 << 16, device="cuda").sum()
         torch.cuda.synchronize()
         assert torch.isfinite(junk)
+
+
+@pytest.mark.parametrize("fused", [False, True])
+def test_verify_pass_over_a_tree(card, fused):
+    """a pass of several rows as a tree (speculative verify): the rows on a root-to-leaf path see exactly what they see
+    as a chain pass of that path's tokens, so their logits agree with that pass's - to the step's bar, not to the bit:
+    the attention folds the same keys in batches cut elsewhere - and a tree that is a chain is the chain pass bit for
+    bit"""
+    _, dev, kv = make_weights(card, False)
+    par, toks = [-1, 0, 0, 2, 2], [17, 5, 901, 33, 4]
+
+    def run(T, tokens, tree):
+        step = DecodeStep(card, CFG, dev, CAP, T=T, fused=fused, fold_silu=fused)
+        step.kv.copy_(kv.cuda())
+        step.reset(N0, tokens[0])
+        step.ids.copy_(torch.tensor(tokens, dtype=torch.int32))
+        if tree is not None:
+            step.set_tree(tree)
+        step.body()
+        torch.cuda.synchronize()
+        return step.logits.float().clone()
+
+    tree = run(5, toks, par)
+    for path in ([0, 1], [0, 2, 3], [0, 2, 4]):
+        chain = run(len(path), [toks[t] for t in path], None)
+        for i, t in enumerate(path):
+            assert float((tree[t] - chain[i]).abs().max()) <= 3e-2 * float(chain[i].abs().max()), (path, t)
+    a = run(4, toks[:4], [-1, 0, 1, 2])
+    b = run(4, toks[:4], None)
+    assert torch.equal(a, b)
