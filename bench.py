@@ -49,10 +49,19 @@ def cpu_baseline(budget_s: float = 12.0) -> dict:
         oracle.gemv_bf16(pool[calls % len(pool)], x, threads=0)
         calls += 1
     dt = time.perf_counter() - t0
-    gbs = calls * (R * C * 2 + C * 4 + R * 4) / dt / 1e9
+    per_call = R * C * 2 + C * 4 + R * 4
+    gbs = calls * per_call / dt / 1e9
+    # the same matvec on one thread (the reference's own criterion bench pins one: native/benches/gemv.rs:8-10)
+    t1 = time.perf_counter()
+    solo = 0
+    while time.perf_counter() - t1 < budget_s / 4:
+        oracle.gemv_bf16(pool[solo % len(pool)], x, threads=1)
+        solo += 1
+    d1 = time.perf_counter() - t1
     return {"value": round(gbs, 2), "unit": "GB/s", "cores": cores, "kind": "port", "isa": oracle.isa(),
+            "one_thread_gbs": round(solo * per_call / d1 / 1e9, 2),
             "sample": f"{calls} bf16 matvecs [{R}x{C}] (the gate_up shape), 12 distinct matrices (1.2 GB) in rotation, "
-                      f"f32 x and y, all {cores} host threads, {dt:.1f} s"}
+                      f"f32 x and y, all {cores} host threads, {dt:.1f} s; then {solo} on one thread, {d1:.1f} s"}
 
 
 def kernel_workload(args: argparse.Namespace) -> int:
@@ -83,9 +92,9 @@ def kernel_workload(args: argparse.Namespace) -> int:
 
     name = args.workload
     if name == "moe":
-        # two layers' stacks (3.6 GB) and eight sets of rows: every call routes to other experts, so a pass streams
-        # 0.6 GB (one token) to 3 GB of distinct expert matrices - nothing comes back out of the 256 MB cache
-        E, k, H, I, pool = 128, 8, 2048, 768, 8
+        # two layers' stacks (3.6 GB) and sixteen sets of rows: every call routes to other experts, so a pass streams
+        # 1.2 GB (one token) and more of distinct expert matrices - nothing comes back out of the 256 MB cache
+        E, k, H, I, pool = 128, 8, 2048, 768, 16
         sets = [(Router(card, normal(E, H).to(torch.bfloat16), k), Experts(card, normal(E, 2 * I, H).to(torch.bfloat16),
                                                                            normal(E, H, I).to(torch.bfloat16)))
                 for _ in range(2)]
@@ -107,9 +116,10 @@ def kernel_workload(args: argparse.Namespace) -> int:
         dtype = "bf16 weights and activations, f32 accumulate"
     else:
         R, C = (9728, 2560) if name in ("gemv_bf16", "gemv_p12") else (18432, 7168)
-        # operands of a pass: at least 600 MB of stored weights, well past the 256 MB last-level cache
+        # operands of a pass: over 1 GiB of stored weights, past four times the 256 MB last-level cache (the reference's
+        # own rule for its timing pools: btb/machine.py:384-426)
         per = {"gemv_bf16": 2.0, "gemv_p12": 1.5, "gemv_fp8": 1.0, "gemv_mxfp4": 17 / 32}[name] * R * C
-        pool = max(4, -(-600_000_000 // int(per)))
+        pool = max(4, -(-1_100_000_000 // int(per)))
         mats = []
         for _ in range(pool):
             t = normal(R, C)
