@@ -195,4 +195,101 @@ __device__ __forceinline__ void fold_streams(float (&m)[G], float (&l)[G], float
     }
 }
 
+// The S spans' states of one (row, kv head) folded in span order by a workgroup of 256 into G * 128 outputs
+// bf16(O / L). Every state a thread needs in the first pass - the spans' maxima and sums, and 32 spans' partial
+// outputs of its G / 2 outputs (one, for a single query head) - is requested before anything waits: one round trip.
+// Then every span's factor exp2(m_s - M) and scaled sum are made once, in parallel, and each output adds up its spans
+// in order. DEV: the states were written by other workgroups of the same launch (st_dev) and are read with ld_dev.
+// lds: 2 * S * G floats. `out` is the row's attention output, [Hq * 128]; `base` the state index of the head's span 0.
+template <int G, bool DEV>
+__device__ __forceinline__ void merge_spans(uint16_t* out, int g, int S, size_t base, const float* part_m,
+                                            const float* part_l, const float* part_acc, float* lds, int tid) {
+    constexpr int NOUT = G >= 2 ? G / 2 : 1;  // outputs a thread makes: (j, d) = ((tid + 256 q) / 128, tid % 128)
+    constexpr int MS = NOUT <= 2 ? 32 : 16;   // spans a pass
+    const float ninf = bits_f32(0xff800000u);
+    auto ld = [](const float* p) { return DEV ? ld_dev(p) : *p; };
+    float* f_m = lds;          // [S][G] maxima, then the factors
+    float* f_l = lds + S * G;  // [S][G] sums, then the scaled sums
+    const int d = tid & (AD - 1);
+    int jq[NOUT];
+#pragma unroll
+    for (int q = 0; q < NOUT; ++q) jq[q] = min((tid + 256 * q) / AD, G - 1);
+    const bool mine = tid < G * AD;  // a single query head: half the workgroup has no output
+    float v[NOUT][MS];
+    const int s_first = min(S, MS);
+#pragma unroll
+    for (int s2 = 0; s2 < MS; ++s2)
+#pragma unroll
+        for (int q = 0; q < NOUT; ++q)
+            v[q][s2] = ld(&part_acc[((base + min(s2, s_first - 1)) * G + jq[q]) * AD + d]);  // past the last: it again
+    for (int o = tid; o < S * G; o += 256) {
+        f_m[o] = ld(&part_m[base * G + o]);
+        f_l[o] = ld(&part_l[base * G + o]);
+    }
+    __syncthreads();
+    // each state's factor and scaled sum, by the thread that brought it in
+    float fac[4], lsc[4];  // S * G <= 1024 states over 256 threads
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int o = tid + 256 * r;
+        fac[r] = lsc[r] = 0.f;
+        if (o < S * G) {
+            const int j = o % G;
+            float M = ninf;
+            for (int s2 = 0; s2 < S; ++s2) M = fmaxf(M, f_m[s2 * G + j]);
+            const float pm = f_m[o];
+            fac[r] = pm == ninf ? 0.f : __builtin_amdgcn_exp2f(pm - M);
+            lsc[r] = f_l[o] * fac[r];
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int o = tid + 256 * r;
+        if (o < S * G) {
+            f_m[o] = fac[r];
+            f_l[o] = lsc[r];
+        }
+    }
+    __syncthreads();
+    float A[NOUT], L[NOUT];
+#pragma unroll
+    for (int q = 0; q < NOUT; ++q) {
+        A[q] = 0.f;
+        L[q] = 0.f;
+        for (int s2 = 0; s2 < S; ++s2) L[q] += f_l[s2 * G + jq[q]];
+    }
+#pragma unroll
+    for (int s2 = 0; s2 < MS; ++s2)
+        if (s2 < s_first) {
+#pragma unroll
+            for (int q = 0; q < NOUT; ++q) A[q] = fmaf(v[q][s2], f_m[s2 * G + jq[q]], A[q]);
+        }
+    for (int s0 = MS; s0 < S; s0 += MS) {
+        const int left = min(S - s0, MS);
+#pragma unroll
+        for (int s2 = 0; s2 < MS; ++s2)
+#pragma unroll
+            for (int q = 0; q < NOUT; ++q)
+                v[q][s2] = ld(&part_acc[((base + s0 + min(s2, left - 1)) * G + jq[q]) * AD + d]);
+#pragma unroll
+        for (int s2 = 0; s2 < MS; ++s2)
+            if (s2 < left) {
+#pragma unroll
+                for (int q = 0; q < NOUT; ++q) A[q] = fmaf(v[q][s2], f_m[(s0 + s2) * G + jq[q]], A[q]);
+            }
+    }
+    if (mine) {
+#pragma unroll
+        for (int q = 0; q < NOUT; ++q) {
+            const uint16_t o = f32_bf16(A[q] * (1.f / L[q]));
+            uint16_t* dst = &out[((size_t)g * G + jq[q]) * AD + d];
+            if (DEV)
+                st_dev(dst, o);
+            else
+                *dst = o;
+        }
+    }
+}
+
 }  // namespace btb

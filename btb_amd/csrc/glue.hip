@@ -286,38 +286,10 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(uint16_t* __restrict__ 
                                                          const float* __restrict__ part_m,
                                                          const float* __restrict__ part_l,
                                                          const float* __restrict__ part_acc) {
-    constexpr int D = ATT_D;
-    extern __shared__ float f_m[];  // [S][G] maxima, then the factors exp2(m_s - M); then [S][G] sums
-    __shared__ float s_L[G];
-    float* f_l = f_m + S * G;
+    extern __shared__ float f_m[];  // [S][G] maxima / factors, then [S][G] sums
     const int g = blockIdx.x, t = blockIdx.y;
-    const size_t base = ((size_t)t * Hk + g) * S;
-    for (int o = threadIdx.x; o < S * G; o += 256) {
-        f_m[o] = part_m[base * G + o];
-        f_l[o] = part_l[base * G + o];
-    }
-    __syncthreads();
-    if (threadIdx.x < G) {
-        const int j = threadIdx.x;
-        float M = bits_f32(0xff800000u);
-        for (int s2 = 0; s2 < S; ++s2) M = fmaxf(M, f_m[s2 * G + j]);
-        float L = 0.f;
-        for (int s2 = 0; s2 < S; ++s2) {
-            const float pm = f_m[s2 * G + j];
-            const float f = pm == bits_f32(0xff800000u) ? 0.f : exp2f(pm - M);
-            L = fmaf(f_l[s2 * G + j], f, L);
-            f_m[s2 * G + j] = f;
-        }
-        s_L[j] = L;
-    }
-    __syncthreads();
-    for (int o = threadIdx.x; o < G * D; o += 256) {
-        const int j = o / D, d = o - j * D;
-        float A = 0.f;
-#pragma unroll 8
-        for (int s2 = 0; s2 < S; ++s2) A = fmaf(part_acc[((base + s2) * G + j) * D + d], f_m[s2 * G + j], A);
-        att[((size_t)t * Hq + (size_t)g * G + j) * D + d] = f32_bf16(A * (1.f / s_L[j]));
-    }
+    merge_spans<G, false>(att + (size_t)t * Hq * ATT_D, g, S, ((size_t)t * Hk + g) * S, part_m, part_l, part_acc, f_m,
+                          threadIdx.x);
 }
 
 __global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ m,

@@ -370,86 +370,13 @@ __device__ __forceinline__ void matvec_phase(PRE_T& pre, const StepMat& mat, con
 // fold (attn_merge). head_dim 128, G = Hq / Hk = 4.
 // ------------------------------------------------------------------------------------------------------------
 
-// the spans of kv head g folded in span order (attn_merge_kernel's arithmetic) by the workgroup that finished the
-// head's last span. Thread (j, d) makes two output values; the states' loads are all requested before any is used.
+// the spans of kv head g folded in span order (the merge kernel's routine) by the workgroup that finished the head's
+// last span
 template <int G>
 __device__ __forceinline__ void merge_head(const StepArgs& a, int g, float* lds) {
-    const int tid = phase_tid();
-    constexpr int MS = 32;  // spans folded per pass
     const int S = a.S, Hq = a.Hq;
-    float* f_m = lds;          // [S][G] maxima, then the factors exp2(m_s - M)
-    float* f_l = lds + S * G;  // [S][G]
-    float* s_L = f_l + S * G;  // [G]
-    const float* part_m = a.part;
-    const float* part_l = a.part + (size_t)Hq * S;
-    const float* part_acc = a.part + 2 * (size_t)Hq * S;
-    const size_t base = (size_t)g * S;
-    float pm[2] = {0.f, 0.f}, pl[2] = {0.f, 0.f};
-    // S * G <= 512 states' maxima and sums: two a thread
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-        const int o = tid + q * 256;
-        if (o < S * G) {
-            pm[q] = ld_dev(&part_m[base * G + o]);
-            pl[q] = ld_dev(&part_l[base * G + o]);
-        }
-    }
-    const int d = tid & 127, j0 = tid >> 7;  // outputs (j0, d) and (j0 + 2, d)
-    float v[2][MS] = {};
-    const int s_first = min(S, MS);
-#pragma unroll
-    for (int s2 = 0; s2 < MS; ++s2)
-        if (s2 < s_first) {
-#pragma unroll
-            for (int q = 0; q < 2; ++q) v[q][s2] = ld_dev(&part_acc[((base + s2) * G + j0 + 2 * q) * AD + d]);
-        }
-#pragma unroll
-    for (int q = 0; q < 2; ++q) {
-        const int o = tid + q * 256;
-        if (o < S * G) {
-            f_m[o] = pm[q];
-            f_l[o] = pl[q];
-        }
-    }
-    __syncthreads();
-    if (tid < G) {
-        const int j = tid;
-        float M = bits_f32(0xff800000u);
-        for (int s2 = 0; s2 < S; ++s2) M = fmaxf(M, f_m[s2 * G + j]);
-        float Lsum = 0.f;
-        for (int s2 = 0; s2 < S; ++s2) {
-            const float x = f_m[s2 * G + j];
-            const float f = x == bits_f32(0xff800000u) ? 0.f : exp2f(x - M);
-            Lsum = fmaf(f_l[s2 * G + j], f, Lsum);
-            f_m[s2 * G + j] = f;
-        }
-        s_L[j] = Lsum;
-    }
-    __syncthreads();
-    float A[2] = {0.f, 0.f};
-#pragma unroll
-    for (int s2 = 0; s2 < MS; ++s2)
-        if (s2 < s_first) {
-#pragma unroll
-            for (int q = 0; q < 2; ++q) A[q] = fmaf(v[q][s2], f_m[s2 * G + j0 + 2 * q], A[q]);
-        }
-    for (int s0 = MS; s0 < S; s0 += MS) {
-#pragma unroll
-        for (int s2 = 0; s2 < MS; ++s2)
-            if (s0 + s2 < S) {
-#pragma unroll
-                for (int q = 0; q < 2; ++q) v[q][s2] = ld_dev(&part_acc[((base + s0 + s2) * G + j0 + 2 * q) * AD + d]);
-            }
-#pragma unroll
-        for (int s2 = 0; s2 < MS; ++s2)
-            if (s0 + s2 < S) {
-#pragma unroll
-                for (int q = 0; q < 2; ++q) A[q] = fmaf(v[q][s2], f_m[(s0 + s2) * G + j0 + 2 * q], A[q]);
-            }
-    }
-#pragma unroll
-    for (int q = 0; q < 2; ++q)
-        st_dev(&a.att[((size_t)g * G + j0 + 2 * q) * AD + d], f32_bf16(A[q] * (1.f / s_L[j0 + 2 * q])));
+    merge_spans<G, true>(a.att, g, S, (size_t)g * S, a.part, a.part + (size_t)Hq * S, a.part + 2 * (size_t)Hq * S, lds,
+                         phase_tid());
     __syncthreads();
 }
 
