@@ -174,8 +174,11 @@ __device__ __forceinline__ void fold_streams(float (&m)[G], float (&l)[G], float
         for (int s2 = 0; s2 < 16; ++s2) M = fmaxf(M, s_m[s2 * G + j]);
         const float f = m[j] == ninf ? 0.f : __builtin_amdgcn_exp2f(m[j] - M);
         if (dl == 0) s_l[grp * G + j] = l[j] * f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) s_acc[(grp * G + j) * AD + dl * 8 + e] = acc[j][e] * f;
+        // the lane's eight values as two 16-byte stores (s_acc is 16-byte aligned): one value a store would put
+        // lanes four apart on one bank
+        float4* dst = reinterpret_cast<float4*>(s_acc + (grp * G + j) * AD + dl * 8);
+        dst[0] = make_float4(acc[j][0] * f, acc[j][1] * f, acc[j][2] * f, acc[j][3] * f);
+        dst[1] = make_float4(acc[j][4] * f, acc[j][5] * f, acc[j][6] * f, acc[j][7] * f);
     }
     __syncthreads();
     for (int o = tid; o < G * AD; o += 256) {

@@ -132,7 +132,7 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
                                                           int span) {
     constexpr int D = ATT_D;
     __shared__ float s_m[16][G], s_l[16][G];
-    __shared__ float s_acc[16][G][D];
+    __shared__ __align__(16) float s_acc[16][G][D];
     const int g = blockIdx.x, sp = blockIdx.y, t = blockIdx.z, S = gridDim.y;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int sub = lane >> 4, dl = lane & 15;   // the lane's key within a quad of keys, its 8 dims
@@ -208,7 +208,7 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
     __shared__ uint32_t s_q[G][D / 2];  // the heads' q after norm and rope, bf16 pairs
     __shared__ __align__(16) uint16_t s_k[D], s_v[D];
     __shared__ float s_m[16][G], s_l[16][G];
-    __shared__ float s_acc[16][G][D];
+    __shared__ __align__(16) float s_acc[16][G][D];
     const int g = blockIdx.x, sp = blockIdx.y, S = gridDim.y;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int sub = lane >> 4, dl = lane & 15, grp = wv * 4 + sub;
