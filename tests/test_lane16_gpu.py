@@ -101,3 +101,27 @@ def test_group_equals_single_calls_and_refusals(card):
     w0, x0, y0 = ws[0], x[0], y[0]
     assert L.btb_hip_gemv_bf16_rows(card.ptr(w0), 12, 64, ctypes.c_void_p(x0.data_ptr() + 2), 2, card.ptr(y0), None) == -6
     assert L.btb_hip_gemv_bf16_rows(None, 0, 64, card.ptr(x0), 2, card.ptr(y0), None) == -1
+
+
+@pytest.mark.parametrize("rows,cols", [(128, 2048), (67, 1100)])
+@pytest.mark.parametrize("b", [1, 8, 17])
+def test_bf16_rows_at_an_odd_address_and_width(card, rows, cols, b):
+    """the reference's sweep moves every pointer by one element and takes 17 vectors (native/tests/gemv.rs:20-45,
+    262-329): the bits do not move - here the matrix one element off a 16-byte boundary leaves the wide-load kernel
+    for the element-load one, which must give the very same bits"""
+    w = weights_bf16(rows, cols, seed=440, std=1.0)
+    x = xs(b, cols, 441)
+    want = oracle.gemv_bf16(bits16(w), x.numpy(), threads=0)
+    wbuf = torch.zeros(rows * cols + 1, dtype=torch.bfloat16, device="cuda")
+    wbuf[1:] = w.reshape(-1).cuda()
+    xbuf = torch.zeros(b * cols + 1, dtype=torch.float32, device="cuda")
+    xbuf[1:] = x.reshape(-1).cuda()
+    ybuf = torch.zeros(b * rows + 1, dtype=torch.float32, device="cuda")
+    rc = card.lib.btb_hip_gemv_bf16_rows(ctypes.c_void_p(wbuf.data_ptr() + 2), rows, cols,
+                                         ctypes.c_void_p(xbuf.data_ptr() + 4), b, ctypes.c_void_p(ybuf.data_ptr() + 4),
+                                         ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    assert rc == 0
+    torch.cuda.synchronize()
+    got = ybuf[1:].reshape(b, rows).cpu().numpy()
+    assert np.array_equal(f32_bits(got), f32_bits(want))
+    assert np.array_equal(f32_bits(card.gemv_lane16(w.cuda(), x.cuda()).cpu().numpy()), f32_bits(want))
