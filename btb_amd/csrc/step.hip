@@ -1,7 +1,7 @@
 // The whole decode step as ONE persistent kernel.
 //
 // Why: on MI355X every kernel launch costs 3-4 us of ramp and drain during which HBM idles, and a Qwen3-4B-shaped step
-// is ~220 launches of 5-30 us each even after fusion. Here the grid (three workgroups a CU, all resident) walks the
+// is ~220 launches of 5-30 us each even after fusion. Here the grid (two workgroups a CU, all resident) walks the
 // step's phases itself and meets at a grid-wide barrier between them; before a wave waits at the barrier in front of a
 // matvec it has already requested the first items of its share of that matvec, so weights keep streaming while
 // the barrier resolves. The arithmetic of every phase is the arithmetic of the stand-alone kernels (gemv.hip,
@@ -18,9 +18,12 @@
 // and read with device-scope relaxed loads (cache-bypassing); weights and the cache's old rows are read-only during the
 // step and take ordinary loads. No cache-flushing fence is issued anywhere: on this GPU such a fence costs ~0.8 us per
 // workgroup and the workgroups of a die queue behind one another. The barrier is a two-level counter tree (16
-// workgroups a leaf), ~2.5-3 us per crossing at 768 workgroups. Every wait is bounded: a barrier that does not
-// complete within its spin limit raises the step's error word and every later barrier falls through, so the kernel
-// always ends.
+// workgroups a leaf), ~2.5-3 us per crossing. Every wait is bounded: a barrier that does not complete within its spin
+// limit raises the step's error word and every later barrier falls through, so the kernel always ends.
+//
+// Measured on MI355X the step comes out slower this way than as a replayed graph of the stand-alone kernels (about
+// 4 ms against 2.3 ms): a barrier and the skew of its arrivals cost what a kernel boundary costs, and the phases lose
+// the stand-alone kernels' per-shape tile choices. It is kept as an option, not as the default.
 
 #include <cstring>
 
@@ -481,7 +484,7 @@ __device__ __forceinline__ void phase_end(const StepArgs& a, unsigned nb, int& s
 }
 
 template <class F, int LQ, int LO, int LD>
-__global__ void __launch_bounds__(256, 3) decode_step_kernel(StepArgs a) {
+__global__ void __launch_bounds__(256, 2) decode_step_kernel(StepArgs a) {
     extern __shared__ __align__(16) uint32_t lds[];
     __shared__ float red[4];
     constexpr int G = 4;

@@ -150,7 +150,7 @@ class DecodeStep:
 
     def _bind_persistent(self, workgroups: int | None, trace: bool = False) -> None:
         """the argument block of `card.decode_step`: the layers' pointer table on the device, the buffers the phases
-        hand to one another, the barrier words. Three workgroups a CU unless told otherwise."""
+        hand to one another, the barrier words. Two workgroups a CU unless told otherwise."""
         from .native import StepArgs, StepLayer, StepMat
 
         if self.T != 1:
@@ -179,7 +179,7 @@ class DecodeStep:
                                  ptr(w[L + "ln1"]), ptr(w[L + "ln2"]), ptr(w.get(L + "wq")), ptr(w.get(L + "wk")),
                                  ptr(self.kv[i, 0]), ptr(self.kv[i, 1]))
         self._layer_table = torch.frombuffer(bytearray(bytes(table)), dtype=torch.uint8).to(dev)
-        self.workgroups = int(workgroups) if workgroups else 3 * int(self.card.sms)
+        self.workgroups = int(workgroups) if workgroups else 2 * int(self.card.sms)
         self.part = torch.zeros(2 * Hq * self.S + Hq * self.S * D, dtype=torch.float32, device=dev)
         self.cand_v = torch.zeros(4 * self.workgroups, dtype=torch.float32, device=dev)
         self.cand_i = torch.zeros(4 * self.workgroups, dtype=torch.int32, device=dev)
