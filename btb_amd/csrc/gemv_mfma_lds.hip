@@ -28,8 +28,20 @@ namespace btb {
 
 // ---- the stored forms: bytes a row contributes to a 32-column step, and the step's A fragment out of LDS ----------
 
-struct MfBf16 {
+// STEPB2 > 0: a second byte stream per row (its own slab), for the form that keeps a weight in two arrays
+struct MfNoTail {
+    static constexpr int TWO_TILES_STEPS = 128;  // the longest row (in steps) whose kernel holds two tiles of x rows
+    static constexpr int STEPB2 = 0;
+    static constexpr bool TAIL = false;
+    static constexpr int TAIL_BYTES = 0;
+    struct Tail {};
+    __device__ static __forceinline__ int2 tail_span(...) { return make_int2(0, 0); }
+    __device__ static __forceinline__ bool tail_any(const Tail&) { return false; }
+};
+
+struct MfBf16 : MfNoTail {
     static constexpr int STEPB = 64;
+    static constexpr int SB_NARROW = 8, SB_WIDE = 8;  // steps per sub-block: rows up to 4096 columns, wider rows
     struct Mat {
         const uint8_t* w;
     };
@@ -45,8 +57,9 @@ struct MfBf16 {
     }
 };
 
-struct MfF8 {
+struct MfF8 : MfNoTail {
     static constexpr int STEPB = 32;
+    static constexpr int SB_NARROW = 16, SB_WIDE = 8;  // the wide rows' x fragments leave room for four loads in flight
     struct Mat {
         const uint8_t* w;
         const float* scales;
@@ -107,8 +120,9 @@ struct MfF8 {
     }
 };
 
-struct MfMx4 {
+struct MfMx4 : MfNoTail {
     static constexpr int STEPB = 16;
+    static constexpr int SB_NARROW = 16, SB_WIDE = 16;
     struct Mat {
         const uint8_t* w;
         const uint8_t* scales;
@@ -146,6 +160,137 @@ struct MfMx4 {
     }
 };
 
+// 12 bits a weight: the low bytes (32 a step) and the code nibbles (16 a step) are two arrays, each streamed into a
+// slab of its own; a fragment is eight low bytes and eight codes zipped through the 16-entry table of high bytes
+// (FmtP12::widen8). The escapes - weights whose high byte is not in the table - are rare: the matrix cores multiply the
+// table's last entry in their place, and after the fold each escape of the tile's sixteen rows takes that term out and
+// puts the true one in, in list order, whatever M is.
+struct MfP12 {
+    static constexpr int STEPB = 32;
+    static constexpr int STEPB2 = 16;
+    static constexpr bool TAIL = true;
+    static constexpr int TAIL_BYTES = 32 * 16 * 4 + 32 * 4;
+    static constexpr int TWO_TILES_STEPS = 80;
+    static constexpr int SB_NARROW = 8, SB_WIDE = 8;
+    struct Mat {
+        const uint8_t* w;   // lo
+        const uint8_t* w2;  // hi4
+        const uint8_t* table;
+        const int32_t* esc_idx;
+        const uint8_t* esc_val;
+        const int32_t* row_ptr;
+    };
+    struct RowInfo {};
+    __device__ static __forceinline__ RowInfo row_info(const Mat&, int, int) { return RowInfo{}; }
+    template <int SB>
+    __device__ static __forceinline__ void scales(const Mat&, const RowInfo&, int, int, int, uint32_t (&)[SB]) {}
+    __device__ static __forceinline__ uint4 table(const Mat& m) { return FmtP12::load_table(m.table); }
+    __device__ static __forceinline__ bf16x8 frag2(const uint8_t* p, const uint8_t* p2, int g, const uint4& tbl) {
+        const uint2 l = *reinterpret_cast<const uint2*>(p + g * 8);
+        const uint32_t c = *reinterpret_cast<const uint32_t*>(p2 + g * 4);
+        uint32_t w[4];
+        FmtP12::widen8(tbl, c, l.x, l.y, w);
+        return __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
+    }
+    // The escapes of a tile: each of the KS waves takes those of 16 / KS of the tile's rows into its own partial tile
+    // (lane: x row li, the tile's rows 4 lg .. 4 lg + 3), thirty-two at a time. Lane j takes escape j % 32 and eight
+    // of the sixteen x rows (j / 32): its index and value are requested when the tile starts, its low byte and x
+    // values while the tile's first sub-block is multiplied, so the products wait for neither. The terms go through
+    // LDS (a small buffer of the wave's own) and are added in list order, whatever M is.
+    struct Tail {
+        int e0, e1;
+        uint32_t idx, val, lo;
+        int row;         // of the whole matrix
+        uint32_t xv[4];  // eight x values, two a register
+    };
+    // Every load below is unconditional - a lane with no escape reads a harmless place (the row index, the table,
+    // weight 0) - and so is every use of what the tile-ahead requests bring: a load whose only use sits in a branch
+    // would be moved into that branch, behind the loads issued after it.
+    __device__ static __forceinline__ void tail_request(const Mat& mat, Tail& t, int first, int lane) {
+        const int e = first + (lane & 31);
+        const bool ok = e < t.e1;
+        const int32_t* pi = ok ? mat.esc_idx + e : mat.row_ptr;
+        const uint8_t* pv = ok ? mat.esc_val + e : mat.table;
+        const uint32_t i = (uint32_t)*pi;
+        t.val = *pv;
+        t.idx = ok ? i : 0u;
+    }
+    // the list positions of the escapes of rows row .. row + nrows - 1: asked for well ahead of tail_begin, which
+    // cannot form an address without them
+    __device__ static __forceinline__ int2 tail_span(const Mat& mat, int row, int nrows) {
+        return make_int2(mat.row_ptr[row], mat.row_ptr[row + nrows]);
+    }
+    __device__ static __forceinline__ bool tail_any(const Tail& t) {
+        return __builtin_amdgcn_readfirstlane(t.e0) < __builtin_amdgcn_readfirstlane(t.e1);
+    }
+    __device__ static __forceinline__ Tail tail_begin(const Mat& mat, int2 span, int lane) {
+        Tail t;
+        t.e0 = span.x;
+        t.e1 = span.y;
+        tail_request(mat, t, t.e0, lane);
+        return t;
+    }
+    // xrows: the first of the sixteen x rows, of which `have` exist
+    __device__ static __forceinline__ void tail_loads(const Mat& mat, Tail& t, const uint16_t* xrows, int C, int have,
+                                                      int lane) {
+        t.lo = mat.w[t.idx];
+        t.row = (int)(t.idx / (uint32_t)C);
+        const uint32_t col = t.idx - (uint32_t)t.row * (uint32_t)C;
+        const int m0 = (lane >> 5) * 8;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {  // sixteen rows of at most 2^24 columns: the offsets fit 32 bits
+            const uint32_t o0 = (uint32_t)min(m0 + 2 * q, have - 1) * (uint32_t)C + col;
+            const uint32_t o1 = (uint32_t)min(m0 + 2 * q + 1, have - 1) * (uint32_t)C + col;
+            t.xv[q] = (uint32_t)xrows[o0] | ((uint32_t)xrows[o1] << 16);
+        }
+    }
+    // the thirty-two escapes in t: their terms into LDS, then added to the lane's rows in list order
+    __device__ static __forceinline__ void tail_chunk(const uint4& tbl, const Tail& t, int tile, int first, int C,
+                                                      int lane, uint8_t* scratch, f32x4& s) {
+        float* dl = reinterpret_cast<float*>(scratch);            // [32 escapes][16 x rows]
+        int* rw = reinterpret_cast<int*>(scratch + 32 * 16 * 4);  // [32] the escape's row within the tile
+        const uint32_t t15 = tbl.w >> 24;
+        const int li = lane & 15, row0 = (lane >> 4) * 4;
+        const float streamed = bits_f32((t15 << 24) | (t.lo << 16));
+        const float truth = bits_f32((t.val << 24) | (t.lo << 16));
+        float d[8];
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+            const float xv = (q & 1) ? bf16hi_f32(t.xv[q / 2]) : bf16lo_f32(t.xv[q / 2]);
+            d[q] = fmaf(truth, xv, -(streamed * xv));
+        }
+        float4* o = reinterpret_cast<float4*>(dl + (lane & 31) * 16 + (lane >> 5) * 8);
+        o[0] = make_float4(d[0], d[1], d[2], d[3]);
+        o[1] = make_float4(d[4], d[5], d[6], d[7]);
+        rw[lane & 31] = t.row - tile * 16;  // both halves write the same value
+        const int cnt = max(min(32, t.e1 - first), 0);
+#pragma unroll 2
+        for (int j = 0; j < cnt; ++j) {
+            const int k = rw[j] - row0;
+            const float v = dl[j * 16 + li];
+            s.x = k == 0 ? s.x + v : s.x;
+            s.y = k == 1 ? s.y + v : s.y;
+            s.z = k == 2 ? s.z + v : s.z;
+            s.w = k == 3 ? s.w + v : s.w;
+        }
+    }
+    // fetched: the first thirty-two are already in t (tail_begin, tail_loads with these x rows)
+    __device__ static __forceinline__ void tail_apply(const Mat& mat, const uint4& tbl, Tail& t, int tile,
+                                                      const uint16_t* xrows, int C, int have, int lane, uint8_t* scratch,
+                                                      bool fetched, f32x4& s) {
+        if (!fetched) {  // other x rows than the ones asked for ahead
+            tail_request(mat, t, t.e0, lane);
+            tail_loads(mat, t, xrows, C, have, lane);
+        }
+        tail_chunk(tbl, t, tile, t.e0, C, lane, scratch, s);
+        for (int first = t.e0 + 32; first < t.e1; first += 32) {  // a crowd: fetched here
+            tail_request(mat, t, first, lane);
+            tail_loads(mat, t, xrows, C, have, lane);
+            tail_chunk(tbl, t, tile, first, C, lane, scratch, s);
+        }
+    }
+};
+
 // ---- the kernel -----------------------------------------------------------------------------------------------------
 
 // KS waves a workgroup; MT 16-row tiles of x; SPW the steps a wave holds x fragments for (MT * SPW fragments in
@@ -160,12 +305,23 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
     constexpr int NLD = 16 * ROWB / 1024;     // 16-byte-per-lane loads a sub-block takes
     constexpr int MAXSB = (SPW + SB - 1) / SB;
     static_assert((16 * ROWB) % 1024 == 0 && NLD >= 1, "a sub-block is a whole number of wave loads");
-    extern __shared__ __align__(16) uint8_t lds[];  // KS slabs, then two sets of KS * MT partial tiles
+    // the second stream of a two-array form, the same way
+    constexpr int STEPB2 = MF::STEPB2;
+    constexpr bool TWO = STEPB2 > 0;
+    constexpr int ROWB2 = TWO ? SB * STEPB2 : 1024;
+    constexpr int STRIDE2 = ROWB2 + 16;
+    constexpr int SLAB2 = TWO ? 16 * STRIDE2 : 0;
+    constexpr int NLD2 = TWO ? 16 * ROWB2 / 1024 : 0;
+    static_assert(!TWO || ((16 * ROWB2) % 1024 == 0 && NLD2 >= 1 && 1024 % ROWB2 == 0), "the second stream's sub-block");
+    extern __shared__ __align__(16) uint8_t lds[];  // KS slabs (and second slabs), then two sets of KS * MT partial tiles
     const int lane = threadIdx.x & (WAVE - 1);
     const int wv = __builtin_amdgcn_readfirstlane(threadIdx.x / WAVE);
     const int li = lane & 15, lg = lane >> 4;
     uint8_t* slab = lds + wv * SLAB;
-    f32x4* part = reinterpret_cast<f32x4*>(lds + KS * SLAB);
+    uint8_t* slab2 = lds + KS * SLAB + wv * SLAB2;
+    constexpr int TAILB = MF::TAIL ? MF::TAIL_BYTES : 0;  // a wave's exchange buffer for the escapes' terms
+    [[maybe_unused]] uint8_t* tailbuf = lds + KS * (SLAB + SLAB2) + wv * TAILB;
+    f32x4* part = reinterpret_cast<f32x4*>(lds + KS * (SLAB + SLAB2 + TAILB));
 
     const int chunk4 = C / 8;  // uint4 per row of x
     const int nsteps = C / 32;
@@ -190,7 +346,15 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
     const uint32_t lane_row = (uint32_t)(lane * 16) / ROWB, lane_byte = (uint32_t)(lane * 16) % ROWB;
     const uint32_t goff = lane_row * (uint32_t)rowbytes + lane_byte;
     const uint32_t loff = lane_row * STRIDE + lane_byte;
+    constexpr int RPI2 = 1024 / ROWB2;
+    const uint32_t lane_row2 = (uint32_t)(lane * 16) / ROWB2, lane_byte2 = (uint32_t)(lane * 16) % ROWB2;
+    const size_t rowbytes2 = (size_t)nsteps * STEPB2;
+    const uint32_t goff2 = lane_row2 * (uint32_t)rowbytes2 + lane_byte2;
+    const uint32_t loff2 = lane_row2 * STRIDE2 + lane_byte2;
+    uint4 tbl = make_uint4(0, 0, 0, 0);  // the table of a form that looks its weights up
+    if constexpr (TWO) tbl = MF::table(mat);
     uint4 raw[NLD] = {};
+    uint4 raw2[TWO ? NLD2 : 1] = {};
     uint32_t scl[SB] = {};  // the scales of the sub-block in flight, one per step, for this lane's row and column group
     auto request = [&](int tile, int sb) {  // the loads of sub-block sb of the tile (R is a multiple of 16)
         const uint32_t valid = (uint32_t)(min(SB, n - sb * SB) * MF::STEPB);
@@ -201,42 +365,94 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
             const uint8_t* base = mat.w + (size_t)(tile * 16 + q * RPI) * rowbytes + (size_t)(s0 + sb * SB) * MF::STEPB;
             if (lane_byte < valid) raw[q] = load_stream16(reinterpret_cast<const uint4*>(base + goff));
         }
+        if constexpr (TWO) {
+            const uint32_t valid2 = (uint32_t)(min(SB, n - sb * SB) * STEPB2);
+#pragma unroll
+            for (int q = 0; q < NLD2; ++q) {
+                const uint8_t* base =
+                    mat.w2 + (size_t)(tile * 16 + q * RPI2) * rowbytes2 + (size_t)(s0 + sb * SB) * STEPB2;
+                if (lane_byte2 < valid2) raw2[q] = load_stream16(reinterpret_cast<const uint4*>(base + goff2));
+            }
+        }
     };
 
     const int ntiles = R / 16;
     const int nsb = (n + SB - 1) / SB;
     int tile = blockIdx.x;
+    // the escapes of the wave's rows of a tile: their indices are asked for a tile ahead, the rest of what they need
+    // while the tile's first sub-block is multiplied
+    [[maybe_unused]] typename MF::Tail tl, tnext;
+    [[maybe_unused]] int2 span_next = make_int2(0, 0);
+    constexpr int TROWS = 16 / KS;  // the rows of a tile whose escapes this wave takes
+    if constexpr (MF::TAIL) {
+        if (tile < ntiles) tnext = MF::tail_begin(mat, MF::tail_span(mat, tile * 16 + wv * TROWS, TROWS), lane);
+    }
     if (tile < ntiles && nsb > 0) request(tile, 0);
     for (int turn = 0; tile < ntiles; tile += gridDim.x, ++turn) {
         f32x4 acc[MT];
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
         const bool more = tile + (int)gridDim.x < ntiles;
+        [[maybe_unused]] const uint16_t* xrows = reinterpret_cast<const uint16_t*>(x);
+        if constexpr (MF::TAIL) tl = tnext;
 #pragma unroll
         for (int sb = 0; sb < MAXSB; ++sb) {
             if (sb < nsb) {
                 // the sub-block's bytes into the slab, as stored
 #pragma unroll
                 for (int q = 0; q < NLD; ++q) *reinterpret_cast<uint4*>(slab + q * RPI * STRIDE + loff) = raw[q];
+                if constexpr (TWO) {
+#pragma unroll
+                    for (int q = 0; q < NLD2; ++q)
+                        *reinterpret_cast<uint4*>(slab2 + q * RPI2 * STRIDE2 + loff2) = raw2[q];
+                }
                 uint32_t sc[SB];
 #pragma unroll
                 for (int t = 0; t < SB; ++t) sc[t] = scl[t];
+                if constexpr (MF::TAIL) {
+                    if (sb == 0) {
+                        MF::tail_loads(mat, tl, xrows, C, min(M, 16), lane);
+                        span_next = MF::tail_span(mat, min(tile + (int)gridDim.x, ntiles - 1) * 16 + wv * TROWS, TROWS);
+                    }
+                }
                 // the next sub-block - of this tile, or the first of the workgroup's next tile - on its way
-                if (sb + 1 < nsb)
+                if (sb + 1 < nsb) {
                     request(tile, sb + 1);
-                else if (more)
+                } else if (more) {
+                    if constexpr (MF::TAIL) tnext = MF::tail_begin(mat, span_next, lane);
                     request(tile + (int)gridDim.x, 0);
+                }
 #pragma unroll
                 for (int t = 0; t < SB; ++t) {
                     const int i = sb * SB + t;  // the wave's step (a compile-time index into xb)
                     if (i < SPW && i < n) {
-                        const bf16x8 a = MF::frag(slab + li * STRIDE + t * MF::STEPB, lg, sc[t]);
+                        bf16x8 a;
+                        if constexpr (TWO)
+                            a = MF::frag2(slab + li * STRIDE + t * MF::STEPB, slab2 + li * STRIDE2 + t * STEPB2, lg,
+                                          tbl);
+                        else
+                            a = MF::frag(slab + li * STRIDE + t * MF::STEPB, lg, sc[t]);
 #pragma unroll
                         for (int m = 0; m < MT; ++m)
                             acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
                                 a, __builtin_bit_cast(bf16x8, xb[m][i < SPW ? i : 0]), acc[m], 0, 0, 0);
                     }
                 }
+            }
+        }
+        if constexpr (MF::TAIL) {
+            // a wave with no step of its own (a short row) has not been through the loop above
+            if (nsb == 0) {
+                MF::tail_loads(mat, tl, xrows, C, min(M, 16), lane);
+                if (more)
+                    tnext = MF::tail_begin(mat, MF::tail_span(mat, (tile + (int)gridDim.x) * 16 + wv * TROWS, TROWS), lane);
+            }
+            if (MF::tail_any(tl)) {  // the same for the whole wave
+#pragma unroll
+                for (int t = 0; t < MT; ++t)
+                    if (t == 0 || t * 16 < M)
+                        MF::tail_apply(mat, tbl, tl, tile, xrows + (size_t)t * 16 * C, C, min(M - t * 16, 16), lane,
+                                       tailbuf, t == 0, acc[t]);
             }
         }
         // the KS partial tiles, folded in wave order; two sets of partials alternate so one barrier a tile suffices
@@ -268,7 +484,7 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
 
 template <class MF, int KS, int MT, int SPW, int SB>
 static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st) {
-    constexpr int SLAB = 16 * (SB * MF::STEPB + 16);
+    constexpr int SLAB = 16 * (SB * MF::STEPB + 16) + (MF::STEPB2 > 0 ? 16 * (SB * MF::STEPB2 + 16) : 0) + MF::TAIL_BYTES;
     const size_t lds = (size_t)KS * SLAB + 2 * (size_t)KS * MT * WAVE * sizeof(f32x4);
     const int ntiles = R / 16;
     int per_cu = tuning("mfma_wgs_per_cu");
@@ -302,7 +518,7 @@ bool mfma_lds_fits_packed(int R, int C) { return lds_fits<MfF8>(R, C); }
 
 template <class MF, int MT>
 static int32_t run_narrow(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st) {
-    constexpr int SB = MF::STEPB == 64 ? 8 : 16;  // eight (bf16, FP8) or four (MXFP4) loads of a sub-block in flight
+    constexpr int SB = MF::SB_NARROW;
     const int nsteps = C / 32;
     if (nsteps <= 20) return launch_lds<MF, 2, MT, 10, 8>(mat, x, y, R, C, M, st);
     if (nsteps <= 40) return launch_lds<MF, 4, MT, 10, 8>(mat, x, y, R, C, M, st);
@@ -312,12 +528,19 @@ static int32_t run_narrow(const typename MF::Mat& mat, const void* x, void* y, i
 
 template <class MF>
 static int32_t run_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st) {
-    constexpr int SB = MF::STEPB == 64 ? 8 : 16;
     const int nsteps = C / 32;
-    if (nsteps <= 128) return M <= 16 ? run_narrow<MF, 1>(mat, x, y, R, C, M, st) : run_narrow<MF, 2>(mat, x, y, R, C, M, st);
+    if (nsteps <= MF::TWO_TILES_STEPS)
+        return M <= 16 ? run_narrow<MF, 1>(mat, x, y, R, C, M, st) : run_narrow<MF, 2>(mat, x, y, R, C, M, st);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     uint16_t* yp = static_cast<uint16_t*>(y);
-    constexpr int SBW = MF::STEPB == 16 ? 16 : 8;  // the wide rows' x fragments leave room for four loads in flight
+    if (nsteps <= 128) {  // sixteen steps a wave, registers for one tile of x rows
+        for (int m0 = 0; m0 < M; m0 += 16) {
+            int32_t rc = run_narrow<MF, 1>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * R, R, C, M - m0 < 16 ? M - m0 : 16, st);
+            if (rc != OK) return rc;
+        }
+        return OK;
+    }
+    constexpr int SBW = MF::SB_WIDE;
     for (int m0 = 0; m0 < M; m0 += 16) {
         int32_t rc = launch_lds<MF, 8, 1, 28, SBW>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * R, R, C,
                                                   M - m0 < 16 ? M - m0 : 16, st);
@@ -334,6 +557,11 @@ int32_t gemv_mfma_lds_bf16(const void* w, const void* x, void* y, int R, int C, 
 int32_t gemv_mfma_lds_fp8(const void* w, const float* scales, int sc, int bm, int bn, const void* x, void* y, int R,
                           int C, int M, hipStream_t st) {
     return run_lds<MfF8>(MfF8::Mat{static_cast<const uint8_t*>(w), scales, sc, bm, bn}, x, y, R, C, M, st);
+}
+int32_t gemv_mfma_lds_p12(const uint8_t* lo, const uint8_t* hi4, const uint8_t* table, const int32_t* esc_idx,
+                          const uint8_t* esc_val, const int32_t* row_ptr, const void* x, void* y, int R, int C, int M,
+                          hipStream_t st) {
+    return run_lds<MfP12>(MfP12::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr}, x, y, R, C, M, st);
 }
 int32_t gemv_mfma_lds_mxfp4(const void* blocks, const void* scales, const void* x, void* y, int R, int C, int M,
                             hipStream_t st) {

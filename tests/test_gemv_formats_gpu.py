@@ -170,18 +170,35 @@ def test_full_shape_one_row_and_linearity(card, form):
     assert np.abs(total - want).max() <= 1e-2 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("M", [8, 16])
-def test_gemv_p12_verify_widths(card, M):
-    """12-bit matrices at the verify widths (passes of four rows of x): the oracle's bar, and row m's bits are those of
-    its one-row pass"""
-    R, C = 9728, 2560
+@pytest.mark.parametrize("R,C", [(9728, 2560), (2560, 4096), (1024, 7168), (2048, 768), (64, 256), (50, 96)])
+@pytest.mark.parametrize("M", [8, 16, 12, 24])
+def test_gemv_p12_verify_widths(card, R, C, M):
+    """12-bit matrices at the verify widths: the matrix-core kernel's forms (rows of 2, 4, 8 waves; the wide form; two
+    tiles of x rows at M = 24) and its fall-back (rows not a multiple of 16), with escapes forced on top of the natural
+    ones so that every 16-row tile holds some"""
     w = weights_bf16(R, C, seed=360)
+    wb = bits16(w).copy().reshape(-1)
+    at = np.arange(0, wb.size, max(1, wb.size // 4001))
+    wb[at] = (wb[at] & 0x00FF) | ((0x30 + np.arange(at.size) % 24).astype(np.uint16) << 8)
+    w = torch.from_numpy(wb.view(np.int16).reshape(R, C)).view(torch.bfloat16)
     pw = P12Weight.pack(w.cuda(), card)
+    assert pw.esc_idx.numel() > 0
     x = acts_bf16(M, C, seed=361)
+    ref = oracle.gemv_p12(*codecs.pack12_pack(wb), R, C, x.float().numpy(), threads=0)
+    _width_law(card, card.gemv_p12, pw, x.cuda(), ref)
+
+
+def test_gemv_p12_verify_width_many_escapes(card):
+    """a matrix whose high bytes are spread over far more than fifteen values: a sixth of the weights are escapes, and
+    the matrix-core pass still meets the bar against the matvec over the unpacked matrix"""
+    R, C, M = 256, 1024, 8
+    g = torch.Generator().manual_seed(362)
+    w = (torch.randn(R, C, generator=g) * torch.exp2(torch.randint(-12, 4, (R, C), generator=g).float())).to(torch.bfloat16)
+    pw = P12Weight.pack(w.cuda(), card)
+    assert pw.esc_idx.numel() > R * C // 10
+    x = acts_bf16(M, C, seed=363)
     y = card.gemv_p12(pw, x.cuda())
     check(y, oracle.gemv_bf16(bits16(w), x.float().numpy()))
-    solo = card.gemv_p12(pw, x[M - 1 :].contiguous().cuda())
-    assert torch.equal(solo[0].view(torch.int16), y[M - 1].view(torch.int16))
 
 
 @pytest.mark.parametrize("packed", [False, True])
