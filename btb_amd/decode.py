@@ -6,7 +6,8 @@ Per layer, as the reference sequences it: add_rmsnorm -> qkv matvec -> q/k norm 
 attention -> o matvec -> add_rmsnorm -> gate_up matvec -> activation -> down matvec; then the final norm, the head
 matvec, the greedy pick and the publish. The default (`fused`) form issues the same arithmetic in six launches a
 layer instead of eight: every add_rmsnorm rides in the following matvec's x load and gate / up / activation are one
-kernel. `DecodeStep.capture()` records the whole step with
+kernel; passes of four rows and more (a speculative verify) take the plain sequence, whose matvecs run on the matrix
+cores. `DecodeStep.capture()` records the whole step with
 torch's graph capture (a hipGraph on ROCm); afterwards the host only replays it and reads the token from pinned
 memory.
 """
@@ -101,7 +102,7 @@ class DecodeStep:
     (`Linear`), `embed` (bf16 [V, H]), `norm` and `head` (`Linear`)."""
 
     def __init__(self, card: Any, cfg: StackConfig, weights: dict[str, Any], cap: int, T: int = 1,
-                 attn_spans: int | None = None, fold_silu: bool = True, fused: bool = True,
+                 attn_spans: int | None = None, fold_silu: bool | None = None, fused: bool | None = None,
                  persistent: bool = False, workgroups: int | None = None, trace: bool = False) -> None:
         dev = torch.device("cuda")
         self.card, self.cfg, self.w, self.cap, self.T = card, cfg, weights, int(cap), int(T)
@@ -129,6 +130,14 @@ class DecodeStep:
             attn_spans = max(1, min(self.cap // 64, (card.sms + Hk - 1) // Hk))
         self.S = int(attn_spans)
         self.scratch = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
+        # Which sequence: up to three rows the fused launches win (fewer launches, every matvec on the streaming
+        # kernel); from four rows on the one-launch-per-operator sequence does, whose matvecs take the matrix cores
+        # at eight rows and more while a fused matvec runs as passes of four rows (measured on the 36-layer
+        # [2560 / 9728] stack, bf16: 4.3 against 4.0 ms at 4 rows, 7.1 against 4.6 at 8, 12.6 against 5.9 at 16).
+        if fused is None:
+            fused = T <= 3
+        if fold_silu is None:
+            fold_silu = fused
         self.fold_silu = bool(fold_silu)
         # the fused launches exist for bf16 and 12-bit matrices; any other stored form takes one launch per operator
         lins = [weights[f"layers.{i}.{k}"] for i in range(cfg.layers) for k in ("qkv", "o", "gu", "down")] + [weights["head"]]

@@ -216,3 +216,24 @@ def test_verify_pass_over_a_tree(card, fused):
     a = run(4, toks[:4], [-1, 0, 1, 2])
     b = run(4, toks[:4], None)
     assert torch.equal(a, b)
+
+
+def test_sequence_by_width(card):
+    """the sequence a step takes when none is asked for - fused launches up to three rows, one launch per operator (its
+    matvecs on the matrix cores) from four - and that a pass of eight rows gives the same logits either way, to the
+    step's bar"""
+    _, dev, kv = make_weights(card, False)
+    assert DecodeStep(card, CFG, dev, CAP).fused and DecodeStep(card, CFG, dev, CAP, T=3).fused
+    toks = [17, 5, 901, 33, 4, 250, 7, 12]
+    out = []
+    for fused in (None, True):
+        step = DecodeStep(card, CFG, dev, CAP, T=8, fused=fused)
+        assert step.fused == bool(fused) and step.fold_silu == bool(fused)
+        step.kv.copy_(kv.cuda())
+        step.reset(N0, toks[0])
+        step.ids.copy_(torch.tensor(toks, dtype=torch.int32))
+        step.body()
+        torch.cuda.synchronize()
+        out.append(step.logits.float().clone())
+    assert float((out[0] - out[1]).abs().max()) <= 3e-2 * float(out[1].abs().max())
+    assert torch.equal(out[0].argmax(dim=1), out[1].argmax(dim=1))
