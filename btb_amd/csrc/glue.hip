@@ -29,6 +29,9 @@ __global__ void __launch_bounds__(256) embed_kernel(const uint4* __restrict__ ta
     for (int i = threadIdx.x; i < H8; i += 256) h[(size_t)t * H8 + i] = table[(size_t)id * H8 + i];
 }
 
+// FAST: rows of a whole number of 8-byte words, at most 4096 values, every pointer 8-byte aligned - a thread's words
+// come in with 8-byte loads, all issued together, and stay in registers between the sum and the scaling
+template <bool FAST>
 __global__ void __launch_bounds__(256) add_rmsnorm_kernel(uint16_t* __restrict__ h, const uint16_t* __restrict__ y,
                                                           const uint16_t* __restrict__ w, float eps,
                                                           uint16_t* __restrict__ x, int H, int centered) {
@@ -39,6 +42,52 @@ __global__ void __launch_bounds__(256) add_rmsnorm_kernel(uint16_t* __restrict__
     uint16_t* xr = x + (size_t)t * H;
     // thread i takes the 4-element words i, i + 256, ... of the row, a word's elements in order (the order the matvec's
     // fused staging sums in, where a word is one 8-byte load)
+    if constexpr (FAST) {
+        constexpr int PER = 4;
+        const int n4 = H / 4;
+        const uint2* h2 = reinterpret_cast<const uint2*>(hr);
+        const uint2* y2 = reinterpret_cast<const uint2*>(yr == nullptr ? hr : yr);
+        const uint2* w2 = reinterpret_cast<const uint2*>(w);
+        uint2 hv[PER], yv[PER], wv[PER];
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {  // unconditional, past the row's end the last word again
+            const int wd = min(tid + 256 * k, n4 - 1);
+            hv[k] = h2[wd];
+            yv[k] = y2[wd];
+            wv[k] = w2[wd];
+        }
+        float f[PER][4];
+        float ss = 0.f;
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const bool live = tid + 256 * k < n4;
+            const uint32_t hw[2] = {hv[k].x, hv[k].y}, yw[2] = {yv[k].x, yv[k].y};
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float v = (e & 1) ? bf16hi_f32(hw[e / 2]) : bf16lo_f32(hw[e / 2]);
+                if (yr != nullptr) v = bfround(v + ((e & 1) ? bf16hi_f32(yw[e / 2]) : bf16lo_f32(yw[e / 2])));
+                f[k][e] = v;
+                ss = live ? fmaf(v, v, ss) : ss;
+            }
+            if (yr != nullptr && live)
+                reinterpret_cast<uint2*>(hr)[tid + 256 * k] =
+                    make_uint2(f32_bf16(f[k][0]) | (f32_bf16(f[k][1]) << 16), f32_bf16(f[k][2]) | (f32_bf16(f[k][3]) << 16));
+        }
+        const float rstd = rsqrtf(block_sum256(ss, red) / (float)H + eps);
+#pragma unroll
+        for (int k = 0; k < PER; ++k) {
+            const uint32_t ww[2] = {wv[k].x, wv[k].y};
+            uint32_t o[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float wf = (e & 1) ? bf16hi_f32(ww[e / 2]) : bf16lo_f32(ww[e / 2]);
+                o[e] = f32_bf16(f[k][e] * rstd * (centered ? 1.f + wf : wf));
+            }
+            if (tid + 256 * k < n4)
+                reinterpret_cast<uint2*>(xr)[tid + 256 * k] = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+        }
+        return;
+    }
     float ss = 0.f;
     for (int wd = tid; 4 * wd < H; wd += 256) {
         for (int i = 4 * wd; i < min(4 * wd + 4, H); ++i) {
@@ -412,9 +461,10 @@ int32_t btb_hip_add_rmsnorm(void* h, const void* y, const void* w, float eps, vo
     if (h == nullptr || w == nullptr || x == nullptr) return ERR_NULL;
     if (T == 0 || H == 0 || T > 0x7FFFFFFFull || H > 0x7FFFFFFFull || !(eps >= 0.f)) return ERR_DOMAIN;
     if (!al(h, 2) || !al(y, 2) || !al(w, 2) || !al(x, 2)) return ERR_DOMAIN;
-    hipLaunchKernelGGL(add_rmsnorm_kernel, dim3((unsigned)T), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       static_cast<uint16_t*>(h), static_cast<const uint16_t*>(y), static_cast<const uint16_t*>(w), eps,
-                       static_cast<uint16_t*>(x), (int)H, centered);
+    const bool fast = H % 4 == 0 && H <= 4096 && al(h, 8) && al(y, 8) && al(w, 8) && al(x, 8);
+    auto kern = fast ? add_rmsnorm_kernel<true> : add_rmsnorm_kernel<false>;
+    hipLaunchKernelGGL(kern, dim3((unsigned)T), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<uint16_t*>(h), static_cast<const uint16_t*>(y),
+                       static_cast<const uint16_t*>(w), eps, static_cast<uint16_t*>(x), (int)H, centered);
     return hip_status(hipGetLastError(), "add_rmsnorm launch");
 }
 
