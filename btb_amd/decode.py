@@ -125,9 +125,11 @@ class DecodeStep:
         self.kv = torch.zeros(cfg.layers, 2, Hk, self.cap, D, **bf)
         self.cos, self.sin = rope_tables(cfg, self.cap, dev)
         self.scale = 1.0 / math.sqrt(D)
-        # key spans: enough workgroups (kv heads x spans) to cover the CUs once, a span at least 64 keys
+        # key spans: enough workgroups (kv heads x spans) to cover the CUs once, a span at least 64 keys; a pass of T
+        # rows launches T times the workgroups, so it takes longer spans - two workgroups a CU in all (measured on
+        # the [2560 / 9728] stack at 4096 keys: 8 rows 4.32 ms a pass with 32 spans, 3.83 with 8; 16 rows 5.6 / 4.7)
         if attn_spans is None:
-            attn_spans = max(1, min(self.cap // 64, (card.sms + Hk - 1) // Hk))
+            attn_spans = max(1, min(self.cap // 64, (card.sms + Hk - 1) // Hk, (2 * card.sms) // (Hk * self.T)))
         self.S = int(attn_spans)
         self.scratch = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
         # Which sequence: up to three rows the fused launches win (fewer launches, every matvec on the streaming
