@@ -66,6 +66,7 @@ static Knob g_knobs[] = {
     {"mfma_wgs_per_cu", {-1}},
     {"mfma_classic", {-1}},
     {"mfma_lds", {-1}},
+    {"mfma_stream_x", {-1}},
     {"moe_wgs_per_cu", {-1}},
     {"attn_split", {-1}},
 };

@@ -294,8 +294,10 @@ struct MfP12 {
 // ---- the kernel -----------------------------------------------------------------------------------------------------
 
 // KS waves a workgroup; MT 16-row tiles of x; SPW the steps a wave holds x fragments for (MT * SPW fragments in
-// registers); SB steps per sub-block (a slab holds 16 rows x SB steps)
-template <class MF, int KS, int MT, int SPW, int SB>
+// registers); SB steps per sub-block (a slab holds 16 rows x SB steps). XS: the x fragments are not held - each
+// sub-block's come in with its weights (x is small and stays in L2), so a row may be as long as SPW allows without
+// the registers x-stationary rows of that length would take
+template <class MF, int KS, int MT, int SPW, int SB, bool XS = false>
 __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, const uint4* __restrict__ x,
                                                          uint16_t* __restrict__ y, int R, int C, int M) {
     constexpr int ROWB = SB * MF::STEPB;      // bytes a row contributes to a sub-block
@@ -330,13 +332,17 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
     const int n = max(min(s0 + spw, nsteps) - s0, 0);  // this wave's steps: s0 .. s0 + n - 1
     const size_t rowbytes = (size_t)nsteps * MF::STEPB;
 
-    uint4 xb[MT][SPW];
+    uint4 xb[MT][XS ? 1 : SPW];
+    const uint4* xr[MT];
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
-        const uint4* xr = x + (size_t)min(t * 16 + li, M - 1) * chunk4 + lg + (size_t)s0 * 4;
+        xr[t] = x + (size_t)min(t * 16 + li, M - 1) * chunk4 + lg + (size_t)s0 * 4;
+        if constexpr (!XS) {
 #pragma unroll
-        for (int i = 0; i < SPW; ++i) xb[t][i] = i < n ? xr[i * 4] : make_uint4(0, 0, 0, 0);
+            for (int i = 0; i < SPW; ++i) xb[t][i] = i < n ? xr[t][i * 4] : make_uint4(0, 0, 0, 0);
+        }
     }
+    [[maybe_unused]] uint4 xs[MT][XS ? SB : 1];  // XS: the x fragments of the sub-block in flight
 
     // A load instruction covers RPI whole rows of the sub-block (ROWB bytes each); the lane's place in it - row and
     // byte within the row - is the same for every load of the kernel, so every address is a uniform base (tile, load,
@@ -357,6 +363,18 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
     uint4 raw2[TWO ? NLD2 : 1] = {};
     uint32_t scl[SB] = {};  // the scales of the sub-block in flight, one per step, for this lane's row and column group
     auto request = [&](int tile, int sb) {  // the loads of sub-block sb of the tile (R is a multiple of 16)
+        if constexpr (XS) {  // out of L2, ahead of the weights they will meet: a step past the wave's last takes the last
+            // the same addresses every tile: a zero the compiler cannot see through keeps it from loading them all
+            // once, ahead of the loop, into the registers this form is there to save
+            int zero = 0;
+            asm volatile("" : "+s"(zero));
+#pragma unroll
+            for (int t = 0; t < SB; ++t) {
+                const int i = min(sb * SB + t, n - 1) + zero;
+#pragma unroll
+                for (int m = 0; m < MT; ++m) xs[m][t] = xr[m][i * 4];
+            }
+        }
         const uint32_t valid = (uint32_t)(min(SB, n - sb * SB) * MF::STEPB);
         const typename MF::RowInfo rn = MF::row_info(mat, tile * 16 + li, nsteps);
         MF::template scales<SB>(mat, rn, lg, s0 + sb * SB, nsteps, scl);
@@ -409,6 +427,13 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
                 uint32_t sc[SB];
 #pragma unroll
                 for (int t = 0; t < SB; ++t) sc[t] = scl[t];
+                [[maybe_unused]] uint4 xc[MT][XS ? SB : 1];
+                if constexpr (XS) {
+#pragma unroll
+                    for (int m = 0; m < MT; ++m)
+#pragma unroll
+                        for (int t = 0; t < SB; ++t) xc[m][t] = xs[m][t];
+                }
                 if constexpr (MF::TAIL) {
                     if (sb == 0) {
                         MF::tail_loads(mat, tl, xrows, C, min(M, 16), lane);
@@ -435,7 +460,8 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
 #pragma unroll
                         for (int m = 0; m < MT; ++m)
                             acc[m] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(
-                                a, __builtin_bit_cast(bf16x8, xb[m][i < SPW ? i : 0]), acc[m], 0, 0, 0);
+                                a, __builtin_bit_cast(bf16x8, XS ? xc[m][t] : xb[m][XS ? 0 : (i < SPW ? i : 0)]), acc[m],
+                                0, 0, 0);
                     }
                 }
             }
@@ -482,7 +508,7 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
     }
 }
 
-template <class MF, int KS, int MT, int SPW, int SB>
+template <class MF, int KS, int MT, int SPW, int SB, bool XS = false>
 static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st) {
     constexpr int SLAB = 16 * (SB * MF::STEPB + 16) + (MF::STEPB2 > 0 ? 16 * (SB * MF::STEPB2 + 16) : 0) + MF::TAIL_BYTES;
     const size_t lds = (size_t)KS * SLAB + 2 * (size_t)KS * MT * WAVE * sizeof(f32x4);
@@ -493,7 +519,7 @@ static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, i
     // whole turns of the grid over the tiles: the smallest grid that walks them in ceil(ntiles / cap) turns
     const int turns = (ntiles + cap - 1) / cap;
     const int grid = (ntiles + turns - 1) / turns;
-    auto kern = gemv_mfma_lds<MF, KS, MT, SPW, SB>;
+    auto kern = gemv_mfma_lds<MF, KS, MT, SPW, SB, XS>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -507,11 +533,11 @@ static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, i
 // The split of the columns over a workgroup's waves comes from the row length alone: at most eight waves (a workgroup
 // of sixteen would leave each wave 128 registers, less than the x fragments and a sub-block in flight need), each
 // holding x for 10, 16 or 28 steps. Up to 16 steps a wave there is room for two tiles of x rows; at 28 for one, and a
-// pass of more than 16 rows runs as two. Rows up to 7168 wide fit; wider ones stay with the column-interleaved kernel
-// (bf16) or the vector-ALU passes (packed forms).
+// pass of more than 16 rows runs as two. Rows up to 7168 wide fit that way; up to 10240 the x fragments are streamed
+// (XS); wider ones stay with the column-interleaved kernel (bf16) or the vector-ALU passes (packed forms).
 template <class MF>
 static bool lds_fits(int R, int C) {
-    return R % 16 == 0 && C % 32 == 0 && C / 32 <= 8 * 28;
+    return R % 16 == 0 && C % 32 == 0 && C / 32 <= 8 * 40;
 }
 bool mfma_lds_fits_bf16(int R, int C) { return lds_fits<MfBf16>(R, C); }
 bool mfma_lds_fits_packed(int R, int C) { return lds_fits<MfF8>(R, C); }
@@ -541,9 +567,14 @@ static int32_t run_lds(const typename MF::Mat& mat, const void* x, void* y, int 
         return OK;
     }
     constexpr int SBW = MF::SB_WIDE;
+    // up to 28 steps a wave the x fragments stay in registers; longer rows (to 40 steps: 10240 columns) stream them
+    const bool stream_x = nsteps > 8 * 28 || tuning("mfma_stream_x") > 0;
     for (int m0 = 0; m0 < M; m0 += 16) {
-        int32_t rc = launch_lds<MF, 8, 1, 28, SBW>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * R, R, C,
-                                                  M - m0 < 16 ? M - m0 : 16, st);
+        const int mm = M - m0 < 16 ? M - m0 : 16;
+        int32_t rc = stream_x ? (nsteps > 8 * 28
+                                     ? launch_lds<MF, 8, 1, 40, 8, true>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * R, R, C, mm, st)
+                                     : launch_lds<MF, 8, 1, 28, 8, true>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * R, R, C, mm, st))
+                              : launch_lds<MF, 8, 1, 28, SBW>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * R, R, C, mm, st);
         if (rc != OK) return rc;
     }
     return OK;

@@ -119,11 +119,13 @@ def _width_law(card, op, w, x, ref):
 
 
 @pytest.mark.parametrize("R,C,block", [(18432, 7168, (128, 128)), (2048, 7168, (128, 128)), (512, 1024, (128, 128)),
-                                       (1024, 2560, (128, 128)), (64, 256, (16, 16)), (50, 96, (50, 96))])
+                                       (1024, 2560, (128, 128)), (64, 256, (16, 16)), (50, 96, (50, 96)),
+                                       (256, 9728, (128, 128))])
 @pytest.mark.parametrize("M", [8, 16, 12])
 def test_gemv_fp8_verify_widths(card, R, C, block, M):
     """config C5a at its full shape and at shapes that take each of the matrix-core kernel's forms (rows of 2, 4, 8
-    waves; the wide form) and its fall-backs (rows not a multiple of 16)"""
+    waves; the wide form; rows past 7168 columns, whose x fragments are streamed) and its fall-backs (rows not a
+    multiple of 16)"""
     src = weights_bf16(R, C, seed=330).float()
     q, s = fp8.quantize(src, block)
     x = acts_bf16(M, C, seed=331)
@@ -132,7 +134,8 @@ def test_gemv_fp8_verify_widths(card, R, C, block, M):
     _width_law(card, card.gemv_fp8, w, x.cuda(), ref)
 
 
-@pytest.mark.parametrize("R,C", [(18432, 7168), (2048, 7168), (1536, 2048), (2048, 768), (1024, 2560), (24, 64), (48, 32)])
+@pytest.mark.parametrize("R,C", [(18432, 7168), (2048, 7168), (1536, 2048), (2048, 768), (1024, 2560), (24, 64), (48, 32),
+                                 (256, 9728)])
 @pytest.mark.parametrize("M", [8, 16, 12])
 def test_gemv_mxfp4_verify_widths(card, R, C, M):
     """config C5b at its full shape, the MoE expert shapes, and small shapes"""
@@ -170,7 +173,8 @@ def test_full_shape_one_row_and_linearity(card, form):
     assert np.abs(total - want).max() <= 1e-2 * np.abs(want).max()
 
 
-@pytest.mark.parametrize("R,C", [(9728, 2560), (2560, 4096), (1024, 7168), (2048, 768), (64, 256), (50, 96)])
+@pytest.mark.parametrize("R,C", [(9728, 2560), (2560, 4096), (1024, 7168), (2048, 768), (64, 256), (50, 96),
+                                 (2560, 9728)])
 @pytest.mark.parametrize("M", [8, 16, 12, 24])
 def test_gemv_p12_verify_widths(card, R, C, M):
     """12-bit matrices at the verify widths: the matrix-core kernel's forms (rows of 2, 4, 8 waves; the wide form; two
