@@ -220,11 +220,16 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     }
     const uint16_t* Kh = K + (size_t)g * hs + dl * 8;
     const uint16_t* Vh = V + (size_t)g * hs + dl * 8;
-    // eight keys of the stream a batch: their sixteen loads are issued together, then the batch is folded in
+    // eight keys of the stream a batch: their sixteen loads are issued together, and the next batch's before this one
+    // is folded in (past the span's end they fall on its last key again, unused), so a span of several batches - a
+    // pass of many rows takes long spans - pays the trip to memory once
+    KeyBatch kb;
+    load_keys(kb, Kh, Vh, rs, k_begin + grp, max(k_end, 1), -1);
     for (int key0 = k_begin + grp; key0 < k_end; key0 += 16 * KB) {
-        KeyBatch kb;
-        load_keys(kb, Kh, Vh, rs, key0, k_end, -1);
+        KeyBatch nx;
+        load_keys(nx, Kh, Vh, rs, key0 + 16 * KB, k_end, -1);
         use_keys<G>(kb, key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, m, l, acc, tree_base, tree_mask);
+        kb = nx;
     }
     // the 16 streams folded in stream order, the workgroup's state out
     const size_t prow = ((size_t)t * Hk + g) * S + sp;  // this workgroup's slot among the partial states
