@@ -272,6 +272,7 @@ int32_t gemv_mfma_bf16(const void* w, const void* x, void* y, int R, int C, int 
 bool mfma_lds_fits_bf16(int R, int C);
 bool mfma_lds_fits_packed(int R, int C);
 int32_t gemv_mfma_lds_bf16(const void* w, const void* x, void* y, int R, int C, int M, hipStream_t st);
+int32_t gemv_mfma_lds_glu_bf16(const void* w, const void* x, void* y, int I, int C, int M, hipStream_t st);
 int32_t gemv_mfma_lds_fp8(const void* w, const float* scales, int sc, int bm, int bn, const void* x, void* y, int R,
                           int C, int M, hipStream_t st);
 int32_t gemv_mfma_lds_mxfp4(const void* blocks, const void* scales, const void* x, void* y, int R, int C, int M,
@@ -363,6 +364,16 @@ int32_t btb_hip_gemv_glu_silu_bf16(const void* w, const void* x, void* m, size_t
     int32_t rc = check_dims(2 * I, C, M, FmtBf16::UW);
     if (rc != OK) return rc;
     if (!aligned16(w) || !aligned16(x) || !aligned2(m)) return ERR_DOMAIN;
+    if (I % 16 == 0 && wide_pass(M, 2 * I, C, false)) {  // the verify widths: the matrix cores, 32 rows of x a pass
+        const uint16_t* xp = static_cast<const uint16_t*>(x);
+        uint16_t* mp = static_cast<uint16_t*>(m);
+        for (size_t m0 = 0; m0 < M; m0 += 32) {
+            const int mm = (int)(M - m0 < 32 ? M - m0 : 32);
+            rc = gemv_mfma_lds_glu_bf16(w, xp + m0 * C, mp + m0 * I, (int)I, (int)C, mm, static_cast<hipStream_t>(stream));
+            if (rc != OK) return rc;
+        }
+        return OK;
+    }
     FmtBf16::Params p{static_cast<const uint4*>(w)};
     return run_rows<FmtBf16, X_PLAIN, E_GLU>(p, plain_x(x), m, 2 * I, C, M, static_cast<hipStream_t>(stream));
 }

@@ -299,7 +299,7 @@ struct MfP12 {
 // the registers x-stationary rows of that length would take
 template <class MF, int KS, int MT, int SPW, int SB, bool XS = false>
 __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, const uint4* __restrict__ x,
-                                                         uint16_t* __restrict__ y, int R, int C, int M) {
+                                                         uint16_t* __restrict__ y, int R, int C, int M, int half) {
     constexpr int ROWB = SB * MF::STEPB;      // bytes a row contributes to a sub-block
     constexpr int STRIDE = ROWB + 16;         // the slab's row stride: 4 banks past a multiple of 64, so the sixteen
                                               // rows a fragment read touches fall in sixteen different bank groups
@@ -396,7 +396,14 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
 
     const int ntiles = R / 16;
     const int nsb = (n + SB - 1) / SB;
-    int tile = blockIdx.x;
+    // The tiles a workgroup visits: blockIdx.x, + gridDim.x, ... - or, with half > 0 (W is a gate matrix over an up
+    // matrix, half tiles each, and y their fold bf16(bf16(silu(g)) * u), [M, R / 2]), the gate tile and the up tile of
+    // each such pair in turn
+    const int grid = (int)gridDim.x, first = (int)blockIdx.x;
+    auto tile_of = [&](int k) { return half ? first + (k >> 1) * grid + (k & 1) * half : first + k * grid; };
+    auto live = [&](int k) { return half ? first + (k >> 1) * grid < half : first + k * grid < ntiles; };
+    int tile = tile_of(0);
+    f32x4 gate = f32x4{0.f, 0.f, 0.f, 0.f};  // the folding wave's gate sums, kept until the up tile's are there
     // the escapes of the wave's rows of a tile: their indices are asked for a tile ahead, the rest of what they need
     // while the tile's first sub-block is multiplied
     [[maybe_unused]] typename MF::Tail tl, tnext;
@@ -406,11 +413,13 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
         if (tile < ntiles) tnext = MF::tail_begin(mat, MF::tail_span(mat, tile * 16 + wv * TROWS, TROWS), lane);
     }
     if (tile < ntiles && nsb > 0) request(tile, 0);
-    for (int turn = 0; tile < ntiles; tile += gridDim.x, ++turn) {
+    for (int turn = 0; live(turn); ++turn) {
+        tile = tile_of(turn);
         f32x4 acc[MT];
 #pragma unroll
         for (int t = 0; t < MT; ++t) acc[t] = f32x4{0.f, 0.f, 0.f, 0.f};
-        const bool more = tile + (int)gridDim.x < ntiles;
+        const bool more = live(turn + 1);
+        const int next = tile_of(turn + 1);
         [[maybe_unused]] const uint16_t* xrows = reinterpret_cast<const uint16_t*>(x);
         if constexpr (MF::TAIL) tl = tnext;
 #pragma unroll
@@ -437,7 +446,7 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
                 if constexpr (MF::TAIL) {
                     if (sb == 0) {
                         MF::tail_loads(mat, tl, xrows, C, min(M, 16), lane);
-                        span_next = MF::tail_span(mat, min(tile + (int)gridDim.x, ntiles - 1) * 16 + wv * TROWS, TROWS);
+                        span_next = MF::tail_span(mat, min(next, ntiles - 1) * 16 + wv * TROWS, TROWS);
                     }
                 }
                 // the next sub-block - of this tile, or the first of the workgroup's next tile - on its way
@@ -445,7 +454,7 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
                     request(tile, sb + 1);
                 } else if (more) {
                     if constexpr (MF::TAIL) tnext = MF::tail_begin(mat, span_next, lane);
-                    request(tile + (int)gridDim.x, 0);
+                    request(next, 0);
                 }
 #pragma unroll
                 for (int t = 0; t < SB; ++t) {
@@ -471,7 +480,7 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
             if (nsb == 0) {
                 MF::tail_loads(mat, tl, xrows, C, min(M, 16), lane);
                 if (more)
-                    tnext = MF::tail_begin(mat, MF::tail_span(mat, (tile + (int)gridDim.x) * 16 + wv * TROWS, TROWS), lane);
+                    tnext = MF::tail_begin(mat, MF::tail_span(mat, next * 16 + wv * TROWS, TROWS), lane);
             }
             if (MF::tail_any(tl)) {  // the same for the whole wave
 #pragma unroll
@@ -496,23 +505,41 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
                 s.w += o.w;
             }
             const int m = wv * 16 + li;
-            const int row = tile * 16 + lg * 4;
-            if (m < M) {
-                uint16_t* o = y + (size_t)m * R + row;
-                if (row + 0 < R) o[0] = f32_bf16(s.x);
-                if (row + 1 < R) o[1] = f32_bf16(s.y);
-                if (row + 2 < R) o[2] = f32_bf16(s.z);
-                if (row + 3 < R) o[3] = f32_bf16(s.w);
+            if (half) {
+                if ((turn & 1) == 0) {
+                    gate = s;
+                } else if (m < M) {
+                    // the arithmetic of the stand-alone fold over the two rounded outputs (silu_pair)
+                    auto fold = [](float g, float u) {
+                        const float gb = bfround(g), ub = bfround(u);
+                        return f32_bf16(bfround(gb / (1.f + expf(-gb))) * ub);
+                    };
+                    uint16_t* o = y + (size_t)m * (R / 2) + (tile - half) * 16 + lg * 4;
+                    o[0] = fold(gate.x, s.x);
+                    o[1] = fold(gate.y, s.y);
+                    o[2] = fold(gate.z, s.z);
+                    o[3] = fold(gate.w, s.w);
+                }
+            } else {
+                const int row = tile * 16 + lg * 4;
+                if (m < M) {
+                    uint16_t* o = y + (size_t)m * R + row;
+                    if (row + 0 < R) o[0] = f32_bf16(s.x);
+                    if (row + 1 < R) o[1] = f32_bf16(s.y);
+                    if (row + 2 < R) o[2] = f32_bf16(s.z);
+                    if (row + 3 < R) o[3] = f32_bf16(s.w);
+                }
             }
         }
     }
 }
 
 template <class MF, int KS, int MT, int SPW, int SB, bool XS = false>
-static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st) {
+static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st,
+                          int half = 0) {
     constexpr int SLAB = 16 * (SB * MF::STEPB + 16) + (MF::STEPB2 > 0 ? 16 * (SB * MF::STEPB2 + 16) : 0) + MF::TAIL_BYTES;
     const size_t lds = (size_t)KS * SLAB + 2 * (size_t)KS * MT * WAVE * sizeof(f32x4);
-    const int ntiles = R / 16;
+    const int ntiles = half ? half : R / 16;  // the units the grid walks: tiles, or pairs of a gate and an up tile
     int per_cu = tuning("mfma_wgs_per_cu");
     if (per_cu <= 0) per_cu = 12 / KS;  // twelve waves a CU: what the kernel's registers leave resident
     const int cap = device_info().cus * per_cu;
@@ -526,7 +553,7 @@ static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, i
         if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(KS * 64), lds, st, mat, static_cast<const uint4*>(x),
-                       static_cast<uint16_t*>(y), R, C, M);
+                       static_cast<uint16_t*>(y), R, C, M, half);
     return hip_status(hipGetLastError(), "gemv_mfma launch");
 }
 
@@ -543,25 +570,28 @@ bool mfma_lds_fits_bf16(int R, int C) { return lds_fits<MfBf16>(R, C); }
 bool mfma_lds_fits_packed(int R, int C) { return lds_fits<MfF8>(R, C); }
 
 template <class MF, int MT>
-static int32_t run_narrow(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st) {
+static int32_t run_narrow(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st,
+                          int half = 0) {
     constexpr int SB = MF::SB_NARROW;
     const int nsteps = C / 32;
-    if (nsteps <= 20) return launch_lds<MF, 2, MT, 10, 8>(mat, x, y, R, C, M, st);
-    if (nsteps <= 40) return launch_lds<MF, 4, MT, 10, 8>(mat, x, y, R, C, M, st);
-    if (nsteps <= 80) return launch_lds<MF, 8, MT, 10, 8>(mat, x, y, R, C, M, st);
-    return launch_lds<MF, 8, MT, 16, SB>(mat, x, y, R, C, M, st);
+    if (nsteps <= 20) return launch_lds<MF, 2, MT, 10, 8>(mat, x, y, R, C, M, st, half);
+    if (nsteps <= 40) return launch_lds<MF, 4, MT, 10, 8>(mat, x, y, R, C, M, st, half);
+    if (nsteps <= 80) return launch_lds<MF, 8, MT, 10, 8>(mat, x, y, R, C, M, st, half);
+    return launch_lds<MF, 8, MT, 16, SB>(mat, x, y, R, C, M, st, half);
 }
 
 template <class MF>
-static int32_t run_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st) {
+static int32_t run_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st,
+                          int half = 0) {
     const int nsteps = C / 32;
     if (nsteps <= MF::TWO_TILES_STEPS)
-        return M <= 16 ? run_narrow<MF, 1>(mat, x, y, R, C, M, st) : run_narrow<MF, 2>(mat, x, y, R, C, M, st);
+        return M <= 16 ? run_narrow<MF, 1>(mat, x, y, R, C, M, st, half) : run_narrow<MF, 2>(mat, x, y, R, C, M, st, half);
     const uint16_t* xp = static_cast<const uint16_t*>(x);
     uint16_t* yp = static_cast<uint16_t*>(y);
+    const int yrow = half ? R / 2 : R;  // values a row of y holds
     if (nsteps <= 128) {  // sixteen steps a wave, registers for one tile of x rows
         for (int m0 = 0; m0 < M; m0 += 16) {
-            int32_t rc = run_narrow<MF, 1>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * R, R, C, M - m0 < 16 ? M - m0 : 16, st);
+            int32_t rc = run_narrow<MF, 1>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * yrow, R, C, M - m0 < 16 ? M - m0 : 16, st, half);
             if (rc != OK) return rc;
         }
         return OK;
@@ -572,9 +602,9 @@ static int32_t run_lds(const typename MF::Mat& mat, const void* x, void* y, int 
     for (int m0 = 0; m0 < M; m0 += 16) {
         const int mm = M - m0 < 16 ? M - m0 : 16;
         int32_t rc = stream_x ? (nsteps > 8 * 28
-                                     ? launch_lds<MF, 8, 1, 40, 8, true>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * R, R, C, mm, st)
-                                     : launch_lds<MF, 8, 1, 28, 8, true>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * R, R, C, mm, st))
-                              : launch_lds<MF, 8, 1, 28, SBW>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * R, R, C, mm, st);
+                                     ? launch_lds<MF, 8, 1, 40, 8, true>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * yrow, R, C, mm, st, half)
+                                     : launch_lds<MF, 8, 1, 28, 8, true>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * yrow, R, C, mm, st, half))
+                              : launch_lds<MF, 8, 1, 28, SBW>(mat, xp + (size_t)m0 * C, yp + (size_t)m0 * yrow, R, C, mm, st, half);
         if (rc != OK) return rc;
     }
     return OK;
@@ -584,6 +614,10 @@ static int32_t run_lds(const typename MF::Mat& mat, const void* x, void* y, int 
 // they come here
 int32_t gemv_mfma_lds_bf16(const void* w, const void* x, void* y, int R, int C, int M, hipStream_t st) {
     return run_lds<MfBf16>(MfBf16::Mat{static_cast<const uint8_t*>(w)}, x, y, R, C, M, st);
+}
+// W = [gate; up], 2I rows: y [M, I] = bf16(bf16(silu(g)) * u)
+int32_t gemv_mfma_lds_glu_bf16(const void* w, const void* x, void* y, int I, int C, int M, hipStream_t st) {
+    return run_lds<MfBf16>(MfBf16::Mat{static_cast<const uint8_t*>(w)}, x, y, 2 * I, C, M, st, I / 16);
 }
 int32_t gemv_mfma_lds_fp8(const void* w, const float* scales, int sc, int bm, int bn, const void* x, void* y, int R,
                           int C, int M, hipStream_t st) {

@@ -108,6 +108,23 @@ def test_silu_fold_equals_two_steps(card, M):
     assert frac < 0.02, frac
 
 
+@pytest.mark.parametrize("I,C", [(9728, 2560), (768, 2048), (96, 4096), (64, 9728), (40, 64)])
+@pytest.mark.parametrize("M", [8, 16, 24])
+def test_glu_kernel_at_the_verify_widths(card, I, C, M):
+    """gate, up and the activation in the matrix-core kernel: the bits of its matvec followed by silu_mul, for each of
+    the kernel's forms (and the vector passes where I is no multiple of 16)"""
+    w = weights_bf16(2 * I, C, seed=152).cuda()
+    x = acts_bf16(M, C, seed=153).cuda()
+    gu = card.gemv(w, x)
+    want = torch.empty(M, I, dtype=torch.bfloat16, device="cuda")
+    card.silu_mul(gu, want)
+    got = card.gemv_glu_silu(w, x)
+    if I % 16 == 0:
+        assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+    else:  # vector passes against a matrix-core matvec: the bar, not the bits
+        assert float((got.float() - want.float()).abs().max()) <= 2.0**-7 * float(want.float().abs().max())
+
+
 @pytest.mark.parametrize("M", [1, 3])
 def test_glu_kernel_equals_matvec_then_silu_mul(card, M):
     I, C = 9728, 2560
