@@ -53,9 +53,10 @@ def test_gemv_p12_no_escapes(card):
     w = (weights_bf16(R, C, seed=302).float().clamp(0.011, 0.03)).to(torch.bfloat16)  # few high bytes: no escapes
     pw = P12Weight.pack(w.cuda(), card)
     assert pw.esc_idx.numel() == 0
-    x = acts_bf16(2, C, seed=303)
+    x = acts_bf16(8, C, seed=303)
     ref = oracle.gemv_bf16(bits16(w), x.float().numpy())
-    check(card.gemv_p12(pw, x.cuda()), ref)
+    check(card.gemv_p12(pw, x[:2].contiguous().cuda()), ref[:2])
+    check(card.gemv_p12(pw, x.cuda()), ref)  # eight rows: the matrix-core kernel, whose escape lists are null here
 
 
 @pytest.mark.parametrize("R,C,block", [(2048, 7168, (128, 128)), (512, 1024, (128, 128)), (64, 256, (16, 16)),

@@ -62,6 +62,11 @@ def test_matvec_outputs_stay_inside(card, R, C, M):
     f = Fenced((M, R), torch.float32)
     card.gemv_lane16(w, fin(x.float()), f.t)
     f.check("gemv_lane16")
+    if R % 2 == 0:
+        g = Fenced((M, R // 2), torch.bfloat16)
+        card.gemv_glu_silu(w, x, g.t)
+        g.check("gemv_glu_silu")
+        assert torch.equal(g.t, card.gemv_glu_silu(w.clone(), x.clone()))
     if C % 16 == 0:
         pw = P12Weight.pack(w.clone(), card)
         y = Fenced((M, R), torch.bfloat16)
