@@ -317,7 +317,8 @@ static int32_t p12_params(const void* lo, const void* hi4, const void* table, co
         return ERR_DOMAIN;
     *p = FmtP12::Params{static_cast<const uint8_t*>(lo),      static_cast<const uint8_t*>(hi4),
                         static_cast<const uint8_t*>(table),   static_cast<const int32_t*>(esc_idx),
-                        static_cast<const uint8_t*>(esc_val), static_cast<const int32_t*>(row_ptr)};
+                        static_cast<const uint8_t*>(esc_val), static_cast<const int32_t*>(row_ptr),
+                        make_uint4(0, 0, 0, 0)};
     return OK;
 }
 

@@ -245,8 +245,8 @@ struct MfP12 {
         }
     }
     // the thirty-two escapes in t: their terms into LDS, then added to the lane's rows in list order
-    __device__ static __forceinline__ void tail_chunk(const uint4& tbl, const Tail& t, int tile, int first, int C,
-                                                      int lane, uint8_t* scratch, f32x4& s) {
+    __device__ static __forceinline__ void tail_chunk(const uint4& tbl, const Tail& t, int tile, int first, int lane,
+                                                      uint8_t* scratch, f32x4& s) {
         float* dl = reinterpret_cast<float*>(scratch);            // [32 escapes][16 x rows]
         int* rw = reinterpret_cast<int*>(scratch + 32 * 16 * 4);  // [32] the escape's row within the tile
         const uint32_t t15 = tbl.w >> 24;
@@ -282,11 +282,11 @@ struct MfP12 {
             tail_request(mat, t, t.e0, lane);
             tail_loads(mat, t, xrows, C, have, lane);
         }
-        tail_chunk(tbl, t, tile, t.e0, C, lane, scratch, s);
+        tail_chunk(tbl, t, tile, t.e0, lane, scratch, s);
         for (int first = t.e0 + 32; first < t.e1; first += 32) {  // a crowd: fetched here
             tail_request(mat, t, first, lane);
             tail_loads(mat, t, xrows, C, have, lane);
-            tail_chunk(tbl, t, tile, first, C, lane, scratch, s);
+            tail_chunk(tbl, t, tile, first, lane, scratch, s);
         }
     }
 };

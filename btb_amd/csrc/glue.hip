@@ -503,7 +503,8 @@ int32_t btb_hip_norm_rope_kv(const void* qkv, const void* wq, const void* wk, fl
 }
 
 size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, size_t S) {
-    // part_m and part_l [T, Hk, S, G], part_acc [T, Hk, S, G, D]
+    // part_m and part_l [T, Hk, S, G], part_acc [T, Hk, S, G, D]: Hk * G = Hq
+    (void)Hk;
     return T * Hq * S * (2 + D);
 }
 

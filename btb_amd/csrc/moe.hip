@@ -332,7 +332,7 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__
 
     // the token's picks by ascending expert id: pick j goes to place #{i : id_i < id_j} (ids of a row are distinct; a
     // repeated id keeps its rank order)
-    if (threadIdx.x < k) {
+    if ((int)threadIdx.x < k) {
         const int j = threadIdx.x;
         const int mine = idx[(size_t)token * k + j];
         int place = 0;

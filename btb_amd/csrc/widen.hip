@@ -145,7 +145,7 @@ int32_t btb_hip_p12_widen(const void* lo, const void* hi4, const void* table, co
     hipStream_t st = static_cast<hipStream_t>(stream);
     FmtP12::Params p{static_cast<const uint8_t*>(lo),      static_cast<const uint8_t*>(hi4),
                      static_cast<const uint8_t*>(table),   static_cast<const int32_t*>(esc_idx),
-                     static_cast<const uint8_t*>(esc_val), nullptr};
+                     static_cast<const uint8_t*>(esc_val), nullptr, make_uint4(0, 0, 0, 0)};
     const size_t threads = n / FmtP12::UW + 1;
     hipLaunchKernelGGL(p12_widen_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, p, n,
                        static_cast<uint16_t*>(out));
