@@ -154,6 +154,7 @@ class DecodeStep:
         self.par = torch.arange(-1, self.T - 1, dtype=torch.int32, device=dev) if self.T > 1 else None
         self.depth = torch.arange(self.T, dtype=torch.int32, device=dev) if self.T > 1 else None
         self.persistent = bool(persistent)
+        self._rows: int | None = None  # set by reset()
         if self.persistent:
             self._bind_persistent(workgroups, trace)
 
@@ -228,6 +229,7 @@ class DecodeStep:
             raise ValueError(f"[decode] {n0} cached rows and a pass of {self.T} do not fit a cache of {self.cap}")
         self.n0.fill_(int(n0))
         self.ids.fill_(int(token))
+        self._rows = int(n0)  # the host's count of the cache's rows: every step run or replayed adds one
 
     def set_tree(self, par: list[int] | None) -> None:
         """the pass's rows as a tree (a speculative verify pass: the reference's `par` / `depth` arguments,
@@ -257,7 +259,18 @@ class DecodeStep:
 
     # -- the kernel sequence ---------------------------------------------------------------------------------------
 
+    def _advance(self) -> None:
+        """refuse a step whose rows would be written past the cache's end (the kernels do not look: the slot is
+        n0 + t on the device), counting from the last `reset`"""
+        if self._rows is None:
+            return
+        if self._rows + self.T > self.cap:
+            raise RuntimeError(f"[decode] the cache is full: {self._rows} rows of {self.cap}, and the step writes {self.T}")
+        self._rows += 1
+
     def body(self) -> None:
+        if not torch.cuda.is_current_stream_capturing():  # a step being recorded runs nothing
+            self._advance()
         if self.persistent:
             self.card.decode_step(self._step_args, self.packed, self.workgroups)
         elif self.fused:
@@ -343,6 +356,7 @@ class DecodeStep:
     def replay(self) -> None:
         if self.graph is None:
             raise RuntimeError("[decode] capture() the step before replaying it")
+        self._advance()
         self.graph.replay()
 
     def token(self) -> int:

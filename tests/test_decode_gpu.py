@@ -237,3 +237,22 @@ def test_sequence_by_width(card):
         out.append(step.logits.float().clone())
     assert float((out[0] - out[1]).abs().max()) <= 3e-2 * float(out[1].abs().max())
     assert torch.equal(out[0].argmax(dim=1), out[1].argmax(dim=1))
+
+
+def test_a_step_past_the_cache_is_refused(card):
+    """the kernels write the pass's rows at n0 + t without looking; the host counts the cache's rows from the last reset
+    and refuses the step - eager or replayed - that would write past the end"""
+    _, dev, kv = make_weights(card, False)
+    step = DecodeStep(card, CFG, dev, CAP, T=2)
+    step.reset(CAP - 3, 5)
+    step.body()          # rows CAP-3, CAP-2
+    step.body()          # rows CAP-2, CAP-1
+    with pytest.raises(RuntimeError, match="cache is full"):
+        step.body()
+    torch.cuda.synchronize()
+    step.reset(CAP - 3, 5)
+    step.capture(warmup=1)
+    step.replay()
+    with pytest.raises(RuntimeError, match="cache is full"):
+        step.replay()
+    torch.cuda.synchronize()
