@@ -191,6 +191,8 @@ def main() -> int:
     ap.add_argument("--workload", default="decode",
                     choices=["decode", "decode_p12", "gemv_bf16", "gemv_p12", "gemv_fp8", "gemv_mxfp4", "moe"])
     ap.add_argument("--m", type=int, default=1, help="rows of x (tokens) for the single-operator workloads")
+    ap.add_argument("--rows", type=int, default=1,
+                    help="rows of a decode pass: 1 is the step the metric is quoted on, more a speculative verify pass")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -200,6 +202,9 @@ def main() -> int:
         return kernel_workload(args)
     if args.steps < 1 or args.warmup < 0 or args.steps + args.warmup > 480:
         print("bench.py: steps + warmup must stay within the cache's 480 spare rows", file=sys.stderr)
+        return 2
+    if not 1 <= args.rows <= 24:
+        print("bench.py: a pass takes 1 to 24 rows here (the cache keeps 512 rows spare)", file=sys.stderr)
         return 2
 
     import torch
@@ -212,7 +217,7 @@ def main() -> int:
     packed = args.workload == "decode_p12"
     weights = random_stack(card, cfg, packed=packed)
     cap = CTX + 512
-    step = DecodeStep(card, cfg, weights, cap)
+    step = DecodeStep(card, cfg, weights, cap, T=args.rows)
     g = torch.Generator(device="cuda").manual_seed(0x0B7B0200)
     for i in range(cfg.layers):  # seeded K/V ~ N(0, 1) for the context
         step.kv[i, :, :, :CTX].copy_(torch.randn(2, cfg.kv_heads, CTX, cfg.head_dim, generator=g, device="cuda"))
@@ -239,8 +244,9 @@ def main() -> int:
 
     # -- the dominant kernel in a timed region of its own: the streaming matvec at the qkv, gate_up and head shapes
     #    (5.5 of the step's 8.0 GB of bf16 weights), over the model's own matrices, so nothing repeats from cache
-    x = torch.randn(1, cfg.hidden, device="cuda").to(torch.bfloat16)
-    outs = {n: torch.empty(1, r, dtype=torch.bfloat16, device="cuda")
+    M = args.rows
+    x = torch.randn(M, cfg.hidden, device="cuda").to(torch.bfloat16)
+    outs = {n: torch.empty(M, r, dtype=torch.bfloat16, device="cuda")
             for n, r in (("qkv", cfg.qkv_rows), ("gu", 2 * cfg.intermediate), ("head", cfg.vocab))}
 
     def dominant() -> tuple[int, int]:
@@ -250,9 +256,9 @@ def main() -> int:
                 lin = weights[f"layers.{i}.{n}"]
                 lin.matvec(x, outs[n])
                 launches += 1
-                nbytes += lin.nbytes + cfg.hidden * 2 + lin.shape[0] * 2
+                nbytes += lin.nbytes + M * (cfg.hidden * 2 + lin.shape[0] * 2)
         weights["head"].matvec(x, outs["head"])
-        return launches + 1, nbytes + weights["head"].nbytes + cfg.hidden * 2 + cfg.vocab * 2
+        return launches + 1, nbytes + weights["head"].nbytes + M * (cfg.hidden * 2 + cfg.vocab * 2)
 
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
@@ -298,14 +304,19 @@ def main() -> int:
         "config": {
             "workload": ("configs[1]: full decode step of a Qwen3-4B-shaped dense stack, M=1, ctx 4096, one hipGraph"
                          if not packed else
-                         "configs[2]: the same stack with every linear in pack12, widened in registers"),
+                         "configs[2]: the same stack with every linear in pack12, widened in registers")
+                        + ("" if args.rows == 1 else f"; a verify pass of {args.rows} rows"),
+            "rows": args.rows, "rows_per_s": round(args.rows * 1e3 / ms, 1),
             "layers": cfg.layers, "hidden": cfg.hidden, "q_heads": cfg.q_heads, "kv_heads": cfg.kv_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate, "vocab": cfg.vocab, "context": CTX,
-            "weight_bytes_per_step": wbytes, "kv_bytes_per_step": kvbytes, "kernels_per_step": 4 + 6 * cfg.layers,
+            "weight_bytes_per_step": wbytes, "kv_bytes_per_step": kvbytes, "kernels_per_step": (4 + 6 * cfg.layers if args.rows == 1 else
+                                 4 + 7 * cfg.layers if step.fused else 5 + 10 * cfg.layers),
             "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
         },
         "roofline": {
-            "kernel": "gemv_stream (streaming matvec, M=1) at the qkv / gate_up / head shapes",
+            "kernel": ("gemv_stream (streaming matvec, M=1)" if M == 1 else
+                       f"the matvec at M={M} (gemv_stream to 4 rows, gemv_mfma_lds from 8)")
+                      + " at the qkv / gate_up / head shapes",
             "bound": "hbm",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBS,
