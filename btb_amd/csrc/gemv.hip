@@ -1,5 +1,5 @@
 // The decode weight matvec for gfx950: y[m][r] = sum_c W[r][c] * x[m][c], M = 1..4 rows of x on the vector ALUs
-// (M = 8..32 take the MFMA kernel in gemv_mfma.hip). Memory-bound: every weight byte is read once, with 16-byte
+// (M = 5..32 take the MFMA kernels in gemv_mfma_lds.hip / gemv_mfma.hip). Memory-bound: every weight byte is read once, with 16-byte
 // per-lane non-temporal loads, a wave covering 1 KiB of a row per load instruction and keeping RPW * U of them in
 // flight; x is staged once per workgroup in LDS (optionally through the SwiGLU fold) and read from there with
 // ds_read_b128, shared by the RPW rows a lane works on. A row is summed by LPR lanes (64, 32 or 16, chosen from the
@@ -283,7 +283,7 @@ int32_t gemv_mfma_lds_p12(const uint8_t* lo, const uint8_t* hi4, const uint8_t* 
 
 // whether a pass of M rows goes to the matrix cores through the LDS-staged kernel
 static bool wide_pass(size_t M, size_t R, size_t C, bool packed) {
-    return M >= 8 && (packed ? mfma_lds_fits_packed((int)R, (int)C) : mfma_lds_fits_bf16((int)R, (int)C)) &&
+    return M >= 5 && (packed ? mfma_lds_fits_packed((int)R, (int)C) : mfma_lds_fits_bf16((int)R, (int)C)) &&
            tuning("gemv_no_mfma") <= 0 && tuning("mfma_lds") != 0;
 }
 
@@ -333,8 +333,9 @@ int32_t btb_hip_gemv_bf16(const void* w, const void* x, void* y, size_t R, size_
     int32_t rc = check_dims(R, C, M, FmtBf16::UW);
     if (rc != OK) return rc;
     if (!aligned16(w) || !aligned16(x) || !aligned2(y)) return ERR_DOMAIN;
-    // the verify widths go to the matrix cores, 32 rows of x a pass; narrower passes stay on the vector ALUs
-    if (M >= 8 && C % 32 == 0 && tuning("gemv_no_mfma") <= 0) {
+    // the verify widths go to the matrix cores, 32 rows of x a pass (from five rows on where the LDS-staged kernel takes
+    // the shape: one pass there against two of the vector ALUs'); narrower passes stay on the vector ALUs
+    if ((M >= 8 || wide_pass(M, R, C, false)) && C % 32 == 0 && tuning("gemv_no_mfma") <= 0) {
         const uint16_t* xp = static_cast<const uint16_t*>(x);
         uint16_t* yp = static_cast<uint16_t*>(y);
         for (size_t m0 = 0; m0 < M; m0 += 32) {

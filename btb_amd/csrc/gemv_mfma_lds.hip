@@ -1,4 +1,4 @@
-// The verify widths (M = 8..32 rows of x) on the matrix cores, with the weights brought in the way memory likes them.
+// The verify widths (M = 5..32 rows of x) on the matrix cores, with the weights brought in the way memory likes them.
 //
 // A v_mfma_f32_16x16x32_bf16 wants its A operand as "lane l: row l % 16, eight columns"; loading it that way straight
 // from memory makes every load instruction touch sixteen rows, 64 bytes of each, and HBM then runs at half speed

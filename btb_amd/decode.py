@@ -134,7 +134,7 @@ class DecodeStep:
         self.scratch = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
         # Which sequence: up to three rows the fused launches win (fewer launches, every matvec on the streaming
         # kernel); from four rows on the one-launch-per-operator sequence does, whose matvecs take the matrix cores
-        # at eight rows and more while a fused matvec runs as passes of four rows (measured on the 36-layer
+        # at five rows and more while a fused matvec runs as passes of four rows (measured on the 36-layer
         # [2560 / 9728] stack, bf16: 4.3 against 4.0 ms at 4 rows, 7.1 against 4.6 at 8, 12.6 against 5.9 at 16).
         if fused is None:
             fused = T <= 3
