@@ -109,6 +109,8 @@ def _width_law(card, op, w, x, ref):
     check(y, ref)
     y8 = op(w, x[:8].contiguous())
     assert torch.equal(y8.view(torch.int16), y[:8].view(torch.int16))
+    y5 = op(w, x[:5].contiguous())  # the narrowest pass the matrix cores take
+    assert torch.equal(y5.view(torch.int16), y[:5].view(torch.int16))
     card.set_tuning("gemv_no_mfma", 1)
     try:
         v = op(w, x)
