@@ -280,7 +280,7 @@ def main() -> int:
     achieved = dom_bytes / launches / (dom_us * 1e-6) / 1e9
     traffic = None
     tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath):
+    if os.path.exists(tpath) and args.rows == 1:  # the counters were read for the one-row region
         with open(tpath) as f:
             entry = json.load(f).get(args.workload)
             traffic = None if entry is None else entry.get("bytes_per_launch")
