@@ -9,7 +9,15 @@ matvec. Follows:
              -> times the pick's weight -> summed into the row in ASCENDING expert order, every step in the rows'
              dtype
 
+  grouping   btb/engine/host.py:283-296 (`group_picks`): the call's (pick, row) pairs in one stable sort by expert, an
+             expert's pairs pick-major then row, with each expert's offset and count
+
 `dt` is the rows' dtype: "bf16" (the engine running bf16 rows, what the GPU path computes) or "f32".
+
+Pinned on the CPU by tests/test_oracle_moe.py: the f32 layer against an independent plain-torch layer (softmax,
+torch.topk, renormalisation, dense per-token expert sums) to 1e-5; hand cases that a swapped gate / up half, a dropped
+renormalisation, a descending expert sum (bf16, where the order shows) or the wrong tie rule fail; `group_picks`
+against the one-hot / torch.where listing the reference's docstring names.
 """
 
 from __future__ import annotations
@@ -40,6 +48,18 @@ def router(w_router_bits: np.ndarray, x: np.ndarray, k: int, dt: str = "bf16", n
             s = (s + top[:, j]).astype(np.float32)
         top = (top / s[:, None]).astype(np.float32)
     return logits, _as(dt, top), order.astype(np.int64)
+
+
+def group_picks(picks: np.ndarray, num_experts: int):
+    """picks [T, k] -> (pick position, row) of every pair sorted by expert (stable, so pick-major then row within an
+    expert), and each expert's offset and count into them (btb/engine/host.py:283-296)"""
+    picks = np.asarray(picks)
+    T = picks.shape[0]
+    flat = picks.T.reshape(-1)
+    order = np.argsort(flat, kind="stable")
+    counts = np.bincount(flat, minlength=int(num_experts)).astype(np.int64)
+    offs = np.concatenate([[0], np.cumsum(counts)[:-1]]).astype(np.int64)
+    return order // T, order % T, offs, counts
 
 
 def silu(g: np.ndarray) -> np.ndarray:
