@@ -52,8 +52,19 @@ def sources() -> list[str]:
     return sorted(os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hip"))
 
 
-def _compile(src: str) -> str:
+def _fresh(src: str, obj: str) -> bool:
+    """whether obj is newer than its source and every header the sources share"""
+    if not os.path.exists(obj):
+        return False
+    deps = [src] + [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")]
+    deps.append(os.path.join(ROOT, "include", "btb_hip.h"))
+    return all(os.path.getmtime(d) <= os.path.getmtime(obj) for d in deps)
+
+
+def _compile(src: str, incremental: bool = False) -> str:
     obj = os.path.join(OBJ, os.path.basename(src)[:-4] + ".o")
+    if incremental and _fresh(src, obj):
+        return obj
     cmd = [hipcc(), *HIPCC_FLAGS, "-c", src, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     noise = "is not a recognized feature for this target"
@@ -65,11 +76,13 @@ def _compile(src: str) -> str:
     return obj
 
 
-def build_hip(jobs: int = 8) -> str:
-    """compile every csrc/*.hip for gfx950 and link libbtb_hip.so; returns its path"""
+def build_hip(jobs: int = 8, incremental: bool = False) -> str:
+    """compile every csrc/*.hip for gfx950 and link libbtb_hip.so; returns its path. `incremental` (a developer's
+    shortcut, `python -m btb_amd.build hip --incremental`) skips sources whose object is newer than they and the
+    headers are"""
     os.makedirs(OBJ, exist_ok=True)
     with ThreadPoolExecutor(max_workers=jobs) as pool:
-        objs = list(pool.map(_compile, sources()))
+        objs = list(pool.map(lambda s: _compile(s, incremental), sources()))
     tmp = LIB + ".tmp"
     cmd = [hipcc(), f"--offload-arch={ARCH}", "-shared", "-fPIC", "-o", tmp, *objs]
     r = subprocess.run(cmd, capture_output=True, text=True)
@@ -88,9 +101,10 @@ def build_oracle() -> str:
 
 
 def main(argv: list[str]) -> int:
-    what = argv[1:] or ["hip", "oracle"]
+    incremental = "--incremental" in argv
+    what = [a for a in argv[1:] if not a.startswith("--")] or ["hip", "oracle"]
     if "hip" in what:
-        print(build_hip())
+        print(build_hip(incremental=incremental))
     if "oracle" in what:
         print(build_oracle())
     return 0
