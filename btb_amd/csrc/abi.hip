@@ -12,6 +12,8 @@
 
 namespace btb {
 
+int32_t attn_static_bind();  // glue.hip: resolves the static attention scratch on the current device
+
 static DeviceInfo g_dev;
 static std::mutex g_dev_lock;
 static thread_local char g_err[256] = "";
@@ -87,8 +89,12 @@ int32_t btb_hip_init(int32_t device) {
     if (device < 0) return ERR_DOMAIN;
     hipError_t e = hipSetDevice(device);
     if (e != hipSuccess) return hip_status(e, "hipSetDevice");
-    std::lock_guard<std::mutex> hold(g_dev_lock);
-    return bind_current();
+    {
+        std::lock_guard<std::mutex> hold(g_dev_lock);
+        const int32_t rc = bind_current();
+        if (rc != OK) return rc;
+    }
+    return attn_static_bind();
 }
 
 const char* btb_hip_arch(void) { return "gfx950"; }

@@ -12,6 +12,8 @@
 //
 // Every reduction runs in an order fixed by the element's index alone, so a replayed graph repeats its bits.
 
+#include <mutex>
+
 #include "btb_attn.hpp"
 #include "btb_common.hpp"
 #include "btb_stream.hpp"
@@ -19,7 +21,48 @@
 
 #include "../../include/btb_hip.h"
 
+// The partial attention states of btb_hip_attn_decode_noalloc: 4 MiB that every GPU the library runs on holds until
+// the process ends. In host code this name is only a stand-in for the symbol; the array's address on a device comes
+// from hipGetSymbolAddress (scratch_on_device below) and is what the kernels are handed.
+constexpr size_t ATTN_STATIC_FLOATS = BTB_HIP_ATTN_NOALLOC_FLOATS;
+static __device__ __align__(256) float scratch[ATTN_STATIC_FLOATS];
+
 namespace btb {
+
+constexpr int MAX_DEVICES = 64;
+static float* g_scratch_ptr[MAX_DEVICES];  // per device: where that device's copy of `scratch` lies
+static std::mutex g_scratch_lock;
+
+// the current device's copy of `scratch`, looked up once per device (not an allocation: the array is part of the
+// code object the device loaded)
+static int32_t scratch_on_device(float** out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return hip_status(e, "hipGetDevice");
+    if (dev < 0 || dev >= MAX_DEVICES) {
+        set_error("attn_decode_noalloc: device ordinal beyond the table of per-device scratch addresses");
+        return ERR_DOMAIN;
+    }
+    std::lock_guard<std::mutex> hold(g_scratch_lock);
+    if (g_scratch_ptr[dev] == nullptr) {
+        float* p = nullptr;
+        e = hipGetSymbolAddress(reinterpret_cast<void**>(&p), HIP_SYMBOL(scratch));
+        if (e != hipSuccess) return hip_status(e, "hipGetSymbolAddress(scratch)");
+        if (p == nullptr) {
+            set_error("attn_decode_noalloc: the scratch symbol has no address on this device");
+            return ERR_PANIC;
+        }
+        g_scratch_ptr[dev] = p;
+    }
+    *out = g_scratch_ptr[dev];
+    return OK;
+}
+
+// called by btb_hip_init with the device current, so that the first attention call finds the address there already
+int32_t attn_static_bind() {
+    float* p = nullptr;
+    return scratch_on_device(&p);
+}
 
 __global__ void __launch_bounds__(256) embed_kernel(const uint4* __restrict__ table, const int32_t* __restrict__ ids,
                                                     uint4* __restrict__ h, int H8, int vocab) {
@@ -170,6 +213,7 @@ __global__ void __launch_bounds__(64) norm_rope_kv_kernel(const uint16_t* __rest
 // ------------------------------------------------------------------------------------------------------------
 constexpr int ATT_D = 128;
 constexpr int ATT_MAXG = 8;
+constexpr int ATT_MAX_STATES = 1024;  // (span, head) states of one kv head that merge_spans turns into factors
 
 template <int G>
 __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ K,
@@ -508,10 +552,12 @@ size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, siz
     return T * Hq * S * (2 + D);
 }
 
-int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
-                            const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
-                            float scale, size_t cap, size_t S, float* scratch, void* stream) {
-    if (q == nullptr || K == nullptr || V == nullptr || att == nullptr || n0 == nullptr || scratch == nullptr)
+// `work` is the caller's workspace, or nullptr for the library's own static array on the current device
+static int32_t attn_decode_any(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
+                               const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
+                               float scale, size_t cap, size_t S, float* work, bool own_scratch, void* stream) {
+    if (q == nullptr || K == nullptr || V == nullptr || att == nullptr || n0 == nullptr ||
+        (!own_scratch && work == nullptr))
         return ERR_NULL;
     if (T == 0 || Hq == 0 || Hk == 0 || S == 0 || cap == 0 || T > 65535 || S > 1024 || Hq % Hk != 0 || hs <= 0 ||
         rs <= 0 || !(scale == scale))
@@ -526,10 +572,23 @@ int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* a
         set_error("attn_decode: a tree pass holds at most 32 rows");
         return ERR_DOMAIN;
     }
+    if (S * G > (size_t)ATT_MAX_STATES) {
+        set_error("attn_decode: spans * (query heads per kv head) is at most 1024");
+        return ERR_DOMAIN;
+    }
+    if (own_scratch) {
+        if (T * Hq * S > ATTN_STATIC_FLOATS / (2 + D)) {
+            set_error("attn_decode_noalloc: T * Hq * S * (2 + D) floats of partial states exceed the 4 MiB the library "
+                      "holds; use fewer spans or btb_hip_attn_decode with a workspace");
+            return ERR_DOMAIN;
+        }
+        const int32_t rc = scratch_on_device(&work);
+        if (rc != OK) return rc;
+    }
     const int span = (int)((cap + S - 1) / S);
-    float* part_m = scratch;
-    float* part_l = scratch + T * Hq * S;
-    float* part_acc = scratch + 2 * T * Hq * S;
+    float* part_m = work;
+    float* part_l = work + T * Hq * S;
+    float* part_acc = work + 2 * T * Hq * S;
     const float scale_log2 = scale * 1.4426950408889634f;
     const dim3 grid((unsigned)Hk, (unsigned)S, (unsigned)T);
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -554,12 +613,24 @@ int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* a
     return hip_status(hipGetLastError(), "attn_decode launch");
 }
 
+int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
+                            const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
+                            float scale, size_t cap, size_t S, float* workspace, void* stream) {
+    return attn_decode_any(q, K, V, att, n0, par, T, Hq, Hk, D, hs, rs, scale, cap, S, workspace, false, stream);
+}
+
+int32_t btb_hip_attn_decode_noalloc(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
+                                    const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs,
+                                    int64_t rs, float scale, size_t cap, size_t S, void* stream) {
+    return attn_decode_any(q, K, V, att, n0, par, T, Hq, Hk, D, hs, rs, scale, cap, S, nullptr, true, stream);
+}
+
 int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk, float eps, int32_t centered,
                                 const void* cos_t, const void* sin_t, const int32_t* n0, void* K, void* V, void* att,
                                 size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap,
-                                size_t S, float* scratch, void* stream) {
+                                size_t S, float* workspace, void* stream) {
     if (qkv == nullptr || cos_t == nullptr || sin_t == nullptr || n0 == nullptr || K == nullptr || V == nullptr ||
-        att == nullptr || scratch == nullptr)
+        att == nullptr || workspace == nullptr)
         return ERR_NULL;
     if (Hq == 0 || Hk == 0 || S == 0 || cap == 0 || S > 1024 || Hq % Hk != 0 || hs <= 0 || rs <= 0 ||
         !(scale == scale) || !(eps >= 0.f))
@@ -570,10 +641,14 @@ int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk,
         return ERR_DOMAIN;
     }
     if (!al(qkv, 4) || !al(K, 16) || !al(V, 16) || (rs % 8) != 0 || (hs % 8) != 0) return ERR_DOMAIN;
+    if (S * G > (size_t)ATT_MAX_STATES) {
+        set_error("attn_decode_qkv: spans * (query heads per kv head) is at most 1024");
+        return ERR_DOMAIN;
+    }
     const int span = (int)((cap + S - 1) / S);
-    float* part_m = scratch;
-    float* part_l = scratch + Hq * S;
-    float* part_acc = scratch + 2 * Hq * S;
+    float* part_m = workspace;
+    float* part_l = workspace + Hq * S;
+    float* part_acc = workspace + 2 * Hq * S;
     const float scale_log2 = scale * 1.4426950408889634f;
     const dim3 grid((unsigned)Hk, (unsigned)S);
     hipStream_t st = static_cast<hipStream_t>(stream);

@@ -62,6 +62,8 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_attn_scratch_floats": (_sz, [_sz, _sz, _sz, _sz, _sz]),
     "btb_hip_attn_decode": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
                                    ctypes.c_float, _sz, _sz, _vp, _vp]),
+    "btb_hip_attn_decode_noalloc": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64,
+                                           ctypes.c_int64, ctypes.c_float, _sz, _sz, _vp]),
     "btb_hip_attn_decode_qkv": (_i32, [_vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
                                        ctypes.c_int64, ctypes.c_int64, ctypes.c_float, _sz, _sz, _vp, _vp]),
     "btb_hip_silu_mul": (_i32, [_vp, _vp, _sz, _sz, _vp]),
@@ -574,6 +576,27 @@ class HipCard:
         self._call("btb_hip_attn_decode", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0),
                    None if par is None else self.ptr(par), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)),
                    float(scale), int(K.shape[1]), S, self.ptr(scratch), _stream())
+
+    def attn_decode_noalloc(self, q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, att: torch.Tensor,
+                            n0: torch.Tensor, Hq: int, Hk: int, D: int, scale: float, S: int,
+                            par: torch.Tensor | None = None) -> None:
+        """`attn_decode` without a workspace: the spans' states go into the array the library holds on the GPU (4 MiB;
+        larger passes are refused). For callers that may not allocate; calls that overlap on one GPU race on it."""
+        self._need(q, torch.bfloat16, "q")
+        self._need(att, torch.bfloat16, "att")
+        self._need(n0, torch.int32, "n0")
+        if K.dtype != torch.bfloat16 or V.dtype != torch.bfloat16 or K.stride(2) != 1 or K.stride() != V.stride():
+            raise ValueError("[hip] attn_decode_noalloc: K and V are bf16 [Hk, cap, D] views with the same strides")
+        T = int(q.numel()) // (Hq * D)
+        if att.numel() != T * Hq * D:
+            raise ValueError(f"[hip] attn_decode_noalloc: att holds {att.numel()} values, the pass makes {T * Hq * D}")
+        if par is not None:
+            self._need(par, torch.int32, "par")
+            if par.numel() != T:
+                raise ValueError(f"[hip] attn_decode_noalloc: par names {par.numel()} rows, the pass has {T}")
+        self._call("btb_hip_attn_decode_noalloc", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0),
+                   None if par is None else self.ptr(par), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)),
+                   float(scale), int(K.shape[1]), S, _stream())
 
     def attn_decode_qkv(self, qkv: torch.Tensor, wq: torch.Tensor | None, wk: torch.Tensor | None, eps: float,
                         cos_t: torch.Tensor, sin_t: torch.Tensor, n0: torch.Tensor, K: torch.Tensor, V: torch.Tensor,

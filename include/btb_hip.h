@@ -13,7 +13,7 @@
  *
  * Two faces are exported, as in the reference: the device twins of the crate's CPU entry points (f32 x and y, the
  * host's summation order, bit for bit: btb_hip_gemv_*_rows) and the card operators the CUDA backend launches by
- * kernel name (bf16 x and y: btb_hip_gemv_bf16 and friends, also reachable through btb_hip_launch).
+ * kernel name (bf16 x and y: btb_hip_gemv_bf16 and friends).
  */
 #ifndef BTB_HIP_H
 #define BTB_HIP_H
@@ -217,12 +217,26 @@ size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, siz
  * pass's rows, -1 at a root): row t over the cache's keys 0 .. *n0 - 1 and, of the pass's own rows at slots
  * *n0 .. *n0 + T - 1, its ancestors and itself - the reference's TREE form (native/cuda/btb_attn_flash.cuh:284-286,
  * 407-419). The keys (capacity `cap`) are cut into S spans, a workgroup per (kv head, span, row) leaving its
- * online-softmax state in `scratch` (btb_hip_attn_scratch_floats floats); a second small launch folds the spans in
- * span order. head_dim 128, Hq / Hk in {1, 2, 4, 8}, S <= 1024. Replaces btb_attn_flash_d128's decode form
+ * online-softmax state in `workspace` (btb_hip_attn_scratch_floats floats); a second small launch folds the spans in
+ * span order. head_dim 128, Hq / Hk in {1, 2, 4, 8}, S * (Hq / Hk) <= 1024. Replaces btb_attn_flash_d128's decode form
  * (native/cuda/btb_attn_flash.cuh:277-675); the cache's row map (`tbl`) and the window are not taken. */
 int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
                             const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
-                            float scale, size_t cap, size_t S, float* scratch, void* stream);
+                            float scale, size_t cap, size_t S, float* workspace, void* stream);
+
+/* btb_hip_attn_decode for callers that cannot allocate device memory or pass a workspace: code under hipGraph
+ * capture, tight serving loops, harnesses that forbid hipMalloc. No counterpart in the reference. The spans' partial
+ * states go into an array the library itself holds on every GPU it runs on (BTB_HIP_ATTN_NOALLOC_FLOATS floats =
+ * 4 MiB per GPU, until the process ends), so the call allocates nothing and takes no workspace; otherwise the
+ * arguments, limits, kernels and result bits are btb_hip_attn_decode's. BTB_ERR_DOMAIN (and a message) when
+ * btb_hip_attn_scratch_floats(T, Hq, Hk, D, S) exceeds BTB_HIP_ATTN_NOALLOC_FLOATS. The array's address on a device is
+ * looked up once, by btb_hip_init or by the first call there. Every call on a GPU shares that GPU's array: calls that
+ * overlap on one GPU (two streams, two threads) race on it - serialise them or use btb_hip_attn_decode. Nothing in
+ * the array needs clearing between calls: every state a call reads, it has written first. */
+#define BTB_HIP_ATTN_NOALLOC_FLOATS ((size_t)1 << 20)
+int32_t btb_hip_attn_decode_noalloc(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
+                                    const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs,
+                                    int64_t rs, float scale, size_t cap, size_t S, void* stream);
 
 /* The decode step's own attention (one row), straight from the fused qkv row [(Hq + 2 Hk) D] bf16: what
  * btb_hip_norm_rope_kv followed by btb_hip_attn_decode compute at T = 1, bit for bit, in one launch less - the
@@ -232,7 +246,7 @@ int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* a
 int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk, float eps, int32_t centered,
                                 const void* cos_t, const void* sin_t, const int32_t* n0, void* K, void* V, void* att,
                                 size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap,
-                                size_t S, float* scratch, void* stream);
+                                size_t S, float* workspace, void* stream);
 
 /* m [T, I] = bf16(bf16(silu(g)) * u) over gu [T, 2I] (gate then up). Replaces btb_silu_mul
  * (native/cuda/btb_kernels.cu:467-484); the matvec btb_hip_gemv_silu_bf16 folds the same values into its x load. */
