@@ -36,12 +36,24 @@ __global__ void __launch_bounds__(256) p12_widen_kernel(FmtP12::Params p, size_t
 
 // the escapes written over the widened tensor: out[esc_idx[k]] = esc_val[k] << 8 | lo
 __global__ void __launch_bounds__(256) p12_patch_kernel(const uint8_t* __restrict__ lo, const int32_t* __restrict__ esc_idx,
-                                                        const uint8_t* __restrict__ esc_val, size_t n_esc,
+                                                        const uint8_t* __restrict__ esc_val, size_t n_esc, size_t n,
                                                         uint16_t* __restrict__ out) {
     const size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (k >= n_esc) return;
-    const size_t i = (size_t)esc_idx[k];
+    const int32_t at = esc_idx[k];
+    if (at < 0 || (size_t)at >= n) return;  // a list btb_hip_p12_check would refuse: never a write outside the tensor
+    const size_t i = (size_t)at;
     out[i] = (uint16_t)(((uint32_t)esc_val[k] << 8) | lo[i]);
+}
+
+// *bad |= 1 unless the list is strictly ascending inside [0, n): entry k against its left neighbour
+__global__ void __launch_bounds__(256) p12_check_kernel(const int32_t* __restrict__ esc_idx, size_t n_esc, size_t n,
+                                                        int32_t* __restrict__ bad) {
+    const size_t k = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (k >= n_esc) return;
+    const int32_t v = esc_idx[k];
+    const bool ok = v >= 0 && (size_t)v < n && (k == 0 || esc_idx[k - 1] < v);
+    if (!ok) atomicOr(bad, 1);
 }
 
 // row_ptr[r] = the number of escapes below r * cols: a binary search per row over the ascending list
@@ -136,6 +148,28 @@ int32_t btb_hip_p12_row_ptr(const void* esc_idx, size_t n_esc, size_t rows, size
     return hip_status(hipGetLastError(), "p12_row_ptr launch");
 }
 
+int32_t btb_hip_p12_check(const void* esc_idx, size_t n_esc, size_t n, int32_t* flag, void* stream) {
+    if (n_esc == 0) return n == 0 || n > 0x7FFFFFFFull ? ERR_DOMAIN : OK;
+    if (esc_idx == nullptr || flag == nullptr) return ERR_NULL;
+    if (n == 0 || n > 0x7FFFFFFFull || n_esc > n || !al(esc_idx, 4) || !al(flag, 4)) return ERR_DOMAIN;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    hipError_t e = hipMemsetAsync(flag, 0, sizeof(int32_t), st);
+    if (e != hipSuccess) return hip_status(e, "p12_check clear");
+    hipLaunchKernelGGL(p12_check_kernel, dim3((unsigned)((n_esc + 255) / 256)), dim3(256), 0, st,
+                       static_cast<const int32_t*>(esc_idx), n_esc, n, flag);
+    int32_t rc = hip_status(hipGetLastError(), "p12_check launch");
+    if (rc != OK) return rc;
+    int32_t bad = 0;
+    e = hipMemcpyAsync(&bad, flag, sizeof(int32_t), hipMemcpyDeviceToHost, st);
+    if (e == hipSuccess) e = hipStreamSynchronize(st);
+    if (e != hipSuccess) return hip_status(e, "p12_check read-back");
+    if (bad != 0) {
+        set_error("p12_check: the escape list is not strictly ascending inside [0, n)");
+        return ERR_DOMAIN;
+    }
+    return OK;
+}
+
 int32_t btb_hip_p12_widen(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
                           size_t n_esc, size_t n, void* out, void* stream) {
     if (lo == nullptr || hi4 == nullptr || table == nullptr || out == nullptr) return ERR_NULL;
@@ -153,7 +187,7 @@ int32_t btb_hip_p12_widen(const void* lo, const void* hi4, const void* table, co
     if (rc != OK || n_esc == 0) return rc;
     hipLaunchKernelGGL(p12_patch_kernel, dim3((unsigned)((n_esc + 255) / 256)), dim3(256), 0, st,
                        static_cast<const uint8_t*>(lo), static_cast<const int32_t*>(esc_idx),
-                       static_cast<const uint8_t*>(esc_val), n_esc, static_cast<uint16_t*>(out));
+                       static_cast<const uint8_t*>(esc_val), n_esc, n, static_cast<uint16_t*>(out));
     return hip_status(hipGetLastError(), "p12_patch launch");
 }
 

@@ -154,7 +154,7 @@ class DecodeStep:
         self.par = torch.arange(-1, self.T - 1, dtype=torch.int32, device=dev) if self.T > 1 else None
         self.depth = torch.arange(self.T, dtype=torch.int32, device=dev) if self.T > 1 else None
         self.persistent = bool(persistent)
-        self._rows: int | None = None  # set by reset()
+        self._rows = 0  # the host's count of the cache's rows (n0 starts at 0 on the device too); reset() sets both
         if self.persistent:
             self._bind_persistent(workgroups, trace)
 
@@ -262,8 +262,6 @@ class DecodeStep:
     def _advance(self) -> None:
         """refuse a step whose rows would be written past the cache's end (the kernels do not look: the slot is
         n0 + t on the device), counting from the last `reset`"""
-        if self._rows is None:
-            return
         if self._rows + self.T > self.cap:
             raise RuntimeError(f"[decode] the cache is full: {self._rows} rows of {self.cap}, and the step writes {self.T}")
         self._rows += 1

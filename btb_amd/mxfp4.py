@@ -18,44 +18,55 @@ BIAS = 127
 
 
 def blocks_per_row(k: int) -> int:
-    if k % BLOCK:
-        raise ValueError(f"[mxfp4] K = {k} is not a multiple of {BLOCK}")
-    return k // BLOCK
+    """how many 32-weight blocks a row of k weights is cut into"""
+    n, rest = divmod(int(k), BLOCK)
+    if rest or n < 0:
+        raise ValueError(f"[mxfp4] a row of {k} weights is not a whole number of {BLOCK}-weight blocks")
+    return n
 
 
 def matrix_bytes(rows: int, k: int) -> tuple[int, int]:
-    g = blocks_per_row(k)
-    return rows * g * BLOCK_BYTES, rows * g
+    """(bytes of packed codes, bytes of scales) a [rows, k] matrix takes"""
+    blocks = int(rows) * blocks_per_row(k)
+    return blocks * BLOCK_BYTES, blocks
 
 
 def scale_factors(scales: torch.Tensor) -> torch.Tensor:
-    """2^(scale - 127) as f32, exactly, for every uint8 scale (0 is 2^-127)"""
-    s = scales.to(torch.int32)
-    f = (torch.clamp(s, min=1) << 23).view(torch.float32)
-    return torch.where(s == 0, f * 0.5, f)
+    """Every e8m0 byte s as the f32 2^(s - 127), built from its bits so that nothing rounds: s >= 1 is a normal number
+    with exponent field s, s = 0 is the subnormal 2^-127 (mantissa 0x400000), s = 255 comes out as +inf."""
+    field = scales.to(torch.int32)
+    bits = torch.where(field > 0, field * (1 << 23), torch.full_like(field, 0x0040_0000))
+    return bits.view(torch.float32)
+
+
+def _codes_to_values(blocks: torch.Tensor) -> torch.Tensor:
+    """[..., 16] packed bytes -> [..., 32] fp4 values as f32, the low nibble first"""
+    lut = torch.tensor(FP4_VALUES, dtype=torch.float32, device=blocks.device)
+    idx = torch.stack((blocks & 0x0F, blocks >> 4), dim=-1).to(torch.int64)
+    return lut[idx].flatten(-2)
+
+
+def _check_pair(blocks: torch.Tensor, scales: torch.Tensor) -> None:
+    if blocks.shape[-1] != BLOCK_BYTES:
+        raise ValueError(f"[mxfp4] the last dim of blocks is the {BLOCK_BYTES} bytes of one block, not {blocks.shape[-1]}")
+    if tuple(blocks.shape[:-1]) != tuple(scales.shape):
+        raise ValueError(f"[mxfp4] one scale a block: blocks {tuple(blocks.shape)} need scales {tuple(blocks.shape[:-1])}, "
+                         f"got {tuple(scales.shape)}")
 
 
 def dequantize(blocks: torch.Tensor, scales: torch.Tensor, dtype: torch.dtype = torch.float32) -> torch.Tensor:
-    """blocks [..., rows, K/32, 16] uint8 and scales [..., rows, K/32] uint8 to [..., rows, K]: one rounding per
-    weight (the f32 product, then `dtype`), as torch.ldexp makes it"""
-    if blocks.shape[:-1] != scales.shape:
-        raise ValueError(f"[mxfp4] blocks {tuple(blocks.shape)} do not match scales {tuple(scales.shape)}")
-    if blocks.shape[-1] != BLOCK_BYTES:
-        raise ValueError(f"[mxfp4] a block is {BLOCK_BYTES} bytes, got {blocks.shape[-1]}")
-    lut = torch.tensor(FP4_VALUES, dtype=torch.float32, device=blocks.device)
-    b = blocks.to(torch.int64)
-    vals = torch.stack([lut[b & 15], lut[b >> 4]], dim=-1).reshape(*blocks.shape[:-1], BLOCK)
-    out = vals * scale_factors(scales)[..., None]
-    return out.reshape(*blocks.shape[:-2], blocks.shape[-2] * BLOCK).to(dtype)
+    """blocks [..., rows, K/32, 16] and scales [..., rows, K/32] (uint8) -> [..., rows, K]: the f32 product
+    fp4 * 2^(scale - 127) - exact but for the subnormal results - cast to `dtype`"""
+    _check_pair(blocks, scales)
+    wide = _codes_to_values(blocks) * scale_factors(scales).unsqueeze(-1)
+    return wide.flatten(-2).to(dtype)
 
 
 def dequant_blocks(blocks: torch.Tensor, scales: torch.Tensor, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
     """the widening the card's `mx4_widen` matches bit for bit: ldexp(fp4, scale - 127) rounded to `dtype`"""
-    lut = torch.tensor(FP4_VALUES, dtype=torch.float32, device=blocks.device)
-    b = blocks.to(torch.int64)
-    vals = torch.stack([lut[b & 15], lut[b >> 4]], dim=-1).reshape(*blocks.shape[:-1], BLOCK)
-    out = torch.ldexp(vals, (scales.to(torch.int32) - BIAS)[..., None])
-    return out.reshape(*blocks.shape[:-2], blocks.shape[-2] * BLOCK).to(dtype)
+    _check_pair(blocks, scales)
+    wide = torch.ldexp(_codes_to_values(blocks), (scales.to(torch.int32) - BIAS).unsqueeze(-1))
+    return wide.flatten(-2).to(dtype)
 
 
 def quantize(t: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:

@@ -40,6 +40,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
                                      _sz, _sz, _sz, _i32, _vp]),
     "btb_hip_gemv_p12": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_p12_row_ptr": (_i32, [_vp, _sz, _sz, _sz, _vp, _vp]),
+    "btb_hip_p12_check": (_i32, [_vp, _sz, _sz, _vp, _vp]),
     "btb_hip_p12_widen": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _vp, _vp]),
     "btb_hip_gemv_fp8": (_i32, [_vp, _vp, _sz, _sz, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_fp8_widen": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _i32, _vp]),
@@ -300,6 +301,18 @@ class HipCard:
             raise ValueError(f"[hip] {what}: y holds {y.numel()} elements, the product has {M * R}")
         return y
 
+    def p12_check(self, esc_idx: torch.Tensor, n: int) -> None:
+        """ValueError unless the escape list is strictly ascending inside [0, n): checked on the GPU, once, at upload"""
+        self._need(esc_idx, torch.int32, "esc_idx")
+        if esc_idx.numel() == 0:
+            return
+        flag = torch.zeros(1, dtype=torch.int32, device=esc_idx.device)
+        rc = self.lib.btb_hip_p12_check(self.ptr(esc_idx), esc_idx.numel(), int(n), self.ptr(flag), _stream())
+        if rc == ERR_DOMAIN:
+            raise ValueError(f"[hip] pack12: {self.lib.btb_hip_last_error().decode(errors='replace')}")
+        if rc != OK:
+            raise HipError(f"[hip] btb_hip_p12_check failed: {rc} {_CODES.get(rc, '?')}")
+
     def p12_row_ptr(self, esc_idx: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
         """int32 [rows + 1]: the first escape at or past each row's first weight (built once at upload)"""
         self._need(esc_idx, torch.int32, "esc_idx")
@@ -321,11 +334,17 @@ class HipCard:
                    self.ptr(x2), self.ptr(y), R, C, M, _stream())
         return y
 
-    def p12_widen(self, lo, hi4, table, esc_idx, esc_val, n: int, shape: Sequence[int]) -> torch.Tensor:
+    def p12_widen(self, lo, hi4, table, esc_idx, esc_val, n: int, shape: Sequence[int],
+                  out: torch.Tensor | None = None) -> torch.Tensor:
         """a packed tensor back to bf16 on the GPU (`unpack_bf16`), through the matvec's own in-register widen"""
         for t, what in ((lo, "lo"), (hi4, "hi4"), (table, "table")):
             self._need(t, torch.uint8, what)
-        out = torch.empty(tuple(shape), dtype=torch.bfloat16, device=lo.device)
+        if out is None:
+            out = torch.empty(tuple(shape), dtype=torch.bfloat16, device=lo.device)
+        else:
+            self._need(out, torch.bfloat16, "out")
+            if out.numel() != int(n):
+                raise ValueError(f"[hip] p12_widen: out holds {out.numel()} values, the tensor has {int(n)}")
         ne = 0 if esc_idx is None else int(esc_idx.numel())
         if ne:
             self._need(esc_idx, torch.int32, "esc_idx")

@@ -82,7 +82,8 @@ int32_t btb_hip_gemv_bf16_norm(const void* w, const void* h_in, const void* y, c
 
 /* The matvec over a pack12 matrix (n = R * C weights): lo u8[n], hi4 u8[(n + 1) / 2] (weight 2k in the low nibble
  * of byte k), table u8[16], esc_idx i32[n_esc] strictly ascending, esc_val u8[n_esc] - the arrays of
- * btb_gemv_p12_rows (native/src/lib.rs:114-135), on the device - plus row_ptr i32[R + 1] from btb_hip_p12_row_ptr.
+ * btb_gemv_p12_rows (native/src/lib.rs:114-135), on the device, the list validated at upload by btb_hip_p12_check -
+ * plus row_ptr i32[R + 1] from btb_hip_p12_row_ptr.
  * x [M, C] bf16, y [M, R] bf16; C a multiple of 16, lo 16-byte and hi4 8-byte aligned. The reference has no card
  * kernel for this form (it widens a packed layer to bf16 before the card holds it: btb/engine/tiers.py:1200-1216). */
 int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
@@ -99,6 +100,14 @@ int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table
  * matvec reads. Run once when a packed matrix is uploaded; replaces the per-call search of p12_cursors
  * (native/src/gemv.rs:719-734). */
 int32_t btb_hip_p12_row_ptr(const void* esc_idx, size_t n_esc, size_t rows, size_t cols, void* row_ptr, void* stream);
+
+/* Validates a packed tensor's escape list on the device, once, when it is uploaded: BTB_ERR_DOMAIN unless esc_idx
+ * i32[n_esc] is strictly ascending with every entry in [0, n) - the lists btb_gemv_p12_rows refuses per call
+ * (native/src/gemv.rs:4171-4189; native/src/lib.rs:114-135 "strictly ascending"). The matvec and widen entry points
+ * index the low bytes and x with these entries and do not re-check them, so a list from an untrusted store goes
+ * through here first. `flag` is one device int32 the check may write. Synchronous (it reads the verdict back and
+ * waits for `stream`), so it is not for graph capture. n_esc == 0 launches nothing. */
+int32_t btb_hip_p12_check(const void* esc_idx, size_t n_esc, size_t n, int32_t* flag, void* stream);
 
 /* A packed tensor of n weights back to bf16 [n], escapes applied: unpack_bf16 (btb/pack12.py:70-97) on the device,
  * through the same in-register widen the matvec uses. out 16-byte aligned. */
@@ -144,7 +153,8 @@ int32_t btb_hip_gemv_bf16_group(size_t n, const uint16_t* const* w, const size_t
                                 const float* const* x, const size_t* b, float* const* y, void* stream);
 
 /* btb_gemv_p12_rows (native/src/lib.rs:114-135) on the device, bit-identical to it and so to the bf16 form. The
- * escape list's ascending order is not re-checked here (that would copy it back to the host). */
+ * escape list is not re-checked per call (that would copy a verdict back to the host every time): validate it once
+ * at upload with btb_hip_p12_check. */
 int32_t btb_hip_gemv_p12_rows(const uint8_t* lo, const uint8_t* hi4, const uint8_t* table, const int32_t* esc_idx,
                               const uint8_t* esc_val, size_t n_esc, size_t rows, size_t cols, const float* x, size_t b,
                               float* y, void* stream);

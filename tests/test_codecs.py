@@ -163,3 +163,37 @@ def test_mxfp4_encoder_round_trip_and_agreement():
     assert torch.equal(mxfp4.dequantize(pb2, ps2), deq)
     unit = mxfp4.scale_factors(ps)[..., None]
     assert torch.all((deq - w).abs().reshape(16, 8, 32) <= 2.0 * unit)
+
+
+# -- a damaged 12-bit store is refused before it reaches a kernel -----------------------------------------------------
+
+
+@pytest.mark.parametrize("bad", [[5, 5], [9, 3], [0, 32], [-1, 4]])   # the lists native/src/gemv.rs:4171-4189 refuses
+def test_pack12_bad_escape_lists_are_refused(bad):
+    with pytest.raises(ValueError):
+        pack12.check_escapes(torch.tensor(bad, dtype=torch.int32), torch.zeros(2, dtype=torch.uint8), 32)
+
+
+def test_pack12_escape_list_checks():
+    pack12.check_escapes(torch.tensor([0, 7, 31], dtype=torch.int32), torch.zeros(3, dtype=torch.uint8), 32)
+    pack12.check_escapes(torch.empty(0, dtype=torch.int32), torch.empty(0, dtype=torch.uint8), 32)
+    with pytest.raises(ValueError):   # as many values as indices
+        pack12.check_escapes(torch.tensor([1, 2], dtype=torch.int32), torch.zeros(3, dtype=torch.uint8), 32)
+
+
+def test_pack12_split_refuses_a_body_of_the_wrong_length(parent):
+    w = parent["model.layers.0.mlp.down_proj.weight"]
+    body, meta = pack12.blob(w)
+    lo, hi4, table, ei, ev, shape = pack12.split(body, meta)
+    assert shape == list(w.shape) and ei.numel() == ev.numel()
+    assert torch.equal(pack12.unpack_bf16(lo, hi4, table, w.numel(), shape, ei, ev).view(torch.int16), w.view(torch.int16))
+    with pytest.raises(ValueError):
+        pack12.split(body[:-4], meta)
+    with pytest.raises(ValueError):
+        pack12.split(torch.cat([body, body.new_zeros(4)]), meta)
+    more = meta.clone()
+    more[16] += 1                      # one more escape than the body holds
+    with pytest.raises(ValueError):
+        pack12.split(body, more)
+    with pytest.raises(ValueError):
+        pack12.entry(bytes(meta[:20].numpy().tobytes()))

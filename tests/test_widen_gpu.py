@@ -67,6 +67,52 @@ def test_p12_row_ptr(card):
     assert torch.all(empty == 0)
 
 
+@pytest.mark.parametrize("bad", [[5, 5], [9, 3], [0, 32], [-1, 4]])   # the lists native/src/gemv.rs:4171-4189 refuses
+def test_p12_bad_escape_lists_are_refused_at_upload(card, bad):
+    """btb_hip_p12_check returns ERR_DOMAIN for them, raw through the C ABI, and `P12Weight` refuses to come into
+    being - so no matvec or widen kernel is ever handed such a list"""
+    import ctypes
+
+    from btb_amd import native
+    from btb_amd.pack12 import P12Weight
+
+    ei = torch.tensor(bad, dtype=torch.int32, device="cuda")
+    flag = torch.zeros(1, dtype=torch.int32, device="cuda")
+    P = lambda t: ctypes.c_void_p(t.data_ptr())
+    st = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    assert card.lib.btb_hip_p12_check(P(ei), 2, 32, P(flag), st) == native.ERR_DOMAIN
+    assert card.lib.btb_hip_p12_check(None, 2, 32, P(flag), st) == native.ERR_NULL
+    assert card.lib.btb_hip_p12_check(P(ei), 33, 32, P(flag), st) == native.ERR_DOMAIN   # more escapes than weights
+    good = torch.tensor([3, 9], dtype=torch.int32, device="cuda")
+    assert card.lib.btb_hip_p12_check(P(good), 2, 32, P(flag), st) == native.OK
+    assert card.lib.btb_hip_p12_check(None, 0, 32, None, st) == native.OK                # no list: nothing to check
+    z = lambda n: torch.zeros(n, dtype=torch.uint8, device="cuda")
+    with pytest.raises(ValueError):
+        P12Weight(z(32), z(16), z(16), ei, z(2), 4, 8, card)
+    with pytest.raises(ValueError):
+        card.p12_check(ei, 32)
+    P12Weight(z(32), z(16), z(16), good, z(2), 4, 8, card)
+
+
+def test_p12_widen_skips_escape_indices_outside_the_tensor(card):
+    """the patch kernel itself never writes outside `out`, whatever the list holds (the fences stay as they were)"""
+    n = 64
+    lo = torch.arange(n, dtype=torch.uint8, device="cuda")
+    hi4 = torch.zeros(n // 2, dtype=torch.uint8, device="cuda")
+    table = torch.zeros(16, dtype=torch.uint8, device="cuda")
+    ei = torch.tensor([-7, 5, n, 2**30], dtype=torch.int32, device="cuda")
+    ev = torch.tensor([1, 2, 3, 4], dtype=torch.uint8, device="cuda")
+    buf = torch.full((n + 64,), 0x7777, dtype=torch.int16, device="cuda")
+    out = buf[32 : 32 + n].view(torch.bfloat16)
+    card.p12_widen(lo, hi4, table, ei, ev, n, (n,), out=out)
+    torch.cuda.synchronize()
+    assert bool((buf[:32] == 0x7777).all()) and bool((buf[32 + n :] == 0x7777).all())
+    got = out.view(torch.int16).cpu().numpy().astype(np.uint16)
+    want = np.arange(n, dtype=np.uint16)
+    want[5] |= 2 << 8
+    assert np.array_equal(got, want)
+
+
 # -- fp8 ---------------------------------------------------------------------------------------------------------------
 
 
