@@ -71,6 +71,7 @@ static Knob g_knobs[] = {
     {"mfma_stream_x", {-1}},
     {"moe_wgs_per_cu", {-1}},
     {"attn_split", {-1}},
+    {"attn_heads_per_wg", {-1}},
 };
 
 int tuning(const char* key) {

@@ -82,6 +82,19 @@ __device__ __forceinline__ void load_keys(KeyBatch& kb, const uint16_t* Kh, cons
     }
 }
 
+// the same batch with addresses that do not depend on how many keys the cache holds: a key at or past `lim` (the end of
+// the span or of the cache's capacity) reads slot lim - 1 again. Which of the batch's keys count is decided when they
+// are used; the step's own slot may be read here before its row has landed - use_keys takes that key from LDS.
+__device__ __forceinline__ void load_keys_upto(KeyBatch& kb, const uint16_t* Kh, const uint16_t* Vh, long long rs,
+                                               int key0, int lim) {
+#pragma unroll
+    for (int b = 0; b < KB; ++b) {
+        const int key = min(key0 + 16 * b, lim - 1);
+        kb.k[b] = *reinterpret_cast<const uint4*>(Kh + (size_t)key * rs);
+        kb.v[b] = *reinterpret_cast<const uint4*>(Vh + (size_t)key * rs);
+    }
+}
+
 // The batch's keys folded into the G query heads' online-softmax states, a batch at a time: the 8 x G scores first
 // (q and the key row meet as bf16 pairs in v_dot2_f32_bf16 - products exact, f32 sums - then the 16 lanes' sums are
 // folded and scaled into log2 units), then per head one new maximum, one correction of the running sum and output for
@@ -89,8 +102,10 @@ __device__ __forceinline__ void load_keys(KeyBatch& kb, const uint16_t* Kh, cons
 // span's end scores -inf and weighs 0. qp: the heads' q, this lane's 8 dims as 4 bf16 pairs. own >= 0: the step's
 // own row is key `own` and is taken from LDS (s_k, s_v) - the cache's copy may not have landed yet.
 // tree_base >= 0: the keys from slot tree_base on are the pass's own rows, and of those the row sees the ones whose
-// bit is set in tree_mask (its ancestors and itself: a verify pass's tree).
-template <int G>
+// bit is set in tree_mask (its ancestors and itself: a verify pass's tree). ZERO_DEAD: a key that does not count may
+// have been loaded from a slot the cache has never written (load_keys_upto), so its value row is taken as zeros -
+// weight 0 times whatever bits lie there must not make a NaN.
+template <int G, bool ZERO_DEAD = false>
 __device__ __forceinline__ void use_keys(KeyBatch& kb, int key0, int k_end, int own, const uint16_t* s_k,
                                          const uint16_t* s_v, int dl, const uint32_t (&qp)[G][4], float scale_log2,
                                          float (&m)[G], float (&l)[G], float (&acc)[G][8], int tree_base = -1,
@@ -111,6 +126,7 @@ __device__ __forceinline__ void use_keys(KeyBatch& kb, int key0, int k_end, int 
         const int key = key0 + 16 * b;
         bool live = key < k_end;
         if (tree_base >= 0) live = live && (key < tree_base || ((tree_mask >> min(key - tree_base, 31)) & 1u) != 0u);
+        if (ZERO_DEAD && !live) kb.v[b] = make_uint4(0u, 0u, 0u, 0u);
 #pragma unroll
         for (int j = 0; j < G; ++j) {
             float sc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr.x), __builtin_bit_cast(bf16x2, qp[j][0]), 0.f, false);

@@ -16,7 +16,9 @@ enum XMode { X_PLAIN = 0, X_SILU = 1, X_ADDNORM = 2 };
 
 // where x comes from. X_PLAIN: x [M, C]. X_SILU: x is gu [M, 2C]. X_ADDNORM: x is the residual h [M, C]; y the block
 // output added to it (or null), norm_w the norm's weight, h_out where the new residual is written (not h itself:
-// other workgroups are still reading it).
+// other workgroups are still reading it). With `ids` (X_ADDNORM only) x is an embedding table [vocab, C] and row m of
+// the residual is table[ids[m]] (an id outside the table is clamped into it): the step's first layer, whose residual
+// is the token's embedding.
 struct XArgs {
     const uint16_t* x;
     const uint16_t* y;
@@ -24,6 +26,8 @@ struct XArgs {
     uint16_t* h_out;
     float eps;
     int centered;
+    const int32_t* ids = nullptr;
+    int vocab = 0;
 };
 
 // the fold the reference's btb_gemv_silu_bf16 makes in its x load (native/cuda/btb_kernels.cu:168-209):
@@ -98,7 +102,9 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
         constexpr int PER = 3;  // words a thread holds at once: rows up to 3072 wide take one pass
         const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr;
         for (int m = 0; m < M; ++m) {
-            const uint2* hs = reinterpret_cast<const uint2*>(a.x + (size_t)m * C);
+            size_t hrow = (size_t)m;
+            if (a.ids != nullptr) hrow = (size_t)min(max(a.ids[m], 0), a.vocab - 1);  // uniform: one scalar load
+            const uint2* hs = reinterpret_cast<const uint2*>(a.x + hrow * C);
             const uint2* ys = a.y == nullptr ? hs : reinterpret_cast<const uint2*>(a.y + (size_t)m * C);
             const uint2* ws = reinterpret_cast<const uint2*>(a.norm_w);
             uint2* row = rows4 + (size_t)m * n4;

@@ -258,7 +258,10 @@ static int32_t run_rows(const typename F::Params& p, XArgs xa, void* y, size_t R
         const int mm = (int)(M - m0 < 4 ? M - m0 : 4);
         int32_t rc = launch_by_m<F, XMODE, EPI>(p, xa, yp + m0 * y_row, (int)R, (int)C, mm, st);
         if (rc != OK) return rc;
-        xa.x += 4 * x_row;
+        if (xa.ids != nullptr)
+            xa.ids += 4;
+        else
+            xa.x += 4 * x_row;
         if (xa.y != nullptr) xa.y += 4 * C;
         if (xa.h_out != nullptr) xa.h_out += 4 * C;
     }
@@ -304,6 +307,17 @@ static int32_t norm_args(const void* h_in, const void* y, const void* norm_w, fl
     if (!aligned2(h_in) || !aligned2(y) || !aligned2(norm_w) || !aligned2(h_out)) return ERR_DOMAIN;
     *xa = XArgs{static_cast<const uint16_t*>(h_in), static_cast<const uint16_t*>(y),
                 static_cast<const uint16_t*>(norm_w), static_cast<uint16_t*>(h_out), eps, centered ? 1 : 0};
+    return OK;
+}
+
+// the arguments of the entry points whose residual is an embedding row per id
+static int32_t embed_args(const void* table, const int32_t* ids, size_t vocab, const void* norm_w, float eps,
+                          int32_t centered, void* h_out, XArgs* xa) {
+    if (table == nullptr || ids == nullptr || norm_w == nullptr) return ERR_NULL;
+    if (!(eps >= 0.f) || vocab == 0 || vocab > 0x7FFFFFFFull) return ERR_DOMAIN;
+    if (!aligned16(table) || (reinterpret_cast<uintptr_t>(ids) & 3u) || !aligned2(norm_w) || !aligned2(h_out)) return ERR_DOMAIN;
+    *xa = XArgs{static_cast<const uint16_t*>(table), nullptr, static_cast<const uint16_t*>(norm_w),
+                static_cast<uint16_t*>(h_out), eps, centered ? 1 : 0, ids, (int)vocab};
     return OK;
 }
 
@@ -396,6 +410,20 @@ int32_t btb_hip_gemv_bf16_norm(const void* w, const void* h_in, const void* y, c
                : run_rows<FmtBf16, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, st);
 }
 
+int32_t btb_hip_gemv_bf16_embed_norm(const void* w, const void* table, const int32_t* ids, size_t vocab,
+                                     const void* norm_w, float eps, int32_t centered, void* h_out, void* out, size_t R,
+                                     size_t C, size_t M, void* stream) {
+    if (w == nullptr || out == nullptr) return ERR_NULL;
+    XArgs xa;
+    int32_t rc = embed_args(table, ids, vocab, norm_w, eps, centered, h_out, &xa);
+    if (rc != OK) return rc;
+    rc = check_dims(R, C, M, FmtBf16::UW);
+    if (rc != OK) return rc;
+    if (!aligned16(w) || !aligned2(out)) return ERR_DOMAIN;
+    FmtBf16::Params p{static_cast<const uint4*>(w)};
+    return run_rows<FmtBf16, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, static_cast<hipStream_t>(stream));
+}
+
 int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
                          size_t n_esc, const void* row_ptr, const void* x, void* y, size_t R, size_t C, size_t M,
                          void* stream) {
@@ -441,6 +469,25 @@ int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table
     hipStream_t st = static_cast<hipStream_t>(stream);
     return glu ? run_rows<FmtP12, X_ADDNORM, E_GLU>(p, xa, out, R, C, M, st)
                : run_rows<FmtP12, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, st);
+}
+
+int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void* table, const void* esc_idx,
+                                    const void* esc_val, size_t n_esc, const void* row_ptr, const void* embed,
+                                    const int32_t* ids, size_t vocab, const void* norm_w, float eps, int32_t centered,
+                                    void* h_out, void* out, size_t R, size_t C, size_t M, void* stream) {
+    if (out == nullptr) return ERR_NULL;
+    FmtP12::Params p;
+    XArgs xa;
+    int32_t rc = embed_args(embed, ids, vocab, norm_w, eps, centered, h_out, &xa);
+    if (rc == ERR_NULL) return rc;
+    const int32_t rp = p12_params(lo, hi4, table, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
+    if (rp == ERR_NULL) return rp;
+    if (rc != OK) return rc;
+    if (rp != OK) return rp;
+    rc = check_dims(R, C, M, FmtP12::UW);
+    if (rc != OK) return rc;
+    if (!aligned2(out)) return ERR_DOMAIN;
+    return run_rows<FmtP12, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, static_cast<hipStream_t>(stream));
 }
 
 int32_t btb_hip_gemv_fp8(const void* w, const void* scales, size_t sr, size_t sc, const void* x, void* y, size_t R,

@@ -287,12 +287,16 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
                     });
 }
 
-// The step's own form (one row): the kernel reads the fused qkv row itself. Each workgroup norms and ropes the G query
-// heads of its kv head (a wave a head; the result never leaves LDS), and the workgroup whose span holds slot *n0 also
-// norms and ropes the new key, copies the new value, writes both into the cache and takes them from LDS where its
-// stream reaches that slot. One launch (norm_rope_kv) less, and the stream's first keys are requested before q is
-// touched. The arithmetic is norm_rope_kv_kernel's followed by attn_decode_kernel's: the states it leaves are theirs.
-template <int G>
+// The step's own form (one row): the kernel reads the fused qkv row itself. A workgroup takes GW of a kv head's query
+// heads (all of them, or fewer: the heads of one kv head then sit in workgroups that share a die's L2, so the keys still
+// leave memory once) and one span of the keys. It norms and ropes its query heads (a wave a head; the result never
+// leaves LDS), and a workgroup whose span holds slot *n0 also norms and ropes the new key and copies the new value
+// into LDS, where its stream takes them from; the first of those workgroups writes both into the cache. One launch
+// (norm_rope_kv) less. The key stream's first batch is requested before anything else and its addresses do not depend
+// on *n0 (they are clamped to the span and the cache's capacity; which keys count is decided afterwards), so the
+// batch travels while *n0, the rope tables and the heads' inputs come in and the heads are prepared. The arithmetic
+// is norm_rope_kv_kernel's followed by attn_decode_kernel's: the states it leaves are theirs.
+template <int GW>
 __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __restrict__ qkv, const uint16_t* __restrict__ wq,
                                                               const uint16_t* __restrict__ wk, float eps, int centered,
                                                               const uint16_t* __restrict__ cos_t,
@@ -301,80 +305,90 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
                                                               uint16_t* __restrict__ V, int Hq, int Hk, long long hs,
                                                               long long rs, float scale_log2, float* __restrict__ part_m,
                                                               float* __restrict__ part_l, float* __restrict__ part_acc,
-                                                              int span) {
+                                                              int span, int cap) {
     constexpr int D = ATT_D;
-    __shared__ uint32_t s_q[G][D / 2];  // the heads' q after norm and rope, bf16 pairs
+    __shared__ uint32_t s_q[GW][D / 2];  // the heads' q after norm and rope, bf16 pairs
     __shared__ __align__(16) uint16_t s_k[D], s_v[D];
-    __shared__ float s_m[16][G], s_l[16][G];
-    __shared__ __align__(16) float s_acc[16][G][D];
-    const int g = blockIdx.x, sp = blockIdx.y, S = gridDim.y;
+    __shared__ float s_m[16][GW], s_l[16][GW];
+    __shared__ __align__(16) float s_acc[16][GW][D];
+    const int Gt = Hq / Hk;                                  // query heads a kv head
+    const int g = blockIdx.x % Hk, part = blockIdx.x / Hk;   // consecutive workgroups: consecutive kv heads
+    const int j0 = part * GW;                                // the first of this workgroup's heads among the Gt
+    const int sp = blockIdx.y, S = gridDim.y;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int sub = lane >> 4, dl = lane & 15, grp = wv * 4 + sub;
-    const int n0 = *n0p;
-    const int k_begin = sp * span, k_end = min(n0 + 1, k_begin + span);
+    const int k_begin = sp * span;
+    const int k_lim = max(min(k_begin + span, cap), 1);      // the last slot of the cache this span may touch, + 1
     const uint16_t* Kh = K + (size_t)g * hs + dl * 8;
     const uint16_t* Vh = V + (size_t)g * hs + dl * 8;
-    // requests in the order their answers are needed (loads come back in order): the heads' inputs - a few words out
-    // of L2 - then the stream's first keys; the norm and rope then run while the keys travel
-    constexpr int NQ = (G + 3) / 4;  // query heads a wave prepares
+    const int key_first = k_begin + grp;
+    KeyBatch kb;
+    load_keys_upto(kb, Kh, Vh, rs, key_first, k_lim);
+
+    const int n0 = *n0p;
+    const int k_end = min(n0 + 1, k_begin + span);
+    constexpr int NQ = (GW + 3) / 4;  // query heads a wave prepares
     HeadIn qin[NQ];
 #pragma unroll
     for (int i = 0; i < NQ; ++i)
-        qin[i] = head_request<false>(qkv + (size_t)(g * G + min(wv + 4 * i, G - 1)) * D, wq, cos_t, sin_t, n0, lane);
+        qin[i] = head_request<false>(qkv + (size_t)(g * Gt + j0 + min(wv + 4 * i, GW - 1)) * D, wq, cos_t, sin_t, n0, lane);
     const bool holds_own = n0 >= k_begin && n0 < k_begin + span;  // this workgroup's span holds the new slot
-    const bool owner = wv == 3 && holds_own;
+    const bool preps_k = wv == 3 && holds_own;
     const HeadIn kin = head_request<false>(qkv + (size_t)(Hq + g) * D, wk, cos_t, sin_t, n0, lane);
     const uint32_t vraw = reinterpret_cast<const uint32_t*>(qkv + (size_t)(Hq + Hk + g) * D)[lane];
-    KeyBatch kb = {};
-    const int key_first = k_begin + grp;
-    load_keys(kb, Kh, Vh, rs, min(key_first, max(k_end - 1, 0)), max(k_end, 1), n0);
 
 #pragma unroll
     for (int i = 0; i < NQ; ++i) {
         const int j = wv + 4 * i;
         uint16_t o[2];
         head_finish(qin[i], wq != nullptr, eps, centered, lane, o);
-        if (j < G) s_q[j][lane] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+        if (j < GW) s_q[j][lane] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
     }
-    if (owner) {
+    if (preps_k) {
         uint16_t o[2];
         head_finish(kin, wk != nullptr, eps, centered, lane, o);
         s_k[lane * 2] = o[0];
         s_k[lane * 2 + 1] = o[1];
         s_v[lane * 2] = (uint16_t)(vraw & 0xFFFFu);
         s_v[lane * 2 + 1] = (uint16_t)(vraw >> 16);
-        reinterpret_cast<uint32_t*>(K + (size_t)g * hs + (size_t)n0 * rs)[lane] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
-        reinterpret_cast<uint32_t*>(V + (size_t)g * hs + (size_t)n0 * rs)[lane] = vraw;
+        if (part == 0) {
+            reinterpret_cast<uint32_t*>(K + (size_t)g * hs + (size_t)n0 * rs)[lane] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+            reinterpret_cast<uint32_t*>(V + (size_t)g * hs + (size_t)n0 * rs)[lane] = vraw;
+        }
     }
     __syncthreads();
 
-    uint32_t qp[G][4];
+    uint32_t qp[GW][4];
 #pragma unroll
-    for (int j = 0; j < G; ++j)
+    for (int j = 0; j < GW; ++j)
 #pragma unroll
         for (int e = 0; e < 4; ++e) qp[j][e] = s_q[j][dl * 4 + e];
-    float m[G], l[G], acc[G][8];
+    float m[GW], l[GW], acc[GW][8];
 #pragma unroll
-    for (int j = 0; j < G; ++j) {
+    for (int j = 0; j < GW; ++j) {
         m[j] = bits_f32(0xff800000u);
         l[j] = 0.f;
 #pragma unroll
         for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
     }
-    for (int key0 = key_first; key0 < k_end;) {
-        use_keys<G>(kb, key0, k_end, holds_own ? n0 : -1, s_k, s_v, dl, qp, scale_log2, m, l, acc);
-        key0 += 16 * KB;
-        if (key0 < k_end) load_keys(kb, Kh, Vh, rs, key0, k_end, n0);
+    // a span of several batches asks for the next one before it folds the current one in (past the span's end the
+    // request falls on its last key again and is dropped)
+    const bool batches = k_begin + 16 * KB < k_end;  // uniform: the span holds more than one batch of live keys
+    for (int key0 = key_first; key0 < k_end; key0 += 16 * KB) {
+        KeyBatch nx;
+        if (batches) load_keys_upto(nx, Kh, Vh, rs, key0 + 16 * KB, k_lim);
+        use_keys<GW, true>(kb, key0, k_end, holds_own ? n0 : -1, s_k, s_v, dl, qp, scale_log2, m, l, acc);
+        if (batches) kb = nx;
     }
     const size_t prow = (size_t)g * S + sp;
-    fold_streams<G>(m, l, acc, grp, dl, &s_m[0][0], &s_l[0][0], &s_acc[0][0][0], threadIdx.x,
-                    [&](int j, int d, float M, float L, float A) {
-                        part_acc[(prow * G + j) * D + d] = A;
-                        if (d == 0) {
-                            part_m[prow * G + j] = M;
-                            part_l[prow * G + j] = L;
-                        }
-                    });
+    fold_streams<GW>(m, l, acc, grp, dl, &s_m[0][0], &s_l[0][0], &s_acc[0][0][0], threadIdx.x,
+                     [&](int j, int d, float M, float L, float A) {
+                         part_acc[((prow * Gt) + j0 + j) * D + d] = A;
+                         if (d == 0) {
+                             part_m[prow * Gt + j0 + j] = M;
+                             part_l[prow * Gt + j0 + j] = L;
+                         }
+                     });
 }
 
 // the spans' states folded in span order: one workgroup per (row, kv head). Launched right after attn_decode_kernel,
@@ -406,8 +420,12 @@ __global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restric
 // it is strictly larger than its best so far (a tie keeps the earlier; a NaN never wins; the scan starts from -inf as
 // native/src/sample.rs:53-67 does), then the (value, index) maximum over the block in the total order value descending,
 // index ascending
+// PUBLISH: one row, and the thread that holds the pick goes on with the step's end (publish_kernel's duties) - one
+// launch less at the end of a step.
+template <bool PUBLISH>
 __global__ void __launch_bounds__(1024) argmax_kernel(const uint16_t* __restrict__ logits, int32_t* __restrict__ out,
-                                                      int V) {
+                                                      int V, int32_t* __restrict__ n0, int32_t* __restrict__ next_ids,
+                                                      int32_t* out_tok, int32_t* out_n0, long long* out_ts) {
     __shared__ float s_v[16];
     __shared__ int s_i[16];
     const int t = blockIdx.x, tid = threadIdx.x;
@@ -467,7 +485,19 @@ __global__ void __launch_bounds__(1024) argmax_kernel(const uint16_t* __restrict
                 bv = s_v[k];
                 bi = s_i[k];
             }
-        out[t] = bi == 0x7fffffff ? 0 : bi;  // nothing above -inf (or only NaNs): index 0, as the reference's scan
+        const int tok = bi == 0x7fffffff ? 0 : bi;  // nothing above -inf (or only NaNs): index 0, as the reference's scan
+        out[t] = tok;
+        if constexpr (PUBLISH) {
+            const int len = *n0 + 1;
+            if (next_ids != nullptr) *next_ids = tok;
+            *n0 = len;
+            if (out_tok != nullptr) {
+                *out_tok = tok;
+                if (out_ts != nullptr) *out_ts = (long long)wall_clock64();
+                __threadfence_system();
+                if (out_n0 != nullptr) *out_n0 = len;
+            }
+        }
     }
 }
 
@@ -650,28 +680,43 @@ int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk,
     float* part_l = workspace + Hq * S;
     float* part_acc = workspace + 2 * Hq * S;
     const float scale_log2 = scale * 1.4426950408889634f;
-    const dim3 grid((unsigned)Hk, (unsigned)S);
     hipStream_t st = static_cast<hipStream_t>(stream);
     const dim3 mgrid((unsigned)Hk, 1);
     const size_t mlds = 2 * S * G * sizeof(float);
-#define ATT(GG)                                                                                                      \
-    hipLaunchKernelGGL(attn_decode_qkv_kernel<GG>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(qkv),        \
+    // query heads a workgroup takes: all G of its kv head, or fewer (the workgroups of one kv head are Hk apart in
+    // the grid, which on this GPU - workgroups dealt to its eight dies in turn - keeps them on one die when Hk is 8)
+    // Measured on MI355X (Qwen3-4B shape, 4096 keys, whole step): two heads a workgroup and 16 spans 2.295 ms, four
+    // heads and 32 spans 2.371, one head and 8 spans 2.351 - each 256 workgroups.
+    int gw = tuning("attn_heads_per_wg");
+    if (gw <= 0 || gw > (int)G || G % gw != 0 || (gw & (gw - 1)) != 0) gw = G >= 4 ? 2 : (int)G;
+    const dim3 grid((unsigned)(Hk * (G / gw)), (unsigned)S);
+#define ATT(GW)                                                                                                      \
+    hipLaunchKernelGGL(attn_decode_qkv_kernel<GW>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(qkv),        \
                        static_cast<const uint16_t*>(wq), static_cast<const uint16_t*>(wk), eps, centered ? 1 : 0,    \
                        static_cast<const uint16_t*>(cos_t), static_cast<const uint16_t*>(sin_t), n0,                 \
                        static_cast<uint16_t*>(K), static_cast<uint16_t*>(V), (int)Hq, (int)Hk, (long long)hs,        \
-                       (long long)rs, scale_log2, part_m, part_l, part_acc, span);                                   \
+                       (long long)rs, scale_log2, part_m, part_l, part_acc, span, (int)cap)
+#define MERGE(GG)                                                                                                    \
     hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,       \
                        (int)Hk, (int)S, part_m, part_l, part_acc)
-    switch (G) {
+    if (G != 1 && G != 2 && G != 4 && G != 8) {
+        set_error("attn_decode_qkv: 1, 2, 4 or 8 query heads per kv head");
+        return ERR_DOMAIN;
+    }
+    switch (gw) {
         case 1: ATT(1); break;
         case 2: ATT(2); break;
         case 4: ATT(4); break;
-        case 8: ATT(8); break;
-        default:
-            set_error("attn_decode_qkv: 1, 2, 4 or 8 query heads per kv head");
-            return ERR_DOMAIN;
+        default: ATT(8); break;
+    }
+    switch (G) {
+        case 1: MERGE(1); break;
+        case 2: MERGE(2); break;
+        case 4: MERGE(4); break;
+        default: MERGE(8); break;
     }
 #undef ATT
+#undef MERGE
     return hip_status(hipGetLastError(), "attn_decode_qkv launch");
 }
 
@@ -688,9 +733,19 @@ int32_t btb_hip_silu_mul(const void* gu, void* m, size_t T, size_t I, void* stre
 int32_t btb_hip_argmax(const void* logits, int32_t* out, size_t T, size_t V, void* stream) {
     if (logits == nullptr || out == nullptr) return ERR_NULL;
     if (T == 0 || V == 0 || T > 0x7FFFFFFFull || V > 0x7FFFFFFEull) return ERR_DOMAIN;
-    hipLaunchKernelGGL(argmax_kernel, dim3((unsigned)T), dim3(1024), 0, static_cast<hipStream_t>(stream),
-                       static_cast<const uint16_t*>(logits), out, (int)V);
+    hipLaunchKernelGGL(argmax_kernel<false>, dim3((unsigned)T), dim3(1024), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t*>(logits), out, (int)V, nullptr, nullptr, nullptr, nullptr, nullptr);
     return hip_status(hipGetLastError(), "argmax launch");
+}
+
+int32_t btb_hip_argmax_publish(const void* logits, size_t V, int32_t* picked, int32_t* n0, int32_t* next_ids,
+                               int32_t* out_tok, int32_t* out_n0, int64_t* out_ts, void* stream) {
+    if (logits == nullptr || picked == nullptr || n0 == nullptr) return ERR_NULL;
+    if (V == 0 || V > 0x7FFFFFFEull) return ERR_DOMAIN;
+    hipLaunchKernelGGL(argmax_kernel<true>, dim3(1), dim3(1024), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint16_t*>(logits), picked, (int)V, n0, next_ids, out_tok, out_n0,
+                       reinterpret_cast<long long*>(out_ts));
+    return hip_status(hipGetLastError(), "argmax_publish launch");
 }
 
 int32_t btb_hip_publish(int32_t* n0, const int32_t* picked, int32_t* next_ids, int32_t* out_tok, int32_t* out_n0,

@@ -130,6 +130,10 @@ class DecodeStep:
         # the [2560 / 9728] stack at 4096 keys: 8 rows 4.32 ms a pass with 32 spans, 3.83 with 8; 16 rows 5.6 / 4.7)
         if attn_spans is None:
             attn_spans = max(1, min(self.cap // 64, (card.sms + Hk - 1) // Hk, (2 * card.sms) // (Hk * self.T)))
+            if self.T == 1 and D == 128 and Hq // Hk >= 4:
+                # the step's own attention kernel splits a kv head's query heads over workgroups of two heads: one
+                # workgroup a CU then means a CU's worth of (kv head, head pair, span) triples
+                attn_spans = max(1, min(self.cap // 64, card.sms // (Hk * (Hq // Hk // 2))))
         self.S = int(attn_spans)
         self.scratch = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
         # Which sequence: up to three rows the fused launches win (fewer launches, every matvec on the streaming
@@ -313,12 +317,14 @@ class DecodeStep:
         k, cfg, w = self.card, self.cfg, self.w
         Hq, Hk, D = cfg.q_heads, cfg.kv_heads, cfg.head_dim
         ha, hb = self.h, self.h2
-        k.embed(w["embed"], self.ids, ha)
         y_prev = None
         for i in range(cfg.layers):
             L = f"layers.{i}."
             K, V = self.kv[i, 0], self.kv[i, 1]
-            k.gemv_norm(w[L + "qkv"].w, ha, y_prev, w[L + "ln1"], cfg.eps, hb, self.qkv)
+            if i == 0:  # the residual starts as the tokens' embedding rows, gathered by the first matvec itself
+                k.gemv_embed_norm(w[L + "qkv"].w, w["embed"], self.ids, w[L + "ln1"], cfg.eps, hb, self.qkv)
+            else:
+                k.gemv_norm(w[L + "qkv"].w, ha, y_prev, w[L + "ln1"], cfg.eps, hb, self.qkv)
             if self.T == 1 and D == 128:
                 k.attn_decode_qkv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K,
                                   V, self.att, Hq, Hk, D, self.scale, self.S, self.scratch)
@@ -332,8 +338,11 @@ class DecodeStep:
             w[L + "down"].matvec(self.m, self.y)
             y_prev = self.y
         k.gemv_norm(w["head"].w, ha, y_prev, w["norm"], cfg.eps, None, self.logits)
-        k.argmax(self.logits, self.picked)
-        k.publish(self.n0, self.picked, self.ids, self.host_tok, self.host_n0, self.host_ts)
+        if self.T == 1:
+            k.argmax_publish(self.logits, self.picked, self.n0, self.ids, self.host_tok, self.host_n0, self.host_ts)
+        else:
+            k.argmax(self.logits, self.picked)
+            k.publish(self.n0, self.picked, self.ids, self.host_tok, self.host_n0, self.host_ts)
 
     def capture(self, warmup: int = 2) -> torch.cuda.CUDAGraph:
         """run the step eagerly (on a side stream, as a capture requires), then record it: the hipGraph the host

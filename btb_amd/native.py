@@ -36,6 +36,9 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_gemv_silu_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_gemv_glu_silu_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_gemv_bf16_norm": (_i32, [_vp, _vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp, _sz, _sz, _sz, _i32, _vp]),
+    "btb_hip_gemv_bf16_embed_norm": (_i32, [_vp, _vp, _vp, _sz, _vp, ctypes.c_float, _i32, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_gemv_p12_embed_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _vp, ctypes.c_float, _i32,
+                                           _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_gemv_p12_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp,
                                      _sz, _sz, _sz, _i32, _vp]),
     "btb_hip_gemv_p12": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
@@ -70,6 +73,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_silu_mul": (_i32, [_vp, _vp, _sz, _sz, _vp]),
     "btb_hip_argmax": (_i32, [_vp, _vp, _sz, _sz, _vp]),
     "btb_hip_publish": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "btb_hip_argmax_publish": (_i32, [_vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_step_sync_bytes": (_sz, []),
     "btb_hip_decode_step": (_i32, [_vp, _i32, _i32, _vp]),
 }
@@ -289,6 +293,32 @@ class HipCard:
                        self.ptr(w.esc_idx) if ne else None, self.ptr(w.esc_val) if ne else None, ne, self.ptr(w.row_ptr),
                        self.ptr(h_in), p(y), self.ptr(norm_w), float(eps), int(centered), p(h_out), self.ptr(out), R, C,
                        M, int(glu), _stream())
+        return out
+
+    def gemv_embed_norm(self, w: Any, table: torch.Tensor, ids: torch.Tensor, norm_w: torch.Tensor, eps: float,
+                        h_out: torch.Tensor | None, out: torch.Tensor, centered: bool = False) -> torch.Tensor:
+        """`embed` + `gemv_norm` in one launch: the residual rows are table[ids], written to `h_out`; out = W . rmsnorm"""
+        for t, what in ((table, "table"), (norm_w, "norm_w"), (out, "out")):
+            self._need(t, torch.bfloat16, what)
+        self._need(ids, torch.int32, "ids")
+        if h_out is not None:
+            self._need(h_out, torch.bfloat16, "h_out")
+        R, C = (int(s) for s in w.shape)
+        M, vocab = int(ids.numel()), int(table.shape[0])
+        if table.dim() != 2 or table.shape[1] != C or norm_w.numel() != C or out.numel() != M * R \
+                or (h_out is not None and h_out.numel() != M * C):
+            raise ValueError("[hip] gemv_embed_norm: the table, the norm weight and the outputs do not fit the matrix")
+        p = lambda t: None if t is None else self.ptr(t)
+        if isinstance(w, torch.Tensor):
+            self._need(w, torch.bfloat16, "w")
+            self._call("btb_hip_gemv_bf16_embed_norm", self.ptr(w), self.ptr(table), self.ptr(ids), vocab,
+                       self.ptr(norm_w), float(eps), int(centered), p(h_out), self.ptr(out), R, C, M, _stream())
+        else:
+            ne = int(w.esc_idx.numel())
+            self._call("btb_hip_gemv_p12_embed_norm", self.ptr(w.lo), self.ptr(w.hi4), self.ptr(w.table),
+                       self.ptr(w.esc_idx) if ne else None, self.ptr(w.esc_val) if ne else None, ne, self.ptr(w.row_ptr),
+                       self.ptr(table), self.ptr(ids), vocab, self.ptr(norm_w), float(eps), int(centered), p(h_out),
+                       self.ptr(out), R, C, M, _stream())
         return out
 
     # -- the stored forms ---------------------------------------------------------------------------------------
@@ -667,6 +697,20 @@ class HipCard:
         p = lambda t: None if t is None else self.ptr(t)
         self._call("btb_hip_publish", self.ptr(n0), self.ptr(picked), p(next_ids), p(out_tok), p(out_n0), p(out_ts),
                    _stream())
+
+    def argmax_publish(self, logits: torch.Tensor, picked: torch.Tensor, n0: torch.Tensor,
+                       next_ids: torch.Tensor | None = None, out_tok: torch.Tensor | None = None,
+                       out_n0: torch.Tensor | None = None, out_ts: torch.Tensor | None = None) -> None:
+        """`argmax` over one row and `publish` in one launch"""
+        self._need(logits, torch.bfloat16, "logits")
+        self._need(picked, torch.int32, "picked")
+        self._need(n0, torch.int32, "n0")
+        V = int(logits.shape[-1])
+        if logits.numel() != V:
+            raise ValueError("[hip] argmax_publish: one row of logits")
+        p = lambda t: None if t is None else self.ptr(t)
+        self._call("btb_hip_argmax_publish", self.ptr(logits), V, self.ptr(picked), self.ptr(n0), p(next_ids),
+                   p(out_tok), p(out_n0), p(out_ts), _stream())
 
     # -- the step as one persistent launch ------------------------------------------------------------------------
 

@@ -78,6 +78,14 @@ int32_t btb_hip_gemv_bf16_norm(const void* w, const void* h_in, const void* y, c
                                int32_t centered, void* h_out, void* out, size_t R, size_t C, size_t M, int32_t glu,
                                void* stream);
 
+/* btb_hip_gemv_bf16_norm for the step's first layer, whose residual is the tokens' embedding rows: h' [m] =
+ * table[ids[m]] (table [vocab, C] bf16, ids i32 [M] on the device, an id outside the table clamped into it), no y;
+ * h' goes to h_out, out = W rmsnorm(h'). The bits of btb_hip_embed followed by btb_hip_gemv_bf16_norm, in one launch
+ * (the reference gathers the row with torch before its graph: btb/engine/cuda.py:1722-1729). */
+int32_t btb_hip_gemv_bf16_embed_norm(const void* w, const void* table, const int32_t* ids, size_t vocab,
+                                     const void* norm_w, float eps, int32_t centered, void* h_out, void* out, size_t R,
+                                     size_t C, size_t M, void* stream);
+
 /* ---- the stored weight forms, widened in registers inside the matvec ------------------------------------ */
 
 /* The matvec over a pack12 matrix (n = R * C weights): lo u8[n], hi4 u8[(n + 1) / 2] (weight 2k in the low nibble
@@ -95,6 +103,12 @@ int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table
                               const void* esc_val, size_t n_esc, const void* row_ptr, const void* h_in, const void* y,
                               const void* norm_w, float eps, int32_t centered, void* h_out, void* out, size_t R,
                               size_t C, size_t M, int32_t glu, void* stream);
+
+/* btb_hip_gemv_bf16_embed_norm over a pack12 matrix (`table` is the matrix's 16 high bytes, `embed` the embedding). */
+int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void* table, const void* esc_idx,
+                                    const void* esc_val, size_t n_esc, const void* row_ptr, const void* embed,
+                                    const int32_t* ids, size_t vocab, const void* norm_w, float eps, int32_t centered,
+                                    void* h_out, void* out, size_t R, size_t C, size_t M, void* stream);
 
 /* row_ptr[r] = how many escapes lie below weight r * cols, r = 0..rows: the per-row slices of the escape list the
  * matvec reads. Run once when a packed matrix is uploaded; replaces the per-call search of p12_cursors
@@ -265,6 +279,12 @@ int32_t btb_hip_silu_mul(const void* gu, void* m, size_t T, size_t I, void* stre
 /* out[t] = the index of row t's largest logit, the lowest index on ties (native/src/sample.rs:53-67). logits
  * [T, V] bf16. */
 int32_t btb_hip_argmax(const void* logits, int32_t* out, size_t T, size_t V, void* stream);
+
+/* btb_hip_argmax over one row followed by btb_hip_publish, in one launch: the thread that ends up with the pick
+ * writes it to *picked and goes on with the step's end. Replaces the greedy pick (native/src/sample.rs:53-67) and
+ * btb_publish (native/cuda/btb_kernels.cu:448-465) at the end of the reference's step graph. */
+int32_t btb_hip_argmax_publish(const void* logits, size_t V, int32_t* picked, int32_t* n0, int32_t* next_ids,
+                               int32_t* out_tok, int32_t* out_n0, int64_t* out_ts, void* stream);
 
 /* The step's end, one thread: *next_ids = *picked (the next step's input, when not NULL), *n0 += 1, and with
  * out_tok not NULL (pinned host memory) the token and the GPU's clock, then - after a system fence - the new
