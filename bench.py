@@ -7,10 +7,19 @@ A step is one decode step of a random-init Qwen3-4B-shaped dense stack (36 layer
 of 128, SwiGLU 9728, vocab 151936; weights ~N(0, 0.02) in bf16, seeded N(0, 1) K/V for a 4096-token context), M = 1
 token, replayed as one captured hipGraph with every operand already resident in HBM. It prints ONE JSON line:
 `value` is the step's HBM stream in GB/s - the linear weights plus the K/V rows one step reads, divided by the step's
-time - next to tokens/s and the fraction of the 8 TB/s HBM3E peak; `roofline` prices the dominant kernel (the bf16
-streaming matvec at the qkv / gate_up / head shapes) from its own timed region, measured with device events on the
-launch stream; `cpu_baseline` times the CPU oracle's AVX-512 / AVX2 matvec (a port of the reference's CPU path) on the
-host's cores over a bounded sample of the same matrices.
+time - next to tokens/s and the fraction of the 8 TB/s HBM3E peak.
+
+`roofline` prices the kernels the step itself launches. Each class of launch - the qkv matvec with the residual add
+and norm in its x load, the attention pair, the o matvec, the gate/up matvec with the add + norm and the SwiGLU fold,
+the down matvec, the head matvec with the final norm - is timed in a graph region of its own over the model's own 36
+matrices (so nothing repeats from cache), with device events on the launch stream; `roofline.kernels` lists them,
+`roofline.kernel` / `achieved` / `frac` are those of the class that takes the most of the step's time, and
+`roofline.all_matvecs` is the byte-weighted figure over every matvec class. `traffic` is not measured by this run: it
+is the HBM bytes per launch of the dominant class from `rocprofv3 --pmc` runs of this same command, kept in
+profiles/traffic.json (`traffic_source` names the summary).
+
+`cpu_baseline` times the CPU oracle's AVX-512 / AVX2 matvec of the same stored form (a port of the reference's CPU
+path, as `btb bench` times it per stored form: btb/machine.py:1000, 1018) on the host's cores over a bounded sample.
 """
 
 from __future__ import annotations
@@ -28,40 +37,121 @@ if ROOT not in sys.path:
 HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 CTX = 4096
 METRIC = "decode GEMV HBM GB/s (% of peak) + decode tok/s, Qwen3-4B-shape bf16 M=1"
+TRAFFIC = os.path.join(ROOT, "profiles", "traffic.json")
 
 
-def cpu_baseline(budget_s: float = 12.0) -> dict:
-    """the oracle's bf16 matvec (the reference's CPU arithmetic, ported) over gate_up-shaped matrices drawn from a
-    pool larger than 4x the last-level cache, every core, for about `budget_s` seconds"""
+# ---------------------------------------------------------------------------------------------------------------
+# the CPU leg: the oracle (a port of the reference's CPU kernels) on the host's cores, a bounded sample
+# ---------------------------------------------------------------------------------------------------------------
+
+
+def cpu_baseline(workload: str = "decode", m: int = 1, budget_s: float = 12.0) -> dict:
+    """The oracle's matvec of the workload's stored form over matrices drawn in rotation from a pool (so the last-level
+    cache does not hold them), every core, for about `budget_s` seconds, then a quarter of that on one thread.
+    GB/s of the same algorithmic bytes the GPU figure counts."""
     import numpy as np
 
     import oracle
+    from oracle import codecs
 
-    R, C = 19456, 2560
     rng = np.random.default_rng(0x0B7B)
-    pool = [rng.integers(0x3A00, 0x3D00, (R, C), dtype=np.uint16) for _ in range(12)]  # 1.2 GB of bf16 patterns
-    x = rng.standard_normal((1, C)).astype(np.float32)
     cores = os.cpu_count() or 1
-    oracle.gemv_bf16(pool[0], x, threads=0)
+
+    def bf16_bits(rows: int, cols: int) -> np.ndarray:
+        return codecs.f32_to_bf16_bits((rng.standard_normal((rows, cols), dtype=np.float32) * np.float32(0.02)))
+
+    if workload in ("decode", "gemv_bf16"):
+        R, C = (19456, 2560) if workload == "decode" else (9728, 2560)
+        pool = [rng.integers(0x3A00, 0x3D00, (R, C), dtype=np.uint16) for _ in range(12 if workload == "decode" else 24)]
+        x = rng.standard_normal((m, C)).astype(np.float32)
+        call = lambda i, t: oracle.gemv_bf16(pool[i % len(pool)], x, threads=t)
+        per_call = R * C * 2 + m * (C + R) * 4
+        what = f"bf16 matvecs [{R}x{C}]" + (" (the gate_up shape)" if workload == "decode" else "")
+    elif workload in ("decode_p12", "gemv_p12"):
+        R, C = (19456, 2560) if workload == "decode_p12" else (9728, 2560)
+        lo, hi4, table, ei, ev = codecs.pack12_pack(bf16_bits(R, C))
+        pool = [(lo.copy(), hi4.copy()) for _ in range(16 if workload == "decode_p12" else 32)]
+        x = rng.standard_normal((m, C)).astype(np.float32)
+        call = lambda i, t: oracle.gemv_p12(pool[i % len(pool)][0], pool[i % len(pool)][1], table, ei, ev, R, C, x, threads=t)
+        per_call = lo.size + hi4.size + 16 + 5 * ei.size + m * (C + R) * 4
+        what = f"pack12 matvecs [{R}x{C}] ({ei.size} escapes)"
+    elif workload == "gemv_fp8":
+        # random e4m3 bytes (no NaN patterns) and scales of the size quantising N(0, 0.02) gives: the kernel's speed
+        # does not depend on the values, and encoding 132 M weights in numpy would take longer than the sample
+        R, C = 18432, 7168
+        q = rng.integers(0, 0x7F, (R, C), dtype=np.uint8) | (rng.integers(0, 2, (R, C), dtype=np.uint8) << 7)
+        s = (rng.random((R // 128, C // 128), dtype=np.float32) + np.float32(0.5)) * np.float32(2e-4)
+        pool = [q.copy() for _ in range(9)]
+        x = rng.standard_normal((m, C)).astype(np.float32)
+        call = lambda i, t: oracle.gemv_fp8(pool[i % len(pool)], s, x, threads=t)
+        per_call = R * C + s.size * 4 + m * (C + R) * 4
+        what = f"FP8 e4m3 matvecs [{R}x{C}], 128x128 scale blocks (random bytes)"
+    elif workload == "gemv_mxfp4":
+        R, C = 18432, 7168
+        b = rng.integers(0, 256, (R, C // 32, 16), dtype=np.uint8)
+        s = rng.integers(115, 123, (R, C // 32), dtype=np.uint8)
+        pool = [b.copy() for _ in range(16)]
+        x = rng.standard_normal((m, C)).astype(np.float32)
+        call = lambda i, t: oracle.gemv_mxfp4(pool[i % len(pool)], s, R, C, x, threads=t)
+        per_call = b.size + s.size + m * (C + R) * 4
+        what = f"MXFP4 matvecs [{R}x{C}] (random bytes)"
+    elif workload == "moe":
+        from oracle import moe as omoe
+
+        E, k, H, I = 128, 8, 2048, 768
+        bits = lambda *shape: (rng.integers(0x3A00, 0x3D00, shape, dtype=np.uint16)
+                               | (rng.integers(0, 2, shape, dtype=np.uint16) << 15))   # +-2^-11 .. 2^-5
+        wr, gu, dn = bits(E, H), bits(E, 2 * I, H), bits(E, H, I)
+        xs = [codecs.round_bf16(rng.standard_normal((m, H)).astype(np.float32)) for _ in range(16)]
+        distinct = []
+
+        def call(i, t):  # the oracle's layer runs its matvecs on every core (threads = 0 inside oracle/moe.py)
+            _, _, _, picks = omoe.layer(wr, gu, dn, xs[i % len(xs)], k, dt="bf16")
+            distinct.append(len(set(picks.reshape(-1).tolist())))
+
+        per_call = None
+        what = f"MoE layers: top-{k} of {E} experts, gate_up [{2 * I}x{H}] + down [{H}x{I}] bf16, {m} tokens"
+    else:
+        raise ValueError(workload)
+
+    call(0, 0)
+    if workload == "moe":
+        distinct.clear()
     t0 = time.perf_counter()
     calls = 0
     while time.perf_counter() - t0 < budget_s:
-        oracle.gemv_bf16(pool[calls % len(pool)], x, threads=0)
+        call(calls, 0)
         calls += 1
     dt = time.perf_counter() - t0
-    per_call = R * C * 2 + C * 4 + R * 4
+    if workload == "moe":
+        nbytes = sum(128 * 2048 * 2 + d * (2 * 768 * 2048 + 2048 * 768) * 2 for d in distinct)
+        return {"value": round(nbytes / dt / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port", "isa": oracle.isa(),
+                "sample": f"{calls} {what} through the oracle's numpy + C layer, matvecs on all {cores} host threads, "
+                          f"{dt:.1f} s; bytes = the router and every distinct picked expert"}
     gbs = calls * per_call / dt / 1e9
-    # the same matvec on one thread (the reference's own criterion bench pins one: native/benches/gemv.rs:8-10)
     t1 = time.perf_counter()
     solo = 0
     while time.perf_counter() - t1 < budget_s / 4:
-        oracle.gemv_bf16(pool[solo % len(pool)], x, threads=1)
+        call(solo, 1)
         solo += 1
     d1 = time.perf_counter() - t1
     return {"value": round(gbs, 2), "unit": "GB/s", "cores": cores, "kind": "port", "isa": oracle.isa(),
             "one_thread_gbs": round(solo * per_call / d1 / 1e9, 2),
-            "sample": f"{calls} bf16 matvecs [{R}x{C}] (the gate_up shape), 12 distinct matrices (1.2 GB) in rotation, "
-                      f"f32 x and y, all {cores} host threads, {dt:.1f} s; then {solo} on one thread, {d1:.1f} s"}
+            "sample": f"{calls} {what}, {len(pool)} operand copies in rotation, f32 x and y (M={m}), all {cores} host "
+                      f"threads, {dt:.1f} s; then {solo} on one thread, {d1:.1f} s"}
+
+
+def traffic_entry(workload: str, key: str) -> dict | None:
+    """HBM bytes per launch from the committed rocprofv3 --pmc summaries (a profile constant, not measured here)"""
+    if not os.path.exists(TRAFFIC):
+        return None
+    with open(TRAFFIC) as f:
+        return (json.load(f).get(workload) or {}).get(key)
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# the single-operator configs
+# ---------------------------------------------------------------------------------------------------------------
 
 
 def kernel_workload(args: argparse.Namespace) -> int:
@@ -114,6 +204,7 @@ def kernel_workload(args: argparse.Namespace) -> int:
         what = f"C4: top-{k} of {E} experts, gate_up [{2 * I}, {H}] + down [{H}, {I}] bf16, M={M} tokens"
         extra = {"distinct_experts": distinct}
         dtype = "bf16 weights and activations, f32 accumulate"
+        kernel = "the routed layer: router matvec + routing, gate/up with the SwiGLU fold, down with the weighted sum"
     else:
         R, C = (9728, 2560) if name in ("gemv_bf16", "gemv_p12") else (18432, 7168)
         # operands of a pass: over 1 GiB of stored weights, past four times the 256 MB last-level cache (the reference's
@@ -148,6 +239,8 @@ def kernel_workload(args: argparse.Namespace) -> int:
         dtype = {"gemv_bf16": "bf16", "gemv_p12": "pack12 widened to bf16 in registers",
                  "gemv_fp8": "fp8 e4m3 x f32 block scale -> bf16 in registers",
                  "gemv_mxfp4": "mxfp4 -> bf16 in registers"}[name] + ", f32 accumulate"
+        kernel = ("gemv_stream (vector ALUs, v_dot2_f32_bf16)" if M <= 4 else
+                  "gemv_mfma_lds (matrix cores, v_mfma_f32_16x16x32_bf16; taken from 5 rows on)")
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
         for i in range(pool):
@@ -161,26 +254,114 @@ def kernel_workload(args: argparse.Namespace) -> int:
     for _ in range(max(1, args.warmup // pool)):
         graph.replay()
     torch.cuda.synchronize()
+    stream = torch.cuda.current_stream()
     e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    e0.record()
+    e0.record(stream)
     for _ in range(passes):
         graph.replay()
-    e1.record()
+    e1.record(stream)
     torch.cuda.synchronize()
     us = e0.elapsed_time(e1) * 1e3 / (passes * pool)
     mean_bytes = sum(nbytes) / len(nbytes)
     gbs = mean_bytes / (us * 1e-6) / 1e9
+    tr = traffic_entry(name, f"m{M}")
     print(json.dumps({
         "metric": "decode matvec HBM GB/s (% of peak), one operator", "value": round(gbs, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": passes * pool, "warmup": args.warmup, "ms_per_step": round(us * 1e-3, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
         "data": "synthetic: N(0, 0.02) weights, N(0, 1) x, seeded", "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
         "config": {"workload": what, "pool": pool, "algorithmic_bytes_per_step": int(mean_bytes), **extra},
-        "roofline": {"bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(gbs / HBM_PEAK_GBS, 4), "traffic": None},
-        "cpu_baseline": None,
+        "roofline": {"kernel": kernel, "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(gbs / HBM_PEAK_GBS, 4), "avg_launch_us": round(us, 3),
+                     "bytes_per_launch": int(mean_bytes),
+                     "traffic": None if tr is None else tr.get("bytes_per_launch"),
+                     "traffic_source": None if tr is None else tr.get("source")},
+        "cpu_baseline": None if args.no_cpu else cpu_baseline(name, M),
     }))
     return 0
+
+
+# ---------------------------------------------------------------------------------------------------------------
+# the decode step
+# ---------------------------------------------------------------------------------------------------------------
+
+
+def step_classes(step, card) -> list[dict]:
+    """The classes of launch one step makes, each as a closure that issues that class over the model's 36 layers (the
+    head: once) on the step's own buffers, with its launches and algorithmic bytes per pass. The calls are the ones
+    `DecodeStep._body_fused` makes."""
+    cfg, w = step.cfg, step.w
+    Hq, Hk, D, H, I = cfg.q_heads, cfg.kv_heads, cfg.head_dim, cfg.hidden, cfg.intermediate
+    L = cfg.layers
+    lay = [f"layers.{i}." for i in range(L)]
+    n_keys = int(step.n0[0]) + 1
+    norm_in = 3 * H * 2  # residual row, block output row and norm weight read by an add + norm x load
+
+    def qkv():
+        for p in lay:
+            card.gemv_norm(w[p + "qkv"].w, step.h, step.y, w[p + "ln1"], cfg.eps, step.h2, step.qkv)
+
+    def attn():
+        for i, p in enumerate(lay):
+            card.attn_decode_qkv(step.qkv, w.get(p + "wq"), w.get(p + "wk"), cfg.eps, step.cos, step.sin, step.n0,
+                                 step.kv[i, 0], step.kv[i, 1], step.att, Hq, Hk, D, step.scale, step.S, step.scratch)
+
+    def o():
+        for p in lay:
+            w[p + "o"].matvec(step.att, step.y)
+
+    def gu():
+        for p in lay:
+            card.gemv_norm(w[p + "gu"].w, step.h2, step.y, w[p + "ln2"], cfg.eps, step.h, step.m, glu=True)
+
+    def down():
+        for p in lay:
+            w[p + "down"].matvec(step.m, step.y)
+
+    def head():
+        card.gemv_norm(w["head"].w, step.h, step.y, w["norm"], cfg.eps, None, step.logits)
+
+    wb = lambda name: sum(w[p + name].nbytes for p in lay)
+    kv = 2 * Hk * n_keys * D * 2
+    return [
+        {"name": "qkv matvec + residual add + RMSNorm (gemv_stream, X_ADDNORM)", "fn": qkv, "launches": L, "matvec": True,
+         "bytes": wb("qkv") + L * (norm_in + H * 2 + cfg.qkv_rows * 2)},
+        {"name": "decode attention: q/k norm + rope + cache write + attention over the spans, then the span merge "
+                 "(attn_decode_qkv_kernel + attn_merge_kernel, two launches)", "fn": attn, "launches": L, "matvec": False,
+         "kernels_per_launch": 2, "bytes": L * (kv + cfg.qkv_rows * 2 + Hq * D * 2)},
+        {"name": "o matvec (gemv_stream)", "fn": o, "launches": L, "matvec": True,
+         "bytes": wb("o") + L * (Hq * D * 2 + H * 2)},
+        {"name": "gate/up matvec + residual add + RMSNorm + SwiGLU fold (gemv_stream, X_ADDNORM, E_GLU)", "fn": gu,
+         "launches": L, "matvec": True, "bytes": wb("gu") + L * (norm_in + H * 2 + I * 2)},
+        {"name": "down matvec (gemv_stream)", "fn": down, "launches": L, "matvec": True,
+         "bytes": wb("down") + L * (I * 2 + H * 2)},
+        {"name": "head matvec + final RMSNorm (gemv_stream, X_ADDNORM)", "fn": head, "launches": 1, "matvec": True,
+         "bytes": w["head"].nbytes + norm_in + cfg.vocab * 2},
+    ]
+
+
+def time_region(torch, fn, launches: int, reps: int) -> float:
+    """average microseconds per launch of `fn`'s launches, replayed as a hipGraph `reps` times between two device
+    events recorded on the stream the graph runs on"""
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        fn()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        fn()
+    g.replay()
+    torch.cuda.synchronize()
+    stream = torch.cuda.current_stream()
+    e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    e0.record(stream)
+    for _ in range(reps):
+        g.replay()
+    e1.record(stream)
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) * 1e3 / (reps * launches)
 
 
 def main() -> int:
@@ -242,48 +423,46 @@ def main() -> int:
     wbytes, kvbytes = step.weight_bytes(), step.kv_bytes(int(n_keys))
     gbs = (wbytes + kvbytes) / (ms * 1e-3) / 1e9
 
-    # -- the dominant kernel in a timed region of its own: the streaming matvec at the qkv, gate_up and head shapes
-    #    (5.5 of the step's 8.0 GB of bf16 weights), over the model's own matrices, so nothing repeats from cache
-    M = args.rows
-    x = torch.randn(M, cfg.hidden, device="cuda").to(torch.bfloat16)
-    outs = {n: torch.empty(M, r, dtype=torch.bfloat16, device="cuda")
-            for n, r in (("qkv", cfg.qkv_rows), ("gu", 2 * cfg.intermediate), ("head", cfg.vocab))}
-
-    def dominant() -> tuple[int, int]:
-        launches = nbytes = 0
-        for i in range(cfg.layers):
-            for n in ("qkv", "gu"):
-                lin = weights[f"layers.{i}.{n}"]
-                lin.matvec(x, outs[n])
-                launches += 1
-                nbytes += lin.nbytes + M * (cfg.hidden * 2 + lin.shape[0] * 2)
-        weights["head"].matvec(x, outs["head"])
-        return launches + 1, nbytes + weights["head"].nbytes + M * (cfg.hidden * 2 + cfg.vocab * 2)
-
-    side = torch.cuda.Stream()
-    with torch.cuda.stream(side):
-        launches, dom_bytes = dominant()
-    torch.cuda.synchronize()
-    gd = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(gd):
-        dominant()
-    gd.replay()
-    torch.cuda.synchronize()
-    reps = 10
-    d0, d1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    d0.record(stream)
-    for _ in range(reps):
-        gd.replay()
-    d1.record(stream)
-    torch.cuda.synchronize()
-    dom_us = d0.elapsed_time(d1) * 1e3 / (reps * launches)
-    achieved = dom_bytes / launches / (dom_us * 1e-6) / 1e9
-    traffic = None
-    tpath = os.path.join(ROOT, "profiles", "traffic.json")
-    if os.path.exists(tpath) and args.rows == 1:  # the counters were read for the one-row region
-        with open(tpath) as f:
-            entry = json.load(f).get(args.workload)
-            traffic = None if entry is None else entry.get("bytes_per_launch")
+    # -- the step's own launches, class by class, each in a timed graph region over the model's 36 layers
+    roofline: dict = {"bound": "hbm", "peak": HBM_PEAK_GBS, "unit": "GB/s"}
+    if args.rows == 1 and step.fused:
+        step.reset(CTX, 0)
+        torch.cuda.synchronize()
+        kernels = []
+        for c in step_classes(step, card):
+            us = time_region(torch, c["fn"], c["launches"], reps=10)
+            per = c["bytes"] / c["launches"]
+            kernels.append({"name": c["name"], "launches_per_step": c["launches"] * c.get("kernels_per_launch", 1),
+                            "avg_launch_us": round(us, 3), "bytes_per_launch": int(per),
+                            "achieved": round(per / (us * 1e-6) / 1e9, 1),
+                            "frac": round(per / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                            "us_per_step": round(us * c["launches"], 1), "matvec": c["matvec"]})
+        total_us = sum(k["us_per_step"] for k in kernels)
+        for k in kernels:
+            k["step_share"] = round(k["us_per_step"] / total_us, 4)
+        dom = max(kernels, key=lambda k: k["us_per_step"])
+        mv = [k for k in kernels if k["matvec"]]
+        mv_bytes = sum(k["bytes_per_launch"] * k["launches_per_step"] for k in mv)
+        mv_us = sum(k["us_per_step"] for k in mv)
+        tr = traffic_entry(args.workload, "dominant")
+        roofline.update({
+            "kernel": dom["name"], "achieved": dom["achieved"], "frac": dom["frac"],
+            "avg_launch_us": dom["avg_launch_us"], "bytes_per_launch": dom["bytes_per_launch"],
+            "launches": dom["launches_per_step"], "step_share": dom["step_share"],
+            "traffic": None if tr is None else tr.get("bytes_per_launch"),
+            "traffic_source": None if tr is None else tr.get("source"),
+            "all_matvecs": {"bytes_per_step": int(mv_bytes), "us_per_step": round(mv_us, 1),
+                            "achieved": round(mv_bytes / (mv_us * 1e-6) / 1e9, 1),
+                            "frac": round(mv_bytes / (mv_us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},
+            "regions_us_per_step": round(total_us, 1),
+            "kernels": [{k2: v for k2, v in k.items() if k2 != "matvec"} for k in kernels],
+        })
+    else:
+        # a verify pass: the whole pass is the region (its matvecs run as gemv_stream up to 4 rows and on the matrix
+        # cores, gemv_mfma_lds, from 5 rows on)
+        roofline.update({"kernel": f"the whole pass of {args.rows} rows (matvecs: gemv_stream to 4 rows, gemv_mfma_lds "
+                                   f"from 5)", "achieved": round(gbs, 1), "frac": round(gbs / HBM_PEAK_GBS, 4),
+                         "traffic": None, "traffic_source": None})
 
     line = {
         "metric": METRIC,
@@ -309,25 +488,13 @@ def main() -> int:
             "rows": args.rows, "rows_per_s": round(args.rows * 1e3 / ms, 1),
             "layers": cfg.layers, "hidden": cfg.hidden, "q_heads": cfg.q_heads, "kv_heads": cfg.kv_heads,
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate, "vocab": cfg.vocab, "context": CTX,
-            "weight_bytes_per_step": wbytes, "kv_bytes_per_step": kvbytes, "kernels_per_step": (4 + 6 * cfg.layers if args.rows == 1 else
-                                 4 + 7 * cfg.layers if step.fused else 5 + 10 * cfg.layers),
+            "weight_bytes_per_step": wbytes, "kv_bytes_per_step": kvbytes,
+            "kernels_per_step": (2 + 6 * cfg.layers if args.rows == 1 else
+                                 3 + 7 * cfg.layers if step.fused else 5 + 10 * cfg.layers),
             "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
         },
-        "roofline": {
-            "kernel": ("gemv_stream (streaming matvec, M=1)" if M == 1 else
-                       f"the matvec at M={M} (gemv_stream to 4 rows, gemv_mfma_lds from 8)")
-                      + " at the qkv / gate_up / head shapes",
-            "bound": "hbm",
-            "achieved": round(achieved, 1),
-            "peak": HBM_PEAK_GBS,
-            "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBS, 4),
-            "traffic": traffic,
-            "launches": launches,
-            "avg_launch_us": round(dom_us, 3),
-            "bytes_per_launch": int(dom_bytes / launches),
-        },
-        "cpu_baseline": None if args.no_cpu else cpu_baseline(),
+        "roofline": roofline,
+        "cpu_baseline": None if args.no_cpu else cpu_baseline(args.workload, 1),
     }
     print(json.dumps(line))
     return 0

@@ -95,23 +95,105 @@ __device__ __forceinline__ void load_keys_upto(KeyBatch& kb, const uint16_t* Kh,
     }
 }
 
-// The batch's keys folded into the G query heads' online-softmax states, a batch at a time: the 8 x G scores first
-// (q and the key row meet as bf16 pairs in v_dot2_f32_bf16 - products exact, f32 sums - then the 16 lanes' sums are
-// folded and scaled into log2 units), then per head one new maximum, one correction of the running sum and output for
-// the whole batch, and the batch's weights; then each value row, widened once, meets all G heads. A key past the
-// span's end scores -inf and weighs 0. qp: the heads' q, this lane's 8 dims as 4 bf16 pairs. own >= 0: the step's
-// own row is key `own` and is taken from LDS (s_k, s_v) - the cache's copy may not have landed yet.
-// tree_base >= 0: the keys from slot tree_base on are the pass's own rows, and of those the row sees the ones whose
-// bit is set in tree_mask (its ancestors and itself: a verify pass's tree). ZERO_DEAD: a key that does not count may
-// have been loaded from a slot the cache has never written (load_keys_upto), so its value row is taken as zeros -
-// weight 0 times whatever bits lie there must not make a NaN.
+// ------------------------------------------------------------------------------------------------------------
+// A key stream's state and the fold of one batch of keys into it.
+//
+// A stream is a group of 16 lanes; a lane holds 8 dims of every key row it loads. A batch is 8 keys; with G query heads
+// that is 8 G scores, each a sum over the 16 lanes. They are summed "transposed": the 16 lanes start with 8 G partial
+// sums each and end with 8 G / 16 finished scores each (lane dl: key dl % 8, head 2 r + dl / 8 in slot r; one head: both
+// halves of the group hold the same 8), so a score is scaled, masked and exponentiated once, by one lane, and a
+// batch's maximum is a three-step exchange among the 8 lanes of a head. The weights then go back to all 16 lanes through
+// a few words of LDS (the stream's exchange area; a wave's own LDS traffic is served in order, so no barrier), two
+// neighbouring keys' weights rounded to bf16 and packed in a word: the value rows of the two keys are zipped into bf16
+// pairs as well and meet the weights in v_dot2_f32_bf16 (products exact, f32 sums). The running sum is made of the
+// same rounded weights, so the weights of a head still add up to one - the reference's card kernel rounds its
+// weights to bf16 for its tensor cores in the same way (native/cuda/btb_attn_flash.cuh:90-125).
+// ------------------------------------------------------------------------------------------------------------
+constexpr int attn_slots(int G) { return G <= 2 ? 1 : G / 2; }
+constexpr int XCH = 48;  // floats of LDS a stream exchanges through: weight pairs at 0.., corrections at 32.., heads' state
+
+template <int G>
+struct AttnState {
+    static constexpr int R = attn_slots(G);
+    float ms[R];      // running maximum of the slot's head, log2 units (the same in the 8 lanes of a head)
+    float ls[R];      // this lane's share of the running sum: its own key slot's weights
+    float acc[G][8];  // the heads' outputs, this lane's 8 dims
+    __device__ __forceinline__ void init() {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            ms[r] = bits_f32(0xff800000u);
+            ls[r] = 0.f;
+        }
+#pragma unroll
+        for (int j = 0; j < G; ++j)
+#pragma unroll
+            for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
+    }
+};
+template <int G>
+__device__ __forceinline__ int slot_head(int r, int dl) {
+    return G == 1 ? 0 : 2 * r + (dl >> 3);
+}
+
+// 16 values a lane, summed over the 16 lanes of the group: lane dl ends up with the sum of value dl. Each step pairs
+// the lanes off (15 - i, then 7 - i within 8, i ^ 2, i ^ 1), a lane keeping the half of its values its side of the
+// pairing owns, plus the partner's same half.
+__device__ __forceinline__ float tsum16(const float* v, int dl) {
+    float a[8], b[4], c[2];
+    const bool u1 = dl >= 8, u2 = (dl & 7) >= 4, u3 = (dl & 3) >= 2, u4 = (dl & 1) != 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const float lo = v[k] + dpp_f32<0x140>(v[k]), hi = v[k + 8] + dpp_f32<0x140>(v[k + 8]);
+        a[k] = u1 ? hi : lo;
+    }
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float lo = a[k] + dpp_f32<0x141>(a[k]), hi = a[k + 4] + dpp_f32<0x141>(a[k + 4]);
+        b[k] = u2 ? hi : lo;
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const float lo = b[k] + dpp_f32<0x4E>(b[k]), hi = b[k + 2] + dpp_f32<0x4E>(b[k + 2]);
+        c[k] = u3 ? hi : lo;
+    }
+    const float lo = c[0] + dpp_f32<0xB1>(c[0]), hi = c[1] + dpp_f32<0xB1>(c[1]);
+    return u4 ? hi : lo;
+}
+// 8 values a lane: lane dl ends up with the sum of value dl % 8
+__device__ __forceinline__ float tsum8(const float* v, int dl) {
+    float a[8], b[4], c[2];
+    const bool u2 = (dl & 7) >= 4, u3 = (dl & 3) >= 2, u4 = (dl & 1) != 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) a[k] = v[k] + dpp_f32<0x140>(v[k]);
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const float lo = a[k] + dpp_f32<0x141>(a[k]), hi = a[k + 4] + dpp_f32<0x141>(a[k + 4]);
+        b[k] = u2 ? hi : lo;
+    }
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+        const float lo = b[k] + dpp_f32<0x4E>(b[k]), hi = b[k + 2] + dpp_f32<0x4E>(b[k + 2]);
+        c[k] = u3 ? hi : lo;
+    }
+    const float lo = c[0] + dpp_f32<0xB1>(c[0]), hi = c[1] + dpp_f32<0xB1>(c[1]);
+    return u4 ? hi : lo;
+}
+
+// The batch's keys folded into the stream's state. A key past the span's end scores -inf and weighs 0. qp: the heads'
+// q, this lane's 8 dims as 4 bf16 pairs. own >= 0: the step's own row is key `own` and is taken from LDS (s_k, s_v) -
+// the cache's copy may not have landed yet. tree_base >= 0: the keys from slot tree_base on are the pass's own rows,
+// and of those the row sees the ones whose bit is set in tree_mask (its ancestors and itself: a verify pass's tree).
+// ZERO_DEAD: a key that does not count may have been loaded from a slot the cache has never written
+// (load_keys_upto), so its value row is taken as zeros - weight 0 times whatever bits lie there must not make a NaN.
+// xch: the stream's XCH floats of LDS.
 template <int G, bool ZERO_DEAD = false>
 __device__ __forceinline__ void use_keys(KeyBatch& kb, int key0, int k_end, int own, const uint16_t* s_k,
                                          const uint16_t* s_v, int dl, const uint32_t (&qp)[G][4], float scale_log2,
-                                         float (&m)[G], float (&l)[G], float (&acc)[G][8], int tree_base = -1,
-                                         uint32_t tree_mask = 0u) {
+                                         AttnState<G>& st, float* xch, int tree_base = -1, uint32_t tree_mask = 0u) {
+    constexpr int R = attn_slots(G);
+    static_assert(G == 1 || G == 2 || G == 4 || G == 8, "1, 2, 4 or 8 query heads a stream");
     const float ninf = bits_f32(0xff800000u);
-    if (own >= 0) {  // uniform: only the workgroup whose span holds the slot gets here with own set
+    if (own >= 0) {  // uniform: only a workgroup whose span holds the slot gets here with own set
 #pragma unroll
         for (int b = 0; b < KB; ++b)
             if (key0 + 16 * b == own) {
@@ -119,65 +201,128 @@ __device__ __forceinline__ void use_keys(KeyBatch& kb, int key0, int k_end, int 
                 kb.v[b] = *reinterpret_cast<const uint4*>(s_v + dl * 8);
             }
     }
-    float w[KB][G];  // scores, then weights
+    // this lane's 8 dims of every (head, key) score
+    float part[(G == 1 ? 1 : G) * KB];
 #pragma unroll
-    for (int b = 0; b < KB; ++b) {
-        const uint4 kr = kb.k[b];
-        const int key = key0 + 16 * b;
-        bool live = key < k_end;
-        if (tree_base >= 0) live = live && (key < tree_base || ((tree_mask >> min(key - tree_base, 31)) & 1u) != 0u);
-        if (ZERO_DEAD && !live) kb.v[b] = make_uint4(0u, 0u, 0u, 0u);
+    for (int j = 0; j < G; ++j)
 #pragma unroll
-        for (int j = 0; j < G; ++j) {
+        for (int b = 0; b < KB; ++b) {
+            const uint4 kr = kb.k[b];
             float sc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr.x), __builtin_bit_cast(bf16x2, qp[j][0]), 0.f, false);
             sc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr.y), __builtin_bit_cast(bf16x2, qp[j][1]), sc, false);
             sc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr.z), __builtin_bit_cast(bf16x2, qp[j][2]), sc, false);
             sc = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, kr.w), __builtin_bit_cast(bf16x2, qp[j][3]), sc, false);
-            sc = group_sum<16>(sc) * scale_log2;
-            w[b][j] = live ? sc : ninf;
+            part[j * KB + b] = sc;
         }
+    // the lane's own key slot
+    const int bk = dl & 7;
+    const int key = key0 + 16 * bk;
+    bool live = key < k_end;
+    if (tree_base >= 0) live = live && (key < tree_base || ((tree_mask >> min(key - tree_base, 31)) & 1u) != 0u);
+    uint32_t* xw = reinterpret_cast<uint32_t*>(xch);
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float raw = G == 1 ? tsum8(part, dl) : tsum16(part + 16 * r, dl);
+        const float s = live ? raw * scale_log2 : ninf;
+        float bm = s;  // the batch's maximum for this slot's head: over the 8 lanes that hold its keys
+        bm = fmaxf(bm, dpp_f32<0xB1>(bm));
+        bm = fmaxf(bm, dpp_f32<0x4E>(bm));
+        bm = fmaxf(bm, dpp_f32<0x141>(bm));
+        const float mn = fmaxf(st.ms[r], bm);
+        // nothing seen yet and nothing live in the batch: mn is still -inf, the weight 0 and the state as it was
+        const float p = s == ninf ? 0.f : __builtin_amdgcn_exp2f(s - mn);
+        const float corr = st.ms[r] == ninf ? 0.f : __builtin_amdgcn_exp2f(st.ms[r] - mn);
+        const float pn = dpp_f32<0xB1>(p);  // the neighbouring key's weight
+        const bool odd = (dl & 1) != 0;
+        const bf16x2 pr = {(__bf16)(odd ? pn : p), (__bf16)(odd ? p : pn)};  // keys 2 i and 2 i + 1, rounded to bf16
+        const uint32_t pw = __builtin_bit_cast(uint32_t, pr);
+        st.ls[r] = fmaf(st.ls[r], corr, odd ? bf16hi_f32(pw) : bf16lo_f32(pw));
+        st.ms[r] = mn;
+        const int j = slot_head<G>(r, dl);
+        xw[j * 4 + (bk >> 1)] = pw;       // both lanes of a pair write the same word
+        if (bk == 0) xch[32 + j] = corr;
     }
+    __builtin_amdgcn_wave_barrier();  // the writes above before the reads below, as written (one wave: served in order)
+    uint4 pw4[G];
+    float corr_all[G];
 #pragma unroll
     for (int j = 0; j < G; ++j) {
-        float mn = m[j];
+        pw4[j] = reinterpret_cast<const uint4*>(xch)[j];
+        corr_all[j] = xch[32 + j];
+    }
+    __builtin_amdgcn_wave_barrier();  // and these reads before the next batch's writes
 #pragma unroll
-        for (int b = 0; b < KB; ++b) mn = fmaxf(mn, w[b][j]);
-        // a tree pass can hand a stream a batch none of whose keys the row sees while the stream has seen none yet:
-        // the maximum is still -inf then, and the batch must leave the state as it is (not -inf - -inf)
-        const bool none = tree_base >= 0 && mn == ninf;
-        const float corr = none ? 1.f : __builtin_amdgcn_exp2f(m[j] - mn);  // 0 on the stream's first keys (m = -inf)
-        float lj = l[j] * corr;
+    for (int j = 0; j < G; ++j)
 #pragma unroll
-        for (int b = 0; b < KB; ++b) {
-            w[b][j] = none ? 0.f : __builtin_amdgcn_exp2f(w[b][j] - mn);
-            lj += w[b][j];
+        for (int e = 0; e < 8; ++e) st.acc[j][e] *= corr_all[j];
+    if (ZERO_DEAD) {
+        if (key0 + 16 * (KB - 1) >= k_end) {
+#pragma unroll
+            for (int b = 0; b < KB; ++b)
+                if (key0 + 16 * b >= k_end) kb.v[b] = make_uint4(0u, 0u, 0u, 0u);
         }
-        l[j] = lj;
-        m[j] = mn;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[j][e] *= corr;
     }
 #pragma unroll
-    for (int b = 0; b < KB; ++b) {
-        const uint4 vr = kb.v[b];
-        const float vf[8] = {bf16lo_f32(vr.x), bf16hi_f32(vr.x), bf16lo_f32(vr.y), bf16hi_f32(vr.y),
-                             bf16lo_f32(vr.z), bf16hi_f32(vr.z), bf16lo_f32(vr.w), bf16hi_f32(vr.w)};
+    for (int pi = 0; pi < KB / 2; ++pi) {
+        const uint4 va = kb.v[2 * pi], vb = kb.v[2 * pi + 1];
+        const uint32_t wa[4] = {va.x, va.y, va.z, va.w}, wb[4] = {vb.x, vb.y, vb.z, vb.w};
+        uint32_t zl[4], zh[4];  // (dim 2 q of key a, of key b), (dim 2 q + 1 of key a, of key b)
 #pragma unroll
-        for (int j = 0; j < G; ++j)
+        for (int q = 0; q < 4; ++q) {
+            zl[q] = __builtin_amdgcn_perm(wb[q], wa[q], 0x05040100u);
+            zh[q] = __builtin_amdgcn_perm(wb[q], wa[q], 0x07060302u);
+        }
 #pragma unroll
-            for (int e = 0; e < 8; ++e) acc[j][e] = fmaf(w[b][j], vf[e], acc[j][e]);
+        for (int j = 0; j < G; ++j) {
+            const uint32_t pj = pi == 0 ? pw4[j].x : pi == 1 ? pw4[j].y : pi == 2 ? pw4[j].z : pw4[j].w;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                st.acc[j][2 * q] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, zl[q]),
+                                                                  __builtin_bit_cast(bf16x2, pj), st.acc[j][2 * q], false);
+                st.acc[j][2 * q + 1] = __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2, zh[q]),
+                                                                      __builtin_bit_cast(bf16x2, pj), st.acc[j][2 * q + 1], false);
+            }
+        }
     }
+}
+
+// the stream's state per head, in every lane: the maximum, and the sum over the head's 8 key slots
+template <int G>
+__device__ __forceinline__ void heads_state(const AttnState<G>& st, int dl, float* xch, float (&m)[G], float (&l)[G]) {
+    constexpr int R = attn_slots(G);
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        float ls = st.ls[r];
+        ls += dpp_f32<0xB1>(ls);
+        ls += dpp_f32<0x4E>(ls);
+        ls += dpp_f32<0x141>(ls);
+        if ((dl & 7) == 0) {
+            const int j = slot_head<G>(r, dl);
+            xch[j] = st.ms[r];
+            xch[8 + j] = ls;
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int j = 0; j < G; ++j) {
+        m[j] = xch[j];
+        l[j] = xch[8 + j];
+    }
+    __builtin_amdgcn_wave_barrier();
 }
 
 // A workgroup's 16 key streams folded into one state per query head, in stream order. Each stream first brings its own
 // state to the workgroup's maximum (the 16 maxima meet in LDS; one exp2 per head and lane), then the scaled sums and
 // outputs are added up in stream order: thread (j, d) of 256 makes output d of head j, G * 128 / 256 of them a
 // thread, and hands it to `store(j, d, M, L, A)` (M and L are the head's; use them where d == 0). s_m and s_l hold
-// 16 * G floats, s_acc 16 * G * 128. 256 threads, all of them call.
+// 16 * G floats, s_acc 16 * G * 128; xch is the stream's exchange area. 256 threads, all of them call.
 template <int G, class Store>
-__device__ __forceinline__ void fold_streams(float (&m)[G], float (&l)[G], float (&acc)[G][8], int grp, int dl,
-                                             float* s_m, float* s_l, float* s_acc, int tid, Store store) {
+__device__ __forceinline__ void fold_streams(const AttnState<G>& st, int grp, int dl, float* xch, float* s_m, float* s_l,
+                                             float* s_acc, int tid, Store store) {
     const float ninf = bits_f32(0xff800000u);
+    float m[G], l[G];
+    heads_state<G>(st, dl, xch, m, l);
     if (dl == 0) {
 #pragma unroll
         for (int j = 0; j < G; ++j) s_m[grp * G + j] = m[j];
@@ -193,8 +338,8 @@ __device__ __forceinline__ void fold_streams(float (&m)[G], float (&l)[G], float
         // the lane's eight values as two 16-byte stores (s_acc is 16-byte aligned): one value a store would put
         // lanes four apart on one bank
         float4* dst = reinterpret_cast<float4*>(s_acc + (grp * G + j) * AD + dl * 8);
-        dst[0] = make_float4(acc[j][0] * f, acc[j][1] * f, acc[j][2] * f, acc[j][3] * f);
-        dst[1] = make_float4(acc[j][4] * f, acc[j][5] * f, acc[j][6] * f, acc[j][7] * f);
+        dst[0] = make_float4(st.acc[j][0] * f, st.acc[j][1] * f, st.acc[j][2] * f, st.acc[j][3] * f);
+        dst[1] = make_float4(st.acc[j][4] * f, st.acc[j][5] * f, st.acc[j][6] * f, st.acc[j][7] * f);
     }
     __syncthreads();
     for (int o = tid; o < G * AD; o += 256) {

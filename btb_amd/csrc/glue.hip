@@ -226,6 +226,7 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     constexpr int D = ATT_D;
     __shared__ float s_m[16][G], s_l[16][G];
     __shared__ __align__(16) float s_acc[16][G][D];
+    __shared__ __align__(16) float s_x[16][XCH];  // the streams' exchange areas
     const int g = blockIdx.x, sp = blockIdx.y, t = blockIdx.z, S = gridDim.y;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int sub = lane >> 4, dl = lane & 15;   // the lane's key within a quad of keys, its 8 dims
@@ -254,14 +255,8 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
         qp[j][2] = raw.z;
         qp[j][3] = raw.w;
     }
-    float m[G], l[G], acc[G][8];
-#pragma unroll
-    for (int j = 0; j < G; ++j) {
-        m[j] = bits_f32(0xff800000u);
-        l[j] = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
-    }
+    AttnState<G> st;
+    st.init();
     const uint16_t* Kh = K + (size_t)g * hs + dl * 8;
     const uint16_t* Vh = V + (size_t)g * hs + dl * 8;
     // eight keys of the stream a batch: their sixteen loads are issued together, and the next batch's before this one
@@ -272,12 +267,12 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     for (int key0 = k_begin + grp; key0 < k_end; key0 += 16 * KB) {
         KeyBatch nx;
         load_keys(nx, Kh, Vh, rs, key0 + 16 * KB, k_end, -1);
-        use_keys<G>(kb, key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, m, l, acc, tree_base, tree_mask);
+        use_keys<G>(kb, key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, st, &s_x[grp][0], tree_base, tree_mask);
         kb = nx;
     }
     // the 16 streams folded in stream order, the workgroup's state out
     const size_t prow = ((size_t)t * Hk + g) * S + sp;  // this workgroup's slot among the partial states
-    fold_streams<G>(m, l, acc, grp, dl, &s_m[0][0], &s_l[0][0], &s_acc[0][0][0], threadIdx.x,
+    fold_streams<G>(st, grp, dl, &s_x[grp][0], &s_m[0][0], &s_l[0][0], &s_acc[0][0][0], threadIdx.x,
                     [&](int j, int d, float M, float L, float A) {
                         part_acc[(prow * G + j) * D + d] = A;
                         if (d == 0) {
@@ -311,6 +306,7 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
     __shared__ __align__(16) uint16_t s_k[D], s_v[D];
     __shared__ float s_m[16][GW], s_l[16][GW];
     __shared__ __align__(16) float s_acc[16][GW][D];
+    __shared__ __align__(16) float s_x[16][XCH];  // the streams' exchange areas
     const int Gt = Hq / Hk;                                  // query heads a kv head
     const int g = blockIdx.x % Hk, part = blockIdx.x / Hk;   // consecutive workgroups: consecutive kv heads
     const int j0 = part * GW;                                // the first of this workgroup's heads among the Gt
@@ -363,25 +359,19 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
     for (int j = 0; j < GW; ++j)
 #pragma unroll
         for (int e = 0; e < 4; ++e) qp[j][e] = s_q[j][dl * 4 + e];
-    float m[GW], l[GW], acc[GW][8];
-#pragma unroll
-    for (int j = 0; j < GW; ++j) {
-        m[j] = bits_f32(0xff800000u);
-        l[j] = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
-    }
+    AttnState<GW> st;
+    st.init();
     // a span of several batches asks for the next one before it folds the current one in (past the span's end the
     // request falls on its last key again and is dropped)
     const bool batches = k_begin + 16 * KB < k_end;  // uniform: the span holds more than one batch of live keys
     for (int key0 = key_first; key0 < k_end; key0 += 16 * KB) {
         KeyBatch nx;
         if (batches) load_keys_upto(nx, Kh, Vh, rs, key0 + 16 * KB, k_lim);
-        use_keys<GW, true>(kb, key0, k_end, holds_own ? n0 : -1, s_k, s_v, dl, qp, scale_log2, m, l, acc);
+        use_keys<GW, true>(kb, key0, k_end, holds_own ? n0 : -1, s_k, s_v, dl, qp, scale_log2, st, &s_x[grp][0]);
         if (batches) kb = nx;
     }
     const size_t prow = (size_t)g * S + sp;
-    fold_streams<GW>(m, l, acc, grp, dl, &s_m[0][0], &s_l[0][0], &s_acc[0][0][0], threadIdx.x,
+    fold_streams<GW>(st, grp, dl, &s_x[grp][0], &s_m[0][0], &s_l[0][0], &s_acc[0][0][0], threadIdx.x,
                      [&](int j, int d, float M, float L, float A) {
                          part_acc[((prow * Gt) + j0 + j) * D + d] = A;
                          if (d == 0) {
@@ -615,7 +605,9 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
         const int32_t rc = scratch_on_device(&work);
         if (rc != OK) return rc;
     }
-    const int span = (int)((cap + S - 1) / S);
+    // a span is a whole number of the workgroup's batches of keys (16 streams by 8 keys): a batch is the unit of its
+    // work, and a span that ends inside one pays for all of it
+    const int span = (int)(((cap + S - 1) / S + 127) / 128 * 128);
     float* part_m = work;
     float* part_l = work + T * Hq * S;
     float* part_acc = work + 2 * T * Hq * S;
@@ -675,7 +667,9 @@ int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk,
         set_error("attn_decode_qkv: spans * (query heads per kv head) is at most 1024");
         return ERR_DOMAIN;
     }
-    const int span = (int)((cap + S - 1) / S);
+    // a span is a whole number of the workgroup's batches of keys (16 streams by 8 keys): a batch is the unit of its
+    // work, and a span that ends inside one pays for all of it
+    const int span = (int)(((cap + S - 1) / S + 127) / 128 * 128);
     float* part_m = workspace;
     float* part_l = workspace + Hq * S;
     float* part_acc = workspace + 2 * Hq * S;
@@ -685,8 +679,8 @@ int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk,
     const size_t mlds = 2 * S * G * sizeof(float);
     // query heads a workgroup takes: all G of its kv head, or fewer (the workgroups of one kv head are Hk apart in
     // the grid, which on this GPU - workgroups dealt to its eight dies in turn - keeps them on one die when Hk is 8)
-    // Measured on MI355X (Qwen3-4B shape, 4096 keys, whole step): two heads a workgroup and 16 spans 2.295 ms, four
-    // heads and 32 spans 2.371, one head and 8 spans 2.351 - each 256 workgroups.
+    // Measured on MI355X (Qwen3-4B shape, 4096 keys of 4608 slots, whole step): two heads a workgroup and 18 spans (of
+    // 256 keys) 2.215 ms, four heads 2.249, one head 2.333; two heads with 16 spans (288 keys: 2.25 batches) 2.274.
     int gw = tuning("attn_heads_per_wg");
     if (gw <= 0 || gw > (int)G || G % gw != 0 || (gw & (gw - 1)) != 0) gw = G >= 4 ? 2 : (int)G;
     const dim3 grid((unsigned)(Hk * (G / gw)), (unsigned)S);

@@ -397,6 +397,8 @@ __device__ __forceinline__ void attention_item(const StepArgs& a, const StepLaye
     float* s_m = lds + G * AD + AD;  // [16][G]
     float* s_l = s_m + 16 * G;       // [16][G]
     float* s_acc = s_l + 16 * G;     // [16][G][128]
+    __shared__ __align__(16) float s_xs[16 * XCH];  // the streams' exchange areas
+    float* s_x = s_xs;
     __shared__ int s_last;
     const int lane = tid & 63, wv = tid >> 6;
     const int Hq = a.Hq, Hk = a.Hk;
@@ -437,16 +439,10 @@ __device__ __forceinline__ void attention_item(const StepArgs& a, const StepLaye
     for (int j = 0; j < G; ++j)
 #pragma unroll
         for (int e = 0; e < 4; ++e) qp[j][e] = reinterpret_cast<const uint32_t*>(s_q)[j * (AD / 2) + dl * 4 + e];
-    float m[G], l[G], acc[G][8];
-#pragma unroll
-    for (int j = 0; j < G; ++j) {
-        m[j] = bits_f32(0xff800000u);
-        l[j] = 0.f;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) acc[j][e] = 0.f;
-    }
+    AttnState<G> st;
+    st.init();
     for (int key0 = key_first; key0 < k_end;) {
-        use_keys<G>(kb, key0, k_end, (n0 >= k_begin && n0 < k_begin + a.span) ? n0 : -1, s_k, s_v, dl, qp, a.scale_log2, m, l, acc);
+        use_keys<G>(kb, key0, k_end, (n0 >= k_begin && n0 < k_begin + a.span) ? n0 : -1, s_k, s_v, dl, qp, a.scale_log2, st, s_x + grp * XCH);
         key0 += 16 * KB;
         if (key0 < k_end) load_keys(kb, Kh, Vh, a.rs, key0, k_end, n0);
     }
@@ -454,7 +450,7 @@ __device__ __forceinline__ void attention_item(const StepArgs& a, const StepLaye
     float* part_l = a.part + (size_t)Hq * a.S;
     float* part_acc = a.part + 2 * (size_t)Hq * a.S;
     const size_t prow = (size_t)g * a.S + sp;
-    fold_streams<G>(m, l, acc, grp, dl, s_m, s_l, s_acc, tid, [&](int j, int d, float M, float Lsum, float A) {
+    fold_streams<G>(st, grp, dl, s_x + grp * XCH, s_m, s_l, s_acc, tid, [&](int j, int d, float M, float Lsum, float A) {
         st_dev(&part_acc[(prow * G + j) * AD + d], A);
         if (d == 0) {
             st_dev(&part_m[prow * G + j], M);

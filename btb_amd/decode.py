@@ -131,9 +131,11 @@ class DecodeStep:
         if attn_spans is None:
             attn_spans = max(1, min(self.cap // 64, (card.sms + Hk - 1) // Hk, (2 * card.sms) // (Hk * self.T)))
             if self.T == 1 and D == 128 and Hq // Hk >= 4:
-                # the step's own attention kernel splits a kv head's query heads over workgroups of two heads: one
-                # workgroup a CU then means a CU's worth of (kv head, head pair, span) triples
-                attn_spans = max(1, min(self.cap // 64, card.sms // (Hk * (Hq // Hk // 2))))
+                # the step's own attention kernel splits a kv head's query heads over workgroups of two heads, and a
+                # workgroup folds its span 128 keys at a time: about a CU's worth of (kv head, head pair, span)
+                # triples, each span a whole number of those batches (the library rounds a span up to one)
+                per = max(128, self.cap // max(1, card.sms // (Hk * (Hq // Hk // 2))) // 128 * 128)
+                attn_spans = max(1, -(-self.cap // per))
         self.S = int(attn_spans)
         self.scratch = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
         # Which sequence: up to three rows the fused launches win (fewer launches, every matvec on the streaming
@@ -205,7 +207,7 @@ class DecodeStep:
         a = StepArgs()
         a.layers = ptr(self._layer_table)
         a.nlayers, a.H, a.Hq, a.Hk, a.I, a.vocab = cfg.layers, H, Hq, Hk, I, cfg.vocab
-        a.S, a.span = self.S, (self.cap + self.S - 1) // self.S
+        a.S, a.span = self.S, ((self.cap + self.S - 1) // self.S + 127) // 128 * 128  # the library's rule for a span
         a.hs, a.rs = int(K0.stride(0)), int(K0.stride(1))
         a.eps = cfg.eps
         a.scale_log2 = float(np.float32(self.scale) * np.float32(1.4426950408889634))
