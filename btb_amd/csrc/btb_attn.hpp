@@ -71,12 +71,14 @@ struct KeyBatch {
     uint4 k[KB], v[KB];
 };
 __device__ __forceinline__ void load_keys(KeyBatch& kb, const uint16_t* Kh, const uint16_t* Vh, long long rs, int key0,
-                                          int k_end, int n0) {
+                                          int k_end, int n0, const int32_t* tbl = nullptr) {
 #pragma unroll
     for (int b = 0; b < KB; ++b) {
         const int key = min(key0 + 16 * b, k_end - 1);  // a key past the span's end is loaded again, not used
         // slot n0 is this step's own row: it is taken from LDS, the cache's copy may not have landed yet
-        const int safe = key == n0 ? max(n0 - 1, 0) : key;
+        int safe = key == n0 ? max(n0 - 1, 0) : key;
+        // the cache's row map (the reference's `tbl`, native/cuda/btb_attn_flash.cuh:34): logical slot -> cache row
+        if (tbl != nullptr) safe = tbl[safe];
         kb.k[b] = *reinterpret_cast<const uint4*>(Kh + (size_t)safe * rs);
         kb.v[b] = *reinterpret_cast<const uint4*>(Vh + (size_t)safe * rs);
     }
@@ -189,7 +191,8 @@ __device__ __forceinline__ float tsum8(const float* v, int dl) {
 template <int G, bool ZERO_DEAD = false>
 __device__ __forceinline__ void use_keys(KeyBatch& kb, int key0, int k_end, int own, const uint16_t* s_k,
                                          const uint16_t* s_v, int dl, const uint32_t (&qp)[G][4], float scale_log2,
-                                         AttnState<G>& st, float* xch, int tree_base = -1, uint32_t tree_mask = 0u) {
+                                         AttnState<G>& st, float* xch, int tree_base = -1, uint32_t tree_mask = 0u,
+                                         int k_first = 0) {
     constexpr int R = attn_slots(G);
     static_assert(G == 1 || G == 2 || G == 4 || G == 8, "1, 2, 4 or 8 query heads a stream");
     const float ninf = bits_f32(0xff800000u);
@@ -217,8 +220,13 @@ __device__ __forceinline__ void use_keys(KeyBatch& kb, int key0, int k_end, int 
     // the lane's own key slot
     const int bk = dl & 7;
     const int key = key0 + 16 * bk;
+    // a cache key counts from the window's first key on (k_first; 0: no window); one of the pass's own rows counts when
+    // the mask names it (the window is already in the mask: those rows stand at their depth, not at their slot)
     bool live = key < k_end;
-    if (tree_base >= 0) live = live && (key < tree_base || ((tree_mask >> min(key - tree_base, 31)) & 1u) != 0u);
+    if (tree_base >= 0 && key >= tree_base)
+        live = live && ((tree_mask >> min(key - tree_base, 31)) & 1u) != 0u;
+    else
+        live = live && key >= k_first;
     uint32_t* xw = reinterpret_cast<uint32_t*>(xch);
 #pragma unroll
     for (int r = 0; r < R; ++r) {

@@ -157,11 +157,13 @@ __global__ void __launch_bounds__(64) norm_rope_kv_kernel(const uint16_t* __rest
                                                           const uint16_t* __restrict__ sin_t, const int32_t* __restrict__ n0p,
                                                           const int32_t* __restrict__ depth, uint16_t* __restrict__ K,
                                                           uint16_t* __restrict__ V, uint16_t* __restrict__ qo, int Hq,
-                                                          int Hk, long long hs, long long rs, int centered) {
+                                                          int Hk, long long hs, long long rs, int centered,
+                                                          const int32_t* __restrict__ tbl) {
     constexpr int E = D / 64;
     const int head = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
     const int n0 = *n0p;
-    const int slot = n0 + t;
+    int slot = n0 + t;
+    if (tbl != nullptr) slot = tbl[slot];  // the cache's row map: the row lands where the attention's walk reads it
     const int pos = n0 + (depth != nullptr ? depth[t] : t);
     const int width = (Hq + 2 * Hk) * D;
     const uint16_t* src = qkv + (size_t)t * width + (size_t)head * D + lane * E;
@@ -222,7 +224,7 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
                                                           const int32_t* __restrict__ par, int T, int Hq, int Hk, long long hs,
                                                           long long rs, float scale_log2, float* __restrict__ part_m,
                                                           float* __restrict__ part_l, float* __restrict__ part_acc,
-                                                          int span) {
+                                                          int span, int win, const int32_t* __restrict__ tbl) {
     constexpr int D = ATT_D;
     __shared__ float s_m[16][G], s_l[16][G];
     __shared__ __align__(16) float s_acc[16][G][D];
@@ -238,11 +240,21 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     int tree_base = -1;
     uint32_t tree_mask = 0u;
     int n = n0 + t + 1;
+    int last = n0 + t;  // the row's own logical position: a chain's row t stands at n0 + t, a tree's at n0 + its depth
     if (par != nullptr) {
         tree_base = n0;
         n = n0 + T;
-        for (int p = t, hops = 0; p >= 0 && p < T && hops < 32; p = par[p], ++hops) tree_mask |= 1u << p;
+        int depth = -1;
+        for (int p = t, hops = 0; p >= 0 && p < T && hops < 32; p = par[p], ++hops) ++depth;
+        last = n0 + depth;
+        // the row's keys among the pass's rows: itself and its ancestors, the one at depth d standing at n0 + d - under
+        // a window (the reference's `first = last + 1 - win`, native/cuda/btb_attn_flash.cuh:437) those at or past it
+        const int first_depth = win > 0 ? last + 1 - win - n0 : 0;
+        int d = depth;
+        for (int p = t, hops = 0; p >= 0 && p < T && hops < 32; p = par[p], ++hops, --d)
+            if (d >= first_depth) tree_mask |= 1u << p;
     }
+    const int k_first = win > 0 ? max(last + 1 - win, 0) : 0;
     const int k_begin = sp * span, k_end = min(n, k_begin + span);
 
     // the row's G query heads, the lane's 8 dims of each as bf16 pairs (the scale meets the folded score)
@@ -263,11 +275,12 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     // is folded in (past the span's end they fall on its last key again, unused), so a span of several batches - a
     // pass of many rows takes long spans - pays the trip to memory once
     KeyBatch kb;
-    load_keys(kb, Kh, Vh, rs, k_begin + grp, max(k_end, 1), -1);
+    load_keys(kb, Kh, Vh, rs, k_begin + grp, max(k_end, 1), -1, tbl);
     for (int key0 = k_begin + grp; key0 < k_end; key0 += 16 * KB) {
         KeyBatch nx;
-        load_keys(nx, Kh, Vh, rs, key0 + 16 * KB, k_end, -1);
-        use_keys<G>(kb, key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, st, &s_x[grp][0], tree_base, tree_mask);
+        load_keys(nx, Kh, Vh, rs, key0 + 16 * KB, k_end, -1, tbl);
+        use_keys<G>(kb, key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, st, &s_x[grp][0], tree_base, tree_mask,
+                    k_first);
         kb = nx;
     }
     // the 16 streams folded in stream order, the workgroup's state out
@@ -494,12 +507,12 @@ __global__ void __launch_bounds__(1024) argmax_kernel(const uint16_t* __restrict
 // the step's end: the picked token becomes the next step's input and the cache grows by one on the device; with
 // pinned host buffers, the token, the GPU clock and then (after a system fence) the new length go to the host
 __global__ void publish_kernel(int32_t* __restrict__ n0, const int32_t* __restrict__ picked, int32_t* __restrict__ next_ids,
-                               int32_t* out_tok, int32_t* out_n0, long long* out_ts) {
+                               int32_t* out_tok, int32_t* out_n0, long long* out_ts, int advance) {
     if (threadIdx.x != 0 || blockIdx.x != 0) return;
     const int tok = *picked;
-    const int len = *n0 + 1;
+    const int len = *n0 + (advance ? 1 : 0);
     if (next_ids != nullptr) *next_ids = tok;
-    *n0 = len;
+    if (advance) *n0 = len;
     if (out_tok != nullptr) {
         *out_tok = tok;
         if (out_ts != nullptr) *out_ts = (long long)wall_clock64();
@@ -537,15 +550,15 @@ int32_t btb_hip_add_rmsnorm(void* h, const void* y, const void* w, float eps, vo
     return hip_status(hipGetLastError(), "add_rmsnorm launch");
 }
 
-int32_t btb_hip_norm_rope_kv(const void* qkv, const void* wq, const void* wk, float eps, const void* cos_t,
-                             const void* sin_t, const int32_t* n0, const int32_t* depth, void* K, void* V, void* q,
-                             size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered,
-                             void* stream) {
+static int32_t norm_rope_kv_any(const void* qkv, const void* wq, const void* wk, float eps, const void* cos_t,
+                                const void* sin_t, const int32_t* n0, const int32_t* depth, void* K, void* V, void* q,
+                                size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered,
+                                const int32_t* tbl, void* stream) {
     if (qkv == nullptr || cos_t == nullptr || sin_t == nullptr || n0 == nullptr || K == nullptr || V == nullptr ||
         q == nullptr)
         return ERR_NULL;
     if (T == 0 || Hq == 0 || Hk == 0 || T > 65535 || Hq + 2 * Hk > 0x7FFFFFFFull || hs <= 0 || rs <= 0 ||
-        !(eps >= 0.f))
+        !(eps >= 0.f) || !al(tbl, 4))
         return ERR_DOMAIN;
     if (D != 64 && D != 128 && D != 256) return ERR_DOMAIN;
     const dim3 grid((unsigned)(Hq + 2 * Hk), (unsigned)T);
@@ -555,7 +568,7 @@ int32_t btb_hip_norm_rope_kv(const void* qkv, const void* wq, const void* wk, fl
                        static_cast<const uint16_t*>(wq), static_cast<const uint16_t*>(wk), eps,                      \
                        static_cast<const uint16_t*>(cos_t), static_cast<const uint16_t*>(sin_t), n0, depth,          \
                        static_cast<uint16_t*>(K), static_cast<uint16_t*>(V), static_cast<uint16_t*>(q), (int)Hq,      \
-                       (int)Hk, (long long)hs, (long long)rs, centered)
+                       (int)Hk, (long long)hs, (long long)rs, centered, tbl)
     if (D == 64)
         NRK(64);
     else if (D == 128)
@@ -564,6 +577,23 @@ int32_t btb_hip_norm_rope_kv(const void* qkv, const void* wq, const void* wk, fl
         NRK(256);
 #undef NRK
     return hip_status(hipGetLastError(), "norm_rope_kv launch");
+}
+
+int32_t btb_hip_norm_rope_kv(const void* qkv, const void* wq, const void* wk, float eps, const void* cos_t,
+                             const void* sin_t, const int32_t* n0, const int32_t* depth, void* K, void* V, void* q,
+                             size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered,
+                             void* stream) {
+    return norm_rope_kv_any(qkv, wq, wk, eps, cos_t, sin_t, n0, depth, K, V, q, T, Hq, Hk, D, hs, rs, centered, nullptr,
+                            stream);
+}
+
+int32_t btb_hip_norm_rope_kv_tbl(const void* qkv, const void* wq, const void* wk, float eps, const void* cos_t,
+                                 const void* sin_t, const int32_t* n0, const int32_t* depth, void* K, void* V, void* q,
+                                 size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered,
+                                 const int32_t* tbl, void* stream) {
+    if (tbl == nullptr) return ERR_NULL;
+    return norm_rope_kv_any(qkv, wq, wk, eps, cos_t, sin_t, n0, depth, K, V, q, T, Hq, Hk, D, hs, rs, centered, tbl,
+                            stream);
 }
 
 size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, size_t S) {
@@ -575,7 +605,8 @@ size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, siz
 // `work` is the caller's workspace, or nullptr for the library's own static array on the current device
 static int32_t attn_decode_any(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
                                const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
-                               float scale, size_t cap, size_t S, float* work, bool own_scratch, void* stream) {
+                               float scale, size_t cap, size_t S, float* work, bool own_scratch, void* stream,
+                               int64_t win = 0, const int32_t* tbl = nullptr) {
     if (q == nullptr || K == nullptr || V == nullptr || att == nullptr || n0 == nullptr ||
         (!own_scratch && work == nullptr))
         return ERR_NULL;
@@ -587,7 +618,9 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
         set_error("attn_decode: head_dim 128 and at most 8 query heads per kv head");
         return ERR_DOMAIN;
     }
-    if (!al(q, 16) || !al(K, 16) || !al(V, 16) || !al(par, 4) || (rs % 8) != 0 || (hs % 8) != 0) return ERR_DOMAIN;
+    if (!al(q, 16) || !al(K, 16) || !al(V, 16) || !al(par, 4) || !al(tbl, 4) || (rs % 8) != 0 || (hs % 8) != 0 ||
+        win < 0 || win > 0x7FFFFFFF)
+        return ERR_DOMAIN;
     if (par != nullptr && T > 32) {
         set_error("attn_decode: a tree pass holds at most 32 rows");
         return ERR_DOMAIN;
@@ -619,7 +652,8 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
 #define ATT(GG)                                                                                                      \
     hipLaunchKernelGGL(attn_decode_kernel<GG>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(q),              \
                        static_cast<const uint16_t*>(K), static_cast<const uint16_t*>(V), n0, par, (int)T, (int)Hq,   \
-                       (int)Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, span);            \
+                       (int)Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, span, (int)win,   \
+                       tbl);                                                                                         \
     hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,       \
                        (int)Hk, (int)S, part_m, part_l, part_acc)
     switch (G) {
@@ -639,6 +673,14 @@ int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* a
                             const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
                             float scale, size_t cap, size_t S, float* workspace, void* stream) {
     return attn_decode_any(q, K, V, att, n0, par, T, Hq, Hk, D, hs, rs, scale, cap, S, workspace, false, stream);
+}
+
+int32_t btb_hip_attn_decode_win(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
+                                const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
+                                float scale, size_t cap, size_t S, int64_t win, const int32_t* tbl, float* workspace,
+                                void* stream) {
+    return attn_decode_any(q, K, V, att, n0, par, T, Hq, Hk, D, hs, rs, scale, cap, S, workspace, false, stream, win,
+                           tbl);
 }
 
 int32_t btb_hip_attn_decode_noalloc(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
@@ -746,7 +788,15 @@ int32_t btb_hip_publish(int32_t* n0, const int32_t* picked, int32_t* next_ids, i
                         int64_t* out_ts, void* stream) {
     if (n0 == nullptr || picked == nullptr) return ERR_NULL;
     hipLaunchKernelGGL(publish_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), n0, picked, next_ids,
-                       out_tok, out_n0, reinterpret_cast<long long*>(out_ts));
+                       out_tok, out_n0, reinterpret_cast<long long*>(out_ts), 1);
+    return hip_status(hipGetLastError(), "publish launch");
+}
+
+int32_t btb_hip_publish_only(const int32_t* n0, const int32_t* ids, int32_t* out_tok, int32_t* out_n0, int64_t* out_ts,
+                             void* stream) {
+    if (n0 == nullptr || ids == nullptr || out_tok == nullptr) return ERR_NULL;
+    hipLaunchKernelGGL(publish_kernel, dim3(1), dim3(64), 0, static_cast<hipStream_t>(stream), const_cast<int32_t*>(n0),
+                       ids, static_cast<int32_t*>(nullptr), out_tok, out_n0, reinterpret_cast<long long*>(out_ts), 0);
     return hip_status(hipGetLastError(), "publish launch");
 }
 

@@ -9,6 +9,9 @@ stored forms are taken as they are, none widened to bf16 in memory:
               a 12-bit store holds only `layers.*` and names its       the per-row escape index is built on the GPU at
               parent under `config.json: btb.source`)                   load)
   fp8 e4m3    `<name>.weight` float8_e4m3fn + `<name>.weight_scale_inv` -> `F8Weight` (bytes + the f32 scale grid)
+  mxfp4       `<name>_blocks` u8 [E, rows, K/32, 16] + `<name>_scales`  -> `MxExperts`: a layer's expert stacks as stored
+              u8 [E, rows, K/32] (gpt-oss's routed experts,              (17 bytes per 32 weights), an expert's matrix an
+              btb/mxfp4.py:4-29, 127-168)                               `MxWeight` view into them
 
 The card's step multiplies q/k/v as one matrix and gate/up as one (btb/engine/cuda.py:1722-1834), so the loader
 stacks them by rows: bf16 rows are concatenated; FP8 bytes and their scale grids are concatenated (every part holds a
@@ -30,6 +33,7 @@ from safetensors import safe_open
 from . import pack12
 from .decode import Linear, StackConfig
 from .fp8 import E4M3, F8Weight, scale_grid
+from .mxfp4 import BLOCK, BLOCK_BYTES, MxWeight
 from .pack12 import P12Weight
 
 
@@ -193,3 +197,66 @@ def load_stack(card: Any, path: str, fuse: bool = True, device: Any = "cuda") ->
     tied = bool(raw.get("tie_word_embeddings", False)) or not store.has("lm_head.weight")
     w["head"] = Linear(card, w["embed"] if tied else _matrix(store, card, "lm_head.weight", dev))
     return cfg, w
+
+
+class MxExperts:
+    """One layer's routed experts as an MXFP4 checkpoint stores them, in VRAM unchanged: `gate_up_blocks` u8
+    [E, 2I, H/32, 16] with `gate_up_scales` u8 [E, 2I, H/32], `down_blocks` u8 [E, H, I/32, 16] with `down_scales`
+    (btb/mxfp4.py:4-29: 32 weights along K share 16 bytes and one e8m0 exponent; the slot order of an expert is
+    gate_up blocks, gate_up scales, down blocks, down scales). gpt-oss interleaves its gate and up rows (gate at the
+    even rows); the rows are kept as stored. `gate_up(e)` / `down(e)` are expert e's matrices as `MxWeight` views
+    (no copy) for `HipCard.gemv_mx4`; `widen` is `HipCard.mx4_widen` over a whole stack or the experts at `seats`."""
+
+    __slots__ = ("down_blocks", "down_scales", "experts", "gate_up_blocks", "gate_up_scales", "hidden", "intermediate")
+
+    def __init__(self, gate_up_blocks: torch.Tensor, gate_up_scales: torch.Tensor, down_blocks: torch.Tensor,
+                 down_scales: torch.Tensor) -> None:
+        for b, sc, what in ((gate_up_blocks, gate_up_scales, "gate_up"), (down_blocks, down_scales, "down")):
+            if b.dtype != torch.uint8 or sc.dtype != torch.uint8 or b.dim() != 4 or b.shape[-1] != BLOCK_BYTES \
+                    or tuple(b.shape[:-1]) != tuple(sc.shape):
+                raise ValueError(f"[load] {what}: MXFP4 stacks are uint8 blocks [E, rows, K/32, {BLOCK_BYTES}] with "
+                                 f"scales [E, rows, K/32], got {tuple(b.shape)} {b.dtype} and {tuple(sc.shape)} {sc.dtype}")
+        E, rows_gu, g_h = (int(v) for v in gate_up_scales.shape)
+        E2, rows_dn, g_i = (int(v) for v in down_scales.shape)
+        H, I = g_h * BLOCK, g_i * BLOCK
+        if E != E2 or rows_dn != H or rows_gu != 2 * I:
+            raise ValueError(f"[load] gate_up [{E}, {rows_gu}, {H}] and down [{E2}, {rows_dn}, {I}] are not one layer's "
+                             f"experts")
+        self.gate_up_blocks, self.gate_up_scales = gate_up_blocks.contiguous(), gate_up_scales.contiguous()
+        self.down_blocks, self.down_scales = down_blocks.contiguous(), down_scales.contiguous()
+        self.experts, self.hidden, self.intermediate = E, H, I
+
+    def gate_up(self, e: int) -> MxWeight:
+        return MxWeight(self.gate_up_blocks[e].reshape(-1), self.gate_up_scales[e].reshape(-1), 2 * self.intermediate,
+                        self.hidden)
+
+    def down(self, e: int) -> MxWeight:
+        return MxWeight(self.down_blocks[e].reshape(-1), self.down_scales[e].reshape(-1), self.hidden, self.intermediate)
+
+    @property
+    def nbytes(self) -> int:
+        return sum(int(t.numel()) for t in (self.gate_up_blocks, self.gate_up_scales, self.down_blocks, self.down_scales))
+
+    def widen(self, card: Any, which: str, seats: torch.Tensor | None = None,
+              dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
+        """the `which` ("gate_up" or "down") matrices of every expert, or of those at `seats`, widened on the GPU:
+        [n, rows, K] in `dtype`"""
+        if which not in ("gate_up", "down"):
+            raise ValueError("[load] which is 'gate_up' or 'down'")
+        blocks = self.gate_up_blocks if which == "gate_up" else self.down_blocks
+        scales = self.gate_up_scales if which == "gate_up" else self.down_scales
+        flat = card.mx4_widen(blocks, scales, seats, dtype=dtype)
+        return flat.reshape(flat.shape[0], int(scales.shape[1]), int(scales.shape[2]) * BLOCK)
+
+
+def load_mx_experts(path: str | Store, layer: int, device: Any = "cuda",
+                    prefix: str = "model.layers.{i}.mlp.experts.") -> MxExperts:
+    """layer `layer`'s MXFP4 expert stacks of a store, uploaded as stored (`<prefix>{gate_up,down}_proj_{blocks,scales}`)"""
+    store = path if isinstance(path, Store) else Store(path)
+    base = prefix.format(i=int(layer))
+    names = [base + n for n in ("gate_up_proj_blocks", "gate_up_proj_scales", "down_proj_blocks", "down_proj_scales")]
+    missing = [n for n in names if not store.has(n)]
+    if missing:
+        raise KeyError(f"[load] not an MXFP4 expert layer: {missing[0]} is not in {store.path}")
+    dev = torch.device(device)
+    return MxExperts(*(store.get(n).to(dev) for n in names))

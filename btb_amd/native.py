@@ -63,6 +63,11 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_add_rmsnorm": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _sz, _sz, _i32, _vp]),
     "btb_hip_norm_rope_kv": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
                                     _sz, ctypes.c_int64, ctypes.c_int64, _i32, _vp]),
+    "btb_hip_norm_rope_kv_tbl": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
+                                        _sz, ctypes.c_int64, ctypes.c_int64, _i32, _vp, _vp]),
+    "btb_hip_attn_decode_win": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
+                                       ctypes.c_float, _sz, _sz, ctypes.c_int64, _vp, _vp, _vp]),
+    "btb_hip_publish_only": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_attn_scratch_floats": (_sz, [_sz, _sz, _sz, _sz, _sz]),
     "btb_hip_attn_decode": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
                                    ctypes.c_float, _sz, _sz, _vp, _vp]),
@@ -126,26 +131,41 @@ def _launch_table() -> dict[str, tuple[int, Any]]:
     """reference kernel name -> (its parameter count, parameters -> (entry point, its arguments less the stream))"""
     t: dict[str, tuple[int, Any]] = {}
     for M in (1, 2, 4, 8, 16, 32):
-        t[f"btb_gemv_bf16_m{M}"] = (5, lambda v, g, M=M: ("btb_hip_gemv_bf16", (v[0], v[1], v[2], v[3], v[4], M)))
-        t[f"btb_gemv_silu_bf16_m{M}"] = (5, lambda v, g, M=M: ("btb_hip_gemv_silu_bf16", (v[0], v[1], v[2], v[3], v[4], M)))
-        t[f"btb_gemv_lane16_f32_m{M}"] = (5, lambda v, g, M=M: ("btb_hip_gemv_bf16_rows", (v[0], v[3], v[4], v[1], M, v[2])))
+        t[f"btb_gemv_bf16_m{M}"] = (5, lambda v, g, card, M=M: ("btb_hip_gemv_bf16", (v[0], v[1], v[2], v[3], v[4], M)))
+        t[f"btb_gemv_silu_bf16_m{M}"] = (5, lambda v, g, card, M=M: ("btb_hip_gemv_silu_bf16", (v[0], v[1], v[2], v[3], v[4], M)))
+        t[f"btb_gemv_lane16_f32_m{M}"] = (5, lambda v, g, card, M=M: ("btb_hip_gemv_bf16_rows", (v[0], v[3], v[4], v[1], M, v[2])))
         t[f"btb_gemv_lane16_mx4_f32_m{M}"] = (
-            6, lambda v, g, M=M: ("btb_hip_gemv_mxfp4_rows", (v[0], v[1], v[4], v[5], v[2], M, v[3])))
+            6, lambda v, g, card, M=M: ("btb_hip_gemv_mxfp4_rows", (v[0], v[1], v[4], v[5], v[2], M, v[3])))
     for n in ("btb_gemv_mma_bf16", "btb_gemv_mma8_bf16"):
-        t[n] = (6, lambda v, g: ("btb_hip_gemv_bf16", (v[0], v[1], v[2], v[3], v[4], v[5])))
-    t["btb_gemv_mma_glu_silu"] = (6, lambda v, g: ("btb_hip_gemv_glu_silu_bf16", (v[0], v[1], v[2], v[3], v[4], v[5])))
-    t["btb_silu_mul"] = (4, lambda v, g: ("btb_hip_silu_mul", (v[0], v[1], v[2], v[3])))
+        t[n] = (6, lambda v, g, card: ("btb_hip_gemv_bf16", (v[0], v[1], v[2], v[3], v[4], v[5])))
+    t["btb_gemv_mma_glu_silu"] = (6, lambda v, g, card: ("btb_hip_gemv_glu_silu_bf16", (v[0], v[1], v[2], v[3], v[4], v[5])))
+    t["btb_silu_mul"] = (4, lambda v, g, card: ("btb_hip_silu_mul", (v[0], v[1], v[2], v[3])))
     # btb_add_rmsnorm(h, y, w, eps, x, H, centered), a block a row
-    t["btb_add_rmsnorm"] = (7, lambda v, g: ("btb_hip_add_rmsnorm", (v[0], v[1], v[2], v[3], v[4], g[0], v[5], v[6])))
+    t["btb_add_rmsnorm"] = (7, lambda v, g, card: ("btb_hip_add_rmsnorm", (v[0], v[1], v[2], v[3], v[4], g[0], v[5], v[6])))
     for D in (64, 128, 256):
         # (qkv, wq, wk, eps, cos, sin, n0, depth, K, V, q, T, Hq, Hk, hs, rs, centered)
-        t[f"btb_norm_rope_kv_d{D}"] = (17, lambda v, g, D=D: ("btb_hip_norm_rope_kv", (
+        t[f"btb_norm_rope_kv_d{D}"] = (17, lambda v, g, card, D=D: ("btb_hip_norm_rope_kv", (
             v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], v[9], v[10], v[11], v[12], v[13], D, v[14], v[15], v[16])))
     # btb_moe_route(logits bf16, ls, E, k, idx, w, hidx, hw, cnt, seq, hseq), a block a row; the host copies are the
     # reference's way of fetching experts from the host tier and are not made here
-    t["btb_moe_route"] = (11, lambda v, g: ("btb_hip_moe_route", (v[0], 0, v[1], v[2], v[3], g[0], v[4], v[5], None)))
+    t["btb_moe_route"] = (11, lambda v, g, card: ("btb_hip_moe_route", (v[0], 0, v[1], v[2], v[3], g[0], v[4], v[5], None)))
+    for D in (64, 128, 256):  # the same with the cache's row map as the last parameter
+        t[f"btb_norm_rope_kv_tbl_d{D}"] = (18, lambda v, g, card, D=D: ("btb_hip_norm_rope_kv_tbl", (
+            v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], v[9], v[10], v[11], v[12], v[13], D, v[14], v[15], v[16],
+            v[17])))
+    # btb_attn_flash_d128(q, K, V, out, n0p, par, T, Hq, Hk, hs, rs, scale, part_m, part_l, part_acc, cnt, win, tbl) on
+    # a grid (row tiles, key groups, kv heads): grid[1] key groups of 512 keys each reach the cache's capacity. The
+    # caller's partial-state arrays and arrival counter are not used (see HipCard._flash_work).
+    def flash(v, g, card):
+        T, Hq, S = int(v[6] or 1), int(v[7] or 1), max(int(g[1]), 1)
+        work = None if card is None else card._flash_work(T * Hq * S * 130)
+        return "btb_hip_attn_decode_win", (v[0], v[1], v[2], v[3], v[4], v[5], T, Hq, v[8], 128, v[9], v[10], v[11],
+                                           S * 512, S, v[16], v[17], work)
+    t["btb_attn_flash_d128"] = (18, flash)
+    # btb_publish(n0, ids, out_tok, out_n0, out_ts)
+    t["btb_publish"] = (5, lambda v, g, card: ("btb_hip_publish_only", (v[0], v[1], v[2], v[3], v[4])))
     # btb_mx4_widen(blocks, scales, seats, groups, out), grid.y seats
-    t["btb_mx4_widen"] = (5, lambda v, g: ("btb_hip_mx4_widen", (v[0], v[1], v[2], g[1], v[3], v[4], 0)))
+    t["btb_mx4_widen"] = (5, lambda v, g, card: ("btb_hip_mx4_widen", (v[0], v[1], v[2], g[1], v[3], v[4], 0)))
     return t
 
 
@@ -207,16 +227,27 @@ class HipCard:
             raise ValueError(f"[hip] {name} takes {count} parameters, got {len(args)}")
         vals = [a.value if isinstance(a, ctypes._SimpleCData) else a for a in args]
         st = ctypes.c_void_p((stream or torch.cuda.current_stream()).cuda_stream)
-        sym, cargs = call(vals, tuple(int(g) for g in grid))
+        sym, cargs = call(vals, tuple(int(g) for g in grid), self)
         self._call(sym, *cargs, st)
 
     @property
     def fn(self) -> dict[str, str]:
         """kernel name -> the library entry point that serves it (the reference keeps its loaded kernels here)"""
-        return {n: call([0] * count, (1, 1, 1))[0] for n, (count, call) in _LAUNCH.items()}
+        return {n: call([0] * count, (1, 1, 1), None)[0] for n, (count, call) in _LAUNCH.items()}
 
     def close(self) -> None:
-        """nothing to release (the library stays loaded for the process); may be called any number of times"""
+        """drops the card's own scratch (the library stays loaded for the process); may be called any number of times"""
+        self._flash_scratch = None
+
+    def _flash_work(self, floats: int) -> ctypes.c_void_p:
+        """the partial-state scratch behind `btb_attn_flash_d128` launched by name: the reference's caller passes
+        three arrays in its own layout (part_m / part_l / part_acc, [S, T, Hq(, D)]) and an arrival counter; this
+        library keeps one array in its own layout, owned by the card and grown on demand"""
+        cur = getattr(self, "_flash_scratch", None)
+        if cur is None or cur.numel() < floats:
+            cur = torch.empty(max(floats, 1), dtype=torch.float32, device="cuda")
+            self._flash_scratch = cur
+        return ctypes.c_void_p(cur.data_ptr())
 
     # -- bf16 matvec ------------------------------------------------------------------------------------------
 
@@ -583,19 +614,24 @@ class HipCard:
     def norm_rope_kv(self, qkv: torch.Tensor, wq: torch.Tensor | None, wk: torch.Tensor | None, eps: float,
                      cos: torch.Tensor, sin: torch.Tensor, n0: torch.Tensor, K: torch.Tensor, V: torch.Tensor,
                      q: torch.Tensor, Hq: int, Hk: int, D: int, depth: torch.Tensor | None = None,
-                     centered: bool = False) -> None:
+                     centered: bool = False, tbl: torch.Tensor | None = None) -> None:
         """q/k norm, rope and the cache write for the pass's rows (`btb_norm_rope_kv_d{D}`); K, V are one layer's
-        [Hk, cap, D] views (any strides with D contiguous)"""
+        [Hk, cap, D] views (any strides with D contiguous). `tbl` (int32, one entry a logical slot): the cache's row
+        map - row t lands in cache row tbl[n0 + t] (`btb_norm_rope_kv_tbl_d{D}`)"""
         for t, what in ((qkv, "qkv"), (cos, "cos"), (sin, "sin"), (q, "q")):
             self._need(t, torch.bfloat16, what)
         self._need(n0, torch.int32, "n0")
         if K.dtype != torch.bfloat16 or V.dtype != torch.bfloat16 or K.stride(2) != 1 or K.stride() != V.stride():
             raise ValueError("[hip] norm_rope_kv: K and V are bf16 [Hk, cap, D] views with the same strides")
         T = int(qkv.numel()) // ((Hq + 2 * Hk) * D)
-        self._call("btb_hip_norm_rope_kv", self.ptr(qkv), None if wq is None else self.ptr(wq),
-                   None if wk is None else self.ptr(wk), float(eps), self.ptr(cos), self.ptr(sin), self.ptr(n0),
-                   None if depth is None else self.ptr(depth), self.ptr(K), self.ptr(V), self.ptr(q), T, Hq, Hk, D,
-                   int(K.stride(0)), int(K.stride(1)), int(bool(centered)), _stream())
+        args = (self.ptr(qkv), None if wq is None else self.ptr(wq), None if wk is None else self.ptr(wk), float(eps),
+                self.ptr(cos), self.ptr(sin), self.ptr(n0), None if depth is None else self.ptr(depth), self.ptr(K),
+                self.ptr(V), self.ptr(q), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)), int(bool(centered)))
+        if tbl is None:
+            self._call("btb_hip_norm_rope_kv", *args, _stream())
+        else:
+            self._need(tbl, torch.int32, "tbl")
+            self._call("btb_hip_norm_rope_kv_tbl", *args, self.ptr(tbl), _stream())
 
     def attn_scratch(self, T: int, Hq: int, Hk: int, D: int, S: int, device: Any = "cuda") -> torch.Tensor:
         """the f32 scratch `attn_decode` leaves its spans' states in, at these sizes"""
@@ -604,10 +640,11 @@ class HipCard:
 
     def attn_decode(self, q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, att: torch.Tensor, n0: torch.Tensor,
                     Hq: int, Hk: int, D: int, scale: float, S: int, scratch: torch.Tensor,
-                    par: torch.Tensor | None = None) -> None:
+                    par: torch.Tensor | None = None, win: int = 0, tbl: torch.Tensor | None = None) -> None:
         """att [T, Hq * D] = the rows' attention over the cache: row t sees keys 0 .. n0 + t, or with `par` (int32 [T],
         a verify pass's tree: the row's parent among the pass's rows, -1 at a root) the cache's n0 keys and, of the
-        pass's rows, its ancestors and itself"""
+        pass's rows, its ancestors and itself. `win` > 0: only the last `win` positions up to the row's own; `tbl`
+        (int32, one entry a logical slot): the cache's row map"""
         self._need(q, torch.bfloat16, "q")
         self._need(att, torch.bfloat16, "att")
         self._need(n0, torch.int32, "n0")
@@ -622,6 +659,16 @@ class HipCard:
             self._need(par, torch.int32, "par")
             if par.numel() != T:
                 raise ValueError(f"[hip] attn_decode: par names {par.numel()} rows, the pass has {T}")
+        if win or tbl is not None:
+            if tbl is not None:
+                self._need(tbl, torch.int32, "tbl")
+                if tbl.numel() < int(K.shape[1]):
+                    raise ValueError(f"[hip] attn_decode: tbl maps {tbl.numel()} slots, the cache has {int(K.shape[1])}")
+            self._call("btb_hip_attn_decode_win", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0),
+                       None if par is None else self.ptr(par), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)),
+                       float(scale), int(K.shape[1]), S, int(win), None if tbl is None else self.ptr(tbl),
+                       self.ptr(scratch), _stream())
+            return
         self._call("btb_hip_attn_decode", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0),
                    None if par is None else self.ptr(par), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)),
                    float(scale), int(K.shape[1]), S, self.ptr(scratch), _stream())
@@ -697,6 +744,12 @@ class HipCard:
         p = lambda t: None if t is None else self.ptr(t)
         self._call("btb_hip_publish", self.ptr(n0), self.ptr(picked), p(next_ids), p(out_tok), p(out_n0), p(out_ts),
                    _stream())
+
+    def publish_only(self, n0: torch.Tensor, ids: torch.Tensor, out_tok: torch.Tensor, out_n0: torch.Tensor | None = None,
+                     out_ts: torch.Tensor | None = None) -> None:
+        """the reference's `btb_publish`: token, clock and length into pinned host tensors, nothing else"""
+        p = lambda t: None if t is None else self.ptr(t)
+        self._call("btb_hip_publish_only", self.ptr(n0), self.ptr(ids), self.ptr(out_tok), p(out_n0), p(out_ts), _stream())
 
     def argmax_publish(self, logits: torch.Tensor, picked: torch.Tensor, n0: torch.Tensor,
                        next_ids: torch.Tensor | None = None, out_tok: torch.Tensor | None = None,

@@ -233,6 +233,14 @@ int32_t btb_hip_norm_rope_kv(const void* qkv, const void* wq, const void* wk, fl
                              size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered,
                              void* stream);
 
+/* btb_hip_norm_rope_kv with the cache's row map: row t of the pass lands in cache row tbl[*n0 + t] (tbl i32 on the
+ * device, one entry per logical slot), where btb_hip_attn_decode_win's walk reads it. Replaces
+ * btb_norm_rope_kv_tbl_d{D} (native/cuda/btb_kernels.cu:268-283, 347-354). */
+int32_t btb_hip_norm_rope_kv_tbl(const void* qkv, const void* wq, const void* wk, float eps, const void* cos_t,
+                                 const void* sin_t, const int32_t* n0, const int32_t* depth, void* K, void* V, void* q,
+                                 size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered,
+                                 const int32_t* tbl, void* stream);
+
 /* floats of scratch btb_hip_attn_decode needs for T rows and S key spans */
 size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, size_t S);
 
@@ -243,10 +251,20 @@ size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, siz
  * 407-419). The keys (capacity `cap`) are cut into S spans, a workgroup per (kv head, span, row) leaving its
  * online-softmax state in `workspace` (btb_hip_attn_scratch_floats floats); a second small launch folds the spans in
  * span order. head_dim 128, Hq / Hk in {1, 2, 4, 8}, S * (Hq / Hk) <= 1024. Replaces btb_attn_flash_d128's decode form
- * (native/cuda/btb_attn_flash.cuh:277-675); the cache's row map (`tbl`) and the window are not taken. */
+ * (native/cuda/btb_attn_flash.cuh:277-675); its window and row map arguments are btb_hip_attn_decode_win's. */
 int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
                             const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
                             float scale, size_t cap, size_t S, float* workspace, void* stream);
+
+/* btb_hip_attn_decode under a sliding window and through the cache's row map, the two remaining arguments of the
+ * reference's decode form (native/cuda/btb_attn_flash.cuh:372-379, 437, 517, 537). win > 0: a row standing at logical
+ * position `last` (*n0 + t in a chain, *n0 + its depth in a tree) sees the positions last + 1 - win .. last only; 0: no
+ * window. tbl (NULL: none): logical slot j of the cache is its row tbl[j] (i32 on the device, `cap` entries) - an
+ * address, never a bit: the result is the unmapped cache's. */
+int32_t btb_hip_attn_decode_win(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
+                                const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
+                                float scale, size_t cap, size_t S, int64_t win, const int32_t* tbl, float* workspace,
+                                void* stream);
 
 /* btb_hip_attn_decode for callers that cannot allocate device memory or pass a workspace: code under hipGraph
  * capture, tight serving loops, harnesses that forbid hipMalloc. No counterpart in the reference. The spans' partial
@@ -291,6 +309,11 @@ int32_t btb_hip_argmax_publish(const void* logits, size_t V, int32_t* picked, in
  * length, so a host that sees the length sees the token. Replaces btb_publish (native/cuda/btb_kernels.cu:448-465). */
 int32_t btb_hip_publish(int32_t* n0, const int32_t* picked, int32_t* next_ids, int32_t* out_tok, int32_t* out_n0,
                         int64_t* out_ts, void* stream);
+
+/* The reference's btb_publish as it is (native/cuda/btb_kernels.cu:455-465): the step's token *ids and the card's
+ * clock into pinned host memory, then - after a system fence - the cache's length *n0; nothing on the device changes. */
+int32_t btb_hip_publish_only(const int32_t* n0, const int32_t* ids, int32_t* out_tok, int32_t* out_n0, int64_t* out_ts,
+                             void* stream);
 
 /* ---- the whole decode step as one persistent launch ---------------------------------------------------------- */
 

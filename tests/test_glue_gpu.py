@@ -11,6 +11,7 @@ import numpy as np
 import pytest
 import torch
 
+from btb_amd.decode import StackConfig, rope_tables
 from oracle import codecs
 from oracle import decode as od
 
@@ -221,3 +222,109 @@ def test_publish(card):
     card.publish(n0, picked, nxt, tok, ln, ts)
     torch.cuda.synchronize()
     assert int(tok[0]) == 1234 and int(ln[0]) == 42 and int(n0[0]) == 42 and int(nxt[0]) == 1234 and int(ts[0]) != 0
+
+
+@pytest.mark.parametrize("n0,T,Hq,Hk,S,win,tree", [(300, 1, 32, 8, 3, 128, False), (300, 6, 8, 2, 2, 17, False),
+                                                    (40, 8, 16, 2, 1, 3, True), (700, 8, 32, 8, 5, 500, True),
+                                                    (5, 4, 8, 8, 1, 64, False)])
+def test_attn_decode_under_a_window(card, n0, T, Hq, Hk, S, win, tree):
+    """the reference's window (native/cuda/btb_attn_flash.cuh:437: first = last + 1 - win): a row at logical position
+    `last` - n0 + t in a chain, n0 + its depth in a tree - sees positions first .. last only; against f64 attention
+    over exactly those keys"""
+    D = 128
+    cap = n0 + T + 3
+    g = gen(680 + n0 + win)
+    K = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    V = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    q = torch.randn(T, Hq * D, generator=g).to(torch.bfloat16)
+    par = [-1, 0, 1, 2, 1, 4, 0, 6][:T] if tree else None
+    part = None if par is None else torch.tensor(par, dtype=torch.int32, device="cuda")
+    att = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    scale = 1.0 / np.sqrt(D)
+    card.attn_decode(q.cuda(), K.cuda(), V.cuda(), att, n0t, Hq, Hk, D, scale, S, card.attn_scratch(T, Hq, Hk, D, S),
+                     par=part, win=win)
+    got = att.float().cpu().numpy()
+    for t in range(T):
+        if par is None:
+            slots = list(range(n0 + t + 1))            # slot = position in a chain
+            pos = slots
+        else:
+            path, p_ = [], t
+            while p_ >= 0:
+                path.append(p_)
+                p_ = par[p_]
+            path = path[::-1]                            # root first: depth d at position n0 + d
+            slots = list(range(n0)) + [n0 + p for p in path]
+            pos = list(range(n0)) + [n0 + d for d in range(len(path))]
+        last = pos[-1]
+        keep = [s for s, ps in zip(slots, pos) if ps >= last + 1 - win]
+        want = od.attention(q[t].float().numpy().reshape(Hq, D), K[:, keep].float().numpy(), V[:, keep].float().numpy(),
+                            scale)
+        worst = np.abs(got[t].reshape(Hq, D) - want).max() / np.abs(want).max()
+        assert worst <= 2.0**-7, (t, worst)
+
+
+def test_attn_and_rope_through_the_caches_row_map(card):
+    """`tbl` maps a logical slot to its cache row - an address, never a bit (native/cuda/btb_attn_flash.cuh:34): the
+    pass over a cache whose rows were shuffled by the map gives the unshuffled cache's bits, and norm_rope_kv with the
+    map writes the pass's rows where the map says"""
+    D, Hq, Hk, T, n0, S = 128, 16, 4, 5, 200, 3
+    cap = 256
+    cfg = StackConfig(layers=1, hidden=64, q_heads=Hq, kv_heads=Hk, head_dim=D, intermediate=64, vocab=8)
+    g = gen(690)
+    K = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda()
+    V = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda()
+    qkv = torch.randn(T, (Hq + 2 * Hk) * D, generator=g).to(torch.bfloat16).cuda()
+    wq = (1.0 + 0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).cuda()
+    wk = (1.0 + 0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).cuda()
+    cos, sin = rope_tables(cfg, cap, "cuda")
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    perm = torch.randperm(cap, generator=g).to(torch.int32)
+    tbl = perm.cuda()
+    Kp, Vp = torch.zeros_like(K), torch.zeros_like(V)
+    Kp[:, perm.long()] = K                              # logical slot j lives in row perm[j]
+    Vp[:, perm.long()] = V
+    scale = 1.0 / np.sqrt(D)
+    scratch = card.attn_scratch(T, Hq, Hk, D, S)
+    par = torch.tensor([-1, 0, 0, 2, 3], dtype=torch.int32, device="cuda")
+    outs = []
+    for Kc, Vc, m in ((K.clone(), V.clone(), None), (Kp, Vp, tbl)):
+        q = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+        card.norm_rope_kv(qkv, wq, wk, 1e-6, cos, sin, n0t, Kc, Vc, q, Hq, Hk, D, tbl=m)
+        att = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+        card.attn_decode(q, Kc, Vc, att, n0t, Hq, Hk, D, scale, S, scratch, par=par, win=150, tbl=m)
+        outs.append((q, att, Kc, Vc))
+    assert torch.equal(outs[0][0], outs[1][0]) and torch.equal(outs[0][1], outs[1][1])
+    # the pass's rows landed in their mapped cache rows
+    for t in range(T):
+        assert torch.equal(outs[1][2][:, int(perm[n0 + t])], outs[0][2][:, n0 + t])
+        assert torch.equal(outs[1][3][:, int(perm[n0 + t])], outs[0][3][:, n0 + t])
+    assert bool(outs[0][1].float().abs().sum() > 0)
+
+
+def test_attn_span_count_limit(card):
+    """spans * (query heads per kv head) is at most 1024 - the states the span fold turns into factors: the maximum
+    is taken and right, one more span is refused (nothing is launched)"""
+    D, Hq, Hk, n0 = 128, 8, 2, 2100
+    G = Hq // Hk
+    cap = n0 + 8
+    g = gen(695)
+    K = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    V = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    q = torch.randn(1, Hq * D, generator=g).to(torch.bfloat16)
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    scale = 1.0 / np.sqrt(D)
+    S = 1024 // G
+    att = torch.zeros(1, Hq * D, dtype=torch.bfloat16, device="cuda")
+    card.attn_decode(q.cuda(), K.cuda(), V.cuda(), att, n0t, Hq, Hk, D, scale, S, card.attn_scratch(1, Hq, Hk, D, S))
+    want = od.attention(q[0].float().numpy().reshape(Hq, D), K[:, : n0 + 1].float().numpy(),
+                        V[:, : n0 + 1].float().numpy(), scale)
+    got = att[0].float().cpu().numpy().reshape(Hq, D)
+    assert np.abs(got - want).max() / np.abs(want).max() <= 2.0**-7
+    att.fill_(3.0)
+    with pytest.raises(Exception):
+        card.attn_decode(q.cuda(), K.cuda(), V.cuda(), att, n0t, Hq, Hk, D, scale, S + 1,
+                         card.attn_scratch(1, Hq, Hk, D, S + 1))
+    torch.cuda.synchronize()
+    assert bool((att == 3.0).all())

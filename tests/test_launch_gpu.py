@@ -93,3 +93,61 @@ def test_launcher_refusals(card):
     assert "btb_gemv_bf16_m32" in card.fn and "btb_moe_route" in card.fn
     card.close()
     card.close()
+
+
+def test_attention_rope_and_publish_kernels_by_name(card):
+    """btb_norm_rope_kv_tbl_d128, btb_attn_flash_d128 and btb_publish with the reference's own parameter lists
+    (btb/engine/card_launch.py:469-523, 2152-2212, 2334-2347): the typed wrappers' bits. The attention's partial-state
+    arrays and arrival counter are the caller's in the reference's layout and go unused here - the card keeps its own."""
+    import numpy as np
+
+    from btb_amd.decode import StackConfig, rope_tables
+
+    D, Hq, Hk, T, n0 = 128, 16, 4, 4, 700
+    G = Hq // Hk
+    S = 2                                              # key groups of 512: the graph's capacity is 1024 slots
+    cap = S * 512
+    cfg = StackConfig(layers=1, hidden=64, q_heads=Hq, kv_heads=Hk, head_dim=D, intermediate=64, vocab=8)
+    g = gen(820)
+    K = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda()
+    V = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda()
+    qkv = torch.randn(T, (Hq + 2 * Hk) * D, generator=g).to(torch.bfloat16).cuda()
+    wq = (1.0 + 0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).cuda()
+    wk = (1.0 + 0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).cuda()
+    cos, sin = rope_tables(cfg, cap, "cuda")
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    par = torch.tensor([-1, 0, 1, 0], dtype=torch.int32, device="cuda")
+    depth = torch.tensor([0, 1, 2, 1], dtype=torch.int32, device="cuda")
+    tbl = torch.randperm(cap, generator=g).to(torch.int32).cuda()
+    scale = 1.0 / np.sqrt(D)
+    hs, rs = int(K.stride(0)), int(K.stride(1))
+
+    K1, V1, K2, V2 = K.clone(), V.clone(), K.clone(), V.clone()
+    q1 = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+    q2 = torch.zeros_like(q1)
+    card.norm_rope_kv(qkv, wq, wk, 1e-6, cos, sin, n0t, K1, V1, q1, Hq, Hk, D, depth=depth, tbl=tbl)
+    card.launch("btb_norm_rope_kv_tbl_d128", (Hq + 2 * Hk, T, 1), (32, 1, 1),
+                [p(qkv), p(wq), p(wk), F(1e-6), p(cos), p(sin), p(n0t), p(depth), p(K2), p(V2), p(q2), I(T), I(Hq), I(Hk),
+                 I(hs), I(rs), I(0), p(tbl)])
+    assert torch.equal(q1, q2) and torch.equal(K1, K2) and torch.equal(V1, V2)
+
+    a1 = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+    a2 = torch.zeros_like(a1)
+    card.attn_decode(q1, K1, V1, a1, n0t, Hq, Hk, D, scale, S, card.attn_scratch(T, Hq, Hk, D, S), par=par, win=300, tbl=tbl)
+    part_m = torch.zeros(S * T * Hq, dtype=torch.float32, device="cuda")
+    part_acc = torch.zeros(S * T * Hq * D, dtype=torch.float32, device="cuda")
+    cnt = torch.zeros(T * Hq, dtype=torch.int32, device="cuda")
+    card.launch("btb_attn_flash_d128", ((T * G + 7) // 8, S, Hk), (256, 1, 1),
+                [p(q1), p(K1), p(V1), p(a2), p(n0t), p(par), I(T), I(Hq), I(Hk), I(hs), I(rs), F(scale), p(part_m),
+                 p(part_m.clone()), p(part_acc), p(cnt), I(300), p(tbl)], shared=8192)
+    assert torch.equal(a1, a2) and bool(a1.float().abs().sum() > 0)
+
+    ids = torch.tensor([4242], dtype=torch.int32, device="cuda")
+    out_tok = torch.zeros(1, dtype=torch.int32).pin_memory()
+    out_n0 = torch.zeros(1, dtype=torch.int32).pin_memory()
+    out_ts = torch.zeros(1, dtype=torch.int64).pin_memory()
+    card.launch("btb_publish", (1, 1, 1), (32, 1, 1), [p(n0t), p(ids), p(out_tok), p(out_n0), p(out_ts)])
+    torch.cuda.synchronize()
+    assert int(out_tok[0]) == 4242 and int(out_n0[0]) == n0 and int(out_ts[0]) > 0 and int(n0t[0]) == n0
+    for name in ("btb_attn_flash_d128", "btb_publish", "btb_norm_rope_kv_tbl_d64"):
+        assert name in card.fn

@@ -7,6 +7,7 @@ from __future__ import annotations
 import os
 
 import numpy as np
+import pytest
 import torch
 
 from btb_amd.load import Store, read_config
@@ -51,3 +52,24 @@ def test_the_f32_forward_reproduces_the_bf16_receipts():
     want = torch.load(os.path.join(GOLDEN, "receipts_qwen3.pt"), weights_only=True)["bf16"]["prompt_logits"].numpy()
     got = reference_logits(cfg, lambda n: store.get(n).float(), PROMPT)
     assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max() + 1e-4
+
+
+def test_mxfp4_expert_store_reads_as_stored():
+    """the reference's tiny gpt-oss fixture (its MXFP4 expert tensors, copied as data): shapes, views, refusals"""
+    from btb_amd.load import MxExperts, load_mx_experts
+
+    path = os.path.join(GOLDEN, "tiny_gpt_oss")
+    ex = load_mx_experts(path, 1, device="cpu")
+    assert (ex.experts, ex.hidden, ex.intermediate) == (8, 64, 64)
+    assert tuple(ex.gate_up_blocks.shape) == (8, 128, 2, 16) and tuple(ex.down_scales.shape) == (8, 64, 2)
+    w = ex.gate_up(3)
+    assert w.shape == (128, 64) and w.blocks.data_ptr() == ex.gate_up_blocks[3].data_ptr()      # a view, not a copy
+    assert ex.down(7).shape == (64, 64) and ex.nbytes == 8 * (128 + 64) * 2 * 17
+    # the views dequantise to what transformers makes of the same bytes
+    tm = pytest.importorskip("transformers.integrations.mxfp4")
+    want = tm.convert_moe_packed_tensors(ex.down_blocks, ex.down_scales, dtype=torch.float32).transpose(1, 2)
+    assert torch.equal(ex.down(5).dequantize().view(torch.int32), want[5].contiguous().view(torch.int32))
+    with pytest.raises(KeyError):
+        load_mx_experts(path, 9, device="cpu")
+    with pytest.raises(ValueError):
+        MxExperts(ex.gate_up_blocks, ex.gate_up_scales, ex.gate_up_blocks, ex.gate_up_scales)

@@ -104,3 +104,28 @@ def test_fp8_store_loads_as_stored_and_tracks_its_own_f32_evaluation(card, recei
     assert toks[0] == int(np.argmax(want))
     # quantisation moves the logits a little off the receipts, not far
     check_receipt(logits, receipts["bf16"]["prompt_logits"], 0.25)
+
+
+def test_mxfp4_expert_store_widens_bit_exact_on_the_gpu(card):
+    """every layer of the reference's tiny gpt-oss store: its MXFP4 expert stacks go to VRAM as stored and
+    btb_hip_mx4_widen makes of them, bit for bit, what transformers' convert_moe_packed_tensors does (a library already
+    here, not the reference), whole stacks and picked seats; an expert's matvec over the stored bytes equals the
+    matvec over the widened matrix within the bf16-output bar"""
+    from btb_amd.load import load_mx_experts
+
+    tm = pytest.importorskip("transformers.integrations.mxfp4")
+    path = os.path.join(GOLDEN, "tiny_gpt_oss")
+    for layer in range(4):
+        ex = load_mx_experts(path, layer)
+        for which, blocks, scales in (("gate_up", ex.gate_up_blocks, ex.gate_up_scales),
+                                      ("down", ex.down_blocks, ex.down_scales)):
+            want = tm.convert_moe_packed_tensors(blocks.cpu(), scales.cpu(), dtype=torch.bfloat16).transpose(1, 2)
+            got = ex.widen(card, which)
+            assert torch.equal(got.cpu().view(torch.int16), want.contiguous().view(torch.int16)), (layer, which)
+            seats = torch.tensor([6, 1, 1, 4], dtype=torch.int32, device="cuda")
+            picked = ex.widen(card, which, seats)
+            assert torch.equal(picked.cpu().view(torch.int16), want[[6, 1, 1, 4]].contiguous().view(torch.int16))
+        x = torch.randn(2, ex.hidden, generator=torch.Generator().manual_seed(layer)).to(torch.bfloat16).cuda()
+        y = card.gemv_mx4(ex.gate_up(2), x).float().cpu().numpy()
+        ref = (x.float().cpu() @ ex.widen(card, "gate_up", dtype=torch.float32)[2].cpu().T).numpy()
+        assert np.abs(y - ref).max() <= 2.0**-7 * np.abs(ref).max()
