@@ -101,10 +101,12 @@ def silu_mul(gu: np.ndarray, dt: str = "bf16") -> np.ndarray:
     return R((s * u).astype(np.float32))
 
 
-def step(cfg, W: dict, token: int, kv: np.ndarray, n0: int, dt: str = "bf16"):
+def step(cfg, W: dict, token: int, kv: np.ndarray, n0: int, dt: str = "bf16", trace: list | None = None):
     """One row's step. cfg has layers, hidden, q_heads, kv_heads, head_dim, intermediate, vocab, eps, rope_theta; W
     maps names to bf16 bit patterns; kv [layers, 2, Hk, cap, D] f32 holding values of dt, updated in place at slot n0.
-    Returns (logits as values of dt [vocab], picked token)."""
+    Returns (logits as values of dt [vocab], picked token). `trace`, when a list, receives what stands between the
+    layers: entry i is (h, y) as layer i finds them - the residual and the block output not yet added to it (None
+    before layer 0) - and entry `layers` what the last layer leaves."""
     Hq, Hk, D = cfg.q_heads, cfg.kv_heads, cfg.head_dim
     cos, sin = rope_tables(D, cfg.rope_theta, n0 + 1, dt)
     cos, sin = cos[n0], sin[n0]
@@ -112,6 +114,8 @@ def step(cfg, W: dict, token: int, kv: np.ndarray, n0: int, dt: str = "bf16"):
     y = None
     for i in range(cfg.layers):
         L = f"layers.{i}."
+        if trace is not None:
+            trace.append((h.copy(), None if y is None else y.copy()))
         h, x = add_rmsnorm(h, y, W[L + "ln1"], cfg.eps, dt)
         qkv = matvec(W[L + "qkv"], x, dt)[0]
         q = norm_rope(qkv[: Hq * D].reshape(Hq, D), W.get(L + "wq"), cfg.eps, cos, sin, dt)
@@ -124,6 +128,8 @@ def step(cfg, W: dict, token: int, kv: np.ndarray, n0: int, dt: str = "bf16"):
         h, x = add_rmsnorm(h, y, W[L + "ln2"], cfg.eps, dt)
         gu = matvec(W[L + "gu"], x, dt)
         y = matvec(W[L + "down"], silu_mul(gu, dt), dt)
+    if trace is not None:
+        trace.append((h.copy(), None if y is None else y.copy()))
     h, x = add_rmsnorm(h, y, W["norm"], cfg.eps, dt)
     logits = matvec(W["head"], x, dt)[0]
     return logits, int(np.argmax(logits))

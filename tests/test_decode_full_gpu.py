@@ -93,3 +93,51 @@ def test_full_shape_step_against_the_cpu_path(card):
     packed = _run(card, random_stack(card, cfg, packed=True), kv, graph=True)
     worst, rms = _rel(packed.logits[0].float().cpu().numpy(), got)
     assert worst <= 8e-2 and rms <= 6e-2, (worst, rms)
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_each_full_shape_layer_alone_against_the_cpu_path(card, packed):
+    """Every one of the 36 full-shape layers on its own, at the tight bar: the layer is handed the CPU path's own
+    input - the residual and the pending block output as the oracle's step had them at that depth (teacher forcing) -
+    runs the step's launches (add + norm + qkv, attention over the 4096-key cache, o, add + norm + gate/up + SwiGLU,
+    down) and must leave the oracle's residual and block output within 3e-2 of the largest value, with no drift from
+    the layers before it to lean on. Both stored forms: bf16, and the same weights at 12 bits a weight."""
+    cfg = QWEN3_4B
+    Hq, Hk, D, H, I = cfg.q_heads, cfg.kv_heads, cfg.head_dim, cfg.hidden, cfg.intermediate
+    w16 = random_stack(card, cfg)
+    W = {k: bits16(v.w if hasattr(v, "w") else v) for k, v in w16.items()}
+    w = random_stack(card, cfg, packed=True) if packed else w16
+    g = torch.Generator(device="cuda").manual_seed(0x0B7B0909)
+    kv = torch.randn(cfg.layers, 2, cfg.kv_heads, CAP, cfg.head_dim, generator=g, device="cuda").to(torch.bfloat16)
+    okv = kv.float().cpu().numpy()
+    trace: list = []
+    od.step(cfg, W, TOKEN, okv, N0, trace=trace)
+    assert len(trace) == cfg.layers + 1
+    del W
+
+    step = DecodeStep(card, cfg, w, CAP)          # its buffers, rope tables and attention scratch; the body is not run
+    step.kv.copy_(kv)
+    step.reset(N0, TOKEN)
+    bf = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(torch.bfloat16).cuda()
+    worst_h = worst_y = 0.0
+    for i in range(cfg.layers):
+        L = f"layers.{i}."
+        h_in, y_in = trace[i]
+        h_want, y_want = trace[i + 1]
+        h0 = bf(h_in)
+        hb, ha = torch.zeros_like(h0), torch.zeros_like(h0)
+        card.gemv_norm(w[L + "qkv"].w, h0, None if y_in is None else bf(y_in), w[L + "ln1"], cfg.eps, hb, step.qkv)
+        card.attn_decode_qkv(step.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, step.cos, step.sin, step.n0,
+                             step.kv[i, 0], step.kv[i, 1], step.att, Hq, Hk, D, step.scale, step.S, step.scratch)
+        w[L + "o"].matvec(step.att, step.y)
+        card.gemv_norm(w[L + "gu"].w, hb, step.y, w[L + "ln2"], cfg.eps, ha, step.m, glu=True)
+        w[L + "down"].matvec(step.m, step.y)
+        torch.cuda.synchronize()
+        eh = _rel(ha.float().cpu().numpy(), h_want)[0]
+        ey = _rel(step.y.float().cpu().numpy(), y_want)[0]
+        worst_h, worst_y = max(worst_h, eh), max(worst_y, ey)
+        assert eh <= 3e-2 and ey <= 3e-2, (i, eh, ey)
+        # the layer's new key and value rows are the oracle's too
+        krow = step.kv[i, :, :, N0].float().cpu().numpy()
+        assert np.abs(krow - okv[i, :, :, N0]).max() <= 3e-2 * np.abs(okv[i, :, :, N0]).max(), i
+    print(f"teacher-forced layers ({'pack12' if packed else 'bf16'}): worst residual {worst_h:.2e}, worst block output {worst_y:.2e}")
