@@ -69,6 +69,7 @@ static Knob g_knobs[] = {
     {"mfma_classic", {-1}},
     {"mfma_lds", {-1}},
     {"mfma_stream_x", {-1}},
+    {"mfma_direct", {-1}},
     {"moe_wgs_per_cu", {-1}},
     {"attn_split", {-1}},
     {"attn_heads_per_wg", {-1}},

@@ -284,6 +284,14 @@ int32_t gemv_mfma_lds_p12(const uint8_t* lo, const uint8_t* hi4, const uint8_t* 
                           const uint8_t* esc_val, const int32_t* row_ptr, const void* x, void* y, int R, int C, int M,
                           hipStream_t st);
 
+// the direct-to-LDS form of the matrix-core matvec for the long rows of the block-scaled forms (gemv_mfma_dl.hip)
+bool mfma_dl_fits(int R, int C, int M);
+bool mfma_dl_fits_fp8(int R, int C, int M, int bm, int bn);
+int32_t gemv_mfma_dl_fp8(const void* w, const float* scales, int sc, int bm, int bn, const void* x, void* y, int R,
+                         int C, int M, hipStream_t st);
+int32_t gemv_mfma_dl_mxfp4(const void* blocks, const void* scales, const void* x, void* y, int R, int C, int M,
+                           hipStream_t st);
+
 // whether a pass of M rows goes to the matrix cores through the LDS-staged kernel
 static bool wide_pass(size_t M, size_t R, size_t C, bool packed) {
     return M >= 5 && (packed ? mfma_lds_fits_packed((int)R, (int)C) : mfma_lds_fits_bf16((int)R, (int)C)) &&
@@ -498,6 +506,17 @@ int32_t btb_hip_gemv_fp8(const void* w, const void* scales, size_t sr, size_t sc
     if (rc != OK) return rc;
     if (R % sr != 0 || C % sc != 0 || (C / sc) % FmtF8::UW != 0) return ERR_DOMAIN;
     if (!aligned16(w) || !aligned16(x) || (reinterpret_cast<uintptr_t>(scales) & 3u) || !aligned2(y)) return ERR_DOMAIN;
+    if (wide_pass(M, R, C, true) && mfma_dl_fits_fp8((int)R, (int)C, 16, (int)(R / sr), (int)(C / sc))) {
+        const uint16_t* xp = static_cast<const uint16_t*>(x);  // the long rows: weights straight into LDS, 16 rows a pass
+        uint16_t* yp = static_cast<uint16_t*>(y);
+        for (size_t m0 = 0; m0 < M; m0 += 16) {
+            const int mm = (int)(M - m0 < 16 ? M - m0 : 16);
+            rc = gemv_mfma_dl_fp8(w, static_cast<const float*>(scales), (int)sc, (int)(R / sr), (int)(C / sc), xp + m0 * C,
+                                  yp + m0 * R, (int)R, (int)C, mm, static_cast<hipStream_t>(stream));
+            if (rc != OK) return rc;
+        }
+        return OK;
+    }
     if (wide_pass(M, R, C, true)) {  // the verify widths: the matrix cores, 32 rows of x a pass
         const uint16_t* xp = static_cast<const uint16_t*>(x);
         uint16_t* yp = static_cast<uint16_t*>(y);
@@ -521,6 +540,17 @@ int32_t btb_hip_gemv_mxfp4(const void* blocks, const void* scales, const void* x
     int32_t rc = check_dims(R, C, M, FmtMx4::UW);
     if (rc != OK) return rc;
     if (!aligned16(blocks) || !aligned16(x) || !aligned2(y)) return ERR_DOMAIN;
+    if (wide_pass(M, R, C, true) && mfma_dl_fits((int)R, (int)C, 16) && (reinterpret_cast<uintptr_t>(scales) & 3u) == 0) {
+        const uint16_t* xp = static_cast<const uint16_t*>(x);  // the long rows: weights straight into LDS, 16 rows a pass
+        uint16_t* yp = static_cast<uint16_t*>(y);
+        for (size_t m0 = 0; m0 < M; m0 += 16) {
+            const int mm = (int)(M - m0 < 16 ? M - m0 : 16);
+            rc = gemv_mfma_dl_mxfp4(blocks, scales, xp + m0 * C, yp + m0 * R, (int)R, (int)C, mm,
+                                    static_cast<hipStream_t>(stream));
+            if (rc != OK) return rc;
+        }
+        return OK;
+    }
     if (wide_pass(M, R, C, true)) {
         const uint16_t* xp = static_cast<const uint16_t*>(x);
         uint16_t* yp = static_cast<uint16_t*>(y);

@@ -150,6 +150,42 @@ def test_gemv_mxfp4_verify_widths(card, R, C, M):
     _width_law(card, card.gemv_mx4, w, x.cuda(), ref)
 
 
+@pytest.mark.parametrize("form,block", [("fp8", (128, 128)), ("fp8", (64, 256)), ("fp8", (16, 32)), ("mxfp4", None)])
+@pytest.mark.parametrize("M", [5, 16, 24, 33])
+def test_long_rows_straight_into_lds(card, form, block, M):
+    """Rows of 7168 columns at the verify widths take the kernel whose weights go from memory straight into LDS
+    (sixteen rows of x a pass, so 24 and 33 are two and three passes, the last of 8 and of 1): against the oracle,
+    against the staged kernel it replaces (knob mfma_direct = 0; the two differ in f32 summation order only), and a
+    row's bits do not depend on which pass or which other rows it came with."""
+    R, C = 9728, 7168  # 608 tiles: three turns of a grid of 203 workgroups, the last of which has two
+    src = weights_bf16(R, C, seed=350).float()
+    x = acts_bf16(M, C, seed=351)
+    if form == "fp8":
+        q, s = fp8.quantize(src, block)
+        w = fp8.F8Weight(q.view(torch.uint8).cuda(), s.cuda(), R, C)
+        ref = oracle.gemv_fp8(q.view(torch.uint8).numpy(), s.numpy(), x.float().numpy(), threads=0)
+        op = card.gemv_fp8
+    else:
+        blocks, scales = mxfp4.quantize(src)
+        w = mxfp4.MxWeight(blocks.reshape(-1).cuda(), scales.reshape(-1).cuda(), R, C)
+        ref = oracle.gemv_mxfp4(blocks.numpy(), scales.numpy(), R, C, x.float().numpy(), threads=0)
+        op = card.gemv_mx4
+    xg = x.cuda()
+    y = op(w, xg)
+    check(y, ref)
+    card.set_tuning("mfma_direct", 0)
+    try:
+        staged = op(w, xg)
+    finally:
+        card.set_tuning("mfma_direct", -1)
+    check(staged, ref)
+    peak = float(y.float().abs().max())
+    assert float((staged.float() - y.float()).abs().max()) <= peak * 2.0**-7
+    last = op(w, xg[M - 5:].contiguous())  # the last five rows in a pass of their own (the narrowest wide pass)
+    assert torch.equal(last.view(torch.int16), y[M - 5:].view(torch.int16))
+    assert torch.equal(op(w, xg).view(torch.int16), y.view(torch.int16))  # and the same bits every time
+
+
 @pytest.mark.parametrize("form", ["fp8", "mxfp4"])
 def test_full_shape_one_row_and_linearity(card, form):
     """C5 at M = 1 on the full [18432, 7168] matrix against the oracle, and a size-independent property on top: the
