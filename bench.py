@@ -154,6 +154,16 @@ def traffic_entry(workload: str, key: str) -> dict | None:
 # ---------------------------------------------------------------------------------------------------------------
 
 
+def apply_tuning(card, pairs: list[str]) -> dict[str, int]:
+    """--tune KNOB=VALUE: the library's tuning knobs set before anything is timed; returned for the config record"""
+    out: dict[str, int] = {}
+    for item in pairs:
+        key, _, value = item.partition("=")
+        card.set_tuning(key.strip(), int(value))
+        out[key.strip()] = int(value)
+    return out
+
+
 def kernel_workload(args: argparse.Namespace) -> int:
     """The single-operator configs: one JSON line each, `value` the operator's HBM stream in GB/s. A step is one call
     over the next operand set of a pool larger than the last-level cache (256 MB), so nothing repeats from cache; the
@@ -173,6 +183,7 @@ def kernel_workload(args: argparse.Namespace) -> int:
     from btb_amd.pack12 import P12Weight
 
     card = Native.card_kernels()
+    tuned = apply_tuning(card, args.tune)
     dev, M = torch.device("cuda"), int(args.m)
     g = torch.Generator(device=dev).manual_seed(0x0B7B0500)
     bf = dict(dtype=torch.bfloat16, device=dev)
@@ -270,7 +281,8 @@ def kernel_workload(args: argparse.Namespace) -> int:
         "n_gpus": 1, "steps": passes * pool, "warmup": args.warmup, "ms_per_step": round(us * 1e-3, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
         "data": "synthetic: N(0, 0.02) weights, N(0, 1) x, seeded", "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
-        "config": {"workload": what, "pool": pool, "algorithmic_bytes_per_step": int(mean_bytes), **extra},
+        "config": {"workload": what, "pool": pool, "algorithmic_bytes_per_step": int(mean_bytes), **extra,
+                   **({"tuning": tuned} if tuned else {})},
         "roofline": {"kernel": kernel, "bound": "hbm", "achieved": round(gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(gbs / HBM_PEAK_GBS, 4), "avg_launch_us": round(us, 3),
                      "bytes_per_launch": int(mean_bytes),
@@ -375,6 +387,8 @@ def main() -> int:
     ap.add_argument("--rows", type=int, default=1,
                     help="rows of a decode pass: 1 is the step the metric is quoted on, more a speculative verify pass")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--tune", action="append", default=[], metavar="KNOB=VALUE",
+                    help="set one of the library's tuning knobs before the run (repeatable); recorded in config")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
@@ -394,6 +408,7 @@ def main() -> int:
     from btb_amd.native import Native
 
     card = Native.card_kernels()  # raises where the HIP library or the GPU is missing: there is no fallback
+    tuned = apply_tuning(card, args.tune)
     cfg = QWEN3_4B
     packed = args.workload == "decode_p12"
     weights = random_stack(card, cfg, packed=packed)
@@ -492,6 +507,7 @@ def main() -> int:
             "kernels_per_step": (2 + 6 * cfg.layers if args.rows == 1 else
                                  3 + 7 * cfg.layers if step.fused else 5 + 10 * cfg.layers),
             "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
+            **({"tuning": tuned} if tuned else {}),
         },
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu else cpu_baseline(args.workload, 1),

@@ -71,6 +71,8 @@ static Knob g_knobs[] = {
     {"mfma_stream_x", {-1}},
     {"mfma_direct", {-1}},
     {"moe_wgs_per_cu", {-1}},
+    {"moe_grouped", {-1}},
+    {"moe_fused_router", {-1}},
     {"attn_split", {-1}},
     {"attn_heads_per_wg", {-1}},
 };

@@ -14,6 +14,8 @@ constexpr int32_t ERR_NULL = -1;
 constexpr int32_t ERR_OVERFLOW = -5;
 constexpr int32_t ERR_DOMAIN = -6;
 constexpr int32_t ERR_PANIC = -7;  // a HIP runtime error at the boundary (the crate's "panic caught")
+// between the library's own files only, never across the C ABI: "this form of the kernel does not take the shape"
+constexpr int32_t ERR_UNSUPPORTED = -100;
 
 constexpr int WAVE = 64;
 

@@ -16,6 +16,7 @@
 
 #include "btb_common.hpp"
 #include "btb_formats.hpp"
+#include "btb_route.hpp"
 #include "btb_stream.hpp"
 #include "btb_tuning.hpp"
 
@@ -25,23 +26,14 @@ namespace btb {
 
 int32_t lane16_bf16_rows16(const uint16_t* w, size_t rows, size_t cols, const uint16_t* x, size_t b, float* y,
                            hipStream_t st);  // lane16.hip
+int32_t lane16_bf16_router16(const uint16_t* w, size_t rows, size_t cols, const uint16_t* x, size_t b, float* y,
+                             int32_t* idx, uint16_t* wts, float* w32, uint16_t* logits16, int k, hipStream_t st);
 
 constexpr int ROUTE_MAX_K = 32;  // the reference's ROUTE_MAX_K (native/cuda/btb_kernels.cu:859)
 
 // ------------------------------------------------------------------------------------------------------------
 // route: one wave per token
 // ------------------------------------------------------------------------------------------------------------
-
-template <bool F32>
-__device__ __forceinline__ float logit_at(const void* base, size_t i) {
-    return F32 ? static_cast<const float*>(base)[i] : bf16_f32(static_cast<const uint16_t*>(base)[i]);
-}
-
-__device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int s = 32; s > 0; s >>= 1) v = fmaxf(v, __shfl_xor(v, s, WAVE));
-    return v;
-}
 
 // the (value, index) maximum over the wave in the total order: value descending, then index ascending; an index of
 // NONE is "nothing"
@@ -113,98 +105,12 @@ __global__ void __launch_bounds__(64) moe_route_kernel(const void* __restrict__ 
     }
 }
 
-// Up to 256 experts: the row's probabilities stay in registers, P a lane, and a pick is the maximum of 64-bit keys
-// (the probability's bits above the complement of the index: p >= 0, so the bits order as p does, and of equal p the
-// lower index has the greater key). A taken key is 0, below every live one. The same arithmetic in the same order as
-// the kernel above, so the same picks and weights; a row of NaN probabilities takes the experts 0..k-1.
-__device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v) {
-    auto step = [&](auto ctrl) {
-        constexpr int C = decltype(ctrl)::value;
-        const uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)v, C, 0xF, 0xF, true);
-        const uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)(uint32_t)(v >> 32), C, 0xF, 0xF, true);
-        const unsigned long long o = ((unsigned long long)hi << 32) | lo;
-        v = o > v ? o : v;
-    };
-    step(std::integral_constant<int, 0xB1>{});
-    step(std::integral_constant<int, 0x4E>{});
-    step(std::integral_constant<int, 0x141>{});
-    step(std::integral_constant<int, 0x140>{});
-    unsigned long long best = 0;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)v, 16 * r);
-        const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(v >> 32), 16 * r);
-        const unsigned long long o = ((unsigned long long)hi << 32) | lo;
-        best = o > best ? o : best;
-    }
-    return best;
-}
-
 template <bool F32, int P>
 __global__ void __launch_bounds__(64) moe_route_reg_kernel(const void* __restrict__ logits, size_t ls, int E, int k,
                                                            int32_t* __restrict__ idx, uint16_t* __restrict__ w,
                                                            float* __restrict__ w32, uint16_t* __restrict__ logits16) {
-    const int t = blockIdx.x, lane = threadIdx.x;
-    const size_t base = (size_t)t * ls;
-    float lv[P];
-#pragma unroll
-    for (int s = 0; s < P; ++s) {
-        const int e = lane + WAVE * s;
-        lv[s] = e < E ? logit_at<F32>(logits, base + e) : bits_f32(0xff800000u);
-    }
-    if (logits16 != nullptr) {
-#pragma unroll
-        for (int s = 0; s < P; ++s) {
-            const int e = lane + WAVE * s;
-            if (e < E) logits16[(size_t)t * E + e] = f32_bf16(lv[s]);
-        }
-    }
-    float m = bits_f32(0xff800000u);
-#pragma unroll
-    for (int s = 0; s < P; ++s) m = fmaxf(m, lv[s]);
-    m = wave_max(m);
-    float pr[P], sum_p = 0.f;
-#pragma unroll
-    for (int s = 0; s < P; ++s) {
-        const int e = lane + WAVE * s;
-        pr[s] = e < E ? expf(lv[s] - m) : 0.f;
-        if (e < E) sum_p += pr[s];
-    }
-    sum_p = group_sum<64>(sum_p);
-    sum_p = __shfl(sum_p, 0, WAVE);
-    unsigned long long key[P];
-#pragma unroll
-    for (int s = 0; s < P; ++s) {
-        const int e = lane + WAVE * s;
-        const float p = pr[s] / sum_p;
-        const uint32_t bits = p != p ? 0x7fc00000u : f32_bits(p);
-        key[s] = e < E ? (((unsigned long long)bits << 32) | (0xFFFFFFFFu - (uint32_t)e)) : 0ull;
-    }
-    float topv = 0.f;  // lane j keeps pick j
-    int topi = 0;
-    for (int j = 0; j < k; ++j) {
-        unsigned long long best = key[0];
-#pragma unroll
-        for (int s = 1; s < P; ++s) best = key[s] > best ? key[s] : best;
-        best = wave_max_u64(best);
-        const int e = (int)(0xFFFFFFFFu - (uint32_t)best);
-        if (lane == j) {
-            topv = bits_f32((uint32_t)(best >> 32));
-            topi = e;
-        }
-#pragma unroll
-        for (int s = 0; s < P; ++s)
-            if (lane + WAVE * s == e) key[s] = 0ull;
-    }
-    float sum = 0.f;
-    for (int j = 0; j < k; ++j) sum += __shfl(topv, j, WAVE);
-    if (lane < k) {
-        const float wv = topv / sum;
-        const size_t o = (size_t)t * k + lane;
-        idx[o] = topi;
-        w[o] = f32_bf16(wv);
-        if (w32 != nullptr) w32[o] = wv;
-    }
+    route_row_reg<F32, P, false>(logits, (size_t)blockIdx.x * ls, (int)blockIdx.x, (int)threadIdx.x, E, k, idx, w, w32,
+                                 logits16);
 }
 
 // a row's logits rounded to bf16, for the wide rows the kernel above does not take
@@ -235,6 +141,48 @@ static int32_t launch_route(const void* logits, size_t ls, int E, int k, int T, 
     }
 #undef BTB_ROUTE_REG
     return hip_status(hipGetLastError(), "moe_route launch");
+}
+
+// ------------------------------------------------------------------------------------------------------------
+// group_picks: a call's (pick, row) pairs sorted by expert, stable (btb/engine/host.py:283-296)
+// ------------------------------------------------------------------------------------------------------------
+
+// The pairs in the order of picks.T.reshape(-1) - pick position j outermost, row t within it - are f = j T + t, with
+// expert idx[t k + j]. A thread owns an expert: it counts its pairs, the counts are summed over the experts before it
+// (within the workgroup by a scan; over the workgroups before this one by counting the pairs whose expert lies below
+// the workgroup's first), and a second walk in the same order writes the expert's pairs from its offset on - so an
+// expert's pairs keep the order of f, which is what a stable sort leaves. Every id must lie in [0, E).
+__global__ void __launch_bounds__(256) moe_group_picks_kernel(const int32_t* __restrict__ idx, int T, int k, int E,
+                                                              int32_t* __restrict__ slot, int32_t* __restrict__ token,
+                                                              int32_t* __restrict__ offs, int32_t* __restrict__ counts) {
+    __shared__ int s_wave[4];
+    __shared__ int s_cnt[256];
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), wv = tid / WAVE;
+    const int base = blockIdx.x * 256, e = base + tid;
+    const int n = T * k;
+    int below = 0;
+    for (int p = tid; p < n; p += 256) below += idx[p] < base;  // any order: a count
+    below = (int)group_sum<64>((float)below);                     // exact: n <= 65535
+    below = __shfl(below, 0, WAVE);
+    if (lane == 0) s_wave[wv] = below;
+    int cnt = 0;
+    if (e < E)
+        for (int p = 0; p < n; ++p) cnt += idx[p] == e;
+    s_cnt[tid] = cnt;
+    __syncthreads();
+    int off = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+    for (int i = 0; i < tid; ++i) off += s_cnt[i];
+    if (e >= E) return;
+    counts[e] = cnt;
+    offs[e] = off;
+    if (cnt == 0) return;
+    for (int j = 0; j < k; ++j)
+        for (int t = 0; t < T; ++t)
+            if (idx[(size_t)t * k + j] == e) {
+                slot[off] = j;
+                token[off] = t;
+                ++off;
+            }
 }
 
 // ------------------------------------------------------------------------------------------------------------
@@ -306,6 +254,141 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
         const float g = bfround(group_sum<LPR>(acc[0][0]));
         const float u = bfround(group_sum<LPR>(acc[1][0]));
         if (sl == 0 && rows[0] < I) y[rows[0]] = f32_bf16(bfround(g / (1.f + expf(-g))) * u);
+    }
+}
+
+// The same with the rows that picked an expert taken together: blockIdx.y is still a pair, but only an expert's FIRST
+// pair (in pair order) has work - it gathers every pair of its expert and streams the expert's rows once, MC of the
+// gathered rows of x a pass, where the kernel above streams them once a pair. The workgroups of the later pairs leave
+// before asking memory for anything. A product is a row of x against a row of weights in the lane order above, so
+// each h row has the bits the kernel above gives it. n = T k <= GROUP_MAX_PAIRS.
+constexpr int GROUP_MAX_PAIRS = 1024;
+template <int LPR, int RPW, int U, int MC>
+__global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* __restrict__ stack,
+                                                                  const uint16_t* __restrict__ x,
+                                                                  const int32_t* __restrict__ idx, uint16_t* __restrict__ h,
+                                                                  int R, int C, int k, int E, int n) {
+    static_assert(RPW == 2, "gate and up");
+    extern __shared__ __align__(16) uint32_t xs[];  // [MC][C / 2]
+    __shared__ int s_pairs[GROUP_MAX_PAIRS];        // the expert's pairs, ascending
+    __shared__ unsigned long long s_mask[GROUP_MAX_PAIRS / WAVE];
+    using F = FmtBf16;
+    constexpr int G = WAVE / LPR, ROWS = G;
+    const int pair = blockIdx.y;
+    auto clamp = [E](int v) { return v < 0 ? 0 : (v >= E ? E - 1 : v); };
+    const int expert = clamp(idx[pair]);
+    const int tid = threadIdx.x, lane = tid & (WAVE - 1), sl = lane % LPR, wv = tid / WAVE;
+    // which pairs picked this expert: 64 pairs a ballot, the ballots side by side in LDS
+    for (int q0 = wv * WAVE; q0 < n; q0 += 4 * WAVE) {
+        const int q = q0 + lane;
+        const bool hit = q < n && clamp(idx[q]) == expert;
+        const unsigned long long m = __ballot(hit);
+        if (lane == 0) s_mask[q0 / WAVE] = m;
+    }
+    __syncthreads();
+    // an earlier pair of the same expert does the work
+    {
+        bool earlier = false;
+        for (int b = 0; b * WAVE <= pair; ++b) {
+            unsigned long long m = s_mask[b];
+            if (b == pair / WAVE) m &= (1ull << (pair % WAVE)) - 1ull;
+            earlier |= m != 0ull;
+        }
+        if (earlier) return;  // uniform: every thread sees the same masks
+    }
+    int rows_n = 0;
+    {
+        const int nb = (n + WAVE - 1) / WAVE;
+        for (int b = 0; b < nb; ++b) {
+            const unsigned long long m = s_mask[b];
+            if (tid == 0) {
+                unsigned long long r = m;
+                int at = rows_n;
+                while (r) {
+                    s_pairs[at++] = b * WAVE + __builtin_ctzll(r);
+                    r &= r - 1;
+                }
+            }
+            rows_n += __builtin_popcountll(m);
+        }
+    }
+    __syncthreads();
+
+    const int units = C / F::UW;
+    const int wave = blockIdx.x * (blockDim.x / WAVE) + wv;
+    const int nwaves = gridDim.x * (blockDim.x / WAVE);
+    const int I = R / 2;
+    const int ntiles = (I + ROWS - 1) / ROWS;
+    const int span = U * LPR;
+    F::Params p{stack + (size_t)expert * R * units};
+    const int per = C / 8;  // 16-byte pieces a row of x
+    uint4* xd = reinterpret_cast<uint4*>(xs);
+    const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
+    // one pass: M of the gathered rows against every row of the expert. The wave's first span of weights is asked
+    // for before the rows of x are staged (it needs the expert only), as in the kernel above.
+    auto pass = [&](auto mtag, int r0, int mc) {
+        constexpr int M = decltype(mtag)::value;
+        F::Raw first[U][RPW] = {};
+        {
+            F::RowCtx c0[RPW];
+#pragma unroll
+            for (int j = 0; j < RPW; ++j)
+                c0[j] = F::row_ctx(p, (size_t)(min(min(wave, ntiles - 1) * ROWS + lane / LPR, I - 1) + j * I), units);
+            load_span_always<F, LPR, RPW, U>(first, c0, 0, sl, units);
+        }
+        if (r0 != 0) __syncthreads();  // the previous pass has read its rows
+        // the pass's rows of x, a row past the last being the last again (its sums are dropped)
+        for (int i = tid; i < M * per; i += 256) {
+            const int m = i / per, c = i - m * per;
+            const int tok = s_pairs[r0 + min(m, mc - 1)] / k;
+            xd[i] = reinterpret_cast<const uint4*>(x + (size_t)tok * C)[c];
+        }
+        __syncthreads();
+        for (int tile = wave; tile < ntiles; tile += nwaves) {
+            F::RowCtx ctx[RPW];
+            int rows[RPW];
+#pragma unroll
+            for (int j = 0; j < RPW; ++j) {
+                rows[j] = tile * ROWS + lane / LPR;
+                ctx[j] = F::row_ctx(p, (size_t)(min(rows[j], I - 1) + j * I), units);
+            }
+            float acc[RPW][M];
+#pragma unroll
+            for (int j = 0; j < RPW; ++j)
+#pragma unroll
+                for (int m = 0; m < M; ++m) acc[j][m] = 0.f;
+            int k0 = 0;
+            if (tile == wave) {
+                fma_span<F, M, LPR, RPW, U, true>(first, ctx, 0, sl, units, xs4, C / 8, acc);
+                k0 = span;
+            }
+            for (; k0 < units; k0 += span) {
+                F::Raw raw[U][RPW];
+                if (k0 + span <= units) {
+                    load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
+                    fma_span<F, M, LPR, RPW, U, false>(raw, ctx, k0, sl, units, xs4, C / 8, acc);
+                } else {
+                    load_span<F, LPR, RPW, U, true>(raw, ctx, k0, sl, units);
+                    fma_span<F, M, LPR, RPW, U, true>(raw, ctx, k0, sl, units, xs4, C / 8, acc);
+                }
+            }
+#pragma unroll
+            for (int m = 0; m < M; ++m) {
+                const float g = bfround(group_sum<LPR>(acc[0][m]));
+                const float u = bfround(group_sum<LPR>(acc[1][m]));
+                if (sl == 0 && rows[0] < I && m < mc)
+                    h[(size_t)s_pairs[r0 + m] * I + rows[0]] = f32_bf16(bfround(g / (1.f + expf(-g))) * u);
+            }
+        }
+    };
+    for (int r0 = 0; r0 < rows_n; r0 += MC) {
+        const int mc = min(MC, rows_n - r0);
+        if (mc == 1)
+            pass(std::integral_constant<int, 1>{}, r0, mc);
+        else if (mc == 2)
+            pass(std::integral_constant<int, 2>{}, r0, mc);
+        else
+            pass(std::integral_constant<int, MC>{}, r0, mc);
     }
 }
 
@@ -440,6 +523,25 @@ static int32_t launch_gate_up(const void* stack, const void* x, const int32_t* i
     constexpr int RPW = 2, U = 4, G = WAVE / LPR;
     const int ntiles = (R / 2 + G - 1) / G;
     const int grid = (ntiles + 3) / 4;
+    // From eight rows on, the rows that share an expert go through it together. Fewer rows share few experts (4 rows of
+    // top-8 over 128 experts: 30 distinct of 32 picks) and the gathering costs more than it saves: measured on the
+    // Qwen3-30B-A3B shape, a layer takes 74 against 72 us at 4 rows, 117 against 119 at 8, 190 against 208 at 16, 310
+    // against 384 at 32. The knob moe_grouped forces either (1 / 0).
+    constexpr int MC = 4;
+    const int grouped = tuning("moe_grouped");
+    const bool wanted = grouped >= 0 ? grouped != 0 && pairs > k : pairs >= 8 * k;
+    if (wanted && pairs <= GROUP_MAX_PAIRS && (size_t)MC * C * 2 <= (size_t)device_info().lds_bytes - 16 * 1024) {
+        auto kern = moe_gate_up_grouped_kernel<LPR, RPW, U, MC>;
+        const size_t lds = (size_t)MC * C * 2;
+        if (lds > 48 * 1024) {
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                               hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+            if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
+        }
+        hipLaunchKernelGGL(kern, dim3(grid, pairs), dim3(256), lds, st, static_cast<const uint4*>(stack),
+                           static_cast<const uint16_t*>(x), idx, static_cast<uint16_t*>(gu), R, C, k, E, pairs);
+        return hip_status(hipGetLastError(), "moe gate_up launch");
+    }
     hipLaunchKernelGGL((moe_gate_up_kernel<LPR, RPW, U>), dim3(grid, pairs), dim3(256), (size_t)C * 2, st,
                        static_cast<const uint4*>(stack), static_cast<const uint16_t*>(x), idx,
                        static_cast<uint16_t*>(gu), R, C, k, E);
@@ -485,6 +587,16 @@ int32_t btb_hip_moe_route(const void* logits, int32_t logits_f32, size_t ls, siz
     return launch_route<false>(logits, ls, (int)E, (int)k, (int)T, idx, static_cast<uint16_t*>(w), w32, nullptr, st);
 }
 
+int32_t btb_hip_moe_group_picks(const int32_t* idx, size_t T, size_t k, size_t E, int32_t* slot, int32_t* token,
+                                int32_t* offs, int32_t* counts, void* stream) {
+    if (idx == nullptr || slot == nullptr || token == nullptr || offs == nullptr || counts == nullptr) return ERR_NULL;
+    if (T == 0 || k == 0 || E == 0 || T * k > 65535 || E > (1u << 20)) return ERR_DOMAIN;
+    if (!al(idx, 4) || !al(slot, 4) || !al(token, 4) || !al(offs, 4) || !al(counts, 4)) return ERR_DOMAIN;
+    hipLaunchKernelGGL(moe_group_picks_kernel, dim3((unsigned)((E + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), idx, (int)T, (int)k, (int)E, slot, token, offs, counts);
+    return hip_status(hipGetLastError(), "moe_group_picks launch");
+}
+
 int32_t btb_hip_moe_router_bf16(const void* router, const void* x, size_t T, size_t E, size_t H, size_t k, float* logits,
                                 void* logits16, int32_t* idx, void* w, float* w32, void* stream) {
     if (router == nullptr || x == nullptr || logits == nullptr || idx == nullptr || w == nullptr) return ERR_NULL;
@@ -493,8 +605,12 @@ int32_t btb_hip_moe_router_bf16(const void* router, const void* x, size_t T, siz
     if (!al(router, 2) || !al(x, 2) || !al(logits, 4) || !al(logits16, 2) || !al(idx, 4) || !al(w, 2) || !al(w32, 4))
         return ERR_DOMAIN;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    int32_t rc = lane16_bf16_rows16(static_cast<const uint16_t*>(router), E, H, static_cast<const uint16_t*>(x), T,
-                                    logits, st);
+    // one launch where the matvec's last workgroup can route (up to 256 experts, rows of whole 128-column steps)
+    int32_t rc = lane16_bf16_router16(static_cast<const uint16_t*>(router), E, H, static_cast<const uint16_t*>(x), T,
+                                      logits, idx, static_cast<uint16_t*>(w), w32, static_cast<uint16_t*>(logits16),
+                                      (int)k, st);
+    if (rc != ERR_UNSUPPORTED) return rc;
+    rc = lane16_bf16_rows16(static_cast<const uint16_t*>(router), E, H, static_cast<const uint16_t*>(x), T, logits, st);
     if (rc != OK) return rc;
     return launch_route<true>(logits, E, (int)E, (int)k, (int)T, idx, static_cast<uint16_t*>(w), w32,
                               static_cast<uint16_t*>(logits16), st);

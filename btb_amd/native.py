@@ -57,6 +57,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_gemv_fp8_rows": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _vp]),
     "btb_hip_gemv_fp8_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_moe_route": (_i32, [_vp, _i32, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp]),
+    "btb_hip_moe_group_picks": (_i32, [_vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_moe_router_bf16": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_moe_experts_bf16": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _vp]),
     "btb_hip_embed": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
@@ -545,6 +546,22 @@ class HipCard:
         self._call("btb_hip_moe_route", self.ptr(logits), int(logits.dtype == torch.float32), ls, E, k, T, self.ptr(idx),
                    self.ptr(w), self.ptr(w32), _stream())
         return idx, w, w32
+
+    def moe_group_picks(self, idx: torch.Tensor, num_experts: int):
+        """(pick position i32 [T k], row i32 [T k], offsets i32 [E], counts i32 [E]) of the picks idx i32 [T, k] sorted
+        by expert, stable over idx.T.reshape(-1) (`group_picks`, btb/engine/host.py:283-296), all on the device"""
+        self._need(idx, torch.int32, "idx")
+        if idx.dim() != 2 or not idx.is_contiguous():
+            raise ValueError("[hip] moe_group_picks: idx must be a contiguous [T, k] int32 tensor on the GPU")
+        T, k = (int(s) for s in idx.shape)
+        dev = idx.device
+        slot = torch.empty(T * k, dtype=torch.int32, device=dev)
+        token = torch.empty(T * k, dtype=torch.int32, device=dev)
+        offs = torch.empty(int(num_experts), dtype=torch.int32, device=dev)
+        counts = torch.empty(int(num_experts), dtype=torch.int32, device=dev)
+        self._call("btb_hip_moe_group_picks", self.ptr(idx), T, k, int(num_experts), self.ptr(slot), self.ptr(token),
+                   self.ptr(offs), self.ptr(counts), _stream())
+        return slot, token, offs, counts
 
     def moe_router(self, router: torch.Tensor, x: torch.Tensor, k: int):
         """(logits f32 [T, E], logits bf16 [T, E], idx int32 [T, k], weights bf16 [T, k], weights f32 [T, k]) of bf16

@@ -198,6 +198,14 @@ int32_t btb_hip_gemv_fp8_group(size_t n, const uint8_t* const* w, const float* c
 int32_t btb_hip_moe_route(const void* logits, int32_t logits_f32, size_t ls, size_t E, size_t k, size_t T, int32_t* idx,
                           void* w, float* w32, void* stream);
 
+/* group_picks (btb/engine/host.py:283-296) on the device: the (pick position, row) pairs of idx i32 [T, k] sorted by
+ * expert with a stable sort of idx.T.reshape(-1) - so an expert's pairs come pick-major, then row - into slot i32
+ * [T k] and token i32 [T k], and each expert's first place and count among them into offs i32 [E] and counts i32 [E].
+ * Every id must lie in [0, E) (btb_hip_moe_route's do). T k <= 65535. The experts kernel below does this grouping in
+ * place (an expert's first pair gathers the others); this entry point is the reference's function as data. */
+int32_t btb_hip_moe_group_picks(const int32_t* idx, size_t T, size_t k, size_t E, int32_t* slot, int32_t* token,
+                                int32_t* offs, int32_t* counts, void* stream);
+
 /* Qwen4Router.forward for bf16 rows in two launches (btb/engine/families/qwen4/router.py:43-51): the f32 logits of
  * x [T, H] bf16 against router [E, H] bf16 in the host matvec's order (btb_hip_gemv_bf16_rows of the rows widened to
  * f32, to the bit) into logits f32 [T, E], then btb_hip_moe_route over them. logits16, when not NULL, receives the

@@ -118,14 +118,23 @@ def test_route_in_registers_and_through_lds_agree(card):
     assert idx[0].tolist() == [9, 4, 30] + [i for i in range(40) if i not in (9, 4, 30)][:29]
 
 
-@pytest.mark.parametrize("T,E,H", [(1, 128, 2048), (5, 128, 2048), (3, 60, 520), (2, 384, 256)])
+@pytest.mark.parametrize("T,E,H", [(1, 128, 2048), (5, 128, 2048), (3, 60, 520), (2, 384, 256), (9, 128, 2048),
+                                   (64, 256, 1024), (3, 200, 384), (7, 40, 128)])
 def test_router_in_two_launches_is_the_three_step_form(card, T, E, H):
     """bf16 rows straight into the host-order matvec, the logits rounded inside the routing kernel: the same bits as
-    widening the rows first, routing the f32 logits and rounding them afterwards"""
+    widening the rows first, routing the f32 logits and rounding them afterwards. Up to 256 experts with rows of whole
+    128-column steps it can be one launch (knob moe_fused_router = 1: the matvec's last workgroup routes), and the
+    same bits again: against the three steps, against the two launches, and on a second call (the tickets that
+    find the last workgroup are back at zero)"""
     g = gen(540 + T)
     wr = (torch.randn(E, H, generator=g) * 0.05).to(torch.bfloat16).cuda()
     x = acts_bf16(T, H, seed=545 + T).cuda()
-    logits, logits16, idx, w, w32 = card.moe_router(wr, x, 8)
+    card.set_tuning("moe_fused_router", 1)
+    try:
+        logits, logits16, idx, w, w32 = card.moe_router(wr, x, 8)
+        again = card.moe_router(wr, x, 8)
+    finally:
+        card.set_tuning("moe_fused_router", -1)
     raw = card.gemv_lane16(wr, x.float())
     ridx, rw, rw32 = card.moe_route(raw, 8)
     assert torch.equal(logits.view(torch.int32), raw.view(torch.int32))
@@ -135,3 +144,46 @@ def test_router_in_two_launches_is_the_three_step_form(card, T, E, H):
     want, ow, opicks = omoe.router(bits16(wr.cpu()), x.float().cpu().numpy(), 8, "bf16")
     assert np.array_equal(f32_bits(logits.cpu().numpy()), f32_bits(want))
     assert np.array_equal(idx.cpu().numpy().astype(np.int64), opicks)
+    two = card.moe_router(wr, x, 8)  # the default: two launches
+    for a, b, c in zip((logits, logits16, idx, w, w32), again, two):
+        bits = torch.int16 if a.dtype == torch.bfloat16 else torch.int32
+        assert torch.equal(a.view(bits), b.view(bits)) and torch.equal(a.view(bits), c.view(bits))
+
+
+@pytest.mark.parametrize("T,k,n_experts", [(1, 8, 128), (8, 8, 128), (13, 4, 60), (64, 8, 128), (5, 3, 700), (200, 8, 16)])
+def test_group_picks_is_the_stable_sort(card, T, k, n_experts):
+    """`group_picks` (btb/engine/host.py:283-296) on the device against the oracle's stable argsort, entry for entry:
+    few experts with many rows each, more experts than one workgroup's threads, experts nobody picked"""
+    g = gen(560 + T)
+    picks = torch.stack([torch.randperm(n_experts, generator=g)[:k] for _ in range(T)]).to(torch.int32)
+    slot, token, offs, counts = card.moe_group_picks(picks.cuda(), n_experts)
+    wslot, wtoken, woffs, wcounts = omoe.group_picks(picks.numpy(), n_experts)
+    assert np.array_equal(counts.cpu().numpy(), wcounts)
+    assert np.array_equal(offs.cpu().numpy(), woffs)
+    assert np.array_equal(slot.cpu().numpy(), wslot)
+    assert np.array_equal(token.cpu().numpy(), wtoken)
+
+
+@pytest.mark.parametrize("T,share", [(4, 2), (8, 3), (12, 1), (9, 40)])
+def test_rows_that_share_an_expert_go_through_it_together(card, layer_weights, T, share):
+    """the gate/up kernel that streams an expert once for all the rows that picked it writes the bits of the kernel
+    that streams it once a pair (knob moe_grouped = 0), with picks drawn from `share` + k - 1 experts so that rows
+    share many (an expert picked by more than four rows takes more than one pass), and from all 128"""
+    wr, gu, dn = layer_weights
+    g = gen(570 + T)
+    pool = min(E, share + K - 1)
+    picks = torch.stack([torch.randperm(pool, generator=g)[:K] * (E // pool) for _ in range(T)]).to(torch.int32).cuda()
+    w = torch.rand(T, K, generator=g).to(torch.bfloat16).cuda()
+    x = acts_bf16(T, H, seed=580 + T).cuda()
+    experts = Experts(card, gu.cuda(), dn.cuda())
+    try:
+        card.set_tuning("moe_grouped", 1)  # from eight rows on it is the default; here for every T
+        y = experts(x, picks, w).clone()
+        card.set_tuning("moe_grouped", 0)
+        by_pair = experts(x, picks, w).clone()
+    finally:
+        card.set_tuning("moe_grouped", -1)
+    assert torch.equal(y.view(torch.int16), by_pair.view(torch.int16))
+    want = omoe.experts(bits16(gu), bits16(dn), x.float().cpu().numpy(), picks.cpu().numpy().astype(np.int64),
+                        w.float().cpu().numpy(), "bf16")
+    assert np.abs(y.float().cpu().numpy() - want).max() <= 1e-2 * np.abs(want).max()
