@@ -2,6 +2,7 @@
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode|decode_p12] [--no-cpu]
     python bench.py --workload gemv_bf16|gemv_p12|gemv_fp8|gemv_mxfp4|moe [--m M]      (the other configs, one kernel each)
+    python bench.py --workload copy          (a plain 2^28-byte device copy: the scale of the FETCH_SIZE / WRITE_SIZE counters)
 
 A step is one decode step of a random-init Qwen3-4B-shaped dense stack (36 layers, hidden 2560, 32 query / 8 kv heads
 of 128, SwiGLU 9728, vocab 151936; weights ~N(0, 0.02) in bf16, seeded N(0, 1) K/V for a 4096-token context), M = 1
@@ -162,6 +163,21 @@ def apply_tuning(card, pairs: list[str]) -> dict[str, int]:
         card.set_tuning(key.strip(), int(value))
         out[key.strip()] = int(value)
     return out
+
+
+def copy_workload() -> int:
+    """A device-to-device copy of 2^28 bytes, three times: under `rocprofv3 --pmc FETCH_SIZE` (or WRITE_SIZE) its
+    dispatches read 2^28 bytes and write 2^28 bytes, which gives the unit the counter counts in on this GPU."""
+    import torch
+
+    n = 1 << 28
+    a = torch.empty(n, dtype=torch.uint8, device="cuda")
+    b = torch.randint(0, 255, (n,), dtype=torch.uint8, device="cuda")
+    for _ in range(3):
+        a.copy_(b)
+    torch.cuda.synchronize()
+    print(json.dumps({"workload": "copy", "bytes": n, "copies": 3}))
+    return 0
 
 
 def kernel_workload(args: argparse.Namespace) -> int:
@@ -382,7 +398,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="decode",
-                    choices=["decode", "decode_p12", "gemv_bf16", "gemv_p12", "gemv_fp8", "gemv_mxfp4", "moe"])
+                    choices=["decode", "decode_p12", "gemv_bf16", "gemv_p12", "gemv_fp8", "gemv_mxfp4", "moe", "copy"])
     ap.add_argument("--m", type=int, default=1, help="rows of x (tokens) for the single-operator workloads")
     ap.add_argument("--rows", type=int, default=1,
                     help="rows of a decode pass: 1 is the step the metric is quoted on, more a speculative verify pass")
@@ -393,6 +409,8 @@ def main() -> int:
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU (no collectives, no sharding); use --gpus 1", file=sys.stderr)
         return 2
+    if args.workload == "copy":
+        return copy_workload()
     if args.workload not in ("decode", "decode_p12"):
         return kernel_workload(args)
     if args.steps < 1 or args.warmup < 0 or args.steps + args.warmup > 480:

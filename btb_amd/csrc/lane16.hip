@@ -262,7 +262,9 @@ static int32_t launch_lane16(const W& w, const XT* x, float* y, size_t rows, siz
             bool done = true;
             const size_t fours = std::min<size_t>(b / 4, 65535);
             if (fours > 0) {
-                done = launch_wide<4, 4>(w.w, x, y, rows, cols, 0, b, (unsigned)fours, st);
+                // few rows of weights (a router): every step of a row asked for at once, as the one-row pass does
+                done = rows <= 1024 && launch_wide<4, 16>(w.w, x, y, rows, cols, 0, b, (unsigned)fours, st);
+                if (!done) done = launch_wide<4, 4>(w.w, x, y, rows, cols, 0, b, (unsigned)fours, st);
                 if (done) b0 = 4 * fours;
             }
             while (done && b0 < b) {
