@@ -144,6 +144,43 @@ struct FmtP12 {
     }
 };
 
+// The same form with the table lookups done in LDS: a 256-entry table of PAIRS - entry b holds the high bytes of the
+// two weights whose codes are byte b's nibbles - is built once a workgroup, and a byte of codes becomes its two high
+// bytes with one 16-bit LDS read where the in-register lookup takes two byte-permutes, a select and the nibble split
+// per four codes. Eight weights: 4 byte extractions, 4 LDS reads, 4 byte-permutes that zip high and low bytes (23
+// vector instructions before). prepare() must be followed by a workgroup barrier before the first widen (the
+// streaming kernel's x staging ends with one).
+struct FmtP12L : FmtP12 {
+    __device__ static __forceinline__ uint16_t* pair_table() {
+        __shared__ uint16_t pairs[256];
+        return pairs;
+    }
+    __device__ static __forceinline__ void prepare(Params& p) {
+        FmtP12::prepare(p);
+        uint16_t* t = pair_table();
+        const uint32_t d[4] = {p.tbl.x, p.tbl.y, p.tbl.z, p.tbl.w};
+        for (int b = threadIdx.x; b < 256; b += blockDim.x) {
+            const uint32_t lo = (d[(b & 15) >> 2] >> (8 * (b & 3))) & 0xFFu;
+            const uint32_t hi = (d[(b >> 4) >> 2] >> (8 * ((b >> 4) & 3))) & 0xFFu;
+            t[b] = (uint16_t)(lo | (hi << 8));
+        }
+    }
+    // eight weights: codes c (weight k in nibble k), low bytes l0 (weights 0..3), l1 (4..7)
+    __device__ static __forceinline__ void widen8(uint32_t c, uint32_t l0, uint32_t l1, uint32_t* w) {
+        const uint16_t* t = pair_table();
+        const uint32_t h01 = t[c & 0xFFu], h23 = t[(c >> 8) & 0xFFu], h45 = t[(c >> 16) & 0xFFu], h67 = t[c >> 24];
+        // a byte-permute's selector 0..3 takes a byte of its second operand, 4..7 of its first
+        w[0] = __builtin_amdgcn_perm(h01, l0, 0x05010400u);  // lo0 hi0 lo1 hi1
+        w[1] = __builtin_amdgcn_perm(h23, l0, 0x05030402u);  // lo2 hi2 lo3 hi3
+        w[2] = __builtin_amdgcn_perm(h45, l1, 0x05010400u);
+        w[3] = __builtin_amdgcn_perm(h67, l1, 0x05030402u);
+    }
+    __device__ static __forceinline__ void widen(const RowCtx&, const Raw& r, int /*unit*/, uint32_t (&w)[UW / 2]) {
+        widen8(r.codes.x, r.lo.x, r.lo.y, w);
+        widen8(r.codes.y, r.lo.z, r.lo.w, w + 4);
+    }
+};
+
 // ------------------------------------------------------------------------------------------------------------
 // FP8 e4m3fn with an f32 scale per block of a [sr, sc] grid: a unit is 16 weights, one 16-byte load, under one
 // scale (the block's width is a multiple of 16). weight = bf16_rne(e4m3 * scale): the byte pair is converted by
