@@ -53,6 +53,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_gemv_bf16_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_gemv_p12_rows": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _sz, _vp, _vp]),
     "btb_hip_gemv_mxfp4_rows": (_i32, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _vp]),
+    "btb_hip_gemv_mxfp4_ggml_rows": (_i32, [_vp, _sz, _sz, _vp, _sz, _vp, _vp]),
     "btb_hip_gemv_mxfp4_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_gemv_fp8_rows": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _vp]),
     "btb_hip_gemv_fp8_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
@@ -520,6 +521,17 @@ class HipCard:
         x2, b, y = self._rows_io(x, y, R, C, "gemv_lane16_mx4")
         self._call("btb_hip_gemv_mxfp4_rows", self.ptr(w.blocks), self.ptr(w.scales), R, C, self.ptr(x2), b, self.ptr(y),
                    _stream())
+        return y
+
+    def gemv_lane16_mx4_ggml(self, raw: torch.Tensor, rows: int, cols: int, x: torch.Tensor,
+                             y: torch.Tensor | None = None) -> torch.Tensor:
+        """the same over ggml's layout: raw u8 [rows * cols / 32 * 17], 17-byte blocks with the scale first
+        (`btb_gemv_mxfp4_ggml_rows`, native/src/lib.rs:162-183); the bits of `gemv_lane16_mx4` for the same weights"""
+        self._need(raw, torch.uint8, "raw")
+        if raw.numel() != rows * cols // 32 * 17:
+            raise ValueError(f"[hip] gemv_lane16_mx4_ggml: {raw.numel()} bytes are not {rows} x {cols} weights in 17-byte blocks")
+        x2, b, y = self._rows_io(x, y, rows, cols, "gemv_lane16_mx4_ggml")
+        self._call("btb_hip_gemv_mxfp4_ggml_rows", self.ptr(raw), rows, cols, self.ptr(x2), b, self.ptr(y), _stream())
         return y
 
     def gemv_lane16_fp8(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:

@@ -177,6 +177,11 @@ int32_t btb_hip_gemv_p12_rows(const uint8_t* lo, const uint8_t* hi4, const uint8
  * reference card's btb_gemv_lane16_mx4_f32_m* (native/cuda/btb_kernels.cu:1701-1766). */
 int32_t btb_hip_gemv_mxfp4_rows(const uint8_t* blocks, const uint8_t* scales, size_t rows, size_t cols, const float* x,
                                 size_t b, float* y, void* stream);
+/* btb_gemv_mxfp4_ggml_rows (native/src/lib.rs:162-183) on the device: the same matvec over ggml's MXFP4 layout (a
+ * GGUF's) - raw holds 17-byte blocks, the e8m0 scale first, then 16 bytes whose low nibbles are weights 0..15 and high
+ * nibbles 16..31. The same arithmetic in the same order: the bits of btb_hip_gemv_mxfp4_rows for the same weights. */
+int32_t btb_hip_gemv_mxfp4_ggml_rows(const uint8_t* raw, size_t rows, size_t cols, const float* x, size_t b, float* y,
+                                     void* stream);
 int32_t btb_hip_gemv_mxfp4_group(size_t n, const uint8_t* const* blocks, const uint8_t* const* scales,
                                  const size_t* rows, const size_t* cols, const float* const* x, const size_t* b,
                                  float* const* y, void* stream);

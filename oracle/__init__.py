@@ -33,6 +33,7 @@ _SIGS = {
     "btb_gemv_bf16_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
     "btb_gemv_p12_rows": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
     "btb_gemv_mxfp4_rows": (_i32, [_vp, _vp, _sz, _sz, _vp, _sz, _vp, _sz]),
+    "btb_gemv_mxfp4_ggml_rows": (_i32, [_vp, _sz, _sz, _vp, _sz, _vp, _sz]),
     "btb_gemv_mxfp4_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
     "btb_gemv_fp8_rows": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _sz, _vp, _sz]),
     "btb_gemv_fp8_group": (_i32, [_sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz]),
@@ -109,6 +110,17 @@ def gemv_p12(lo, hi4, table, esc_idx, esc_val, rows: int, cols: int, x: np.ndarr
                                  _p(y), threads)
     if rc != OK:
         raise ValueError(f"btb_gemv_p12_rows: {rc}")
+    return y
+
+
+def gemv_mxfp4_ggml(raw: np.ndarray, rows: int, cols: int, x: np.ndarray, threads: int = 1):
+    """the MXFP4 matvec over ggml's layout: 17-byte blocks, scale first (btb_gemv_mxfp4_ggml_rows, lib.rs:162-183)"""
+    raw = _c(raw, np.uint8)
+    x = _c(np.atleast_2d(x), np.float32)
+    y = np.empty((x.shape[0], rows), dtype=np.float32)
+    rc = lib().btb_gemv_mxfp4_ggml_rows(_p(raw), rows, cols, _p(x), x.shape[0], _p(y), threads)
+    if rc != OK:
+        raise ValueError(f"btb_gemv_mxfp4_ggml_rows: {rc}")
     return y
 
 

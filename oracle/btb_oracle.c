@@ -137,6 +137,7 @@ typedef struct {
     /* mxfp4 */
     const uint8_t* blocks;
     const uint8_t* scales8;
+    int ggml; /* 17-byte blocks, the scale first, low nibbles weights 0..15, high nibbles 16..31 (gemv.rs:1034-1078) */
     /* fp8 */
     const uint8_t* q;
     const float* scales;
@@ -238,6 +239,16 @@ static size_t p12_cursor(const Stored* s, size_t start) {
 static void widen_mx4(const Stored* s, size_t start, size_t n, float* dst) {
     for (size_t blk = 0; blk < n / MX_BLOCK; ++blk) {
         size_t g = start / MX_BLOCK + blk;
+        if (s->ggml) { /* gemv.rs:1147-1151: the same values in the same places, read from the other layout */
+            const uint8_t* raw = s->blocks + g * 17;
+            float sc = mx_scale(raw[0]);
+            float* o = dst + blk * MX_BLOCK;
+            for (int j = 0; j < 16; ++j) {
+                o[j] = fp4_value(raw[1 + j] & 0x0F) * sc;
+                o[16 + j] = fp4_value(raw[1 + j] >> 4) * sc;
+            }
+            continue;
+        }
         const uint8_t* bytes = s->blocks + g * 16;
         float sc = mx_scale(s->scales8[g]);
         float* o = dst + blk * MX_BLOCK;
@@ -634,6 +645,17 @@ EXPORT int32_t btb_gemv_mxfp4_rows(const uint8_t* blocks, const uint8_t* scales,
     Job job;
     int rc = check_mx4(blocks, scales, rows, cols, x, b, y, &job);
     if (rc != OK) return rc;
+    return run_jobs(&job, 1, rows, threads);
+}
+
+/* btb_gemv_mxfp4_ggml_rows (native/src/lib.rs:162-183): the same matvec over ggml's 17-byte blocks */
+EXPORT int32_t btb_gemv_mxfp4_ggml_rows(const uint8_t* raw, size_t rows, size_t cols, const float* x, size_t b, float* y,
+                                        size_t threads) {
+    Job job;
+    int rc = check_mx4(raw, raw, rows, cols, x, b, y, &job);
+    if (rc != OK) return rc;
+    job.w.scales8 = NULL;
+    job.w.ggml = 1;
     return run_jobs(&job, 1, rows, threads);
 }
 

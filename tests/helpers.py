@@ -121,3 +121,17 @@ def reference_logits(cfg, get, prompt):
         x = x + (torch.nn.functional.silu(g) * u) @ get(L + "mlp.down_proj.weight").T
     x = norm(x, "model.norm.weight")
     return (x[-1] @ get("model.embed_tokens.weight").T).numpy()
+
+
+def mx4_ggml(blocks, scales):
+    """a checkpoint-layout MXFP4 matrix (blocks u8 [..., 16], scales u8 [...]) in ggml's layout: 17-byte blocks, the
+    scale first, weights 0..15 in the low nibbles and 16..31 in the high (the reference's own test helper does the
+    same repacking, native/src/gemv.rs:5192-5213)"""
+    import numpy as np
+
+    b = np.asarray(blocks, np.uint8).reshape(-1, 16)
+    codes = np.stack([b & 0x0F, b >> 4], axis=-1).reshape(-1, 32)  # weight order
+    raw = np.empty((b.shape[0], 17), np.uint8)
+    raw[:, 0] = np.asarray(scales, np.uint8).reshape(-1)
+    raw[:, 1:] = codes[:, :16] | (codes[:, 16:] << 4)
+    return raw.reshape(-1)

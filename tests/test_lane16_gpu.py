@@ -66,6 +66,26 @@ def test_mxfp4_rows_bits(card, rows, cols, b):
     assert np.all(same | (np.isnan(got) & np.isnan(want)))
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 32), (17, 1024), (33, 2880)])
+@pytest.mark.parametrize("b", [1, 3, 16])
+def test_mxfp4_ggml_rows_bits(card, rows, cols, b):
+    """`btb_gemv_mxfp4_ggml_rows` on the device: the oracle's bits, which are the checkpoint layout's for the same
+    weights (native/src/gemv.rs:5215-5250)"""
+    from .helpers import mx4_ggml
+
+    rng = np.random.default_rng(rows + b)
+    blocks = rng.integers(0, 256, (rows, cols // 32, 16), dtype=np.uint8)
+    scales = rng.integers(0, 255, (rows, cols // 32), dtype=np.uint8)
+    raw = mx4_ggml(blocks, scales)
+    x = xs(b, cols, 423)
+    got = card.gemv_lane16_mx4_ggml(torch.from_numpy(raw).cuda(), rows, cols, x.cuda()).cpu().numpy()
+    want = oracle.gemv_mxfp4_ggml(raw, rows, cols, x.numpy(), threads=0)
+    assert np.all((f32_bits(got) == f32_bits(want)) | (np.isnan(got) & np.isnan(want)))
+    w = mxfp4.MxWeight(torch.from_numpy(blocks).reshape(-1).cuda(), torch.from_numpy(scales).reshape(-1).cuda(), rows, cols)
+    other = card.gemv_lane16_mx4(w, x.cuda()).cpu().numpy()
+    assert np.all((f32_bits(got) == f32_bits(other)) | (np.isnan(got) & np.isnan(other)))
+
+
 @pytest.mark.parametrize("rows,cols,block", [(256, 512, (128, 128)), (48, 111, (16, 37)), (8, 64, (8, 64))])
 def test_fp8_rows_bits(card, rows, cols, block):
     src = weights_bf16(rows, cols, seed=430).float()

@@ -180,6 +180,32 @@ def test_mxfp4_gemv_against_f64():
     assert conditioned_err(y, w, x.astype(np.float64)) < 1e-6
 
 
+@pytest.mark.parametrize("rows,cols", [(1, 32), (5, 96), (17, 1024), (33, 2880)])
+def test_mxfp4_ggml_layout_gives_the_checkpoint_layouts_bits(rows, cols):
+    """native/src/gemv.rs:5215-5250: the same weights in ggml's 17-byte blocks give the same bits, any b, any threads"""
+    from .helpers import mx4_ggml
+
+    rng = np.random.default_rng(rows)
+    blocks = rng.integers(0, 256, (rows, cols // 32, 16), dtype=np.uint8)
+    scales = rng.integers(0, 255, (rows, cols // 32), dtype=np.uint8)
+    raw = mx4_ggml(blocks, scales)
+    for b in (1, 3, 16):
+        x = rng.uniform(-1, 1, (b, cols)).astype(np.float32)
+        want = oracle.gemv_mxfp4(blocks, scales, rows, cols, x, threads=2)
+        got = oracle.gemv_mxfp4_ggml(raw, rows, cols, x, threads=3)
+        assert np.all((f32_bits(got) == f32_bits(want)) | (np.isnan(got) & np.isnan(want)))
+    # a hand case: scale 127 (2^0), weight 0 = code 2 (1.0) in the low nibble of byte 1, weight 16 = code 4 (2.0) in its high
+    one = np.zeros(17, np.uint8)
+    one[0], one[1] = 127, 0x42
+    xx = np.zeros((1, 32), np.float32)
+    xx[0, 0], xx[0, 16] = 3.0, 5.0
+    assert oracle.gemv_mxfp4_ggml(one, 1, 32, xx)[0, 0] == 1.0 * 3.0 + 2.0 * 5.0
+    L = oracle.lib()
+    y = np.zeros((1, 1), np.float32)
+    assert L.btb_gemv_mxfp4_ggml_rows(None, 1, 32, xx.ctypes.data, 1, y.ctypes.data, 1) == oracle.ERR_NULL
+    assert L.btb_gemv_mxfp4_ggml_rows(one.ctypes.data, 1, 24, xx.ctypes.data, 1, y.ctypes.data, 1) == oracle.ERR_DOMAIN
+
+
 # -- FP8 (native/src/gemv.rs:5383-5430) --------------------------------------------------------------------------
 
 
