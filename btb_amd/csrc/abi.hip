@@ -76,6 +76,7 @@ static Knob g_knobs[] = {
     {"moe_fused_router", {-1}},
     {"attn_split", {-1}},
     {"attn_heads_per_wg", {-1}},
+    {"attn_rows_per_wg", {-1}},
 };
 
 int tuning(const char* key) {

@@ -136,6 +136,12 @@ class DecodeStep:
                 # triples, each span a whole number of those batches (the library rounds a span up to one)
                 per = max(128, self.cap // max(1, card.sms // (Hk * (Hq // Hk // 2))) // 128 * 128)
                 attn_spans = max(1, -(-self.cap // per))
+            elif 2 <= self.T <= 16 and D == 128 and Hq // Hk in (2, 4) and self.cap <= 128 * (1024 // (Hq // Hk)):
+                # a pass of a few rows: spans of 128 keys, one batch of the attention's sixteen streams, which a
+                # workgroup asks for at once and keeps in registers (measured at 4096 keys, ms a pass with this
+                # against the best span count of the general kernel: 2 rows 2.95 / 3.12, 4 rows 3.51 / 3.68, 8 rows
+                # 3.67 / 3.83, 16 rows 4.64 / 4.83)
+                attn_spans = -(-self.cap // 128)
         self.S = int(attn_spans)
         self.scratch = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
         # Which sequence: up to three rows the fused launches win (fewer launches, every matvec on the streaming

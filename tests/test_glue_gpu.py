@@ -137,6 +137,58 @@ def test_attn_decode_over_a_tree_of_rows(card, n0, T, Hq, Hk, S, seed):
                          card.attn_scratch(33, Hq, Hk, D, 1), par=torch.zeros(33, dtype=torch.int32, device="cuda"))
 
 
+@pytest.mark.parametrize("n0,T,Hq,Hk,S,tree,win", [(1000, 8, 32, 8, 9, False, 0), (1000, 8, 32, 8, 5, False, 0),
+                                                    (300, 5, 8, 2, 3, True, 0), (120, 16, 8, 4, 1, False, 0),
+                                                    (700, 6, 16, 4, 6, True, 200), (0, 3, 8, 2, 1, False, 0),
+                                                    (500, 2, 32, 8, 4, False, 37)])
+def test_attn_short_spans_kept_in_registers(card, n0, T, Hq, Hk, S, tree, win):
+    """a pass of several rows whose spans are one or two batches of keys (128 / 256) takes the kernel that asks for a
+    span's keys at once: against f64 attention over the keys each row sees, the bits of the general kernel at the same
+    span count (knob attn_rows_per_wg = 0), and the same bits however many rows a workgroup takes"""
+    D = 128
+    cap = n0 + T + 3
+    span = -(-(-(-cap // S)) // 128) * 128
+    assert span in (128, 256)
+    g = gen(690 + n0 + T)
+    K = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    V = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    q = torch.randn(T, Hq * D, generator=g).to(torch.bfloat16)
+    par = [-1] + [int(torch.randint(-1, t, (1,), generator=g)) for t in range(1, T)] if tree else None
+    part = None if par is None else torch.tensor(par, dtype=torch.int32, device="cuda")
+    scratch = card.attn_scratch(T, Hq, Hk, D, S)
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    scale = 1.0 / np.sqrt(D)
+    outs = {}
+    try:
+        for knob in (-1, 0, 2, 3, T):
+            card.set_tuning("attn_rows_per_wg", knob)
+            att = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+            card.attn_decode(q.cuda(), K.cuda(), V.cuda(), att, n0t, Hq, Hk, D, scale, S, scratch, par=part, win=win)
+            outs[knob] = att.clone()
+    finally:
+        card.set_tuning("attn_rows_per_wg", -1)
+    for knob, a in outs.items():
+        assert torch.equal(a, outs[-1]), knob
+    got = outs[-1].float().cpu().numpy()
+    for t in range(T):
+        if par is None:
+            slots = list(range(n0 + t + 1))            # slot = position in a chain
+            pos = slots
+        else:
+            path, p_ = [], t
+            while p_ >= 0:
+                path.append(p_)
+                p_ = par[p_]
+            path = path[::-1]                            # root first: depth d at position n0 + d
+            slots = list(range(n0)) + [n0 + p for p in path]
+            pos = list(range(n0)) + [n0 + d for d in range(len(path))]
+        keep = [s_ for s_, ps in zip(slots, pos) if win == 0 or ps >= pos[-1] + 1 - win]
+        want = od.attention(q[t].float().numpy().reshape(Hq, D), K[:, keep].float().numpy(), V[:, keep].float().numpy(),
+                            scale)
+        worst = np.abs(got[t].reshape(Hq, D) - want).max() / np.abs(want).max()
+        assert worst <= 2.0**-7, (t, worst)
+
+
 @pytest.mark.parametrize("n0,Hq,Hk,S", [(4096, 32, 8, 36), (100, 32, 8, 4), (0, 8, 8, 1), (63, 16, 2, 7), (64, 16, 2, 2),
                                          (500, 8, 1, 16), (31, 4, 2, 3), (300, 8, 1, 40), (200, 4, 4, 5)])
 @pytest.mark.parametrize("with_norm", [True, False])
