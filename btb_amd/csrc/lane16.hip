@@ -164,10 +164,13 @@ __global__ void __launch_bounds__(256) lane16_bf16_wide_kernel(const uint16_t* _
     const bool live = r < rows;
     const uint4* wrow = reinterpret_cast<const uint4*>(w + (live ? r : rows - 1) * cols);
     const int nchunks = (int)(cols / 128);
-    uint4 raw[NB];
+    // a compiler vector, not HIP's uint4: an array of the struct type that lives across the loop below is kept in scratch
+    // memory - written there as soon as it is loaded, which waits for the loads at once - and a vector's is not
+    u32x4 raw[NB];
     auto request = [&](int n0) {
 #pragma unroll
-        for (int n = 0; n < NB; ++n) raw[n] = wrow[(size_t)min(n0 + n, nchunks - 1) * 16 + j];
+        for (int n = 0; n < NB; ++n)
+            raw[n] = *reinterpret_cast<const u32x4*>(wrow + (size_t)min(n0 + n, nchunks - 1) * 16 + j);
     };
     request(0);
     // x in 16-byte pieces (rows are 16-byte aligned: cols is a multiple of 128), every piece of every row requested
@@ -200,7 +203,7 @@ __global__ void __launch_bounds__(256) lane16_bf16_wide_kernel(const uint16_t* _
     for (int i = 0; i < B; ++i) acc[i] = 0.f;
     for (int n0 = 0; n0 < nchunks; n0 += NB) {
 #pragma unroll
-        for (int n = 0; n < NB; ++n) *reinterpret_cast<uint4*>(mine + n * 256 + 16 * j) = raw[n];
+        for (int n = 0; n < NB; ++n) *reinterpret_cast<u32x4*>(mine + n * 256 + 16 * j) = raw[n];
         if (n0 + NB < nchunks) request(n0 + NB);
 #pragma unroll
         for (int n = 0; n < NB; ++n) {
@@ -275,7 +278,7 @@ static int32_t launch_lane16(const W& w, const XT* x, float* y, size_t rows, siz
             // A few rows of x against a small matrix (a router at the verify widths): a pass a row, all in one launch.
             // The matrix is re-read once a row out of L2, but every row's sums start at once, where passes of four
             // rows take four times the arithmetic each behind a fourfold staging (8 rows against the 128 x 2048
-            // router: 13.2 -> 8.6 us). A (row, vector) sum is the same chain of operations in every form.
+            // router: 13.2 -> 8.9 us). A (row, vector) sum is the same chain of operations in every form.
             if (b > 1 && b <= 16 && rows * cols <= (1u << 20)) {
                 done = launch_wide<1, 16>(w.w, x, y, rows, cols, 0, b, (unsigned)b, st);
                 if (done) b0 = b;
@@ -341,7 +344,7 @@ int32_t lane16_bf16_rows16(const uint16_t* w, size_t rows, size_t cols, const ui
 // a multiple of 128 columns or not 16-byte aligned, more than 256 experts, more passes than tickets) and unless the knob
 // moe_fused_router asks for it: the caller then uses the matvec and the routing kernel one after the other. Off by
 // default because it is no faster: inside a graph the routing kernel's launch costs less than the tail's fence,
-// ticket and barrier cost every workgroup of the matvec (Qwen3-30B-A3B router, one row: 32.8 us a layer against 31.2).
+// ticket and barrier cost every workgroup of the matvec (Qwen3-30B-A3B router, one row: 29.4 us a layer against 27.5).
 int32_t lane16_bf16_router16(const uint16_t* w, size_t rows, size_t cols, const uint16_t* x, size_t b, float* y,
                              int32_t* idx, uint16_t* wts, float* w32, uint16_t* logits16, int k, hipStream_t st) {
     if (!shape_ok(rows, cols, b)) return ERR_DOMAIN;
