@@ -10,6 +10,8 @@
 // The same loop serves every stored form through a policy (btb_widen.hpp semantics, vector forms here): the bytes a
 // lane loads are widened in its registers, never through a dequantised copy in memory.
 
+#include <type_traits>
+
 #include "btb_common.hpp"
 #include "btb_formats.hpp"
 #include "btb_stream.hpp"
@@ -155,14 +157,17 @@ static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void
     // of tiles (the last wave of the grid may walk fewer): tiles_per_wave is the smallest count that fits the cap.
     const int Rout = EPI == E_PLAIN ? R : R / 2;
     const int ntiles = (Rout + ROWS - 1) / ROWS;
+    auto kern = gemv_stream<F, M, LPR, RPW, U, XMODE, EPI>;
     int per_cu = tuning("gemv_wgs_per_cu");
-    if (per_cu <= 0) per_cu = 6;
+    // Six workgroups' worth of waves a CU, measured best for every form (more, smaller workgroups than are resident
+    // even out the grid's tail) but the pack12 form with the pair table, which does better cut for five - the head
+    // matvec [151936 x 2560] takes 97 us instead of 113, the packed step 2.194 ms instead of 2.213.
+    if (per_cu <= 0) per_cu = std::is_same<F, FmtP12L>::value ? 5 : 6;
     const int cap_waves = dev.cus * per_cu * 4;
     const int tiles_per_wave = (ntiles + cap_waves - 1) / cap_waves;
     const int waves = (ntiles + tiles_per_wave - 1) / tiles_per_wave;
     int grid = (waves + 3) / 4;
     if (grid < 1) grid = 1;
-    auto kern = gemv_stream<F, M, LPR, RPW, U, XMODE, EPI>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
