@@ -244,6 +244,49 @@ def test_gemv_p12_verify_width_many_escapes(card):
     check(y, oracle.gemv_bf16(bits16(w), x.float().numpy()))
 
 
+@pytest.mark.parametrize("R,C", [(6144, 2560), (2560, 9728), (512, 4096), (96, 272), (64, 1024)])
+@pytest.mark.parametrize("M,glu,wild", [(1, False, False), (1, True, False), (3, False, True), (2, True, True)])
+def test_packed_norm_forms_with_the_pair_table_change_no_bit(card, R, C, M, glu, wild):
+    """The add + norm matvecs over a pack12 matrix look the high bytes up in a 256-entry pair table in LDS; the plain
+    packed matvec does the lookup in registers. The widened weights are the same bf16 values and the sums run in the
+    same lane order, so: folded form == add_rmsnorm, then the plain packed matvec (then silu_mul), bit for bit; the
+    same with the table switched off (knob p12_pair_table = 0); and within the bar of the oracle's matvec over the
+    unpacked matrix. `wild`: high bytes spread over far more than fifteen values, a sixth of the weights escapes."""
+    g = torch.Generator().manual_seed(370 + R + M)
+    if wild:
+        w = (torch.randn(R, C, generator=g) * torch.exp2(torch.randint(-12, 4, (R, C), generator=g).float())).to(torch.bfloat16)
+    else:
+        w = weights_bf16(R, C, seed=371 + R)
+    pw = P12Weight.pack(w.cuda(), card)
+    if wild:
+        assert pw.esc_idx.numel() > R * C // 10
+    h = acts_bf16(M, C, seed=372).cuda()
+    y = acts_bf16(M, C, seed=373).cuda()
+    nw = (1.0 + 0.1 * torch.randn(C, generator=g)).to(torch.bfloat16).cuda()
+    h1, x1 = h.clone(), torch.empty_like(h)
+    card.add_rmsnorm(h1, y, nw, 1e-6, x1)
+    want = card.gemv_p12(pw, x1)
+    if glu:
+        half = torch.empty(M, R // 2, dtype=torch.bfloat16, device="cuda")
+        card.silu_mul(want, half)
+        want = half
+    outs = []
+    try:
+        for knob in (-1, 0):
+            card.set_tuning("p12_pair_table", knob)
+            h2 = torch.empty_like(h)
+            out = torch.empty(M, R // 2 if glu else R, dtype=torch.bfloat16, device="cuda")
+            card.gemv_norm(pw, h, y, nw, 1e-6, h2, out, glu=glu)
+            assert torch.equal(h2.view(torch.int16), h1.view(torch.int16))
+            outs.append(out)
+    finally:
+        card.set_tuning("p12_pair_table", -1)
+    assert torch.equal(outs[0].view(torch.int16), want.view(torch.int16))
+    assert torch.equal(outs[1].view(torch.int16), want.view(torch.int16))
+    if not glu:
+        check(outs[0], oracle.gemv_bf16(bits16(w), x1.float().cpu().numpy()))
+
+
 @pytest.mark.parametrize("packed", [False, True])
 def test_the_head_shape(card, packed):
     """the largest matrix of the step, the [151936, 2560] head (778 MB of bf16), stored as bf16 and as 12 bits a weight:
