@@ -187,6 +187,42 @@ def test_long_rows_straight_into_lds(card, form, block, M):
 
 
 @pytest.mark.parametrize("form", ["fp8", "mxfp4"])
+def test_long_rows_with_scales_of_every_size(card, form):
+    """the direct-to-LDS kernel's scales travel through LDS by loads of their own: random bytes under scales that differ
+    from block to block by factors up to 2^40 (MXFP4: e8m0 bytes 107..147; FP8: f32 scales 2^-20..2^20, a zero scale
+    and a negative one among them) against the oracle over the same bytes, at 16 rows and at 7 (one pass each)"""
+    R, C = 1024, 7168
+    rng = np.random.default_rng(380)
+    x = acts_bf16(16, C, seed=381)
+    if form == "fp8":
+        q = rng.integers(0, 256, (R, C), dtype=np.uint8)
+        q[(q & 0x7F) == 0x7F] = 0x3C  # no NaN bytes: e4m3fn has no infinities, 0x7F / 0xFF are its NaNs
+        sc = np.exp2(rng.integers(-20, 21, (R // 128, C // 128))).astype(np.float32) * rng.uniform(1.0, 2.0, (R // 128, C // 128)).astype(np.float32)
+        sc[1, 3] = 0.0
+        sc[2, 5] = -sc[2, 5]
+        w = fp8.F8Weight(torch.from_numpy(q).cuda(), torch.from_numpy(sc).cuda(), R, C)
+        ref = oracle.gemv_fp8(q, sc, x.float().numpy(), threads=0)
+        op = card.gemv_fp8
+    else:
+        blocks = rng.integers(0, 256, (R, C // 32, 16), dtype=np.uint8)
+        scales = rng.integers(107, 148, (R, C // 32), dtype=np.uint8)
+        w = mxfp4.MxWeight(torch.from_numpy(blocks).reshape(-1).cuda(), torch.from_numpy(scales).reshape(-1).cuda(), R, C)
+        ref = oracle.gemv_mxfp4(blocks, scales, R, C, x.float().numpy(), threads=0)
+        op = card.gemv_mx4
+    xg = x.cuda()
+    y = op(w, xg)
+    # weight rows of very different size: each weight row's sixteen outputs are held to 2^-6 of the largest of them
+    # (two bf16 ulps: the f32 sums run in another order than the oracle's, and blocks 2^40 apart cancel little)
+    got = y.float().cpu().numpy()
+    want = codecs.round_bf16(ref)
+    assert np.all(np.isfinite(want)) and np.all(np.isfinite(got))
+    peak = np.abs(want).max(axis=0, keepdims=True)  # per weight row, over the x rows
+    assert np.all(np.abs(got - want) <= 2.0**-6 * np.maximum(peak, 1e-30)), float((np.abs(got - want) / np.maximum(peak, 1e-30)).max())
+    y7 = op(w, xg[:7].contiguous())
+    assert torch.equal(y7.view(torch.int16), y[:7].view(torch.int16))
+
+
+@pytest.mark.parametrize("form", ["fp8", "mxfp4"])
 def test_full_shape_one_row_and_linearity(card, form):
     """C5 at M = 1 on the full [18432, 7168] matrix against the oracle, and a size-independent property on top: the
     matvec is linear in x up to the output's rounding - y(x1) + y(x2) against y over the f32 sum, each within the bar"""
