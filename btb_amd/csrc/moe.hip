@@ -262,7 +262,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
 // gathered rows of x a pass, where the kernel above streams them once a pair. The workgroups of the later pairs leave
 // before asking memory for anything. A product is a row of x against a row of weights in the lane order above, so
 // each h row has the bits the kernel above gives it. n = T k <= GROUP_MAX_PAIRS.
-constexpr int GROUP_MAX_PAIRS = 1024;
+constexpr int GROUP_MAX_PAIRS = 256;
 template <int LPR, int RPW, int U, int MC>
 __global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* __restrict__ stack,
                                                                   const uint16_t* __restrict__ x,
@@ -270,49 +270,54 @@ __global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* _
                                                                   int R, int C, int k, int E, int n) {
     static_assert(RPW == 2, "gate and up");
     extern __shared__ __align__(16) uint32_t xs[];  // [MC][C / 2]
-    __shared__ int s_pairs[GROUP_MAX_PAIRS];        // the expert's pairs, ascending
-    __shared__ unsigned long long s_mask[GROUP_MAX_PAIRS / WAVE];
     using F = FmtBf16;
     constexpr int G = WAVE / LPR, ROWS = G;
+    constexpr int NM = GROUP_MAX_PAIRS / WAVE;  // ballots that cover the pairs
     const int pair = blockIdx.y;
     auto clamp = [E](int v) { return v < 0 ? 0 : (v >= E ? E - 1 : v); };
-    const int expert = clamp(idx[pair]);
     const int tid = threadIdx.x, lane = tid & (WAVE - 1), sl = lane % LPR, wv = tid / WAVE;
-    // which pairs picked this expert: 64 pairs a ballot, the ballots side by side in LDS
-    for (int q0 = wv * WAVE; q0 < n; q0 += 4 * WAVE) {
-        const int q = q0 + lane;
-        const bool hit = q < n && clamp(idx[q]) == expert;
-        const unsigned long long m = __ballot(hit);
-        if (lane == 0) s_mask[q0 / WAVE] = m;
-    }
-    __syncthreads();
+    // Which pairs picked this pair's expert: every wave finds out for itself - a lane a pair, 64 pairs a ballot, the
+    // picks asked for together with the pair's own - so there is nothing to exchange and no barrier, and the scan
+    // costs the one trip to the picks that the kernel above makes for its expert anyway.
+    const int own = idx[pair];
+    int picks[NM];
+#pragma unroll
+    for (int i = 0; i < NM; ++i) picks[i] = idx[min(i * WAVE + lane, n - 1)];
+    const int expert = clamp(own);
+    unsigned long long mask[NM];
+#pragma unroll
+    for (int i = 0; i < NM; ++i)
+        mask[i] = i * WAVE < n ? __ballot(i * WAVE + lane < n && clamp(picks[i]) == expert) : 0ull;
     // an earlier pair of the same expert does the work
     {
-        bool earlier = false;
-        for (int b = 0; b * WAVE <= pair; ++b) {
-            unsigned long long m = s_mask[b];
-            if (b == pair / WAVE) m &= (1ull << (pair % WAVE)) - 1ull;
-            earlier |= m != 0ull;
+        unsigned long long earlier = 0ull;
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            unsigned long long m = mask[i];
+            if (i == pair / WAVE) m &= (1ull << (pair % WAVE)) - 1ull;
+            if (i > pair / WAVE) m = 0ull;
+            earlier |= m;
         }
-        if (earlier) return;  // uniform: every thread sees the same masks
+        if (earlier != 0ull) return;  // uniform
     }
     int rows_n = 0;
-    {
-        const int nb = (n + WAVE - 1) / WAVE;
-        for (int b = 0; b < nb; ++b) {
-            const unsigned long long m = s_mask[b];
-            if (tid == 0) {
-                unsigned long long r = m;
-                int at = rows_n;
-                while (r) {
-                    s_pairs[at++] = b * WAVE + __builtin_ctzll(r);
-                    r &= r - 1;
-                }
+#pragma unroll
+    for (int i = 0; i < NM; ++i) rows_n += __builtin_popcountll(mask[i]);
+    // the r-th of the expert's pairs, ascending (uniform arithmetic on the ballots)
+    auto pair_of = [&](int r) {
+        int found = 0;
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            unsigned long long m = mask[i];
+            const int c = __builtin_popcountll(m);
+            if (r >= 0 && r < c) {
+                for (int q = 0; q < r; ++q) m &= m - 1ull;
+                found = i * WAVE + __builtin_ctzll(m);
             }
-            rows_n += __builtin_popcountll(m);
+            r -= c;
         }
-    }
-    __syncthreads();
+        return found;
+    };
 
     const int units = C / F::UW;
     const int wave = blockIdx.x * (blockDim.x / WAVE) + wv;
@@ -338,9 +343,14 @@ __global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* _
         }
         if (r0 != 0) __syncthreads();  // the previous pass has read its rows
         // the pass's rows of x, a row past the last being the last again (its sums are dropped)
+        int prs[M];
+#pragma unroll
+        for (int m = 0; m < M; ++m) prs[m] = pair_of(r0 + min(m, mc - 1));
         for (int i = tid; i < M * per; i += 256) {
             const int m = i / per, c = i - m * per;
-            const int tok = s_pairs[r0 + min(m, mc - 1)] / k;
+            int tok = prs[0] / k;
+#pragma unroll
+            for (int m2 = 1; m2 < M; ++m2) tok = m == m2 ? prs[m2] / k : tok;
             xd[i] = reinterpret_cast<const uint4*>(x + (size_t)tok * C)[c];
         }
         __syncthreads();
@@ -377,7 +387,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* _
                 const float g = bfround(group_sum<LPR>(acc[0][m]));
                 const float u = bfround(group_sum<LPR>(acc[1][m]));
                 if (sl == 0 && rows[0] < I && m < mc)
-                    h[(size_t)s_pairs[r0 + m] * I + rows[0]] = f32_bf16(bfround(g / (1.f + expf(-g))) * u);
+                    h[(size_t)prs[m] * I + rows[0]] = f32_bf16(bfround(g / (1.f + expf(-g))) * u);
             }
         }
     };
@@ -524,9 +534,12 @@ static int32_t launch_gate_up(const void* stack, const void* x, const int32_t* i
     const int ntiles = (R / 2 + G - 1) / G;
     const int grid = (ntiles + 3) / 4;
     // From eight rows on, the rows that share an expert go through it together. Fewer rows share few experts (4 rows of
-    // top-8 over 128 experts: 30 distinct of 32 picks) and the gathering costs more than it saves: measured on the
-    // Qwen3-30B-A3B shape, a layer takes 74 against 72 us at 4 rows, 117 against 119 at 8, 190 against 208 at 16, 310
-    // against 384 at 32. The knob moe_grouped forces either (1 / 0).
+    // top-8 over 128 experts: 30 distinct of 32 picks) and the wider pass costs more than the sharing saves: measured on
+    // the Qwen3-30B-A3B shape, a layer takes 64 against 62 us at 4 rows, 88 against 86 at 6, 106 against 109 at 8, 180
+    // against 198 at 16, 295 against 374 at 32. The knob moe_grouped forces either (1 / 0). Asking for the expert's
+    // first rows before the pairs are sorted out - as the pair kernel does - was tried and loses (8 rows: 122 us): a
+    // wave's first span is its whole share of the expert, so the later pairs of a shared expert ask for everything
+    // they then drop.
     constexpr int MC = 4;
     const int grouped = tuning("moe_grouped");
     const bool wanted = grouped >= 0 ? grouped != 0 && pairs > k : pairs >= 8 * k;
