@@ -28,6 +28,8 @@
 // differs (see the kernel), so the two kernels agree to f32 summation order, not to the bit. Every M of a pass takes
 // the same path here, so a row of x gets the same bits whatever the other rows of the pass are.
 
+#include <type_traits>
+
 #include "btb_common.hpp"
 #include "btb_formats.hpp"
 #include "btb_tuning.hpp"
@@ -66,6 +68,41 @@ __device__ __forceinline__ void wait_behind(int behind, uint32_t& a, uint32_t& b
     else
         wait_loads<0>(a, b);
 }
+// the same with the full MAXB sub-blocks behind and, behind them too, `xparts` (0..6) parts of x of XL loads each
+template <int LOADS, int MAXB, int XL>
+__device__ __forceinline__ void wait_lead(int xparts, uint32_t& a, uint32_t& b) {
+    constexpr int BASE = MAXB * LOADS;
+    auto imm = [](int n) constexpr { return BASE + n * XL < 64 ? BASE + n * XL : 0; };
+    if (xparts == 6)
+        wait_loads<imm(6)>(a, b);
+    else if (xparts == 5)
+        wait_loads<imm(5)>(a, b);
+    else if (xparts == 4)
+        wait_loads<imm(4)>(a, b);
+    else if (xparts == 3)
+        wait_loads<imm(3)>(a, b);
+    else if (xparts == 2)
+        wait_loads<imm(2)>(a, b);
+    else if (xparts == 1)
+        wait_loads<imm(1)>(a, b);
+    else
+        wait_loads<BASE>(a, b);
+}
+
+// A 16-byte load whose being outstanding the compiler does not know of, and the statement that says "these four have
+// landed" (it follows the counted wait that makes it true). The compiler's own wait for a loaded register is exact
+// only while no direct-to-LDS load is outstanding: those are FLAT-encoded instructions that name LDS, after which it
+// takes the order of returns to be unknown and waits for every load there is, the ring's included. The kernel's first
+// tile wants its part of x and nothing younger, so x comes through these two where that tile is on its own straight
+// path. Between the two statements the registers are named by nothing else.
+__device__ __forceinline__ u32x4 load_untracked(const u32x4* p) {
+    u32x4 v;
+    asm volatile("global_load_dwordx4 %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ void landed(u32x4& a, u32x4& b, u32x4& c, u32x4& d) {
+    asm volatile("" : "+v"(a), "+v"(b), "+v"(c), "+v"(d));
+}
 
 // the slot's data: column block gb of 128 bytes at gb * BLK, rows 8..15 of it HALF further on
 constexpr int HALF = 1024 + 128;
@@ -85,17 +122,17 @@ struct DlF8 {
         int bm;  // rows per block (a multiple of 16: a tile's sixteen rows share their scales)
         int bn;  // columns per block (a multiple of 32: a step lies in one block)
     };
-    __host__ __device__ static constexpr int scale_bytes(int sbs) { return (4 * sbs + 15) / 16 * 16; }
+    __host__ __device__ static constexpr int scale_bytes(int /*sbs*/) { return 4 * WAVE; }
     __host__ __device__ static constexpr int scale_words(int sbs) { return sbs; }
-    // lane t < SBS brings the scale of the sub-block's step t: f32 [SBS] in the scale area
+    // lane t brings the scale of the sub-block's step min(t, SBS - 1): f32 [64] in the scale area, the first SBS of
+    // them read. Every lane loads, so that there is no branch round the instruction: the compiler counts the loads
+    // outstanding exactly only through straight-line code, and the kernel's first tile depends on that.
     template <int SBS>
     __device__ static __forceinline__ void issue_scales(const Mat& m, int tile, int /*nsteps*/, int step0, uint8_t* dst,
                                                         int lane) {
         static_assert(SBS <= 64, "a lane a step");
-        if (lane < SBS) {
-            const float* srow = m.scales + (size_t)(tile * 16 / m.bm) * m.sc;
-            __builtin_amdgcn_global_load_lds(srow + (step0 + lane) * 32 / m.bn, (lds_void*)dst, 4, 0, 0);
-        }
+        const float* srow = m.scales + (size_t)(tile * 16 / m.bm) * m.sc;
+        __builtin_amdgcn_global_load_lds(srow + (step0 + min(lane, SBS - 1)) * 32 / m.bn, (lds_void*)dst, 4, 0, 0);
     }
     // where in a slot's data the lane's reads start (row li, 8-column group lg), and what step t adds to that
     __device__ static __forceinline__ uint32_t lane_off(int li, int lg) {
@@ -136,7 +173,7 @@ struct DlMx4 {
                                                         int lane) {
         static_assert(SBS % 4 == 0 && 4 * SBS <= 64, "whole words of scale bytes, a lane a word");
         constexpr int per = SBS / 4;
-        if (lane < 16 * per) {
+        if (16 * per == WAVE || lane < 16 * per) {  // no branch where every lane has a word (the first tile relies on it)
             const int r = lane / per, j = lane - r * per;
             __builtin_amdgcn_global_load_lds(m.scales + (size_t)(tile * 16 + r) * nsteps + step0 + 4 * j, (lds_void*)dst,
                                              4, 0, 0);
@@ -189,11 +226,20 @@ template <class DF, int SPW, int GB, int SBS, int NBUF>
 __device__ __forceinline__ f32x4 sub_block(const typename DF::Mat& mat, const uint8_t* __restrict__ cur,
                                            uint8_t* __restrict__ fill, bool do_fill, int fill_tile, int fill_step0,
                                            int nsteps, size_t rowbytes, int lane, int li, int lg, int behind, int sb,
-                                           const uint4 (&xb)[SPW], f32x4 acc) {
+                                           u32x4 (&xb)[SPW], f32x4 acc, int xparts = -1) {
     if (do_fill) issue_loads<DF, GB, SBS>(mat, fill, fill_tile, fill_step0, nsteps, rowbytes, lane);
     // `cur` has landed once at most the loads issued behind it are outstanding
     uint32_t roff = DF::lane_off(li, lg), soff = DF::scale_off(li, SBS);
-    wait_behind<2 * GB + 1, NBUF - 1>(behind, roff, soff);
+    // xparts >= 0: the kernel's first tile - the full NBUF - 1 sub-blocks are behind this one, and so are that many of
+    // the parts of x (SBS loads each)
+    if (xparts >= 0) {
+        static_assert(SBS % 4 == 0, "parts of x in fours");
+        wait_lead<2 * GB + 1, NBUF - 1, SBS>(xparts, roff, soff);
+#pragma unroll
+        for (int t = 0; t < SBS; t += 4)
+            landed(xb[sb * SBS + t], xb[sb * SBS + t + 1], xb[sb * SBS + t + 2], xb[sb * SBS + t + 3]);
+    } else
+        wait_behind<2 * GB + 1, NBUF - 1>(behind, roff, soff);
     __builtin_amdgcn_sched_barrier(0);
     const uint8_t* rowp = cur + roff;
     uint32_t ew[DF::scale_words(SBS)];  // what the lane needs of the sub-block's scales
@@ -239,7 +285,13 @@ __device__ __forceinline__ void fold_tile(f32x4* __restrict__ mine, f32x4 acc, i
 // KS waves a workgroup, each the owner of SPW steps of every row (C = 32 KS SPW); GB 128-byte column blocks a
 // sub-block; NBUF ring slots a wave. A tile is MAXSB sub-blocks; the tile loop's body covers a multiple of
 // NBUF of them, so every sub-block's slot is a compile-time number. One tile of up to sixteen x rows.
-template <class DF, int KS, int SPW, int GB, int NBUF>
+//
+// LEAD is set by the host when every workgroup has tiles enough that each sub-block of its first tile still has its full
+// NBUF - 1 sub-blocks asked for behind it: the first tile is then straight-line code with nothing conditional in it (the
+// compiler counts the loads outstanding exactly only through such code; with a branch round any of them, or this choice
+// made inside the kernel, it falls back to waiting for all of them), and its waits let the parts of x asked for behind a
+// sub-block's own stay outstanding as well.
+template <class DF, int KS, int SPW, int GB, int NBUF, bool LEAD>
 __global__ void __launch_bounds__(KS * 64) gemv_mfma_dl(typename DF::Mat mat, const uint4* __restrict__ x,
                                                         uint16_t* __restrict__ y, int R, int C, int M) {
     constexpr int SBS = GB * 128 / DF::STEPB;  // steps a sub-block
@@ -247,7 +299,8 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_dl(typename DF::Mat mat, co
     constexpr int MAXSB = SPW / SBS;
     constexpr int TPB = MAXSB >= NBUF ? 1 : NBUF / MAXSB;  // tiles a loop body covers
     static_assert(SPW % SBS == 0 && SLOT % 16 == 0 && (SPW * DF::STEPB) % 128 == 0, "shape");
-    static_assert(NBUF >= 2 && NBUF <= 7, "ring depth");
+    static_assert(NBUF >= 2 && NBUF <= 7 && MAXSB <= 7, "ring depth; at most six parts of x behind a sub-block");
+    static_assert((NBUF - 1) * (2 * GB + 1) + (MAXSB - 1) * SBS < 64, "the first tile's waits count up to 63 loads");
     static_assert((MAXSB >= NBUF && MAXSB % NBUF == 0) || (MAXSB < NBUF && NBUF % MAXSB == 0), "slots by position");
     extern __shared__ __align__(16) uint8_t lds[];  // KS rings of NBUF slots, then two sets of KS partial tiles
     const int lane = threadIdx.x & (WAVE - 1);
@@ -269,22 +322,34 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_dl(typename DF::Mat mat, co
     const int grid = (int)gridDim.x, first = (int)blockIdx.x;
     const int nt = first < ntiles ? (ntiles - first + grid - 1) / grid : 0;  // this workgroup's tiles
     const int total = nt * MAXSB;                                            // and the wave's sub-blocks
-    // sub-block q of the wave: tile first + (q / MAXSB) grid, steps (q % MAXSB) SBS .. of the wave's slice, slot q % NBUF
+    // sub-block q of the wave: tile first + (q / MAXSB) grid, steps (q % MAXSB) SBS .. of the wave's slice, slot q % NBUF.
+    //
+    // The x fragments of the wave's steps stay in registers for the whole kernel (row li of x, the lane's 8 columns of
+    // each step); part j of them - SBS loads - is what sub-block j of any tile multiplies by. They and the ring's first
+    // loads are asked for in the order the first tile uses them: x part 0, sub-block 0, x part 1, sub-block 1, ...
+    // Loads come back in that order, so the first tile's sub-block j can start as soon as its own weights and its own
+    // part of x are there, the later parts still on their way out of L2 (every CU reads all of x, 115 KB at 8 rows,
+    // and all at once: asked for and waited for in one piece it held the first product back by 2.7 us per 8 rows).
+    u32x4 xb[SPW];
+    const u32x4* xr = reinterpret_cast<const u32x4*>(x) + (size_t)min(li, M - 1) * chunk4 + lg + (size_t)s0 * 4;
 #pragma unroll
-    for (int q = 0; q < NBUF - 1; ++q) {
-        if (q < total)
-            issue_loads<DF, GB, SBS>(mat, ring + (q % NBUF) * SLOT, first + (q / MAXSB) * grid,
-                                     s0 + (q % MAXSB) * SB_STEP, nsteps, rowbytes, lane);
-    }
-    // The x fragments of the wave's steps, for the whole kernel (row li of x, the lane's 8 columns of each step): asked
-    // for behind the ring's first loads, so the weights are on their way from memory while x comes out of L2.
-    uint4 xb[SPW];
-    {
-        const uint4* xr = x + (size_t)min(li, M - 1) * chunk4 + lg + (size_t)s0 * 4;
+    for (int q = 0; q < (NBUF - 1 > MAXSB ? NBUF - 1 : MAXSB); ++q) {
+        if (q < MAXSB) {
 #pragma unroll
-        for (int i = 0; i < SPW; ++i) xb[i] = xr[((i / SBS) * SB_STEP + i % SBS) * 4];
+            for (int t = 0; t < SBS; ++t)
+                xb[q * SBS + t] = LEAD ? load_untracked(xr + (q * SB_STEP + t) * 4) : xr[(q * SB_STEP + t) * 4];
+            __builtin_amdgcn_sched_barrier(0);  // issued here, not where the scheduler would like them
+        }
+        if (q < NBUF - 1) {
+            if (LEAD || q < total)
+                issue_loads<DF, GB, SBS>(mat, ring + (q % NBUF) * SLOT, first + (q / MAXSB) * grid,
+                                         s0 + (q % MAXSB) * SB_STEP, nsteps, rowbytes, lane);
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
-    for (int k0 = 0; k0 < nt; k0 += TPB) {
+    // one body of the tile loop: TPB tiles; FIRST: the kernel's first body under LEAD
+    auto body = [&](int k0, auto first_tag) {
+        constexpr bool FIRST = decltype(first_tag)::value;
 #pragma unroll
         for (int kk = 0; kk < TPB; ++kk) {
             const int k = k0 + kk;
@@ -297,15 +362,29 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_dl(typename DF::Mat mat, co
                     // compile-time slots: q % NBUF = (kk * MAXSB + sb) % NBUF, because the body covers a multiple of NBUF
                     const int cur_slot = (kk * MAXSB + sb) % NBUF, fill_slot = (kk * MAXSB + sb + NBUF - 1) % NBUF;
                     const int qf = q + NBUF - 1;  // the sub-block asked for now, into the slot the previous one left
-                    const int behind = min(NBUF - 1, total - 1 - q);
-                    acc = sub_block<DF, SPW, GB, SBS, NBUF>(
-                        mat, ring + cur_slot * SLOT, ring + fill_slot * SLOT, qf < total, first + (qf / MAXSB) * grid,
-                        s0 + (qf % MAXSB) * SB_STEP, nsteps, rowbytes, lane, li, lg, behind, sb, xb, acc);
+                    if (FIRST && kk == 0) {
+                        // x parts sb + 1 .. MAXSB - 1 were asked for behind this sub-block's weights and its part of x
+                        acc = sub_block<DF, SPW, GB, SBS, NBUF>(
+                            mat, ring + cur_slot * SLOT, ring + fill_slot * SLOT, true, first + (qf / MAXSB) * grid,
+                            s0 + (qf % MAXSB) * SB_STEP, nsteps, rowbytes, lane, li, lg, NBUF - 1, sb, xb, acc,
+                            MAXSB - 1 - sb);
+                    } else {
+                        const int behind = min(NBUF - 1, total - 1 - q);
+                        acc = sub_block<DF, SPW, GB, SBS, NBUF>(
+                            mat, ring + cur_slot * SLOT, ring + fill_slot * SLOT, qf < total, first + (qf / MAXSB) * grid,
+                            s0 + (qf % MAXSB) * SB_STEP, nsteps, rowbytes, lane, li, lg, behind, sb, xb, acc);
+                    }
                 }
                 fold_tile<KS>(part + (size_t)(k & 1) * KS * WAVE, acc, wv, lane, li, lg, M, R, tile, y);
             }
         }
+    };
+    int k0 = 0;
+    if (LEAD) {
+        body(0, std::true_type{});
+        k0 = TPB;
     }
+    for (; k0 < nt; k0 += TPB) body(k0, std::false_type{});
 }
 
 template <class DF, int KS, int SPW, int GB, int NBUF>
@@ -320,7 +399,9 @@ static int32_t launch_dl(const typename DF::Mat& mat, const void* x, void* y, in
     const int cap = device_info().cus;  // the rings take most of a CU's LDS: one workgroup a CU
     const int turns = (ntiles + cap - 1) / cap;
     const int grid = (ntiles + turns - 1) / turns;
-    auto kern = gemv_mfma_dl<DF, KS, SPW, GB, NBUF>;
+    constexpr int MAXSB = SPW / (GB * 128 / DF::STEPB);
+    const bool lead = (ntiles / grid) * MAXSB >= MAXSB + NBUF - 1;  // the workgroup with the fewest tiles has enough
+    auto kern = lead ? gemv_mfma_dl<DF, KS, SPW, GB, NBUF, true> : gemv_mfma_dl<DF, KS, SPW, GB, NBUF, false>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
