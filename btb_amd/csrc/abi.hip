@@ -70,6 +70,7 @@ static Knob g_knobs[] = {
     {"mfma_lds", {-1}},
     {"mfma_stream_x", {-1}},
     {"mfma_direct", {-1}},
+    {"mfma_direct_grid", {-1}},
     {"p12_pair_table", {-1}},
     {"moe_wgs_per_cu", {-1}},
     {"moe_grouped", {-1}},

@@ -296,6 +296,11 @@ int32_t gemv_mfma_dl_fp8(const void* w, const float* scales, int sc, int bm, int
                          int C, int M, hipStream_t st);
 int32_t gemv_mfma_dl_mxfp4(const void* blocks, const void* scales, const void* x, void* y, int R, int C, int M,
                            hipStream_t st);
+// and for pack12 rows of the lengths it has shapes for
+bool mfma_dl_fits_p12(int R, int C, int M);
+int32_t gemv_mfma_dl_p12(const uint8_t* lo, const uint8_t* hi4, const uint8_t* table, const int32_t* esc_idx,
+                         const uint8_t* esc_val, const int32_t* row_ptr, const void* x, void* y, int R, int C, int M,
+                         hipStream_t st);
 
 // whether a pass of M rows goes to the matrix cores through the LDS-staged kernel
 static bool wide_pass(size_t M, size_t R, size_t C, bool packed) {
@@ -449,7 +454,21 @@ int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, con
     rc = p12_params(lo, hi4, table, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
     if (rc != OK) return rc;
     if (!aligned16(x) || !aligned2(y)) return ERR_DOMAIN;
-    if (wide_pass(M, R, C, true) && aligned16(hi4)) {  // the verify widths: the matrix cores, 32 rows of x a pass
+    // the verify widths: the matrix cores. Weights straight into LDS, 16 rows of x a pass, where that kernel has a
+    // shape for the row length
+    if (wide_pass(M, R, C, true) && aligned16(hi4) && aligned16(lo) && (reinterpret_cast<uintptr_t>(table) & 3u) == 0 &&
+        mfma_dl_fits_p12((int)R, (int)C, 16)) {
+        const uint16_t* xp = static_cast<const uint16_t*>(x);
+        uint16_t* yp = static_cast<uint16_t*>(y);
+        for (size_t m0 = 0; m0 < M; m0 += 16) {
+            const int mm = (int)(M - m0 < 16 ? M - m0 : 16);
+            rc = gemv_mfma_dl_p12(p.lo, p.hi4, p.table, p.esc_idx, p.esc_val, p.row_ptr, xp + m0 * C, yp + m0 * R, (int)R,
+                                  (int)C, mm, static_cast<hipStream_t>(stream));
+            if (rc != OK) return rc;
+        }
+        return OK;
+    }
+    if (wide_pass(M, R, C, true) && aligned16(hi4)) {  // through registers and LDS, 32 rows of x a pass
         const uint16_t* xp = static_cast<const uint16_t*>(x);
         uint16_t* yp = static_cast<uint16_t*>(y);
         for (size_t m0 = 0; m0 < M; m0 += 32) {
