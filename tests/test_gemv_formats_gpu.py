@@ -186,6 +186,40 @@ def test_long_rows_straight_into_lds(card, form, block, M):
     assert torch.equal(op(w, xg).view(torch.int16), y.view(torch.int16))  # and the same bits every time
 
 
+@pytest.mark.parametrize("R,C", [(9728, 2560), (320, 4096), (208, 9728), (256, 3200), (144, 9216), (96, 10752)])
+@pytest.mark.parametrize("M,crowd", [(5, False), (16, False), (21, True)])
+def test_packed_rows_straight_into_lds(card, R, C, M, crowd):
+    """12-bit rows of the lengths the direct-to-LDS kernel has shapes for - 2560 (ten waves), 3073..4096 (eight) and
+    9217..10752 columns (seven, sub-blocks of 256 columns); 3200, 9216 and 9728 leave some waves without a last
+    sub-block - at the verify widths: against the oracle, against the staged kernel it replaces (knob mfma_direct = 0;
+    the two differ in f32 summation order only), a row's bits whatever pass it came with, the same bits every time.
+    `crowd`: high bytes spread over far more than fifteen values, so that a tile's escapes are many times the
+    thirty-two its escape wave takes at once; otherwise the natural handful, with tiles that have none."""
+    g = torch.Generator().manual_seed(390 + M)
+    if crowd:
+        w = (torch.randn(R, C, generator=g) * torch.exp2(torch.randint(-12, 4, (R, C), generator=g).float())).to(torch.bfloat16)
+    else:
+        w = weights_bf16(R, C, seed=391)
+    pw = P12Weight.pack(w.cuda(), card)
+    assert (pw.esc_idx.numel() > R * C // 10) if crowd else (0 < pw.esc_idx.numel() < R * C // 100)
+    x = acts_bf16(M, C, seed=392)
+    ref = oracle.gemv_bf16(bits16(w), x.float().numpy())  # the packed matrix is the bf16 matrix, bit for bit
+    xg = x.cuda()
+    y = card.gemv_p12(pw, xg)
+    check(y, ref)
+    card.set_tuning("mfma_direct", 0)
+    try:
+        staged = card.gemv_p12(pw, xg)
+    finally:
+        card.set_tuning("mfma_direct", -1)
+    check(staged, ref)
+    peak = float(y.float().abs().max())
+    assert float((staged.float() - y.float()).abs().max()) <= peak * 2.0**-7
+    last = card.gemv_p12(pw, xg[M - 5:].contiguous())
+    assert torch.equal(last.view(torch.int16), y[M - 5:].view(torch.int16))
+    assert torch.equal(card.gemv_p12(pw, xg).view(torch.int16), y.view(torch.int16))
+
+
 @pytest.mark.parametrize("form", ["fp8", "mxfp4"])
 def test_long_rows_with_scales_of_every_size(card, form):
     """the direct-to-LDS kernel's scales travel through LDS by loads of their own: random bytes under scales that differ
