@@ -464,4 +464,37 @@ __device__ __forceinline__ void merge_spans(uint16_t* out, int g, int S, size_t 
     }
 }
 
+// What row t of a pass sees. A chain of rows (par null): the cache's keys and the pass's rows up to itself. A tree
+// (par[t] the row's parent among the pass's rows, -1 at a root; the reference's TREE form,
+// native/cuda/btb_attn_flash.cuh:284-286, 407-419): the cache's keys, and of the pass's rows - slots n0 .. n0 + T - 1 -
+// its ancestors and itself.
+struct RowView {
+    int n;               // one past the last slot the row may see
+    int tree_base;       // -1 for a chain; else the first of the pass's own slots
+    uint32_t tree_mask;  // the pass's rows the row sees (a tree)
+    int k_first;         // the window's first key (0: no window)
+};
+__device__ __forceinline__ RowView row_view(const int32_t* __restrict__ par, int t, int T, int n0, int win) {
+    RowView v;
+    v.tree_base = -1;
+    v.tree_mask = 0u;
+    v.n = n0 + t + 1;
+    int last = n0 + t;  // the row's own logical position: a chain's row t stands at n0 + t, a tree's at n0 + its depth
+    if (par != nullptr) {
+        v.tree_base = n0;
+        v.n = n0 + T;
+        int depth = -1;
+        for (int p = t, hops = 0; p >= 0 && p < T && hops < 32; p = par[p], ++hops) ++depth;
+        last = n0 + depth;
+        // the row's keys among the pass's rows: itself and its ancestors, the one at depth d standing at n0 + d - under
+        // a window (the reference's `first = last + 1 - win`, native/cuda/btb_attn_flash.cuh:437) those at or past it
+        const int first_depth = win > 0 ? last + 1 - win - n0 : 0;
+        int d = depth;
+        for (int p = t, hops = 0; p >= 0 && p < T && hops < 32; p = par[p], ++hops, --d)
+            if (d >= first_depth) v.tree_mask |= 1u << p;
+    }
+    v.k_first = win > 0 ? max(last + 1 - win, 0) : 0;
+    return v;
+}
+
 }  // namespace btb

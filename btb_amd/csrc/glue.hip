@@ -216,39 +216,12 @@ __global__ void __launch_bounds__(64) norm_rope_kv_kernel(const uint16_t* __rest
 constexpr int ATT_D = 128;
 constexpr int ATT_MAXG = 8;
 constexpr int ATT_MAX_STATES = 1024;  // (span, head) states of one kv head that merge_spans turns into factors
-
-// What row t of a pass sees. A chain of rows (par null): the cache's keys and the pass's rows up to itself. A tree
-// (par[t] the row's parent among the pass's rows, -1 at a root; the reference's TREE form,
-// native/cuda/btb_attn_flash.cuh:284-286, 407-419): the cache's keys, and of the pass's rows - slots n0 .. n0 + T - 1 -
-// its ancestors and itself.
-struct RowView {
-    int n;               // one past the last slot the row may see
-    int tree_base;       // -1 for a chain; else the first of the pass's own slots
-    uint32_t tree_mask;  // the pass's rows the row sees (a tree)
-    int k_first;         // the window's first key (0: no window)
-};
-__device__ __forceinline__ RowView row_view(const int32_t* __restrict__ par, int t, int T, int n0, int win) {
-    RowView v;
-    v.tree_base = -1;
-    v.tree_mask = 0u;
-    v.n = n0 + t + 1;
-    int last = n0 + t;  // the row's own logical position: a chain's row t stands at n0 + t, a tree's at n0 + its depth
-    if (par != nullptr) {
-        v.tree_base = n0;
-        v.n = n0 + T;
-        int depth = -1;
-        for (int p = t, hops = 0; p >= 0 && p < T && hops < 32; p = par[p], ++hops) ++depth;
-        last = n0 + depth;
-        // the row's keys among the pass's rows: itself and its ancestors, the one at depth d standing at n0 + d - under
-        // a window (the reference's `first = last + 1 - win`, native/cuda/btb_attn_flash.cuh:437) those at or past it
-        const int first_depth = win > 0 ? last + 1 - win - n0 : 0;
-        int d = depth;
-        for (int p = t, hops = 0; p >= 0 && p < T && hops < 32; p = par[p], ++hops, --d)
-            if (d >= first_depth) v.tree_mask |= 1u << p;
-    }
-    v.k_first = win > 0 ? max(last + 1 - win, 0) : 0;
-    return v;
-}
+// the pass of several rows on the matrix cores (attn_mfma.hip): the partial states of every (row, head, span)
+bool attn_mfma_fits(size_t T, size_t G, int span);
+int32_t attn_decode_mfma(const void* q, const void* K, const void* V, const int32_t* n0, const int32_t* par, size_t T,
+                         size_t Hq, size_t Hk, long long hs, long long rs, float scale_log2, float* part_m,
+                         float* part_l, float* part_acc, size_t S, size_t cap, int win, const int32_t* tbl,
+                         hipStream_t st);
 
 template <int G>
 __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ K,
@@ -740,6 +713,21 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
     // with four, 4.23 with eight: the rows of a workgroup run one after another, each with its own fold of the 16
     // streams, which costs more than the other rows' workgroups reading the same keys out of L2 (the keys leave memory
     // once either way). Against attn_decode_kernel at its best span count the pass takes 3.67 instead of 3.83 ms.
+    // Several rows and spans of 128 keys: the matrix cores, every row of the pass that shares a kv head in one workgroup
+    // (attn_mfma.hip). A pass of 8 rows over 4096 keys: 22.7 us a layer on the vector kernel below, which stays for
+    // spans of 256 keys and behind the knob attn_mfma = 0.
+    if (attn_mfma_fits(T, G, span)) {
+        const int32_t rc = attn_decode_mfma(q, K, V, n0, par, T, Hq, Hk, (long long)hs, (long long)rs, scale_log2, part_m,
+                                            part_l, part_acc, S, cap, (int)win, tbl, st);
+        if (rc != OK) return rc;
+        if (G == 4)
+            hipLaunchKernelGGL(attn_merge_kernel<4>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
+                               (int)Hk, (int)S, part_m, part_l, part_acc);
+        else
+            hipLaunchKernelGGL(attn_merge_kernel<2>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
+                               (int)Hk, (int)S, part_m, part_l, part_acc);
+        return hip_status(hipGetLastError(), "attn_decode launch");
+    }
     const int rows_knob = tuning("attn_rows_per_wg");
     if (T >= 2 && (span == 128 || span == 256) && (G == 2 || G == 4) && rows_knob != 0) {
         int rpw = rows_knob > 0 ? rows_knob : 1;

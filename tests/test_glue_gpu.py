@@ -159,6 +159,7 @@ def test_attn_short_spans_kept_in_registers(card, n0, T, Hq, Hk, S, tree, win):
     n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
     scale = 1.0 / np.sqrt(D)
     outs = {}
+    card.set_tuning("attn_mfma", 0)  # the vector-ALU kernels: the matrix-core form has a test of its own below
     try:
         for knob in (-1, 0, 2, 3, T):
             card.set_tuning("attn_rows_per_wg", knob)
@@ -167,6 +168,7 @@ def test_attn_short_spans_kept_in_registers(card, n0, T, Hq, Hk, S, tree, win):
             outs[knob] = att.clone()
     finally:
         card.set_tuning("attn_rows_per_wg", -1)
+        card.set_tuning("attn_mfma", -1)
     for knob, a in outs.items():
         assert torch.equal(a, outs[-1]), knob
     got = outs[-1].float().cpu().numpy()
@@ -180,6 +182,73 @@ def test_attn_short_spans_kept_in_registers(card, n0, T, Hq, Hk, S, tree, win):
                 path.append(p_)
                 p_ = par[p_]
             path = path[::-1]                            # root first: depth d at position n0 + d
+            slots = list(range(n0)) + [n0 + p for p in path]
+            pos = list(range(n0)) + [n0 + d for d in range(len(path))]
+        keep = [s_ for s_, ps in zip(slots, pos) if win == 0 or ps >= pos[-1] + 1 - win]
+        want = od.attention(q[t].float().numpy().reshape(Hq, D), K[:, keep].float().numpy(), V[:, keep].float().numpy(),
+                            scale)
+        worst = np.abs(got[t].reshape(Hq, D) - want).max() / np.abs(want).max()
+        assert worst <= 2.0**-7, (t, worst)
+
+
+@pytest.mark.parametrize("n0,T,Hq,Hk,tree,win", [(4000, 8, 32, 8, False, 0), (1000, 16, 32, 8, False, 0),
+                                                  (300, 5, 8, 2, True, 0), (120, 2, 8, 4, False, 0),
+                                                  (700, 6, 16, 4, True, 200), (0, 3, 8, 2, False, 0),
+                                                  (500, 2, 32, 8, False, 37), (250, 21, 16, 4, False, 0),
+                                                  (380, 32, 8, 2, True, 0), (127, 9, 32, 8, False, 0),
+                                                  (1, 13, 8, 4, True, 5)])
+def test_attn_rows_on_the_matrix_cores(card, n0, T, Hq, Hk, tree, win):
+    """a pass of several rows with spans of 128 keys takes the matrix-core kernel (every row that shares a kv head in one
+    workgroup; more than 64 (row, head) pairs a kv head are several workgroups): against f64 attention over the keys
+    each row sees - chain, tree, window, the pass's own rows straddling a span's end, a span with nothing to see -
+    within the bar of the vector-ALU kernel it replaces (knob attn_mfma = 0; the two differ in f32 summation order),
+    the same bits on a second call, and a tree that is a chain gives the chain's bits"""
+    D = 128
+    cap = n0 + T + 3
+    S = -(-cap // 128)
+    g = gen(700 + n0 + T)
+    K = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    V = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    # slots the pass has not written hold whatever was there: NaN bits must not leak through weight 0
+    K[:, n0 + T:] = float("nan")
+    V[:, n0 + T:] = float("nan")
+    q = torch.randn(T, Hq * D, generator=g).to(torch.bfloat16)
+    par = [-1] + [int(torch.randint(-1, t, (1,), generator=g)) for t in range(1, T)] if tree else None
+    part = None if par is None else torch.tensor(par, dtype=torch.int32, device="cuda")
+    scratch = card.attn_scratch(T, Hq, Hk, D, S)
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    scale = 1.0 / np.sqrt(D)
+
+    def run(p_=part):
+        att = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+        card.attn_decode(q.cuda(), K.cuda(), V.cuda(), att, n0t, Hq, Hk, D, scale, S, scratch, par=p_, win=win)
+        return att.clone()
+
+    y = run()
+    assert torch.equal(run(), y)
+    card.set_tuning("attn_mfma", 0)
+    try:
+        vec = run()
+    finally:
+        card.set_tuning("attn_mfma", -1)
+    peak = float(vec.float().abs().max())
+    assert float((vec.float() - y.float()).abs().max()) <= peak * 2.0**-7
+    if not tree:
+        chain = torch.arange(-1, T - 1, dtype=torch.int32, device="cuda")
+        if T <= 32:
+            assert torch.equal(run(chain), y)
+    got = y.float().cpu().numpy()
+    assert np.isfinite(got).all()
+    for t in range(T):
+        if par is None:
+            slots = list(range(n0 + t + 1))
+            pos = slots
+        else:
+            path, p_ = [], t
+            while p_ >= 0:
+                path.append(p_)
+                p_ = par[p_]
+            path = path[::-1]
             slots = list(range(n0)) + [n0 + p for p in path]
             pos = list(range(n0)) + [n0 + d for d in range(len(path))]
         keep = [s_ for s_, ps in zip(slots, pos) if win == 0 or ps >= pos[-1] + 1 - win]
