@@ -377,7 +377,7 @@ template <int G, bool DEV>
 __device__ __forceinline__ void merge_spans(uint16_t* out, int g, int S, size_t base, const float* part_m,
                                             const float* part_l, const float* part_acc, float* lds, int tid) {
     constexpr int NOUT = G >= 2 ? G / 2 : 1;  // outputs a thread makes: (j, d) = ((tid + 256 q) / 128, tid % 128)
-    constexpr int MS = NOUT <= 2 ? 32 : 16;   // spans a pass
+    constexpr int MS = NOUT <= 2 ? 40 : 20;   // spans a pass (a 4096-key cache is 33 to 36 spans: one pass)
     const float ninf = bits_f32(0xff800000u);
     auto ld = [](const float* p) { return DEV ? ld_dev(p) : *p; };
     float* f_m = lds;          // [S][G] maxima, then the factors

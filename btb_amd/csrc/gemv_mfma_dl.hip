@@ -1,5 +1,6 @@
-// The verify widths (M = 5..16 rows of x a pass) on the matrix cores for the long rows of the block-scaled forms
-// (FP8 e4m3 + block scales, MXFP4), with the weights going from memory straight into LDS.
+// The verify widths (M = 5..16 rows of x a pass) on the matrix cores with the weights going from memory straight into
+// LDS: the long rows of the block-scaled forms (FP8 e4m3 + block scales, MXFP4: 7168 columns) and pack12 rows of the
+// lengths it has shapes for (2560, up to 4096, around 9728 columns).
 //
 // gemv_mfma_lds.hip brings a sub-block of weights into registers, parks it in LDS and reads it back in the MFMA's
 // layout. On rows as long as 7168 columns the x fragments a wave keeps (x-stationary: 28 steps x 4 registers) leave
@@ -14,15 +15,17 @@
 // within granule: [8 granules][8 rows][16 B] = 1 KB - and that is also what the fragment reads want: a step's read
 // touches one or two granules of all sixteen rows, 8 rows x 16 B = 128 contiguous bytes a half, the upper eight rows'
 // block placed 128 bytes off a multiple of 256 so the two halves fall in different banks. A sub-block is GB such
-// 128-byte column blocks of the tile's sixteen rows: 2 GB load instructions, plus one dword-sized direct load for its
-// scales (the MXFP4 bytes of its rows and steps, or the FP8 block scales of its steps - a tile's sixteen rows share
-// them: blocks are a multiple of 16 rows tall).
+// 128-byte column blocks of the tile's sixteen rows: 2 GB load instructions, plus one or two more direct loads for
+// what goes with them (the MXFP4 scale bytes of its rows and steps; the FP8 block scales of its steps - a tile's
+// sixteen rows share them: blocks are a multiple of 16 rows tall; the pack12 code nibbles).
 //
 // Waiting is by count: loads complete in order, a sub-block is LOADS load instructions, so "sub-block q has landed" is
 // "at most (sub-blocks issued behind it) x LOADS loads outstanding" - an immediate, picked by how many were issued
 // behind it. The output stores of a tile's end count as outstanding too and may complete in any order: they are left
 // out of the immediate, which can only make a wait longer. A slot is asked for again only after the reads of its last
-// use have returned (the MFMAs that take them have been issued).
+// use have returned (the MFMAs that take them have been issued). The waves that stream never load into a register
+// the compiler knows to be outstanding (x comes through load_untracked, a form's constants through scalar loads):
+// behind a direct-to-LDS load the compiler's own wait for such a register is a wait for every load there is.
 //
 // The fold of the KS partial tiles in wave order and every rounding are gemv_mfma_lds's; which steps a wave sums
 // differs (see the kernel), so the two kernels agree to f32 summation order, not to the bit. Every M of a pass takes
@@ -149,8 +152,7 @@ struct DlF8 : DlNoTail {
     __host__ __device__ static constexpr int aux_loads(int /*sbs*/) { return 1; }  // load instructions beside the data's
     __host__ __device__ static constexpr int scale_words(int sbs) { return sbs; }
     // lane t brings the scale of the sub-block's step min(t, SBS - 1): f32 [64] in the scale area, the first SBS of
-    // them read. Every lane loads, so that there is no branch round the instruction: the compiler counts the loads
-    // outstanding exactly only through straight-line code, and the kernel's first tile depends on that.
+    // them read. Every lane loads: no branch round the instruction.
     template <int SBS>
     __device__ static __forceinline__ void issue_scales(const Mat& m, int tile, int /*nsteps*/, int step0, uint8_t* dst,
                                                         int lane) {
@@ -199,7 +201,7 @@ struct DlMx4 : DlNoTail {
                                                         int lane) {
         static_assert(SBS % 4 == 0 && 4 * SBS <= 64, "whole words of scale bytes, a lane a word");
         constexpr int per = SBS / 4;
-        if (16 * per == WAVE || lane < 16 * per) {  // no branch where every lane has a word (the first tile relies on it)
+        if (16 * per == WAVE || lane < 16 * per) {  // no branch where every lane has a word
             const int r = lane / per, j = lane - r * per;
             __builtin_amdgcn_global_load_lds(m.scales + (size_t)(tile * 16 + r) * nsteps + step0 + 4 * j, (lds_void*)dst,
                                              4, 0, 0);
@@ -634,9 +636,13 @@ static int32_t launch_dl(const typename DF::Mat& mat, const void* x, void* y, in
         return ERR_DOMAIN;
     }
     const int ntiles = R / 16;
-    const int cap = device_info().cus;  // the rings take most of a CU's LDS: one workgroup a CU
-    const int turns = (ntiles + cap - 1) / cap;
-    int grid = (ntiles + turns - 1) / turns;
+    // The rings take most of a CU's LDS: one workgroup a CU, and every CU one. What bounds a workgroup is how fast its
+    // own waves turn bytes into products (each CU takes in 21-23 GB/s here, whatever the others do), so the workgroup
+    // with the most tiles sets the time and spreading the tiles evenly over fewer workgroups buys nothing: FP8
+    // [18432, 7168] 231 workgroups of 5 tiles and 256 of 4 or 5 take the same 31 us, pack12 [9728, 2560] 203 of 3 take
+    // 15.2 and 256 of 2 or 3 14.6.
+    const int cap = device_info().cus;
+    int grid = std::min(ntiles, cap);
     if (tuning("mfma_direct_grid") > 0) grid = std::min(std::min(tuning("mfma_direct_grid"), cap), ntiles);
     const bool lead = (ntiles / grid) * MAXSB >= MAXSB + NBUF - 1;  // the workgroup with the fewest tiles has enough
     auto kern = lead ? gemv_mfma_dl<DF, KS, SPW, GB, NBUF, true> : gemv_mfma_dl<DF, KS, SPW, GB, NBUF, false>;
