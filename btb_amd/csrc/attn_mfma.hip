@@ -32,8 +32,6 @@
 
 namespace btb {
 
-namespace {
-
 constexpr int AM_D = 128;     // head_dim
 constexpr int AM_SPAN = 128;  // keys a workgroup
 constexpr int AM_VROW = 272;  // bytes a V row takes in LDS: 256 + 16, so the eight rows a fragment read touches differ in bank
@@ -245,7 +243,7 @@ __global__ void __launch_bounds__(256) attn_decode_mfma_kernel(
 }
 
 template <int G, int NQT>
-void launch_am(const uint16_t* q, const uint16_t* K, const uint16_t* V, const int32_t* n0, const int32_t* par, int T,
+static void launch_am(const uint16_t* q, const uint16_t* K, const uint16_t* V, const int32_t* n0, const int32_t* par, int T,
                int Hq, int Hk, long long hs, long long rs, float scale_log2, float* part_m, float* part_l,
                float* part_acc, int S, int cap, int win, const int32_t* tbl, hipStream_t st) {
     constexpr int NQ = 16 * NQT, TPW = NQ / G;
@@ -258,8 +256,6 @@ void launch_am(const uint16_t* q, const uint16_t* K, const uint16_t* V, const in
         hipLaunchKernelGGL((attn_decode_mfma_kernel<G, NQT, false>), grid, dim3(256), lds, st, q, K, V, n0, par, T, Hq,
                            Hk, hs, rs, scale_log2, part_m, part_l, part_acc, cap, win, tbl);
 }
-
-}  // namespace
 
 // whether the pass takes this kernel: spans of 128 keys, 2 or 4 query heads a kv head
 bool attn_mfma_fits(size_t T, size_t G, int span) {

@@ -261,9 +261,10 @@ size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, siz
  * row t over the keys 0 .. *n0 + t. par given (a verify pass's tree, T <= 32: par[t] the row's parent among the
  * pass's rows, -1 at a root): row t over the cache's keys 0 .. *n0 - 1 and, of the pass's own rows at slots
  * *n0 .. *n0 + T - 1, its ancestors and itself - the reference's TREE form (native/cuda/btb_attn_flash.cuh:284-286,
- * 407-419). The keys (capacity `cap`) are cut into S spans, a workgroup per (kv head, span, row) leaving its
- * online-softmax state in `workspace` (btb_hip_attn_scratch_floats floats); a second small launch folds the spans in
- * span order. head_dim 128, Hq / Hk in {1, 2, 4, 8}, S * (Hq / Hk) <= 1024. Replaces btb_attn_flash_d128's decode form
+ * 407-419). The keys (capacity `cap`: K and V hold at least that many slots) are cut into S spans, a workgroup per
+ * (kv head, span, row) - per (kv head, span) with every row of the pass, on the matrix cores, where the pass has several
+ * rows, spans of 128 keys and 2 or 4 query heads a kv head - leaving its online-softmax state in `workspace`
+ * (btb_hip_attn_scratch_floats floats); a second small launch folds the spans in span order. head_dim 128, Hq / Hk in {1, 2, 4, 8}, S * (Hq / Hk) <= 1024. Replaces btb_attn_flash_d128's decode form
  * (native/cuda/btb_attn_flash.cuh:277-675); its window and row map arguments are btb_hip_attn_decode_win's. */
 int32_t btb_hip_attn_decode(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
                             const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
