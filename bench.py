@@ -267,7 +267,10 @@ def kernel_workload(args: argparse.Namespace) -> int:
                  "gemv_fp8": "fp8 e4m3 x f32 block scale -> bf16 in registers",
                  "gemv_mxfp4": "mxfp4 -> bf16 in registers"}[name] + ", f32 accumulate"
         kernel = ("gemv_stream (vector ALUs, v_dot2_f32_bf16)" if M <= 4 else
-                  "gemv_mfma_lds (matrix cores, v_mfma_f32_16x16x32_bf16; taken from 5 rows on)")
+                  "gemv_mfma_lds (matrix cores, v_mfma_f32_16x16x32_bf16, weights staged through registers into LDS; "
+                  "taken from 5 rows on)" if name == "gemv_bf16" else
+                  "gemv_mfma_dl (matrix cores, v_mfma_f32_16x16x32_bf16, weights from memory straight into a ring in "
+                  "LDS; taken from 5 rows on)")
     side = torch.cuda.Stream()
     with torch.cuda.stream(side):
         for i in range(pool):
