@@ -656,40 +656,65 @@ static int32_t launch_dl(const typename DF::Mat& mat, const void* x, void* y, in
     return hip_status(hipGetLastError(), "gemv_mfma_dl launch");
 }
 
-// the shapes this kernel takes: 16-row tiles, rows of exactly 7168 columns (8 waves x 28 steps for FP8, 7 x 32 for
-// MXFP4), at most sixteen rows of x; FP8 blocks a whole number of tiles tall and of steps wide
-bool mfma_dl_fits(int R, int C, int M) {
-    return R % 16 == 0 && C == 7168 && M >= 1 && M <= 16 && tuning("mfma_direct") != 0;
+// The shapes this kernel takes: 16-row tiles, at most sixteen rows of x, and the row lengths it has shapes for, by steps
+// of 32 columns: 224 (7168 columns, the block-scaled forms' long rows), 80 (2560), 97..128 (to 4096) and 281..336
+// (around 9728) - classes 0..3, -1: none. A row is a whole number of the class's sub-blocks (`unit` steps).
+static int row_class(int C, int unit_narrow, int unit_wide) {
+    if (C % 32 != 0) return -1;
+    const int nsteps = C / 32;
+    if (nsteps == 224) return 0;
+    if (nsteps == 80) return 1;
+    if (nsteps > 96 && nsteps <= 128 && nsteps % unit_narrow == 0) return 2;
+    if (nsteps > 280 && nsteps <= 336 && nsteps % unit_wide == 0) return 3;
+    return -1;
 }
+static bool pass_ok(int R, int M) { return R % 16 == 0 && M >= 1 && M <= 16 && tuning("mfma_direct") != 0; }
 
-int32_t gemv_mfma_dl_fp8(const void* w, const float* scales, int sc, int bm, int bn, const void* x, void* y, int R,
-                         int C, int M, hipStream_t st) {
-    return launch_dl<DlF8, 8, 28, 1, 7>(DlF8::Mat{static_cast<const uint8_t*>(w), scales, sc, bm, bn}, x, y, R, C, M, st);
-}
-bool mfma_dl_fits_fp8(int R, int C, int M, int bm, int bn) {
-    return mfma_dl_fits(R, C, M) && bm % 16 == 0 && bn % 32 == 0;
-}
-
+// MXFP4: sub-blocks of 8 steps on the shorter rows, of 16 on the long ones (19 of them over seven waves at 9728 columns)
+bool mfma_dl_fits(int R, int C, int M) { return pass_ok(R, M) && row_class(C, 8, 16) >= 0; }
 int32_t gemv_mfma_dl_mxfp4(const void* blocks, const void* scales, const void* x, void* y, int R, int C, int M,
                            hipStream_t st) {
-    return launch_dl<DlMx4, 7, 32, 2, 4>(DlMx4::Mat{static_cast<const uint8_t*>(blocks), static_cast<const uint8_t*>(scales)},
-                                         x, y, R, C, M, st);
+    const DlMx4::Mat mat{static_cast<const uint8_t*>(blocks), static_cast<const uint8_t*>(scales)};
+    switch (row_class(C, 8, 16)) {
+        case 0: return launch_dl<DlMx4, 7, 32, 2, 4>(mat, x, y, R, C, M, st);
+        case 1: return launch_dl<DlMx4, 5, 16, 1, 4>(mat, x, y, R, C, M, st);
+        case 2: return launch_dl<DlMx4, 8, 16, 1, 4>(mat, x, y, R, C, M, st);
+        case 3: return launch_dl<DlMx4, 7, 48, 2, 3>(mat, x, y, R, C, M, st);
+        default: set_error("gemv_mfma_dl: a row length this kernel has no shape for"); return ERR_DOMAIN;
+    }
+}
+
+// FP8: sub-blocks of 4 steps, of 8 at 9728 columns; blocks a whole number of tiles tall and of steps wide
+bool mfma_dl_fits_fp8(int R, int C, int M, int bm, int bn) {
+    return pass_ok(R, M) && row_class(C, 4, 8) >= 0 && bm % 16 == 0 && bn % 32 == 0;
+}
+int32_t gemv_mfma_dl_fp8(const void* w, const float* scales, int sc, int bm, int bn, const void* x, void* y, int R,
+                         int C, int M, hipStream_t st) {
+    const DlF8::Mat mat{static_cast<const uint8_t*>(w), scales, sc, bm, bn};
+    switch (row_class(C, 4, 8)) {
+        case 0: return launch_dl<DlF8, 8, 28, 1, 7>(mat, x, y, R, C, M, st);
+        case 1: return launch_dl<DlF8, 10, 8, 1, 4>(mat, x, y, R, C, M, st);
+        case 2: return launch_dl<DlF8, 8, 16, 1, 4>(mat, x, y, R, C, M, st);
+        case 3: return launch_dl<DlF8, 7, 48, 2, 3>(mat, x, y, R, C, M, st);
+        default: set_error("gemv_mfma_dl: a row length this kernel has no shape for"); return ERR_DOMAIN;
+    }
 }
 
 // pack12: rows of 2560 columns (20 sub-blocks of 4 steps: ten waves, two each), 3073..4096 (eight waves, four each),
 // 9217..10752 in whole 256-column sub-blocks (seven waves, six sub-blocks of 8 steps each)
 bool mfma_dl_fits_p12(int R, int C, int M) {
-    if (R % 16 != 0 || M < 1 || M > 16 || C % 128 != 0 || tuning("mfma_direct") == 0) return false;
-    const int nsteps = C / 32;
-    return nsteps == 80 || (nsteps > 96 && nsteps <= 128) || (nsteps % 8 == 0 && nsteps > 280 && nsteps <= 336);
+    const int cls = row_class(C, 4, 8);
+    return pass_ok(R, M) && cls >= 1;
 }
 int32_t gemv_mfma_dl_p12(const uint8_t* lo, const uint8_t* hi4, const uint8_t* table, const int32_t* esc_idx,
                          const uint8_t* esc_val, const int32_t* row_ptr, const void* x, void* y, int R, int C, int M,
                          hipStream_t st) {
-    const int nsteps = C / 32;
-    if (nsteps == 80) return launch_dl<DlP12<4>, 10, 8, 1, 4>(DlP12<4>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr}, x, y, R, C, M, st);
-    if (nsteps <= 128) return launch_dl<DlP12<4>, 8, 16, 1, 4>(DlP12<4>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr}, x, y, R, C, M, st);
-    return launch_dl<DlP12<8>, 7, 48, 2, 3>(DlP12<8>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr}, x, y, R, C, M, st);
+    switch (row_class(C, 4, 8)) {
+        case 1: return launch_dl<DlP12<4>, 10, 8, 1, 4>(DlP12<4>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr}, x, y, R, C, M, st);
+        case 2: return launch_dl<DlP12<4>, 8, 16, 1, 4>(DlP12<4>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr}, x, y, R, C, M, st);
+        case 3: return launch_dl<DlP12<8>, 7, 48, 2, 3>(DlP12<8>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr}, x, y, R, C, M, st);
+        default: set_error("gemv_mfma_dl: a row length this kernel has no shape for"); return ERR_DOMAIN;
+    }
 }
 
 }  // namespace btb

@@ -221,6 +221,41 @@ def test_packed_rows_straight_into_lds(card, R, C, M, crowd):
 
 
 @pytest.mark.parametrize("form", ["fp8", "mxfp4"])
+@pytest.mark.parametrize("R,C", [(4864, 2560), (320, 4096), (208, 9728), (256, 3584), (96, 10752), (144, 9216)])
+@pytest.mark.parametrize("M", [7, 19])
+def test_block_scaled_rows_of_the_models_lengths_straight_into_lds(card, form, R, C, M):
+    """the direct-to-LDS kernel's other row lengths for the block-scaled forms - 2560, up to 4096, around 9728 columns;
+    3584 and 9216 / 9728 leave some waves without a last sub-block: against the oracle, the staged kernel, and a
+    row's bits whatever pass it came with (19 rows: a pass of 16 and one of 3)"""
+    src = weights_bf16(R, C, seed=370).float()
+    x = acts_bf16(M, C, seed=371)
+    if form == "fp8":
+        q, s = fp8.quantize(src, (16, 128) if R % 128 else (128, 128))
+        w = fp8.F8Weight(q.view(torch.uint8).cuda(), s.cuda(), R, C)
+        ref = oracle.gemv_fp8(q.view(torch.uint8).numpy(), s.numpy(), x.float().numpy(), threads=0)
+        op = card.gemv_fp8
+    else:
+        blocks, scales = mxfp4.quantize(src)
+        w = mxfp4.MxWeight(blocks.reshape(-1).cuda(), scales.reshape(-1).cuda(), R, C)
+        ref = oracle.gemv_mxfp4(blocks.numpy(), scales.numpy(), R, C, x.float().numpy(), threads=0)
+        op = card.gemv_mx4
+    xg = x.cuda()
+    y = op(w, xg)
+    check(y, ref)
+    card.set_tuning("mfma_direct", 0)
+    try:
+        staged = op(w, xg)
+    finally:
+        card.set_tuning("mfma_direct", -1)
+    check(staged, ref)
+    peak = float(y.float().abs().max())
+    assert float((staged.float() - y.float()).abs().max()) <= peak * 2.0**-7
+    last = op(w, xg[M - 5:].contiguous())
+    assert torch.equal(last.view(torch.int16), y[M - 5:].view(torch.int16))
+    assert torch.equal(op(w, xg).view(torch.int16), y.view(torch.int16))
+
+
+@pytest.mark.parametrize("form", ["fp8", "mxfp4"])
 def test_long_rows_with_scales_of_every_size(card, form):
     """the direct-to-LDS kernel's scales travel through LDS by loads of their own: random bytes under scales that differ
     from block to block by factors up to 2^40 (MXFP4: e8m0 bytes 107..147; FP8: f32 scales 2^-20..2^20, a zero scale
