@@ -60,7 +60,8 @@ __host__ __device__ constexpr size_t stage_lds_bytes(int xmode, int M, int C) {
 // Leaves the rows in xs (a barrier included). 256 threads. `after_issue` is called once, right after the first loads
 // of the staging have been issued and before anything waits for them: the caller requests its first weights there,
 // so they travel while the staging's own (short) round trip and arithmetic run.
-template <int XMODE, class AfterIssue>
+// MR: the number of rows where the caller knows it at compile time (M is then MR), 0 otherwise.
+template <int XMODE, int MR = 0, class AfterIssue>
 __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C, AfterIssue after_issue) {
     const int tid = threadIdx.x, nt = blockDim.x;
     if (XMODE == X_PLAIN) {
@@ -101,6 +102,69 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
         uint2* wkeep = rows4 + (size_t)M * n4;
         constexpr int PER = 3;  // words a thread holds at once: rows up to 3072 wide take one pass
         const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr;
+        if (MR > 1 && n4 <= PER * 256) {
+            // Several rows, each one pass: every row's words are requested before anything waits - and before the
+            // caller's first weights, which travel behind them. Row by row (the loop below) a row's loads queue
+            // behind those weights, and since loads return in order every further row waited for a span of weights:
+            // [19456 x 2560] with add + norm, 2 / 4 rows: 25.4 / 36.5 us against 18.9 / 21.8 for the plain matvec.
+            // The arithmetic, its order and the stores are the loop's.
+            constexpr int MRC = MR > 1 ? MR : 1;
+            uint2 hv[MRC][PER], yv[MRC][PER], wv[PER];
+            const uint2* ws = reinterpret_cast<const uint2*>(a.norm_w);
+#pragma unroll
+            for (int m = 0; m < MRC; ++m) {
+                size_t hrow = (size_t)m;
+                if (a.ids != nullptr) hrow = (size_t)min(max(a.ids[m], 0), a.vocab - 1);
+                const uint2* hs = reinterpret_cast<const uint2*>(a.x + hrow * C);
+                const uint2* ys = a.y == nullptr ? hs : reinterpret_cast<const uint2*>(a.y + (size_t)m * C);
+#pragma unroll
+                for (int q = 0; q < PER; ++q) {
+                    const int i = min(q * 256 + tid, n4 - 1);
+                    hv[m][q] = hs[i];
+                    yv[m][q] = ys[i];
+                    if (m == 0) wv[q] = ws[i];
+                }
+            }
+            after_issue();
+            const bool has_y = a.y != nullptr;
+#pragma unroll
+            for (int m = 0; m < MRC; ++m) {
+                uint2* row = rows4 + (size_t)m * n4;
+                float ss = 0.f;
+#pragma unroll
+                for (int q = 0; q < PER; ++q) {
+                    const int i = q * 256 + tid;
+                    const bool live = i < n4;
+                    float f[4] = {bf16lo_f32(hv[m][q].x), bf16hi_f32(hv[m][q].x), bf16lo_f32(hv[m][q].y), bf16hi_f32(hv[m][q].y)};
+                    const float g[4] = {bf16lo_f32(yv[m][q].x), bf16hi_f32(yv[m][q].x), bf16lo_f32(yv[m][q].y), bf16hi_f32(yv[m][q].y)};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float sum = bfround(f[e] + g[e]);
+                        f[e] = has_y ? sum : f[e];
+                        const float sq = fmaf(f[e], f[e], ss);
+                        ss = live ? sq : ss;
+                    }
+                    const uint2 hb = make_uint2(f32_bf16(f[0]) | ((uint32_t)f32_bf16(f[1]) << 16),
+                                                f32_bf16(f[2]) | ((uint32_t)f32_bf16(f[3]) << 16));
+                    const int ic = min(i, n4 - 1);
+                    row[ic] = hb;
+                    if (m == 0) wkeep[ic] = wv[q];
+                    if (writer) reinterpret_cast<uint2*>(a.h_out + (size_t)m * C)[ic] = hb;
+                }
+                const float rstd = rsqrtf(block_sum256(ss, red) / (float)C + a.eps);
+                for (int i = tid; i < n4; i += 256) {
+                    const uint2 hb = row[i], wb = wkeep[i];
+                    const float f[4] = {bf16lo_f32(hb.x), bf16hi_f32(hb.x), bf16lo_f32(hb.y), bf16hi_f32(hb.y)};
+                    const float g[4] = {bf16lo_f32(wb.x), bf16hi_f32(wb.x), bf16lo_f32(wb.y), bf16hi_f32(wb.y)};
+                    uint32_t o[4];
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) o[e] = f32_bf16(f[e] * rstd * (a.centered ? 1.f + g[e] : g[e]));
+                    row[i] = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+                }
+            }
+            __syncthreads();
+            return;
+        }
         for (int m = 0; m < M; ++m) {
             size_t hrow = (size_t)m;
             if (a.ids != nullptr) hrow = (size_t)min(max(a.ids[m], 0), a.vocab - 1);  // uniform: one scalar load
@@ -163,7 +227,7 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
 
 template <int XMODE>
 __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C) {
-    stage_x<XMODE>(xs, a, M, C, [] {});
+    stage_x<XMODE, 0>(xs, a, M, C, [] {});
 }
 
 // ------------------------------------------------------------------------------------------------------------

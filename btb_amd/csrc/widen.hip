@@ -134,6 +134,14 @@ static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>
 
 using namespace btb;
 
+namespace btb {
+// f32 values rounded to stored bf16 by the library's own f32_bf16, a thread a value
+__global__ void __launch_bounds__(256) round_bf16_kernel(const float* __restrict__ x, uint16_t* __restrict__ out, size_t n) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) out[i] = f32_bf16(x[i]);
+}
+}  // namespace btb
+
 extern "C" {
 
 int32_t btb_hip_p12_row_ptr(const void* esc_idx, size_t n_esc, size_t rows, size_t cols, void* row_ptr, void* stream) {
@@ -226,6 +234,15 @@ int32_t btb_hip_mx4_widen(const void* blocks, const void* scales, const void* se
         hipLaunchKernelGGL(mx4_widen_kernel<false>, grid, dim3(256), 0, st, p, static_cast<const int32_t*>(seats),
                            (long long)groups, out);
     return hip_status(hipGetLastError(), "mx4_widen launch");
+}
+
+int32_t btb_hip_round_bf16(const void* x, void* out, size_t n, void* stream) {
+    if (x == nullptr || out == nullptr) return ERR_NULL;
+    if (n == 0 || n > (1ull << 40)) return ERR_DOMAIN;
+    if (!al(x, 4) || !al(out, 2)) return ERR_DOMAIN;
+    hipLaunchKernelGGL(round_bf16_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const float*>(x), static_cast<uint16_t*>(out), n);
+    return hip_status(hipGetLastError(), "round_bf16 launch");
 }
 
 }  // extern "C"

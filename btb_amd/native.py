@@ -47,6 +47,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_p12_widen": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _vp, _vp]),
     "btb_hip_gemv_fp8": (_i32, [_vp, _vp, _sz, _sz, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_fp8_widen": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _i32, _vp]),
+    "btb_hip_round_bf16": (_i32, [_vp, _vp, _sz, _vp]),
     "btb_hip_gemv_mxfp4": (_i32, [_vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_mx4_widen": (_i32, [_vp, _vp, _vp, _sz, ctypes.c_int64, _vp, _i32, _vp]),
     "btb_hip_gemv_bf16_rows": (_i32, [_vp, _sz, _sz, _vp, _sz, _vp, _vp]),
@@ -429,6 +430,14 @@ class HipCard:
         self._call("btb_hip_gemv_fp8", self.ptr(w.w), self.ptr(w.scales), sr, sc, self.ptr(x2), self.ptr(y), R, C, M,
                    _stream())
         return y
+
+    def round_bf16(self, x: torch.Tensor) -> torch.Tensor:
+        """float32 values as stored bf16, by the rounding every bf16 output of the library goes through (nearest even,
+        a NaN the quiet NaN of its sign and upper payload: the crate's `round_bf16` with torch's NaN rule)"""
+        self._need(x, torch.float32, "x")
+        out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
+        self._call("btb_hip_round_bf16", self.ptr(x), self.ptr(out), int(x.numel()), _stream())
+        return out
 
     def fp8_widen(self, w: Any, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
         """an `F8Weight` as the held matrix (`fp8.held`), bf16 or the same values as f32"""

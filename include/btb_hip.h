@@ -134,6 +134,11 @@ int32_t btb_hip_p12_widen(const void* lo, const void* hi4, const void* table, co
 int32_t btb_hip_gemv_fp8(const void* w, const void* scales, size_t sr, size_t sc, const void* x, void* y, size_t R,
                          size_t C, size_t M, void* stream);
 
+/* out u16[n] = the stored bf16 nearest to x f32[n], ties to even, a NaN the quiet NaN with its sign and upper payload -
+ * the crate's round_bf16 (native/src/gemv.rs:3003-3007) over an array, with the NaN rule of a torch cast; the rounding
+ * every bf16 output of this library goes through. */
+int32_t btb_hip_round_bf16(const void* x, void* out, size_t n, void* stream);
+
 /* An FP8 matrix widened to the held weights bf16(e4m3 * scale): bf16 [rows, cols] (out_f32 == 0) or the same values
  * as f32 (out_f32 != 0). fp8.held (btb/fp8.py:97-100) on the device. */
 int32_t btb_hip_fp8_widen(const void* w, const void* scales, size_t rows, size_t cols, size_t sr, size_t sc, void* out,

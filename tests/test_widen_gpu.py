@@ -175,3 +175,24 @@ def test_mx4_widen_seats(card):
     assert torch.equal(got.cpu().view(torch.int16), want.reshape(3, -1).view(torch.int16))
     with pytest.raises(ValueError):
         card.mx4_widen(dev(blocks).float(), dev(scales))
+
+
+def test_round_bf16_is_the_integer_rule(card):
+    """the device's f32 -> bf16 rounding (one conversion instruction) against the integer rule the reference and the
+    oracle state (native/src/gemv.rs:3003-3007; a NaN: the quiet NaN a torch cast writes) on bit patterns of every
+    kind: anything, NaNs of every payload and both signs, denormals, exact ties, the values round the largest finite"""
+    rng = np.random.default_rng(960)
+    bits = np.concatenate([
+        rng.integers(0, 2**32, 2_000_000, dtype=np.uint64).astype(np.uint32),
+        (0x7F800000 | rng.integers(1, 2**23, 300_000, dtype=np.uint64)).astype(np.uint32),
+        (0xFF800000 | rng.integers(1, 2**23, 300_000, dtype=np.uint64)).astype(np.uint32),
+        rng.integers(0, 2**23, 300_000, dtype=np.uint64).astype(np.uint32),
+        ((rng.integers(0, 2**16, 300_000, dtype=np.uint64).astype(np.uint32) << 16) | 0x8000).astype(np.uint32),
+        np.array([0x7F800000, 0xFF800000, 0x7F7FFFFF, 0x7F7F8000, 0x7F7F7FFF, 0, 0x80000000, 0x7F800001, 0x7FC00000,
+                  0x7FFFFFFF, 0xFFFFFFFF, 0x00000001, 0x00008000, 0x00018000], dtype=np.uint32),
+    ])
+    x = torch.from_numpy(bits.view(np.float32).copy()).cuda()
+    got = card.round_bf16(x).view(torch.int16).cpu().numpy().view(np.uint16)
+    want = codecs.f32_to_bf16_bits(bits.view(np.float32))
+    assert np.array_equal(got, want)
+
