@@ -69,6 +69,16 @@ __host__ __device__ __forceinline__ uint16_t f32_bf16(float f) {
 #endif
 }
 __host__ __device__ __forceinline__ float bfround(float f) { return bf16_f32(f32_bf16(f)); }
+// two values as a packed pair of stored bf16 (lo in the low half): one conversion instruction on the device
+__host__ __device__ __forceinline__ uint32_t f32x2_bf16(float lo, float hi) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    typedef __attribute__((ext_vector_type(2))) __bf16 pair_t;
+    const pair_t p = {(__bf16)lo, (__bf16)hi};
+    return __builtin_bit_cast(uint32_t, p);
+#else
+    return (uint32_t)f32_bf16(lo) | ((uint32_t)f32_bf16(hi) << 16);
+#endif
+}
 
 // a 16-byte streaming load of weights: read once per token, so it is marked non-temporal
 typedef __attribute__((ext_vector_type(4))) uint32_t u32x4;

@@ -35,9 +35,7 @@ struct XArgs {
 __device__ __forceinline__ uint32_t silu_pair(uint32_t g2, uint32_t u2) {
     const float s0 = bfround(bf16lo_f32(g2) / (1.f + expf(-bf16lo_f32(g2))));
     const float s1 = bfround(bf16hi_f32(g2) / (1.f + expf(-bf16hi_f32(g2))));
-    const uint32_t lo = f32_bf16(s0 * bf16lo_f32(u2));
-    const uint32_t hi = f32_bf16(s1 * bf16hi_f32(u2));
-    return lo | (hi << 16);
+    return f32x2_bf16(s0 * bf16lo_f32(u2), s1 * bf16hi_f32(u2));
 }
 
 // sum over a 256-thread block in a fixed order: each wave's DPP tree, then waves 0..3 in order
@@ -144,8 +142,7 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
                         const float sq = fmaf(f[e], f[e], ss);
                         ss = live ? sq : ss;
                     }
-                    const uint2 hb = make_uint2(f32_bf16(f[0]) | ((uint32_t)f32_bf16(f[1]) << 16),
-                                                f32_bf16(f[2]) | ((uint32_t)f32_bf16(f[3]) << 16));
+                    const uint2 hb = make_uint2(f32x2_bf16(f[0], f[1]), f32x2_bf16(f[2], f[3]));
                     const int ic = min(i, n4 - 1);
                     row[ic] = hb;
                     if (m == 0) wkeep[ic] = wv[q];
@@ -156,10 +153,10 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
                     const uint2 hb = row[i], wb = wkeep[i];
                     const float f[4] = {bf16lo_f32(hb.x), bf16hi_f32(hb.x), bf16lo_f32(hb.y), bf16hi_f32(hb.y)};
                     const float g[4] = {bf16lo_f32(wb.x), bf16hi_f32(wb.x), bf16lo_f32(wb.y), bf16hi_f32(wb.y)};
-                    uint32_t o[4];
+                    float o[4];
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) o[e] = f32_bf16(f[e] * rstd * (a.centered ? 1.f + g[e] : g[e]));
-                    row[i] = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+                    for (int e = 0; e < 4; ++e) o[e] = f[e] * rstd * (a.centered ? 1.f + g[e] : g[e]);
+                    row[i] = make_uint2(f32x2_bf16(o[0], o[1]), f32x2_bf16(o[2], o[3]));
                 }
             }
             __syncthreads();
@@ -202,8 +199,7 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
                         const float sq = fmaf(f[e], f[e], ss);
                         ss = live ? sq : ss;
                     }
-                    const uint2 hb = make_uint2(f32_bf16(f[0]) | ((uint32_t)f32_bf16(f[1]) << 16),
-                                                f32_bf16(f[2]) | ((uint32_t)f32_bf16(f[3]) << 16));
+                    const uint2 hb = make_uint2(f32x2_bf16(f[0], f[1]), f32x2_bf16(f[2], f[3]));
                     const int ic = min(i, n4 - 1);
                     row[ic] = hb;
                     wkeep[ic] = wv[q];
@@ -215,10 +211,10 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
                 const uint2 hb = row[i], wb = wkeep[i];
                 const float f[4] = {bf16lo_f32(hb.x), bf16hi_f32(hb.x), bf16lo_f32(hb.y), bf16hi_f32(hb.y)};
                 const float g[4] = {bf16lo_f32(wb.x), bf16hi_f32(wb.x), bf16lo_f32(wb.y), bf16hi_f32(wb.y)};
-                uint32_t o[4];
+                float o[4];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) o[e] = f32_bf16(f[e] * rstd * (a.centered ? 1.f + g[e] : g[e]));
-                row[i] = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+                for (int e = 0; e < 4; ++e) o[e] = f[e] * rstd * (a.centered ? 1.f + g[e] : g[e]);
+                row[i] = make_uint2(f32x2_bf16(o[0], o[1]), f32x2_bf16(o[2], o[3]));
             }
         }
     }

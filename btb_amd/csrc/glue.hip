@@ -114,20 +114,20 @@ __global__ void __launch_bounds__(256) add_rmsnorm_kernel(uint16_t* __restrict__
             }
             if (yr != nullptr && live)
                 reinterpret_cast<uint2*>(hr)[tid + 256 * k] =
-                    make_uint2(f32_bf16(f[k][0]) | (f32_bf16(f[k][1]) << 16), f32_bf16(f[k][2]) | (f32_bf16(f[k][3]) << 16));
+                    make_uint2(f32x2_bf16(f[k][0], f[k][1]), f32x2_bf16(f[k][2], f[k][3]));
         }
         const float rstd = rsqrtf(block_sum256(ss, red) / (float)H + eps);
 #pragma unroll
         for (int k = 0; k < PER; ++k) {
             const uint32_t ww[2] = {wv[k].x, wv[k].y};
-            uint32_t o[4];
+            float o[4];
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const float wf = (e & 1) ? bf16hi_f32(ww[e / 2]) : bf16lo_f32(ww[e / 2]);
-                o[e] = f32_bf16(f[k][e] * rstd * (centered ? 1.f + wf : wf));
+                o[e] = f[k][e] * rstd * (centered ? 1.f + wf : wf);
             }
             if (tid + 256 * k < n4)
-                reinterpret_cast<uint2*>(xr)[tid + 256 * k] = make_uint2(o[0] | (o[1] << 16), o[2] | (o[3] << 16));
+                reinterpret_cast<uint2*>(xr)[tid + 256 * k] = make_uint2(f32x2_bf16(o[0], o[1]), f32x2_bf16(o[2], o[3]));
         }
         return;
     }
