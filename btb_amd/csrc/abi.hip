@@ -79,6 +79,7 @@ static Knob g_knobs[] = {
     {"attn_heads_per_wg", {-1}},
     {"attn_rows_per_wg", {-1}},
     {"attn_mfma", {-1}},
+    {"attn_rows_fused", {-1}},
 };
 
 int tuning(const char* key) {

@@ -222,6 +222,11 @@ int32_t attn_decode_mfma(const void* q, const void* K, const void* V, const int3
                          size_t Hq, size_t Hk, long long hs, long long rs, float scale_log2, float* part_m,
                          float* part_l, float* part_acc, size_t S, size_t cap, int win, const int32_t* tbl,
                          hipStream_t st);
+bool attn_mfma_qkv_fits(size_t T, size_t G, int span);
+int32_t attn_decode_mfma_qkv(const void* qkv, const void* wq, const void* wk, float eps, int centered, const void* cos_t,
+                             const void* sin_t, const int32_t* n0, const int32_t* depth, const int32_t* par, void* K,
+                             void* V, size_t T, size_t Hq, size_t Hk, long long hs, long long rs, float scale_log2,
+                             float* part_m, float* part_l, float* part_acc, size_t S, size_t cap, hipStream_t st);
 
 template <int G>
 __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __restrict__ q, const uint16_t* __restrict__ K,
@@ -844,6 +849,60 @@ int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk,
 #undef ATT
 #undef MERGE
     return hip_status(hipGetLastError(), "attn_decode_qkv launch");
+}
+
+int32_t btb_hip_attn_rows_fused(size_t T, size_t Hq, size_t Hk, size_t D, size_t cap, size_t S) {
+    if (T == 0 || Hq == 0 || Hk == 0 || S == 0 || cap == 0 || Hq % Hk != 0 || D != (size_t)ATT_D) return 0;
+    const int span = (int)(((cap + S - 1) / S + 127) / 128 * 128);
+    return attn_mfma_qkv_fits(T, Hq / Hk, span) ? 1 : 0;
+}
+
+int32_t btb_hip_attn_decode_qkv_rows(const void* qkv, const void* wq, const void* wk, float eps, int32_t centered,
+                                     const void* cos_t, const void* sin_t, const int32_t* n0, const int32_t* depth,
+                                     const int32_t* par, void* K, void* V, void* att, size_t T, size_t Hq, size_t Hk,
+                                     size_t D, int64_t hs, int64_t rs, float scale, size_t cap, size_t S,
+                                     float* workspace, void* stream) {
+    if (qkv == nullptr || cos_t == nullptr || sin_t == nullptr || n0 == nullptr || K == nullptr || V == nullptr ||
+        att == nullptr || workspace == nullptr)
+        return ERR_NULL;
+    if (T == 0 || Hq == 0 || Hk == 0 || S == 0 || cap == 0 || S > 1024 || Hq % Hk != 0 || hs <= 0 || rs <= 0 ||
+        !(scale == scale) || !(eps >= 0.f))
+        return ERR_DOMAIN;
+    const size_t G = Hq / Hk;
+    if (!al(qkv, 4) || !al(K, 16) || !al(V, 16) || !al(par, 4) || !al(depth, 4) || (rs % 8) != 0 || (hs % 8) != 0)
+        return ERR_DOMAIN;
+    if (par != nullptr && T > 32) {
+        set_error("attn_decode_qkv_rows: a tree pass holds at most 32 rows");
+        return ERR_DOMAIN;
+    }
+    if (S * G > (size_t)ATT_MAX_STATES) {
+        set_error("attn_decode_qkv_rows: spans * (query heads per kv head) is at most 1024");
+        return ERR_DOMAIN;
+    }
+    if (btb_hip_attn_rows_fused(T, Hq, Hk, D, cap, S) == 0) {
+        set_error("attn_decode_qkv_rows: head_dim 128, spans of 128 keys, 2 or 4 query heads per kv head and 2 or more "
+                  "rows with rows * (query heads per kv head) <= 32 (btb_hip_attn_rows_fused tells); otherwise "
+                  "btb_hip_norm_rope_kv + btb_hip_attn_decode");
+        return ERR_DOMAIN;
+    }
+    float* part_m = workspace;
+    float* part_l = workspace + T * Hq * S;
+    float* part_acc = workspace + 2 * T * Hq * S;
+    const float scale_log2 = scale * 1.4426950408889634f;
+    hipStream_t st = static_cast<hipStream_t>(stream);
+    const int32_t rc = attn_decode_mfma_qkv(qkv, wq, wk, eps, centered ? 1 : 0, cos_t, sin_t, n0, depth, par, K, V, T, Hq,
+                                            Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, S, cap,
+                                            st);
+    if (rc != OK) return rc;
+    const dim3 mgrid((unsigned)Hk, (unsigned)T);
+    const size_t mlds = 2 * S * G * sizeof(float);
+    if (G == 4)
+        hipLaunchKernelGGL(attn_merge_kernel<4>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
+                           (int)Hk, (int)S, part_m, part_l, part_acc);
+    else
+        hipLaunchKernelGGL(attn_merge_kernel<2>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
+                           (int)Hk, (int)S, part_m, part_l, part_acc);
+    return hip_status(hipGetLastError(), "attn_decode_qkv_rows launch");
 }
 
 int32_t btb_hip_silu_mul(const void* gu, void* m, size_t T, size_t I, void* stream) {

@@ -148,6 +148,7 @@ class DecodeStep:
         # kernel); from four rows on the one-launch-per-operator sequence does, whose matvecs take the matrix cores
         # at five rows and more while a fused matvec runs as passes of four rows (measured on the 36-layer
         # [2560 / 9728] stack, bf16: 4.3 against 4.0 ms at 4 rows, 7.1 against 4.6 at 8, 12.6 against 5.9 at 16).
+        chosen = fused is None
         if fused is None:
             fused = T <= 3
         if fold_silu is None:
@@ -156,6 +157,10 @@ class DecodeStep:
         # the fused launches exist for bf16 and 12-bit matrices; any other stored form takes one launch per operator
         lins = [weights[f"layers.{i}.{k}"] for i in range(cfg.layers) for k in ("qkv", "o", "gu", "down")] + [weights["head"]]
         self.fused = bool(fused) and all(getattr(m, "fusable", False) for m in lins)
+        # a pass's q / k norm, rope and cache write ride in its attention kernel where that kernel takes the pass's
+        # shape - in the fused sequence, and in the other one too unless the caller asked for a launch per operator
+        self.rows_attn_fused = (chosen or bool(fused)) and T > 1 and bool(
+            card.attn_rows_fused(T, cfg.q_heads, cfg.kv_heads, cfg.head_dim, self.cap, self.S))
         # the handoff to the host: token, cache length and the GPU's clock in pinned memory
         self.host_tok = torch.zeros(1, dtype=torch.int32).pin_memory()
         self.host_n0 = torch.zeros(1, dtype=torch.int32).pin_memory()
@@ -289,7 +294,8 @@ class DecodeStep:
             self._body_plain()
 
     def _body_plain(self) -> None:
-        """one launch per operator, in the reference's order (btb/engine/cuda.py:1722-1834)"""
+        """one launch per operator, in the reference's order (btb/engine/cuda.py:1722-1834) - but for a pass's q / k
+        norm and rope, which ride in its attention kernel unless the step was built with `fused=False`"""
         k, cfg, w = self.card, self.cfg, self.w
         Hq, Hk, D = cfg.q_heads, cfg.kv_heads, cfg.head_dim
         k.embed(w["embed"], self.ids, self.h)
@@ -299,9 +305,15 @@ class DecodeStep:
             K, V = self.kv[i, 0], self.kv[i, 1]
             k.add_rmsnorm(self.h, y_prev, w[L + "ln1"], cfg.eps, self.x)
             w[L + "qkv"].matvec(self.x, self.qkv)
-            k.norm_rope_kv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K, V,
-                           self.q, Hq, Hk, D, depth=self.depth)
-            k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch, par=self.par)
+            if self.rows_attn_fused:
+                k.attn_decode_qkv_rows(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin,
+                                       self.n0, K, V, self.att, Hq, Hk, D, self.scale, self.S, self.scratch,
+                                       depth=self.depth, par=self.par)
+            else:
+                k.norm_rope_kv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K, V,
+                               self.q, Hq, Hk, D, depth=self.depth)
+                k.attn_decode(self.q, K, V, self.att, self.n0, Hq, Hk, D, self.scale, self.S, self.scratch,
+                              par=self.par)
             w[L + "o"].matvec(self.att, self.y)
             k.add_rmsnorm(self.h, self.y, w[L + "ln2"], cfg.eps, self.x)
             w[L + "gu"].matvec(self.x, self.gu)
@@ -336,6 +348,10 @@ class DecodeStep:
             if self.T == 1 and D == 128:
                 k.attn_decode_qkv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K,
                                   V, self.att, Hq, Hk, D, self.scale, self.S, self.scratch)
+            elif self.rows_attn_fused:
+                k.attn_decode_qkv_rows(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin,
+                                       self.n0, K, V, self.att, Hq, Hk, D, self.scale, self.S, self.scratch,
+                                       depth=self.depth, par=self.par)
             else:
                 k.norm_rope_kv(self.qkv, w.get(L + "wq"), w.get(L + "wk"), cfg.eps, self.cos, self.sin, self.n0, K, V,
                                self.q, Hq, Hk, D, depth=self.depth)

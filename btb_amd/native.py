@@ -78,6 +78,10 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
                                            ctypes.c_int64, ctypes.c_float, _sz, _sz, _vp]),
     "btb_hip_attn_decode_qkv": (_i32, [_vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
                                        ctypes.c_int64, ctypes.c_int64, ctypes.c_float, _sz, _sz, _vp, _vp]),
+    "btb_hip_attn_rows_fused": (_i32, [_sz, _sz, _sz, _sz, _sz, _sz]),
+    "btb_hip_attn_decode_qkv_rows": (_i32, [_vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+                                            _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64, ctypes.c_float, _sz,
+                                            _sz, _vp, _vp]),
     "btb_hip_silu_mul": (_i32, [_vp, _vp, _sz, _sz, _vp]),
     "btb_hip_argmax": (_i32, [_vp, _vp, _sz, _sz, _vp]),
     "btb_hip_publish": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
@@ -760,6 +764,48 @@ class HipCard:
         self._call("btb_hip_attn_decode_qkv", self.ptr(qkv), p(wq), p(wk), float(eps), 1 if centered else 0,
                    self.ptr(cos_t), self.ptr(sin_t), self.ptr(n0), self.ptr(K), self.ptr(V), self.ptr(att), Hq, Hk, D,
                    int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S, self.ptr(scratch), _stream())
+
+    def attn_rows_fused(self, T: int, Hq: int, Hk: int, D: int, cap: int, S: int) -> bool:
+        """whether `attn_decode_qkv_rows` takes a pass of this shape"""
+        return bool(self.lib.btb_hip_attn_rows_fused(T, Hq, Hk, D, cap, S))
+
+    def attn_decode_qkv_rows(self, qkv: torch.Tensor, wq: torch.Tensor | None, wk: torch.Tensor | None, eps: float,
+                             cos_t: torch.Tensor, sin_t: torch.Tensor, n0: torch.Tensor, K: torch.Tensor,
+                             V: torch.Tensor, att: torch.Tensor, Hq: int, Hk: int, D: int, scale: float, S: int,
+                             scratch: torch.Tensor, depth: torch.Tensor | None = None,
+                             par: torch.Tensor | None = None, centered: bool = False) -> None:
+        """a pass's attention straight from its fused qkv rows [T, (Hq + 2 Hk) D]: `norm_rope_kv` + `attn_decode`, one
+        launch less (q stays on the chip; the new K / V rows are written by the workgroups whose spans hold them)"""
+        for t, what in ((qkv, "qkv"), (att, "att"), (cos_t, "cos"), (sin_t, "sin")):
+            self._need(t, torch.bfloat16, what)
+        for t, what in ((wq, "wq"), (wk, "wk")):
+            if t is not None:
+                self._need(t, torch.bfloat16, what)
+                if t.numel() != D:
+                    raise ValueError(f"[hip] attn_decode_qkv_rows: {what} holds {t.numel()} values, head_dim is {D}")
+        self._need(n0, torch.int32, "n0")
+        self._need(scratch, torch.float32, "scratch")
+        if K.dtype != torch.bfloat16 or V.dtype != torch.bfloat16 or K.stride(2) != 1 or K.stride() != V.stride():
+            raise ValueError("[hip] attn_decode_qkv_rows: K and V are bf16 [Hk, cap, D] views with the same strides")
+        width = (Hq + 2 * Hk) * D
+        T = qkv.numel() // width
+        if T < 1 or qkv.numel() != T * width or att.numel() != T * Hq * D:
+            raise ValueError("[hip] attn_decode_qkv_rows: qkv is [T, (Hq + 2 Hk) D], att [T, Hq D]")
+        if cos_t.shape[-1] != D or cos_t.shape != sin_t.shape or cos_t.shape[0] < K.shape[1]:
+            raise ValueError("[hip] attn_decode_qkv_rows: rope tables are [positions >= cap, D]")
+        for t, what in ((depth, "depth"), (par, "par")):
+            if t is not None:
+                self._need(t, torch.int32, what)
+                if t.numel() != T:
+                    raise ValueError(f"[hip] attn_decode_qkv_rows: {what} names {t.numel()} rows, the pass has {T}")
+        need = int(self.lib.btb_hip_attn_scratch_floats(T, Hq, Hk, D, S))
+        if scratch.numel() < need:
+            raise ValueError(f"[hip] attn_decode_qkv_rows: scratch holds {scratch.numel()} floats, {need} are needed")
+        p = lambda t: None if t is None else self.ptr(t)
+        self._call("btb_hip_attn_decode_qkv_rows", self.ptr(qkv), p(wq), p(wk), float(eps), 1 if centered else 0,
+                   self.ptr(cos_t), self.ptr(sin_t), self.ptr(n0), p(depth), p(par), self.ptr(K), self.ptr(V),
+                   self.ptr(att), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S,
+                   self.ptr(scratch), _stream())
 
     def silu_mul(self, gu: torch.Tensor, m: torch.Tensor) -> torch.Tensor:
         self._need(gu, torch.bfloat16, "gu")

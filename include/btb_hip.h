@@ -309,6 +309,22 @@ int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk,
                                 size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t cap,
                                 size_t S, float* workspace, void* stream);
 
+/* The same for a pass of T >= 2 rows on the matrix cores: qkv [T, (Hq + 2 Hk) D] bf16, depth (i32 [T], device) the
+ * rows' depths for a tree pass or NULL for a chain (row t stands at *n0 + t), par as for btb_hip_attn_decode. What
+ * btb_hip_norm_rope_kv followed by btb_hip_attn_decode compute, bit for bit, in one launch less: each workgroup
+ * prepares the pass's q heads itself, the workgroups whose key span holds some of slots *n0 .. *n0 + T - 1 prepare
+ * and write those K / V rows. For head_dim 128, spans of 128 keys, 2 or 4 query heads a kv head and
+ * T * (Hq / Hk) <= 32: btb_hip_attn_rows_fused returns 1 for such a pass and 0 otherwise, where this call fails with
+ * BTB_HIP_ERR_DOMAIN and the two calls it replaces remain. Workspace: btb_hip_attn_scratch_floats(T, ...). Replaces
+ * btb_norm_rope_kv_d128 + btb_attn_flash_d128 of the reference's verify pass (btb/engine/cuda.py:1756-1790,
+ * native/cuda/btb_attn_flash.cuh:400-470). */
+int32_t btb_hip_attn_rows_fused(size_t T, size_t Hq, size_t Hk, size_t D, size_t cap, size_t S);
+int32_t btb_hip_attn_decode_qkv_rows(const void* qkv, const void* wq, const void* wk, float eps, int32_t centered,
+                                     const void* cos_t, const void* sin_t, const int32_t* n0, const int32_t* depth,
+                                     const int32_t* par, void* K, void* V, void* att, size_t T, size_t Hq, size_t Hk,
+                                     size_t D, int64_t hs, int64_t rs, float scale, size_t cap, size_t S,
+                                     float* workspace, void* stream);
+
 /* m [T, I] = bf16(bf16(silu(g)) * u) over gu [T, 2I] (gate then up). Replaces btb_silu_mul
  * (native/cuda/btb_kernels.cu:467-484); the matvec btb_hip_gemv_silu_bf16 folds the same values into its x load. */
 int32_t btb_hip_silu_mul(const void* gu, void* m, size_t T, size_t I, void* stream);

@@ -296,6 +296,79 @@ def test_attn_decode_qkv_is_the_two_kernels_in_one(card, n0, Hq, Hk, S, with_nor
         assert not torch.equal(Kb[:, n0], K0[:, n0])  # the row was written
 
 
+@pytest.mark.parametrize("n0,T,Hq,Hk,tree", [(4000, 8, 32, 8, False), (4000, 7, 32, 8, False), (125, 8, 32, 8, False),
+                                              (120, 16, 8, 4, True), (0, 2, 8, 2, False), (127, 3, 8, 4, False),
+                                              (255, 16, 8, 4, True), (300, 5, 8, 2, True), (128, 4, 32, 8, False),
+                                              (250, 9, 16, 8, True), (1, 13, 4, 2, False), (383, 2, 32, 8, False)])
+@pytest.mark.parametrize("with_norm", [True, False])
+def test_attn_rows_from_the_fused_qkv_rows(card, n0, T, Hq, Hk, tree, with_norm):
+    """a pass's attention from its fused qkv rows against norm_rope_kv followed by attn_decode: the same output bits,
+    the same cache rows, nothing else in the cache touched - chain and tree (rows at their depths), the pass's own slots
+    at a span's start, across its end, and past the written part of the cache (which holds NaN bits)"""
+    from btb_amd.decode import StackConfig, rope_tables
+
+    D = 128
+    cap = n0 + T + 5
+    S = -(-cap // 128)
+    assert card.attn_rows_fused(T, Hq, Hk, D, cap, S)
+    g = gen(660 + n0 + T + Hq)
+    K0 = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    V0 = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+    K0[:, n0:] = float("nan")
+    V0[:, n0:] = float("nan")
+    K0, V0 = K0.cuda(), V0.cuda()
+    qkv = torch.randn(T, (Hq + 2 * Hk) * D, generator=g).to(torch.bfloat16).cuda()
+    wq = (1.0 + 0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).cuda() if with_norm else None
+    wk = (1.0 + 0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).cuda() if with_norm else None
+    cfg = StackConfig(layers=1, hidden=256, q_heads=Hq, kv_heads=Hk, head_dim=D, intermediate=256, vocab=256)
+    cos, sin = rope_tables(cfg, cap, "cuda")
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    par = depth = None
+    if tree:
+        pl = [-1] + [int(torch.randint(-1, t, (1,), generator=g)) for t in range(1, T)]
+        dl = []
+        for t in range(T):
+            dl.append(0 if pl[t] < 0 else dl[pl[t]] + 1)
+        par = torch.tensor(pl, dtype=torch.int32, device="cuda")
+        depth = torch.tensor(dl, dtype=torch.int32, device="cuda")
+    scale = 1.0 / np.sqrt(D)
+    scratch = card.attn_scratch(T, Hq, Hk, D, S)
+    Ka, Va = K0.clone(), V0.clone()
+    q = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+    want = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+    card.norm_rope_kv(qkv, wq, wk, 1e-6, cos, sin, n0t, Ka, Va, q, Hq, Hk, D, depth=depth)
+    card.attn_decode(q, Ka, Va, want, n0t, Hq, Hk, D, scale, S, scratch, par=par)
+    assert bool(torch.isfinite(want.float()).all())
+    scratch.fill_(float("nan"))
+    for rep in range(2):
+        Kb, Vb = K0.clone(), V0.clone()
+        got = torch.zeros_like(want)
+        card.attn_decode_qkv_rows(qkv, wq, wk, 1e-6, cos, sin, n0t, Kb, Vb, got, Hq, Hk, D, scale, S, scratch,
+                                  depth=depth, par=par)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), rep
+        same = lambda a, b: torch.equal(a.view(torch.int16), b.view(torch.int16))
+        assert same(Ka, Kb) and same(Va, Vb)
+        assert bool(torch.isfinite(Kb[:, n0:n0 + T].float()).all())  # the rows were written
+
+
+def test_attn_rows_from_the_fused_qkv_rows_only_where_it_fits(card):
+    """shapes the fused pass does not take are named by the query and refused by the call: one row, more than 32
+    (row, head) pairs a kv head, spans of 256 keys, 8 query heads a kv head"""
+    D = 128
+    assert card.attn_rows_fused(8, 32, 8, D, 4608, 36)
+    for T, Hq, Hk, cap, S in ((1, 32, 8, 4608, 36), (9, 32, 8, 4608, 36), (8, 32, 8, 4608, 18), (4, 16, 2, 512, 4)):
+        assert not card.attn_rows_fused(T, Hq, Hk, D, cap, S)
+        qkv = torch.zeros(T, (Hq + 2 * Hk) * D, dtype=torch.bfloat16, device="cuda")
+        K = torch.zeros(Hk, cap, D, dtype=torch.bfloat16, device="cuda")
+        att = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+        tab = torch.zeros(cap, D, dtype=torch.bfloat16, device="cuda")
+        n0t = torch.zeros(1, dtype=torch.int32, device="cuda")
+        with pytest.raises(Exception, match="attn_decode_qkv_rows"):
+            card.attn_decode_qkv_rows(qkv, None, None, 1e-6, tab, tab, n0t, K, K.clone(), att, Hq, Hk, D, 0.1, S,
+                                      card.attn_scratch(T, Hq, Hk, D, S))
+
+
 def test_silu_mul_and_argmax_and_embed(card):
     gu = acts_bf16(3, 2 * 768, seed=630)
     m = torch.empty(3, 768, dtype=torch.bfloat16, device="cuda")

@@ -117,7 +117,7 @@ def test_fused_matvec_outputs_stay_inside(card, M):
     x.check("add_rmsnorm: x")
 
 
-@pytest.mark.parametrize("n0,T,S", [(4095, 1, 32), (100, 1, 5), (63, 3, 7), (0, 1, 1)])
+@pytest.mark.parametrize("n0,T,S", [(4095, 1, 32), (100, 1, 5), (63, 3, 7), (0, 1, 1), (125, 8, 2), (250, 3, 2)])
 def test_attention_outputs_stay_inside(card, n0, T, S):
     Hq, Hk, D = 32, 8, 128
     cap = n0 + T + 2
@@ -142,6 +142,12 @@ def test_attention_outputs_stay_inside(card, n0, T, S):
         for f, what in ((K, "K"), (V, "V"), (att2, "att"), (scratch, "scratch")):
             f.check(f"attn_decode_qkv: {what}")
         assert torch.equal(att2.t, att.t)
+    if card.attn_rows_fused(T, Hq, Hk, D, cap, S):
+        att3 = Fenced((T, Hq * D), torch.bfloat16)
+        card.attn_decode_qkv_rows(qkv, wq, wq, 1e-6, cos, sin, n0t, K.t, V.t, att3.t, Hq, Hk, D, D**-0.5, S, scratch.t)
+        for f, what in ((K, "K"), (V, "V"), (att3, "att"), (scratch, "scratch")):
+            f.check(f"attn_decode_qkv_rows: {what}")
+        assert torch.equal(att3.t, att.t)
 
 
 @pytest.mark.parametrize("T", [1, 5])
