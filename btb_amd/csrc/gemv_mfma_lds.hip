@@ -17,6 +17,8 @@
 // so a row's bits depend on neither M nor R nor the launch.
 // The reference's counterpart is btb_gemv_mma_bf16 (native/cuda/btb_gemv_mma.cuh:1-214); it has no packed forms.
 
+#include <type_traits>
+
 #include "btb_common.hpp"
 #include "btb_formats.hpp"
 #include "btb_tuning.hpp"
@@ -380,7 +382,9 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
         MF::template scales<SB>(mat, rn, lg, s0 + sb * SB, nsteps, scl);
 #pragma unroll
         for (int q = 0; q < NLD; ++q) {
-            const uint8_t* base = mat.w + (size_t)(tile * 16 + q * RPI) * rowbytes + (size_t)(s0 + sb * SB) * MF::STEPB;
+            // half > 0: the tile's rows 0..7 are gate rows 8 tile .., its rows 8..15 the up rows of the same outputs
+            const int row0 = half ? tile * 8 + q * RPI + (q * RPI >= 8 ? half * 16 - 8 : 0) : tile * 16 + q * RPI;
+            const uint8_t* base = mat.w + (size_t)row0 * rowbytes + (size_t)(s0 + sb * SB) * MF::STEPB;
             if (lane_byte < valid) raw[q] = load_stream16(reinterpret_cast<const uint4*>(base + goff));
         }
         if constexpr (TWO) {
@@ -396,14 +400,16 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
 
     const int ntiles = R / 16;
     const int nsb = (n + SB - 1) / SB;
-    // The tiles a workgroup visits: blockIdx.x, + gridDim.x, ... - or, with half > 0 (W is a gate matrix over an up
-    // matrix, half tiles each, and y their fold bf16(bf16(silu(g)) * u), [M, R / 2]), the gate tile and the up tile of
-    // each such pair in turn
+    // The tiles a workgroup visits: blockIdx.x, + gridDim.x, ... With half > 0 (W is a gate matrix over an up matrix,
+    // half tiles of 16 rows each, and y their fold bf16(bf16(silu(g)) * u), [M, R / 2]) a tile is eight gate rows over
+    // the eight up rows of the same outputs: as many tiles as without the fold, so the grid walks them the same way
+    // (taking a gate tile and then its up tile, a pair a workgroup, made the last turn two tiles long: [19456 x 2560]
+    // on 256 CUs took six tiles' time where the plain matvec takes five).
+    static_assert(RPI <= 8 || !std::is_same<MF, MfBf16>::value, "a load's rows lie in one half of a folded tile");
     const int grid = (int)gridDim.x, first = (int)blockIdx.x;
-    auto tile_of = [&](int k) { return half ? first + (k >> 1) * grid + (k & 1) * half : first + k * grid; };
-    auto live = [&](int k) { return half ? first + (k >> 1) * grid < half : first + k * grid < ntiles; };
+    auto tile_of = [&](int k) { return first + k * grid; };
+    auto live = [&](int k) { return first + k * grid < ntiles; };
     int tile = tile_of(0);
-    f32x4 gate = f32x4{0.f, 0.f, 0.f, 0.f};  // the folding wave's gate sums, kept until the up tile's are there
     // the escapes of the wave's rows of a tile: their indices are asked for a tile ahead, the rest of what they need
     // while the tile's first sub-block is multiplied
     [[maybe_unused]] typename MF::Tail tl, tnext;
@@ -506,19 +512,20 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
             }
             const int m = wv * 16 + li;
             if (half) {
-                if ((turn & 1) == 0) {
-                    gate = s;
-                } else if (m < M) {
+                // lanes of row groups 0, 1 hold gate sums, the lanes 32 further on the up sums of the same outputs
+                const f32x4 up = f32x4{__shfl_xor(s.x, 32, WAVE), __shfl_xor(s.y, 32, WAVE), __shfl_xor(s.z, 32, WAVE),
+                                       __shfl_xor(s.w, 32, WAVE)};
+                if (m < M && lg < 2) {
                     // the arithmetic of the stand-alone fold over the two rounded outputs (silu_pair)
                     auto fold = [](float g, float u) {
                         const float gb = bfround(g), ub = bfround(u);
                         return f32_bf16(bfround(gb / (1.f + expf(-gb))) * ub);
                     };
-                    uint16_t* o = y + (size_t)m * (R / 2) + (tile - half) * 16 + lg * 4;
-                    o[0] = fold(gate.x, s.x);
-                    o[1] = fold(gate.y, s.y);
-                    o[2] = fold(gate.z, s.z);
-                    o[3] = fold(gate.w, s.w);
+                    uint16_t* o = y + (size_t)m * (R / 2) + tile * 8 + lg * 4;
+                    o[0] = fold(s.x, up.x);
+                    o[1] = fold(s.y, up.y);
+                    o[2] = fold(s.z, up.z);
+                    o[3] = fold(s.w, up.w);
                 }
             } else {
                 const int row = tile * 16 + lg * 4;
@@ -539,7 +546,7 @@ static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, i
                           int half = 0) {
     constexpr int SLAB = 16 * (SB * MF::STEPB + 16) + (MF::STEPB2 > 0 ? 16 * (SB * MF::STEPB2 + 16) : 0) + MF::TAIL_BYTES;
     const size_t lds = (size_t)KS * SLAB + 2 * (size_t)KS * MT * WAVE * sizeof(f32x4);
-    const int ntiles = half ? half : R / 16;  // the units the grid walks: tiles, or pairs of a gate and an up tile
+    const int ntiles = R / 16;
     int per_cu = tuning("mfma_wgs_per_cu");
     if (per_cu <= 0) per_cu = 12 / KS;  // twelve waves a CU: what the kernel's registers leave resident
     const int cap = device_info().cus * per_cu;

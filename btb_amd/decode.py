@@ -15,6 +15,7 @@ memory.
 from __future__ import annotations
 
 import math
+import os
 from dataclasses import dataclass
 from typing import Any
 
@@ -159,6 +160,8 @@ class DecodeStep:
         self.fused = bool(fused) and all(getattr(m, "fusable", False) for m in lins)
         # a pass's q / k norm, rope and cache write ride in its attention kernel where that kernel takes the pass's
         # shape - in the fused sequence, and in the other one too unless the caller asked for a launch per operator
+        # ... and the activation in the gate / up matvec's epilogue (bf16 matrices)
+        self.glu_fold = (chosen or bool(fused)) and T > 1 and os.environ.get("BTB_GLU_FOLD", "1") != "0"
         self.rows_attn_fused = (chosen or bool(fused)) and T > 1 and bool(
             card.attn_rows_fused(T, cfg.q_heads, cfg.kv_heads, cfg.head_dim, self.cap, self.S))
         # the handoff to the host: token, cache length and the GPU's clock in pinned memory
@@ -316,8 +319,13 @@ class DecodeStep:
                               par=self.par)
             w[L + "o"].matvec(self.att, self.y)
             k.add_rmsnorm(self.h, self.y, w[L + "ln2"], cfg.eps, self.x)
-            w[L + "gu"].matvec(self.x, self.gu)
             down = w[L + "down"]
+            if self.glu_fold and isinstance(w[L + "gu"].w, torch.Tensor):
+                k.gemv_glu_silu(w[L + "gu"].w, self.x, self.m)
+                down.matvec(self.m, self.y)
+                y_prev = self.y
+                continue
+            w[L + "gu"].matvec(self.x, self.gu)
             if self.fold_silu and isinstance(down.w, torch.Tensor):
                 k.gemv_silu(down.w, self.gu, self.y)
             else:
