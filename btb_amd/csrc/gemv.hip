@@ -281,6 +281,8 @@ bool mfma_lds_fits_bf16(int R, int C);
 bool mfma_lds_fits_packed(int R, int C);
 int32_t gemv_mfma_lds_bf16(const void* w, const void* x, void* y, int R, int C, int M, hipStream_t st);
 int32_t gemv_mfma_lds_glu_bf16(const void* w, const void* x, void* y, int I, int C, int M, hipStream_t st);
+bool mfma_lds_norm_fits(int R, int C, int M);
+int32_t gemv_mfma_lds_norm_bf16(const void* w, const XArgs& xa, void* y, int R, int C, int M, int I, hipStream_t st);
 int32_t gemv_mfma_lds_fp8(const void* w, const float* scales, int sc, int bm, int bn, const void* x, void* y, int R,
                           int C, int M, hipStream_t st);
 int32_t gemv_mfma_lds_mxfp4(const void* blocks, const void* scales, const void* x, void* y, int R, int C, int M,
@@ -337,6 +339,14 @@ static int32_t embed_args(const void* table, const int32_t* ids, size_t vocab, c
     *xa = XArgs{static_cast<const uint16_t*>(table), nullptr, static_cast<const uint16_t*>(norm_w),
                 static_cast<uint16_t*>(h_out), eps, centered ? 1 : 0, ids, (int)vocab};
     return OK;
+}
+
+// whether a matvec with the add + norm folded in goes to the matrix cores: a shape that kernel makes the rows for,
+// every row of the residual stream a whole number of 8-byte words at an 8-byte boundary
+static bool norm_on_mfma(const XArgs& xa, size_t R, size_t C, size_t M, bool glu) {
+    auto al8 = [](const void* p) { return (reinterpret_cast<uintptr_t>(p) & 7u) == 0; };
+    return tuning("gemv_no_mfma") <= 0 && tuning("mfma_lds") != 0 && C % 32 == 0 && (!glu || (R / 2) % 16 == 0) &&
+           mfma_lds_norm_fits((int)R, (int)C, (int)M) && al8(xa.x) && al8(xa.y) && al8(xa.norm_w) && al8(xa.h_out);
 }
 
 static int32_t p12_params(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
@@ -424,6 +434,9 @@ int32_t btb_hip_gemv_bf16_norm(const void* w, const void* h_in, const void* y, c
     if (!aligned16(w) || !aligned2(out) || (glu && R % 2 != 0)) return ERR_DOMAIN;
     FmtBf16::Params p{static_cast<const uint4*>(w)};
     hipStream_t st = static_cast<hipStream_t>(stream);
+    // the verify widths: the matrix cores, the rows made by each workgroup ahead of its first tile
+    if (norm_on_mfma(xa, R, C, M, glu != 0))
+        return gemv_mfma_lds_norm_bf16(w, xa, out, (int)R, (int)C, (int)M, glu ? (int)(R / 2) : 0, st);
     return glu ? run_rows<FmtBf16, X_ADDNORM, E_GLU>(p, xa, out, R, C, M, st)
                : run_rows<FmtBf16, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, st);
 }
@@ -439,6 +452,8 @@ int32_t btb_hip_gemv_bf16_embed_norm(const void* w, const void* table, const int
     if (rc != OK) return rc;
     if (!aligned16(w) || !aligned2(out)) return ERR_DOMAIN;
     FmtBf16::Params p{static_cast<const uint4*>(w)};
+    if (norm_on_mfma(xa, R, C, M, false))
+        return gemv_mfma_lds_norm_bf16(w, xa, out, (int)R, (int)C, (int)M, 0, static_cast<hipStream_t>(stream));
     return run_rows<FmtBf16, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, static_cast<hipStream_t>(stream));
 }
 

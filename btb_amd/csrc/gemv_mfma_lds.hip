@@ -21,6 +21,7 @@
 
 #include "btb_common.hpp"
 #include "btb_formats.hpp"
+#include "btb_stream.hpp"
 #include "btb_tuning.hpp"
 
 #include "../../include/btb_hip.h"
@@ -299,9 +300,19 @@ struct MfP12 {
 // registers); SB steps per sub-block (a slab holds 16 rows x SB steps). XS: the x fragments are not held - each
 // sub-block's come in with its weights (x is small and stays in L2), so a row may be as long as SPW allows without
 // the registers x-stationary rows of that length would take
-template <class MF, int KS, int MT, int SPW, int SB, bool XS = false>
+// XN: x is not given but made - the residual add and RMSNorm of a.x (+ a.y) with a.norm_w, as add_rmsnorm_kernel
+// computes them (or the embedding rows a.ids name) - by every workgroup for itself before its first tile, the first
+// workgroup also writing the new residual to a.h_out. 256 threads take a row, word i + 256 k of it thread i (the order
+// that kernel sums in, so the bits are its bits); the rows lie in LDS where the slabs will be, a wave takes its
+// fragments from there and holds them as it holds a given x. Making the rows costs a workgroup 5 us (5 rows) to 8.6 us
+// (16) on MI355X ([6144 x 2560]: 14.3 / 15.6 / 19.3 us at 5 / 8 / 16 rows against 9.2 / 9.7 / 10.7 for the matvec
+// alone), about twice what a launch of add_rmsnorm ahead of the plain matvec adds (2.5 us back to back): this is the
+// entry point's kernel for passes of five rows and more - passes of four rows of the vector kernel took twice as
+// long - not the fastest way to run such a pass, which is the two launches.
+template <class MF, int KS, int MT, int SPW, int SB, bool XS = false, bool XN = false>
 __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, const uint4* __restrict__ x,
-                                                         uint16_t* __restrict__ y, int R, int C, int M, int half) {
+                                                         uint16_t* __restrict__ y, int R, int C, int M, int half,
+                                                         XArgs xa) {
     constexpr int ROWB = SB * MF::STEPB;      // bytes a row contributes to a sub-block
     constexpr int STRIDE = ROWB + 16;         // the slab's row stride: 4 banks past a multiple of 64, so the sixteen
                                               // rows a fragment read touches fall in sixteen different bank groups
@@ -339,9 +350,38 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
 #pragma unroll
     for (int t = 0; t < MT; ++t) {
         xr[t] = x + (size_t)min(t * 16 + li, M - 1) * chunk4 + lg + (size_t)s0 * 4;
-        if constexpr (!XS) {
+        if constexpr (!XS && !XN) {
 #pragma unroll
             for (int i = 0; i < SPW; ++i) xb[t][i] = i < n ? xr[t][i * 4] : make_uint4(0, 0, 0, 0);
+        }
+    }
+    // XN: the rows' words, asked for ahead of the first weights (which would otherwise return first, in order)
+    static_assert(!XN || (KS % 4 == 0 && MT == 1 && !XS), "256 threads a row, one tile of rows, fragments held");
+    constexpr int XN_GROUPS = XN ? KS / 4 : 1;       // rows in the making at once
+    constexpr int XN_RPG = XN ? 16 / XN_GROUPS : 1;  // rows a group of 256 threads makes, one after the other
+    constexpr int XN_PER = 3;                        // 8-byte words of a row a thread takes: rows up to 3072 values
+    const int xn_gid = threadIdx.x >> 8, xn_t = threadIdx.x & 255, xn_n4 = C / 4;
+    const int xn_stride = C * 2 + 16;  // a row's bytes in LDS: 4 banks past a multiple of 64, as a slab's rows
+    [[maybe_unused]] uint2 xn_h[XN_RPG][XN_PER], xn_y[XN_RPG][XN_PER], xn_w[XN_PER];
+    if constexpr (XN) {
+        const uint2* ws = reinterpret_cast<const uint2*>(xa.norm_w);
+#pragma unroll
+        for (int q = 0; q < XN_PER; ++q) xn_w[q] = ws[min(q * 256 + xn_t, xn_n4 - 1)];
+#pragma unroll
+        for (int r = 0; r < XN_RPG; ++r) {
+            const int m = r * XN_GROUPS + xn_gid;
+            if (m < M) {
+                size_t hrow = (size_t)m;
+                if (xa.ids != nullptr) hrow = (size_t)min(max(xa.ids[m], 0), xa.vocab - 1);
+                const uint2* hs = reinterpret_cast<const uint2*>(xa.x + hrow * C);
+                const uint2* ys = xa.y == nullptr ? hs : reinterpret_cast<const uint2*>(xa.y + (size_t)m * C);
+#pragma unroll
+                for (int q = 0; q < XN_PER; ++q) {
+                    const int i = min(q * 256 + xn_t, xn_n4 - 1);
+                    xn_h[r][q] = hs[i];
+                    xn_y[r][q] = ys[i];  // no y: h again, unused
+                }
+            }
         }
     }
     [[maybe_unused]] uint4 xs[MT][XS ? SB : 1];  // XS: the x fragments of the sub-block in flight
@@ -419,6 +459,71 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
         if (tile < ntiles) tnext = MF::tail_begin(mat, MF::tail_span(mat, tile * 16 + wv * TROWS, TROWS), lane);
     }
     if (tile < ntiles && nsb > 0) request(tile, 0);
+    if constexpr (XN) {
+        float* red = reinterpret_cast<float*>(lds + 16 * xn_stride);  // [16 rows][4 waves of the row's group]
+        const bool has_y = xa.y != nullptr;
+        const bool writer = blockIdx.x == 0 && xa.h_out != nullptr;
+#pragma unroll
+        for (int r = 0; r < XN_RPG; ++r) {
+            const int m = r * XN_GROUPS + xn_gid;
+            if (m < M) {
+                float ss = 0.f;
+#pragma unroll
+                for (int q = 0; q < XN_PER; ++q) {
+                    const int i = q * 256 + xn_t;
+                    const bool in_row = i < xn_n4;
+                    float f[4] = {bf16lo_f32(xn_h[r][q].x), bf16hi_f32(xn_h[r][q].x), bf16lo_f32(xn_h[r][q].y),
+                                  bf16hi_f32(xn_h[r][q].y)};
+                    const float g[4] = {bf16lo_f32(xn_y[r][q].x), bf16hi_f32(xn_y[r][q].x), bf16lo_f32(xn_y[r][q].y),
+                                        bf16hi_f32(xn_y[r][q].y)};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const float sum = bfround(f[e] + g[e]);
+                        f[e] = has_y ? sum : f[e];
+                        const float sq = fmaf(f[e], f[e], ss);
+                        ss = in_row ? sq : ss;
+                    }
+                    const uint2 hb = make_uint2(f32x2_bf16(f[0], f[1]), f32x2_bf16(f[2], f[3]));
+                    if (in_row) {
+                        *reinterpret_cast<uint2*>(lds + (size_t)m * xn_stride + (size_t)i * 8) = hb;
+                        if (writer) reinterpret_cast<uint2*>(xa.h_out + (size_t)m * C)[i] = hb;
+                    }
+                }
+                ss = group_sum<64>(ss);
+                if (lane == 0) red[m * 4 + (wv & 3)] = ss;
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int r = 0; r < XN_RPG; ++r) {
+            const int m = r * XN_GROUPS + xn_gid;
+            if (m < M) {
+                const float sum = ((red[m * 4] + red[m * 4 + 1]) + red[m * 4 + 2]) + red[m * 4 + 3];
+                const float rstd = rsqrtf(sum / (float)C + xa.eps);
+#pragma unroll
+                for (int q = 0; q < XN_PER; ++q) {
+                    const int i = q * 256 + xn_t;
+                    if (i < xn_n4) {
+                        uint2* slot = reinterpret_cast<uint2*>(lds + (size_t)m * xn_stride + (size_t)i * 8);
+                        const uint2 hb = *slot;
+                        const float f[4] = {bf16lo_f32(hb.x), bf16hi_f32(hb.x), bf16lo_f32(hb.y), bf16hi_f32(hb.y)};
+                        const float g[4] = {bf16lo_f32(xn_w[q].x), bf16hi_f32(xn_w[q].x), bf16lo_f32(xn_w[q].y),
+                                            bf16hi_f32(xn_w[q].y)};
+                        float o[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o[e] = f[e] * rstd * (xa.centered ? 1.f + g[e] : g[e]);
+                        *slot = make_uint2(f32x2_bf16(o[0], o[1]), f32x2_bf16(o[2], o[3]));
+                    }
+                }
+            }
+        }
+        __syncthreads();
+        const uint8_t* xrow = lds + (size_t)min(li, M - 1) * xn_stride + (size_t)(s0 * 32 + lg * 8) * 2;
+#pragma unroll
+        for (int i = 0; i < SPW; ++i)
+            xb[0][i] = i < n ? *reinterpret_cast<const uint4*>(xrow + i * 64) : make_uint4(0, 0, 0, 0);
+        __syncthreads();  // the rows have been read: the slabs may take their place
+    }
     for (int turn = 0; live(turn); ++turn) {
         tile = tile_of(turn);
         f32x4 acc[MT];
@@ -541,11 +646,15 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
     }
 }
 
-template <class MF, int KS, int MT, int SPW, int SB, bool XS = false>
+template <class MF, int KS, int MT, int SPW, int SB, bool XS = false, bool XN = false>
 static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st,
-                          int half = 0) {
+                          int half = 0, const XArgs& xa = XArgs{}) {
     constexpr int SLAB = 16 * (SB * MF::STEPB + 16) + (MF::STEPB2 > 0 ? 16 * (SB * MF::STEPB2 + 16) : 0) + MF::TAIL_BYTES;
-    const size_t lds = (size_t)KS * SLAB + 2 * (size_t)KS * MT * WAVE * sizeof(f32x4);
+    size_t lds = (size_t)KS * SLAB + 2 * (size_t)KS * MT * WAVE * sizeof(f32x4);
+    if (XN) {  // the made rows (and the sums' exchange) lie where the slabs will be
+        const size_t rows = 16 * ((size_t)C * 2 + 16) + 16 * 4 * sizeof(float);
+        if (rows > lds) lds = rows;
+    }
     const int ntiles = R / 16;
     int per_cu = tuning("mfma_wgs_per_cu");
     if (per_cu <= 0) per_cu = 12 / KS;  // twelve waves a CU: what the kernel's registers leave resident
@@ -553,14 +662,14 @@ static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, i
     // whole turns of the grid over the tiles: the smallest grid that walks them in ceil(ntiles / cap) turns
     const int turns = (ntiles + cap - 1) / cap;
     const int grid = (ntiles + turns - 1) / turns;
-    auto kern = gemv_mfma_lds<MF, KS, MT, SPW, SB, XS>;
+    auto kern = gemv_mfma_lds<MF, KS, MT, SPW, SB, XS, XN>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(KS * 64), lds, st, mat, static_cast<const uint4*>(x),
-                       static_cast<uint16_t*>(y), R, C, M, half);
+                       static_cast<uint16_t*>(y), R, C, M, half, xa);
     return hip_status(hipGetLastError(), "gemv_mfma launch");
 }
 
@@ -625,6 +734,31 @@ int32_t gemv_mfma_lds_bf16(const void* w, const void* x, void* y, int R, int C, 
 // W = [gate; up], 2I rows: y [M, I] = bf16(bf16(silu(g)) * u)
 int32_t gemv_mfma_lds_glu_bf16(const void* w, const void* x, void* y, int I, int C, int M, hipStream_t st) {
     return run_lds<MfBf16>(MfBf16::Mat{static_cast<const uint8_t*>(w)}, x, y, 2 * I, C, M, st, I / 16);
+}
+// ... with x made by the residual add and RMSNorm (XArgs); I > 0: W = [gate; up] and y the fold, as above. Rows of
+// 1312 .. 2560 columns (the widths whose workgroups are 512 threads: two rows in the making at once), 16 rows of the
+// residual stream a pass.
+bool mfma_lds_norm_fits(int R, int C, int M) {
+    return lds_fits<MfBf16>(R, C) && C / 32 > 40 && C / 32 <= 80 && M >= 5 && tuning("mfma_lds_norm") != 0;
+}
+int32_t gemv_mfma_lds_norm_bf16(const void* w, const XArgs& xa, void* y, int R, int C, int M, int I, hipStream_t st) {
+    const MfBf16::Mat mat{static_cast<const uint8_t*>(w)};
+    const int half = I > 0 ? I / 16 : 0;
+    XArgs a = xa;
+    uint16_t* yp = static_cast<uint16_t*>(y);
+    const size_t yrow = I > 0 ? (size_t)I : (size_t)R;
+    for (int m0 = 0; m0 < M; m0 += 16) {
+        const int32_t rc = launch_lds<MfBf16, 8, 1, 10, 8, false, true>(mat, nullptr, yp + (size_t)m0 * yrow, R, C,
+                                                                        M - m0 < 16 ? M - m0 : 16, st, half, a);
+        if (rc != OK) return rc;
+        if (a.ids != nullptr)
+            a.ids += 16;
+        else
+            a.x += (size_t)16 * C;
+        if (a.y != nullptr) a.y += (size_t)16 * C;
+        if (a.h_out != nullptr) a.h_out += (size_t)16 * C;
+    }
+    return OK;
 }
 int32_t gemv_mfma_lds_fp8(const void* w, const float* scales, int sc, int bm, int bn, const void* x, void* y, int R,
                           int C, int M, hipStream_t st) {

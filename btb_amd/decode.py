@@ -15,7 +15,6 @@ memory.
 from __future__ import annotations
 
 import math
-import os
 from dataclasses import dataclass
 from typing import Any
 
@@ -146,9 +145,12 @@ class DecodeStep:
         self.S = int(attn_spans)
         self.scratch = card.attn_scratch(T, Hq, Hk, D, self.S, dev)
         # Which sequence: up to three rows the fused launches win (fewer launches, every matvec on the streaming
-        # kernel); from four rows on the one-launch-per-operator sequence does, whose matvecs take the matrix cores
-        # at five rows and more while a fused matvec runs as passes of four rows (measured on the 36-layer
-        # [2560 / 9728] stack, bf16: 4.3 against 4.0 ms at 4 rows, 7.1 against 4.6 at 8, 12.6 against 5.9 at 16).
+        # kernel); from four rows on the sequence with the residual add + norm as launches of their own does. From
+        # five rows its matvecs take the matrix cores; a matvec with the add + norm folded in does too (every
+        # workgroup then makes the pass's normed rows for itself ahead of its first tile), but what that adds to each
+        # workgroup is more than the launch it saves (measured on the 36-layer [2560 / 9728] stack, bf16: 3.03
+        # against 2.97 ms at 5 rows, 3.28 against 3.12 at 8, 4.30 against 3.87 at 16; at 4 rows, vector kernels
+        # both ways, 4.3 against 4.0).
         chosen = fused is None
         if fused is None:
             fused = T <= 3
@@ -161,7 +163,7 @@ class DecodeStep:
         # a pass's q / k norm, rope and cache write ride in its attention kernel where that kernel takes the pass's
         # shape - in the fused sequence, and in the other one too unless the caller asked for a launch per operator
         # ... and the activation in the gate / up matvec's epilogue (bf16 matrices)
-        self.glu_fold = (chosen or bool(fused)) and T > 1 and os.environ.get("BTB_GLU_FOLD", "1") != "0"
+        self.glu_fold = (chosen or bool(fused)) and T > 1
         self.rows_attn_fused = (chosen or bool(fused)) and T > 1 and bool(
             card.attn_rows_fused(T, cfg.q_heads, cfg.kv_heads, cfg.head_dim, self.cap, self.S))
         # the handoff to the host: token, cache length and the GPU's clock in pinned memory

@@ -137,9 +137,16 @@ def test_glu_kernel_equals_matvec_then_silu_mul(card, M):
     assert torch.equal(got.view(torch.int16), want.view(torch.int16))
 
 
-@pytest.mark.parametrize("M,with_y,glu", [(1, True, False), (1, False, False), (2, True, True), (1, True, True)])
-def test_norm_folded_into_the_x_load_changes_no_bit(card, M, with_y, glu):
-    R, C = 6144, 2560
+@pytest.mark.parametrize("M,with_y,glu,C", [(1, True, False, 2560), (1, False, False, 2560), (2, True, True, 2560),
+                                              (1, True, True, 2560), (5, True, False, 2560), (8, True, True, 2560),
+                                              (8, False, False, 2560), (16, True, True, 2560), (13, True, False, 2560),
+                                              (7, True, True, 2048), (16, True, False, 1536), (4, True, False, 1280),
+                                              (17, True, False, 2560), (35, True, True, 2560)])
+def test_norm_folded_into_the_x_load_changes_no_bit(card, M, with_y, glu, C):
+    """the residual add + norm made by the matvec itself (the vector kernels up to four rows a pass; from five rows
+    the matrix cores, where the kernel makes the rows for rows of 1312 .. 2560 values, 16 rows a launch) against
+    add_rmsnorm followed by the matvec: the same output and the same new residual, bit for bit"""
+    R = 6144
     w = weights_bf16(R, C, seed=160).cuda()
     h = acts_bf16(M, C, seed=161).cuda()
     y = acts_bf16(M, C, seed=162).cuda() if with_y else None
@@ -154,6 +161,29 @@ def test_norm_folded_into_the_x_load_changes_no_bit(card, M, with_y, glu):
     assert torch.equal(h2.view(torch.int16), h1.view(torch.int16))
     with pytest.raises(ValueError):
         card.gemv_norm(w, h, y, nw, 1e-6, h, out, glu=glu)
+
+
+@pytest.mark.parametrize("M", [1, 3, 8, 16])
+def test_embedding_rows_gathered_by_the_first_matvec(card, M):
+    """`gemv_embed_norm` against embed + add_rmsnorm + gemv: the same output and residual rows, ids outside the table
+    clamped into it - on the vector kernels and, from five rows, on the matrix cores"""
+    R, C, vocab = 4096, 2560, 300
+    w = weights_bf16(R, C, seed=170).cuda()
+    table = acts_bf16(vocab, C, seed=171).cuda()
+    nw = (1.0 + 0.1 * torch.randn(C, generator=torch.Generator().manual_seed(172))).to(torch.bfloat16).cuda()
+    ids = torch.randint(0, vocab, (M,), generator=torch.Generator().manual_seed(173), dtype=torch.int32)
+    ids[0] = vocab + 5
+    ids = ids.cuda()
+    h1 = torch.empty(M, C, dtype=torch.bfloat16, device="cuda")
+    card.embed(table, ids, h1)
+    x1 = torch.empty_like(h1)
+    card.add_rmsnorm(h1, None, nw, 1e-6, x1)
+    want = card.gemv(w, x1)
+    h2 = torch.empty_like(h1)
+    out = torch.empty(M, R, dtype=torch.bfloat16, device="cuda")
+    card.gemv_embed_norm(w, table, ids, nw, 1e-6, h2, out)
+    assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+    assert torch.equal(h2.view(torch.int16), h1.view(torch.int16))
 
 
 def test_refusals_launch_nothing(card):
