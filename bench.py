@@ -526,7 +526,8 @@ def main() -> int:
             "head_dim": cfg.head_dim, "intermediate": cfg.intermediate, "vocab": cfg.vocab, "context": CTX,
             "weight_bytes_per_step": wbytes, "kv_bytes_per_step": kvbytes,
             "kernels_per_step": (2 + 6 * cfg.layers if args.rows == 1 else
-                                 3 + 7 * cfg.layers if step.fused else 5 + 10 * cfg.layers),
+                                 3 + (7 - step.rows_attn_fused) * cfg.layers if step.fused else
+                                 5 + (10 - step.rows_attn_fused - (step.glu_fold and not packed)) * cfg.layers),
             "host_wall_ms_per_step": round(wall * 1e3 / args.steps, 4),
             **({"tuning": tuned} if tuned else {}),
         },

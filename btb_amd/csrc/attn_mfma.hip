@@ -266,7 +266,8 @@ __global__ void __launch_bounds__(256) attn_decode_mfma_kernel(
                     *reinterpret_cast<uint4*>(q_lds + (id * 16 + c) * AM_QROW + ds * 64 + a * 16) = out[ds];
             } else {
                 const int tr = task_row(id), slot = n0 + tr;
-                if (tr < T && slot >= k_begin && slot < k_begin + AM_SPAN) {
+                // (a slot at or past the cache's capacity is not written: the caller has let the cache overflow)
+                if (tr < T && slot >= k_begin && slot < min(k_begin + AM_SPAN, cap)) {
                     uint16_t* kc = x.Kw + (size_t)g * hs + (size_t)slot * rs + a * 8;
                     uint16_t* vc = x.Vw + (size_t)g * hs + (size_t)slot * rs + a * 8;
 #pragma unroll
