@@ -352,6 +352,38 @@ def test_attn_rows_from_the_fused_qkv_rows(card, n0, T, Hq, Hk, tree, with_norm)
         assert bool(torch.isfinite(Kb[:, n0:n0 + T].float()).all())  # the rows were written
 
 
+@pytest.mark.parametrize("centered,positions", [(True, False), (False, True), (True, True)])
+def test_attn_rows_from_the_fused_qkv_rows_centered_weights_and_given_positions(card, centered, positions):
+    """the same equality with norm weights stored around zero (`centered`: the factor is 1 + w) and with a chain whose
+    rows stand at given depths"""
+    from btb_amd.decode import StackConfig, rope_tables
+
+    D, Hq, Hk, T, n0 = 128, 16, 4, 6, 200
+    cap = n0 + 24
+    S = -(-cap // 128)
+    g = gen(690)
+    K0 = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda()
+    V0 = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda()
+    qkv = torch.randn(T, (Hq + 2 * Hk) * D, generator=g).to(torch.bfloat16).cuda()
+    wq = (0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).cuda()
+    wk = (0.1 * torch.randn(D, generator=g)).to(torch.bfloat16).cuda()
+    cfg = StackConfig(layers=1, hidden=256, q_heads=Hq, kv_heads=Hk, head_dim=D, intermediate=256, vocab=256)
+    cos, sin = rope_tables(cfg, cap, "cuda")
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    depth = torch.tensor([0, 3, 4, 9, 10, 17], dtype=torch.int32, device="cuda") if positions else None
+    scale = 1.0 / np.sqrt(D)
+    scratch = card.attn_scratch(T, Hq, Hk, D, S)
+    Ka, Va, Kb, Vb = K0.clone(), V0.clone(), K0.clone(), V0.clone()
+    q = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+    want, got = torch.zeros_like(q), torch.zeros_like(q)
+    card.norm_rope_kv(qkv, wq, wk, 1e-6, cos, sin, n0t, Ka, Va, q, Hq, Hk, D, depth=depth, centered=centered)
+    card.attn_decode(q, Ka, Va, want, n0t, Hq, Hk, D, scale, S, scratch)
+    card.attn_decode_qkv_rows(qkv, wq, wk, 1e-6, cos, sin, n0t, Kb, Vb, got, Hq, Hk, D, scale, S, scratch, depth=depth,
+                              centered=centered)
+    assert torch.equal(got, want)
+    assert torch.equal(Ka, Kb) and torch.equal(Va, Vb)
+
+
 def test_attn_rows_from_the_fused_qkv_rows_only_where_it_fits(card):
     """shapes the fused pass does not take are named by the query and refused by the call: one row, more than 32
     (row, head) pairs a kv head, spans of 256 keys, 8 query heads a kv head"""
