@@ -69,6 +69,7 @@ static Knob g_knobs[] = {
     {"mfma_classic", {-1}},
     {"mfma_lds", {-1}},
     {"mfma_lds_norm", {-1}},
+    {"mfma_tile_rows", {-1}},
     {"mfma_stream_x", {-1}},
     {"mfma_direct", {-1}},
     {"mfma_direct_grid", {-1}},

@@ -309,10 +309,14 @@ struct MfP12 {
 // alone), about twice what a launch of add_rmsnorm ahead of the plain matvec adds (2.5 us back to back): this is the
 // entry point's kernel for passes of five rows and more - passes of four rows of the vector kernel took twice as
 // long - not the fastest way to run such a pass, which is the two launches.
-template <class MF, int KS, int MT, int SPW, int SB, bool XS = false, bool XN = false>
+// TR: the rows of a tile that are rows of the matrix (a divisor of R, a multiple of a load's rows): the tile is rows
+// TR tile .. + TR - 1, its other rows are not read and what the matrix cores make of them is not written. A template
+// argument: a load that a run-time test decides on is a load the compiler cannot count, and it then waits for all.
+template <class MF, int KS, int MT, int SPW, int SB, bool XS = false, bool XN = false, int TR = 16>
 __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, const uint4* __restrict__ x,
                                                          uint16_t* __restrict__ y, int R, int C, int M, int half,
                                                          XArgs xa) {
+    constexpr int tr = TR;
     constexpr int ROWB = SB * MF::STEPB;      // bytes a row contributes to a sub-block
     constexpr int STRIDE = ROWB + 16;         // the slab's row stride: 4 banks past a multiple of 64, so the sixteen
                                               // rows a fragment read touches fall in sixteen different bank groups
@@ -423,9 +427,11 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
 #pragma unroll
         for (int q = 0; q < NLD; ++q) {
             // half > 0: the tile's rows 0..7 are gate rows 8 tile .., its rows 8..15 the up rows of the same outputs
-            const int row0 = half ? tile * 8 + q * RPI + (q * RPI >= 8 ? half * 16 - 8 : 0) : tile * 16 + q * RPI;
+            const int row0 = half ? tile * 8 + q * RPI + (q * RPI >= 8 ? half * 16 - 8 : 0) : tile * tr + q * RPI;
             const uint8_t* base = mat.w + (size_t)row0 * rowbytes + (size_t)(s0 + sb * SB) * MF::STEPB;
-            if (lane_byte < valid) raw[q] = load_stream16(reinterpret_cast<const uint4*>(base + goff));
+            if (q * RPI < tr) {
+                if (lane_byte < valid) raw[q] = load_stream16(reinterpret_cast<const uint4*>(base + goff));
+            }
         }
         if constexpr (TWO) {
             const uint32_t valid2 = (uint32_t)(min(SB, n - sb * SB) * STEPB2);
@@ -438,7 +444,7 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
         }
     };
 
-    const int ntiles = R / 16;
+    const int ntiles = R / tr;
     const int nsb = (n + SB - 1) / SB;
     // The tiles a workgroup visits: blockIdx.x, + gridDim.x, ... With half > 0 (W is a gate matrix over an up matrix,
     // half tiles of 16 rows each, and y their fold bf16(bf16(silu(g)) * u), [M, R / 2]) a tile is eight gate rows over
@@ -633,36 +639,33 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
                     o[3] = fold(s.w, up.w);
                 }
             } else {
-                const int row = tile * 16 + lg * 4;
+                const int in_tile = lg * 4, row = tile * tr + in_tile;
                 if (m < M) {
                     uint16_t* o = y + (size_t)m * R + row;
-                    if (row + 0 < R) o[0] = f32_bf16(s.x);
-                    if (row + 1 < R) o[1] = f32_bf16(s.y);
-                    if (row + 2 < R) o[2] = f32_bf16(s.z);
-                    if (row + 3 < R) o[3] = f32_bf16(s.w);
+                    if (in_tile + 0 < tr && row + 0 < R) o[0] = f32_bf16(s.x);
+                    if (in_tile + 1 < tr && row + 1 < R) o[1] = f32_bf16(s.y);
+                    if (in_tile + 2 < tr && row + 2 < R) o[2] = f32_bf16(s.z);
+                    if (in_tile + 3 < tr && row + 3 < R) o[3] = f32_bf16(s.w);
                 }
             }
         }
     }
 }
 
-template <class MF, int KS, int MT, int SPW, int SB, bool XS = false, bool XN = false>
-static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st,
-                          int half = 0, const XArgs& xa = XArgs{}) {
+template <class MF, int KS, int MT, int SPW, int SB, bool XS, bool XN, int TR>
+static int32_t launch_lds_tr(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st,
+                             int half, const XArgs& xa, int cap) {
     constexpr int SLAB = 16 * (SB * MF::STEPB + 16) + (MF::STEPB2 > 0 ? 16 * (SB * MF::STEPB2 + 16) : 0) + MF::TAIL_BYTES;
     size_t lds = (size_t)KS * SLAB + 2 * (size_t)KS * MT * WAVE * sizeof(f32x4);
     if (XN) {  // the made rows (and the sums' exchange) lie where the slabs will be
         const size_t rows = 16 * ((size_t)C * 2 + 16) + 16 * 4 * sizeof(float);
         if (rows > lds) lds = rows;
     }
-    const int ntiles = R / 16;
-    int per_cu = tuning("mfma_wgs_per_cu");
-    if (per_cu <= 0) per_cu = 12 / KS;  // twelve waves a CU: what the kernel's registers leave resident
-    const int cap = device_info().cus * per_cu;
+    const int ntiles = R / TR;
     // whole turns of the grid over the tiles: the smallest grid that walks them in ceil(ntiles / cap) turns
     const int turns = (ntiles + cap - 1) / cap;
     const int grid = (ntiles + turns - 1) / turns;
-    auto kern = gemv_mfma_lds<MF, KS, MT, SPW, SB, XS, XN>;
+    auto kern = gemv_mfma_lds<MF, KS, MT, SPW, SB, XS, XN, TR>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
@@ -671,6 +674,31 @@ static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, i
     hipLaunchKernelGGL(kern, dim3(grid), dim3(KS * 64), lds, st, mat, static_cast<const uint4*>(x),
                        static_cast<uint16_t*>(y), R, C, M, half, xa);
     return hip_status(hipGetLastError(), "gemv_mfma launch");
+}
+
+template <class MF, int KS, int MT, int SPW, int SB, bool XS = false, bool XN = false>
+static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, int R, int C, int M, hipStream_t st,
+                          int half = 0, const XArgs& xa = XArgs{}) {
+    int per_cu = tuning("mfma_wgs_per_cu");
+    if (per_cu <= 0) per_cu = 12 / KS;  // twelve waves a CU: what the kernel's registers leave resident
+    const int cap = device_info().cus * per_cu;
+    // Rows a tile: sixteen, or twelve or ten where that fills the CUs better - what a launch takes is the busiest
+    // workgroup's rows, turns x rows a tile, and 2560 rows are 160 tiles of sixteen (one turn of 160 workgroups on 256
+    // CUs, sixteen rows each) but 256 tiles of ten; 6144 rows two turns of sixteen or of twelve. bf16 rows as they are
+    // and eight waves: a tile's loads are whole rows two at a time, and a row's bits do not depend on the tile it
+    // came in. Measured at 8 rows of x, MI355X: [2560 x 9728] 17.9 -> 15.0 us, [6144 x 2560] 11.2 -> 10.5,
+    // [2560 x 4096] 7.8 -> 7.6.
+    if constexpr (std::is_same<MF, MfBf16>::value && KS == 8 && !XN) {
+        if (half == 0 && tuning("mfma_tile_rows") != 0) {
+            auto rows_of = [&](int t) { return (long)((R / t + cap - 1) / cap) * t; };
+            int tr = 16;
+            if (R % 12 == 0 && rows_of(12) < rows_of(tr)) tr = 12;
+            if (R % 10 == 0 && rows_of(10) < rows_of(tr)) tr = 10;
+            if (tr == 12) return launch_lds_tr<MF, KS, MT, SPW, SB, XS, XN, 12>(mat, x, y, R, C, M, st, half, xa, cap);
+            if (tr == 10) return launch_lds_tr<MF, KS, MT, SPW, SB, XS, XN, 10>(mat, x, y, R, C, M, st, half, xa, cap);
+        }
+    }
+    return launch_lds_tr<MF, KS, MT, SPW, SB, XS, XN, 16>(mat, x, y, R, C, M, st, half, xa, cap);
 }
 
 // The split of the columns over a workgroup's waves comes from the row length alone: at most eight waves (a workgroup
