@@ -692,8 +692,12 @@ static int32_t launch_lds(const typename MF::Mat& mat, const void* x, void* y, i
         if (half == 0 && tuning("mfma_tile_rows") != 0) {
             auto rows_of = [&](int t) { return (long)((R / t + cap - 1) / cap) * t; };
             int tr = 16;
-            if (R % 12 == 0 && rows_of(12) < rows_of(tr)) tr = 12;
-            if (R % 10 == 0 && rows_of(10) < rows_of(tr)) tr = 10;
+            // (a lower tile has fewer bytes in flight a workgroup, which costs where the tiles are many: eight rows a
+            // tile took [9728 x 2560] from 12.7 to 14.2 us and the head [151936 x 2560] from 130 to 173 although both
+            // count fewer rows for the busiest workgroup that way - so only twelve and ten, and only for an eighth
+            // fewer rows or better)
+            if (R % 12 == 0 && rows_of(12) * 8 <= rows_of(16) * 7) tr = 12;
+            if (R % 10 == 0 && rows_of(10) * 8 <= rows_of(16) * 7 && rows_of(10) < rows_of(tr)) tr = 10;
             if (tr == 12) return launch_lds_tr<MF, KS, MT, SPW, SB, XS, XN, 12>(mat, x, y, R, C, M, st, half, xa, cap);
             if (tr == 10) return launch_lds_tr<MF, KS, MT, SPW, SB, XS, XN, 10>(mat, x, y, R, C, M, st, half, xa, cap);
         }
@@ -741,6 +745,7 @@ static int32_t run_lds(const typename MF::Mat& mat, const void* x, void* y, int 
         return OK;
     }
     constexpr int SBW = MF::SB_WIDE;
+    // (sixteen steps a sub-block for the streamed rows - twice the bytes in flight - spills: [2560 x 9728] 13.7 -> 22.5 us)
     // up to 28 steps a wave the x fragments stay in registers; longer rows (to 40 steps: 10240 columns) stream them
     const bool stream_x = nsteps > 8 * 28 || tuning("mfma_stream_x") > 0;
     for (int m0 = 0; m0 < M; m0 += 16) {
