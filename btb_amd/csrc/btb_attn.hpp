@@ -373,14 +373,10 @@ __device__ __forceinline__ void fold_streams(const AttnState<G>& st, int grp, in
 // Then every span's factor exp2(m_s - M) and scaled sum are made once, in parallel, and each output adds up its spans
 // in order. DEV: the states were written by other workgroups of the same launch (st_dev) and are read with ld_dev.
 // lds: 2 * S * G floats. `out` is the row's attention output, [Hq * 128]; `base` the state index of the head's span 0.
-// SPLIT (four query heads): the workgroup makes the outputs of two of them only - those numbered from 2 * part on
-template <int G, bool DEV, bool SPLIT = false>
+template <int G, bool DEV>
 __device__ __forceinline__ void merge_spans(uint16_t* out, int g, int S, size_t base, const float* part_m,
-                                            const float* part_l, const float* part_acc, float* lds, int tid,
-                                            int part = 0) {
-    static_assert(!SPLIT || G == 4, "two heads of four a workgroup");
-    // outputs a thread makes: (j, d) = ((tid + 256 (q + part)) / 128, tid % 128)
-    constexpr int NOUT = SPLIT ? 1 : G >= 2 ? G / 2 : 1;
+                                            const float* part_l, const float* part_acc, float* lds, int tid) {
+    constexpr int NOUT = G >= 2 ? G / 2 : 1;  // outputs a thread makes: (j, d) = ((tid + 256 q) / 128, tid % 128)
     constexpr int MS = NOUT <= 2 ? 40 : 20;   // spans a pass (a 4096-key cache is 33 to 36 spans: one pass)
     const float ninf = bits_f32(0xff800000u);
     auto ld = [](const float* p) { return DEV ? ld_dev(p) : *p; };
@@ -389,7 +385,7 @@ __device__ __forceinline__ void merge_spans(uint16_t* out, int g, int S, size_t 
     const int d = tid & (AD - 1);
     int jq[NOUT];
 #pragma unroll
-    for (int q = 0; q < NOUT; ++q) jq[q] = min((tid + 256 * (q + (SPLIT ? part : 0))) / AD, G - 1);
+    for (int q = 0; q < NOUT; ++q) jq[q] = min((tid + 256 * q) / AD, G - 1);
     const bool mine = tid < G * AD;  // a single query head: half the workgroup has no output
     float v[NOUT][MS];
     const int s_first = min(S, MS);

@@ -452,7 +452,6 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
 
 // the spans' states folded in span order: one workgroup per (row, kv head). Launched right after attn_decode_kernel,
 // it reads what that kernel wrote across a kernel boundary, so no fence or arrival count is needed.
-// With four query heads a kv head: two workgroups per (row, kv head), two heads each (gridDim.z = 2).
 template <int G>
 __global__ void __launch_bounds__(256) attn_merge_kernel(uint16_t* __restrict__ att, int Hq, int Hk, int S,
                                                          const float* __restrict__ part_m,
@@ -460,8 +459,8 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(uint16_t* __restrict__ 
                                                          const float* __restrict__ part_acc) {
     extern __shared__ float f_m[];  // [S][G] maxima / factors, then [S][G] sums
     const int g = blockIdx.x, t = blockIdx.y;
-    merge_spans<G, false, G == 4>(att + (size_t)t * Hq * ATT_D, g, S, ((size_t)t * Hk + g) * S, part_m, part_l, part_acc,
-                                  f_m, threadIdx.x, (int)blockIdx.z);
+    merge_spans<G, false>(att + (size_t)t * Hq * ATT_D, g, S, ((size_t)t * Hk + g) * S, part_m, part_l, part_acc, f_m,
+                          threadIdx.x);
 }
 
 __global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ m,
@@ -704,7 +703,7 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
     const float scale_log2 = scale * 1.4426950408889634f;
     const dim3 grid((unsigned)Hk, (unsigned)S, (unsigned)T);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const dim3 mgrid((unsigned)Hk, (unsigned)T, G == 4 ? 2u : 1u);
+    const dim3 mgrid((unsigned)Hk, (unsigned)T);
     const size_t mlds = 2 * S * G * sizeof(float);
 #define ATT(GG)                                                                                                      \
     hipLaunchKernelGGL(attn_decode_kernel<GG>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(q),              \
@@ -813,7 +812,7 @@ int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk,
     float* part_acc = workspace + 2 * Hq * S;
     const float scale_log2 = scale * 1.4426950408889634f;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const dim3 mgrid((unsigned)Hk, 1, G == 4 ? 2u : 1u);
+    const dim3 mgrid((unsigned)Hk, 1);
     const size_t mlds = 2 * S * G * sizeof(float);
     // query heads a workgroup takes: all G of its kv head, or fewer (the workgroups of one kv head are Hk apart in
     // the grid, which on this GPU - workgroups dealt to its eight dies in turn - keeps them on one die when Hk is 8)
@@ -895,7 +894,7 @@ int32_t btb_hip_attn_decode_qkv_rows(const void* qkv, const void* wq, const void
                                             Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, S, cap,
                                             st);
     if (rc != OK) return rc;
-    const dim3 mgrid((unsigned)Hk, (unsigned)T, G == 4 ? 2u : 1u);
+    const dim3 mgrid((unsigned)Hk, (unsigned)T);
     const size_t mlds = 2 * S * G * sizeof(float);
     if (G == 4)
         hipLaunchKernelGGL(attn_merge_kernel<4>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
