@@ -139,9 +139,9 @@ struct AmQkv {
 };
 constexpr int AM_QROW = 272;  // bytes a prepared q or k row takes in LDS: 256 + 16, as for V
 
-__host__ __device__ constexpr size_t am_lds_bytes(int G, int NQT, bool QKV) {
+__host__ __device__ constexpr size_t am_lds_bytes(int G, int NQT, bool QKV, int ZG = 1) {
     const size_t NQ = 16 * (size_t)NQT, TPW = NQ / (size_t)G;
-    const size_t weights = 4 * NQ * AM_PROW, heads = QKV ? (NQ + TPW) * AM_QROW : 0;
+    const size_t weights = 4 * NQ * AM_PROW, heads = QKV ? (NQ + (size_t)ZG * TPW) * AM_QROW : 0;
     return (size_t)AM_SPAN * AM_VROW + 2 * 4 * NQ * sizeof(float) + (weights > heads ? weights : heads);
 }
 
@@ -149,12 +149,14 @@ __host__ __device__ constexpr size_t am_lds_bytes(int G, int NQT, bool QKV) {
 // TBL: the cache has a row map (a template argument, not a test of the pointer: a branch between two loads makes the
 // compiler wait for the first before it issues the second, and the span's rows then arrive one trip at a time)
 // QKV: the rows come as the fused qkv rows, before the q / k norm and rope (DEPTH: with the rows' depths). The whole
-// pass is one workgroup's pairs then (T G <= 16 NQT <= 32). The q heads are prepared by the workgroup itself, a tile of
+// pass is one workgroup's pairs then (T G <= 16 NQT <= 32; ZG below: two workgroups'). The q heads are prepared by the workgroup itself, a tile of
 // 16 a wave, and passed through LDS - q never reaches memory - and so are the k heads of the pass's rows: the
 // workgroups whose span holds some of the pass's own slots *n0 .. *n0 + T - 1 write those and the raw v rows into the
 // cache, and take them from LDS in place of what they read from the cache, which is not written yet. The arithmetic is
-// norm_rope_kv_kernel's, then this kernel's.
-template <int G, int NQT, bool TBL, bool QKV, bool DEPTH>
+// norm_rope_kv_kernel's, then this kernel's. ZG = 2: the pass's pairs are two workgroups' (gridDim.z = 2, up to 64 pairs
+// a kv head): each prepares the q heads of its own rows and the k heads of all the rows, the first of the two writes
+// the cache.
+template <int G, int NQT, bool TBL, bool QKV, bool DEPTH, int ZG = 1>
 __global__ void __launch_bounds__(256) attn_decode_mfma_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ K, const uint16_t* __restrict__ V,
     const int32_t* __restrict__ n0p, const int32_t* __restrict__ par, int T, int Hq, int Hk, long long hs, long long rs,
@@ -168,7 +170,7 @@ __global__ void __launch_bounds__(256) attn_decode_mfma_kernel(
     float* red_m = reinterpret_cast<float*>(lds + AM_SPAN * AM_VROW);     // [4 waves][NQ]
     float* red_l = red_m + 4 * NQ;                                        // [4 waves][NQ]
     // [4 steps of 32 keys][NQ pairs][AM_PROW]; before the scores are done the prepared heads lie here:
-    // q [NQ][AM_QROW], then the pass's own k rows [TPW][AM_QROW]
+    // q [NQ][AM_QROW], then the pass's own k rows [ZG TPW][AM_QROW]
     uint8_t* p_lds = reinterpret_cast<uint8_t*>(red_l + 4 * NQ);
     const int g = blockIdx.x, sp = blockIdx.y, S = gridDim.y;
     const int t_base = blockIdx.z * TPW;
@@ -196,10 +198,10 @@ __global__ void __launch_bounds__(256) attn_decode_mfma_kernel(
     // then the pass's rows' k heads 16 at a time; wave wv takes tile wv. What does not depend on *n0 (the
     // heads' values, the norm weights, the rows' v) is asked for first, ahead of the span's K and V, so the norms are
     // done while those travel; the rope tables' rows come last.
-    constexpr int NKT = (TPW + 15) / 16, NTASK = QKV ? NQT + NKT : 0;
+    constexpr int NKT = (ZG * TPW + 15) / 16, NTASK = QKV ? NQT + NKT : 0;
     static_assert(NTASK <= 4, "a tile a wave");
     auto task_row = [&](int id) {  // the lane's row of the pass in tile id (a q tile: of its pair); unclamped
-        return id < NQT ? (id * 16 + c) / G : (id - NQT) * 16 + c;
+        return id < NQT ? t_base + (id * 16 + c) / G : (id - NQT) * 16 + c;
     };
     HeadTile task0;
     auto request = [&](int id, HeadTile& h) {
@@ -245,6 +247,10 @@ __global__ void __launch_bounds__(256) attn_decode_mfma_kernel(
         }
     }
     const int n0 = *n0p;
+    const int t_end = min(T, t_base + TPW);
+    // the keys any of the workgroup's rows may see end at n_max (a chain's last row, or the whole pass for a tree)
+    const int n_max = par != nullptr ? n0 + T : n0 + t_end;
+    const int k_lim = min(n_max, k_begin + AM_SPAN);
     if constexpr (QKV) {
         auto tables = [&](int id, HeadTile& h) {
             const int t = min(task_row(id), T - 1);
@@ -270,12 +276,17 @@ __global__ void __launch_bounds__(256) attn_decode_mfma_kernel(
                 if (tr < T && slot >= k_begin && slot < min(k_begin + AM_SPAN, cap)) {
                     uint16_t* kc = x.Kw + (size_t)g * hs + (size_t)slot * rs + a * 8;
                     uint16_t* vc = x.Vw + (size_t)g * hs + (size_t)slot * rs + a * 8;
+                    const bool seen = slot < k_lim;          // by one of this workgroup's rows (else: zeros, as below)
+                    const bool writes = ZG == 1 || blockIdx.z == 0;  // the cache's rows are written once
 #pragma unroll
                     for (int ds = 0; ds < 4; ++ds) {
                         *reinterpret_cast<uint4*>(kn_lds + tr * AM_QROW + ds * 64 + a * 16) = out[ds];
-                        *reinterpret_cast<uint4*>(v_lds + (slot - k_begin) * AM_VROW + ds * 64 + a * 16) = h.vrow[ds];
-                        *reinterpret_cast<uint4*>(kc + ds * 32) = out[ds];
-                        *reinterpret_cast<uint4*>(vc + ds * 32) = h.vrow[ds];
+                        *reinterpret_cast<uint4*>(v_lds + (slot - k_begin) * AM_VROW + ds * 64 + a * 16) =
+                            seen ? h.vrow[ds] : make_uint4(0u, 0u, 0u, 0u);
+                        if (writes) {
+                            *reinterpret_cast<uint4*>(kc + ds * 32) = out[ds];
+                            *reinterpret_cast<uint4*>(vc + ds * 32) = h.vrow[ds];
+                        }
                     }
                 }
             }
@@ -301,10 +312,6 @@ __global__ void __launch_bounds__(256) attn_decode_mfma_kernel(
             }
         }
     }
-    const int t_end = min(T, t_base + TPW);
-    // the keys any of the workgroup's rows may see end at n_max (a chain's last row, or the whole pass for a tree)
-    const int n_max = par != nullptr ? n0 + T : n0 + t_end;
-    const int k_lim = min(n_max, k_begin + AM_SPAN);
 
     // V into LDS, dead slots as zeros (weight 0 times whatever bits lie there must not make a NaN)
 #pragma unroll
@@ -460,19 +467,19 @@ static void launch_am(const uint16_t* q, const uint16_t* K, const uint16_t* V, c
 }
 
 // the variant that starts from the fused qkv rows: one workgroup per (kv head, span), the whole pass in it
-template <int G, int NQT>
+template <int G, int NQT, int ZG>
 static void launch_am_qkv(const AmQkv& x, const int32_t* n0, const int32_t* par, int T, int Hq, int Hk, long long hs,
                           long long rs, float scale_log2, float* part_m, float* part_l, float* part_acc, int S, int cap,
                           hipStream_t st) {
-    const size_t lds = am_lds_bytes(G, NQT, true);
-    static_assert(am_lds_bytes(G, NQT, true) <= 64 * 1024, "within what a workgroup gets without asking for more");
-    const dim3 grid((unsigned)Hk, (unsigned)S, 1u);
+    const size_t lds = am_lds_bytes(G, NQT, true, ZG);
+    static_assert(am_lds_bytes(G, NQT, true, ZG) <= 64 * 1024, "within what a workgroup gets without asking for more");
+    const dim3 grid((unsigned)Hk, (unsigned)S, (unsigned)ZG);
     const uint16_t* none = nullptr;
     if (x.depth != nullptr)
-        hipLaunchKernelGGL((attn_decode_mfma_kernel<G, NQT, false, true, true>), grid, dim3(256), lds, st, none, x.Kw, x.Vw,
-                           n0, par, T, Hq, Hk, hs, rs, scale_log2, part_m, part_l, part_acc, cap, 0, nullptr, x);
+        hipLaunchKernelGGL((attn_decode_mfma_kernel<G, NQT, false, true, true, ZG>), grid, dim3(256), lds, st, none, x.Kw,
+                           x.Vw, n0, par, T, Hq, Hk, hs, rs, scale_log2, part_m, part_l, part_acc, cap, 0, nullptr, x);
     else
-        hipLaunchKernelGGL((attn_decode_mfma_kernel<G, NQT, false, true, false>), grid, dim3(256), lds, st, none, x.Kw,
+        hipLaunchKernelGGL((attn_decode_mfma_kernel<G, NQT, false, true, false, ZG>), grid, dim3(256), lds, st, none, x.Kw,
                            x.Vw, n0, par, T, Hq, Hk, hs, rs, scale_log2, part_m, part_l, part_acc, cap, 0, nullptr, x);
 }
 
@@ -480,12 +487,13 @@ static void launch_am_qkv(const AmQkv& x, const int32_t* n0, const int32_t* par,
 bool attn_mfma_fits(size_t T, size_t G, int span) {
     return T >= 2 && span == AM_SPAN && (G == 2 || G == 4) && tuning("attn_mfma") != 0;
 }
-// ... and starting from the fused qkv rows: the whole pass in one workgroup's pairs, and a tile to prepare for each
-// wave at most - 32 pairs. (With 64 pairs a wave prepares two tiles one after the other and the code of the second no
-// longer overlaps the keys' flight: a pass of 16 rows x 4 heads took 27.2 us a layer so, against 23.4 us for
-// norm_rope_kv + the kernel above + the merge.)
+// ... and starting from the fused qkv rows: a tile to prepare for each wave at most, so 32 pairs a workgroup, and up to
+// 64 as two workgroups per (kv head, span). (64 pairs in one workgroup, a wave preparing two tiles one after the other,
+// loses: the second tile's code no longer overlaps the keys' flight - 27.2 us a layer at 16 rows x 4 heads against
+// 23.4 for norm_rope_kv + the kernel above + the merge.)
 bool attn_mfma_qkv_fits(size_t T, size_t G, int span) {
-    return attn_mfma_fits(T, G, span) && T * G <= 32 && tuning("attn_rows_fused") != 0;
+    const int knob = tuning("attn_rows_fused");  // 0: never; 1: one workgroup's 32 pairs only; else up to 64 in two
+    return attn_mfma_fits(T, G, span) && T * G <= (knob == 1 ? 32 : 64) && knob != 0;
 }
 
 // the partial states of every (row, head, span), for attn_merge_kernel
@@ -530,13 +538,13 @@ int32_t attn_decode_mfma_qkv(const void* qkv, const void* wq, const void* wk, fl
     x.Vw = static_cast<uint16_t*>(V);
     x.eps = eps;
     x.centered = centered;
-#define AMQ(GG, NN)                                                                                                   \
-    launch_am_qkv<GG, NN>(x, n0, par, (int)T, (int)Hq, (int)Hk, hs, rs, scale_log2, part_m, part_l, part_acc, (int)S, \
-                          capi, st)
+#define AMQ(GG, NN, ZZ)                                                                                               \
+    launch_am_qkv<GG, NN, ZZ>(x, n0, par, (int)T, (int)Hq, (int)Hk, hs, rs, scale_log2, part_m, part_l, part_acc,     \
+                              (int)S, capi, st)
     if (G == 4) {
-        if (nqt == 1) AMQ(4, 1); else AMQ(4, 2);
+        if (nqt == 1) AMQ(4, 1, 1); else if (pairs <= 32) AMQ(4, 2, 1); else AMQ(4, 2, 2);
     } else {
-        if (nqt == 1) AMQ(2, 1); else AMQ(2, 2);
+        if (nqt == 1) AMQ(2, 1, 1); else if (pairs <= 32) AMQ(2, 2, 1); else AMQ(2, 2, 2);
     }
 #undef AMQ
     return hip_status(hipGetLastError(), "attn_decode_mfma_qkv launch");

@@ -881,7 +881,7 @@ int32_t btb_hip_attn_decode_qkv_rows(const void* qkv, const void* wq, const void
     }
     if (btb_hip_attn_rows_fused(T, Hq, Hk, D, cap, S) == 0) {
         set_error("attn_decode_qkv_rows: head_dim 128, spans of 128 keys, 2 or 4 query heads per kv head and 2 or more "
-                  "rows with rows * (query heads per kv head) <= 32 (btb_hip_attn_rows_fused tells); otherwise "
+                  "rows with rows * (query heads per kv head) <= 64 (btb_hip_attn_rows_fused tells); otherwise "
                   "btb_hip_norm_rope_kv + btb_hip_attn_decode");
         return ERR_DOMAIN;
     }

@@ -314,7 +314,7 @@ int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk,
  * btb_hip_norm_rope_kv followed by btb_hip_attn_decode compute, bit for bit, in one launch less: each workgroup
  * prepares the pass's q heads itself, the workgroups whose key span holds some of slots *n0 .. *n0 + T - 1 prepare
  * and write those K / V rows. For head_dim 128, spans of 128 keys, 2 or 4 query heads a kv head and
- * T * (Hq / Hk) <= 32: btb_hip_attn_rows_fused returns 1 for such a pass and 0 otherwise, where this call fails with
+ * T * (Hq / Hk) <= 64: btb_hip_attn_rows_fused returns 1 for such a pass and 0 otherwise, where this call fails with
  * BTB_HIP_ERR_DOMAIN and the two calls it replaces remain. Workspace: btb_hip_attn_scratch_floats(T, ...). Replaces
  * btb_norm_rope_kv_d128 + btb_attn_flash_d128 of the reference's verify pass (btb/engine/cuda.py:1756-1790,
  * native/cuda/btb_attn_flash.cuh:400-470). */

@@ -299,10 +299,13 @@ def test_attn_decode_qkv_is_the_two_kernels_in_one(card, n0, Hq, Hk, S, with_nor
 @pytest.mark.parametrize("n0,T,Hq,Hk,tree", [(4000, 8, 32, 8, False), (4000, 7, 32, 8, False), (125, 8, 32, 8, False),
                                               (120, 16, 8, 4, True), (0, 2, 8, 2, False), (127, 3, 8, 4, False),
                                               (255, 16, 8, 4, True), (300, 5, 8, 2, True), (128, 4, 32, 8, False),
-                                              (250, 9, 16, 8, True), (1, 13, 4, 2, False), (383, 2, 32, 8, False)])
+                                              (250, 9, 16, 8, True), (1, 13, 4, 2, False), (383, 2, 32, 8, False),
+                                              (4000, 16, 32, 8, False), (120, 16, 16, 4, True), (255, 32, 8, 4, True),
+                                              (100, 12, 32, 8, False), (126, 9, 8, 2, True), (300, 20, 4, 2, False)])
 @pytest.mark.parametrize("with_norm", [True, False])
 def test_attn_rows_from_the_fused_qkv_rows(card, n0, T, Hq, Hk, tree, with_norm):
-    """a pass's attention from its fused qkv rows against norm_rope_kv followed by attn_decode: the same output bits,
+    """a pass's attention from its fused qkv rows (up to 32 (row, head) pairs a kv head in one workgroup, up to 64 in
+    two) against norm_rope_kv followed by attn_decode: the same output bits,
     the same cache rows, nothing else in the cache touched - chain and tree (rows at their depths), the pass's own slots
     at a span's start, across its end, and past the written part of the cache (which holds NaN bits)"""
     from btb_amd.decode import StackConfig, rope_tables
@@ -385,11 +388,11 @@ def test_attn_rows_from_the_fused_qkv_rows_centered_weights_and_given_positions(
 
 
 def test_attn_rows_from_the_fused_qkv_rows_only_where_it_fits(card):
-    """shapes the fused pass does not take are named by the query and refused by the call: one row, more than 32
+    """shapes the fused pass does not take are named by the query and refused by the call: one row, more than 64
     (row, head) pairs a kv head, spans of 256 keys, 8 query heads a kv head"""
     D = 128
     assert card.attn_rows_fused(8, 32, 8, D, 4608, 36)
-    for T, Hq, Hk, cap, S in ((1, 32, 8, 4608, 36), (9, 32, 8, 4608, 36), (8, 32, 8, 4608, 18), (4, 16, 2, 512, 4)):
+    for T, Hq, Hk, cap, S in ((1, 32, 8, 4608, 36), (17, 32, 8, 4608, 36), (8, 32, 8, 4608, 18), (4, 16, 2, 512, 4)):
         assert not card.attn_rows_fused(T, Hq, Hk, D, cap, S)
         qkv = torch.zeros(T, (Hq + 2 * Hk) * D, dtype=torch.bfloat16, device="cuda")
         K = torch.zeros(Hk, cap, D, dtype=torch.bfloat16, device="cuda")
