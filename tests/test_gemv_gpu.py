@@ -186,6 +186,31 @@ def test_embedding_rows_gathered_by_the_first_matvec(card, M):
     assert torch.equal(h2.view(torch.int16), h1.view(torch.int16))
 
 
+def test_rows_a_tile_change_no_bit_over_drawn_shapes(card):
+    """the matrix-core matvec takes tiles of twelve or ten rows where sixteen would leave CUs idle (knob mfma_tile_rows
+    = 0: always sixteen): over thirty drawn shapes - any multiple of 16 rows, the row lengths of the kernel's classes,
+    5 .. 32 rows of x - the same bits either way, within the bar of an f32 product"""
+    rng = np.random.default_rng(20252)
+    lower = 0
+    for _ in range(30):
+        R = 16 * int(rng.integers(1, 700))
+        C = int(rng.choice([2560, 4096, 1536, 5120, 9728, 7168]))
+        M = int(rng.integers(5, 33))
+        w = weights_bf16(R, C, seed=int(rng.integers(1 << 30))).cuda()
+        x = acts_bf16(M, C, seed=int(rng.integers(1 << 30))).cuda()
+        y = card.gemv(w, x)
+        card.set_tuning("mfma_tile_rows", 0)
+        try:
+            y16 = card.gemv(w, x)
+        finally:
+            card.set_tuning("mfma_tile_rows", -1)
+        assert torch.equal(y.view(torch.int16), y16.view(torch.int16)), (R, C, M)
+        ref = x.float() @ w.float().t()
+        assert float((y.float() - ref).abs().max()) <= 2.0**-7 * float(ref.abs().max()), (R, C, M)
+        lower += int(R % 12 == 0 or R % 10 == 0)
+    assert lower >= 5  # the draw holds row counts the lower tiles apply to
+
+
 def test_refusals_launch_nothing(card):
     w = weights_bf16(16, 64, seed=140).cuda()
     x = acts_bf16(1, 64, seed=141).cuda()

@@ -387,6 +387,61 @@ def test_attn_rows_from_the_fused_qkv_rows_centered_weights_and_given_positions(
     assert torch.equal(Ka, Kb) and torch.equal(Va, Vb)
 
 
+def test_attn_rows_from_the_fused_qkv_rows_over_drawn_shapes(card):
+    """the same equality over a hundred drawn passes: 2 or 4 query heads a kv head, 1 to 8 kv heads, 2 rows up to 64
+    pairs, cache lengths 0 .. 700 with any amount of room behind, chain or tree, with or without (centered) norm
+    weights"""
+    from btb_amd.decode import StackConfig, rope_tables
+
+    rng = np.random.default_rng(20251)
+    D, done = 128, 0
+    same = lambda a, b: torch.equal(a.view(torch.int16), b.view(torch.int16))
+    while done < 100:
+        G = int(rng.choice([2, 4]))
+        Hk = int(rng.choice([1, 2, 4, 8]))
+        Hq = Hk * G
+        T = int(rng.integers(2, 64 // G + 1))
+        n0, pad = int(rng.integers(0, 700)), int(rng.integers(0, 40))
+        cap = n0 + T + pad
+        S = -(-cap // 128)
+        assert card.attn_rows_fused(T, Hq, Hk, D, cap, S)
+        g = gen(int(rng.integers(1 << 30)))
+        K0 = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+        V0 = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16)
+        K0[:, n0:] = float("nan")
+        V0[:, n0:] = float("nan")
+        K0, V0 = K0.cuda(), V0.cuda()
+        qkv = torch.randn(T, (Hq + 2 * Hk) * D, generator=g).to(torch.bfloat16).cuda()
+        with_norm, centered = bool(rng.integers(2)), bool(rng.integers(2))
+        mk = lambda: (0.1 * torch.randn(D, generator=g) + (0.0 if centered else 1.0)).to(torch.bfloat16).cuda()
+        wq, wk = (mk(), mk()) if with_norm else (None, None)
+        cfg = StackConfig(layers=1, hidden=256, q_heads=Hq, kv_heads=Hk, head_dim=D, intermediate=256, vocab=256)
+        cos, sin = rope_tables(cfg, cap, "cuda")
+        n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+        par = depth = None
+        if rng.integers(2):
+            pl = [-1] + [int(rng.integers(-1, t)) for t in range(1, T)]
+            dl = []
+            for t in range(T):
+                dl.append(0 if pl[t] < 0 else dl[pl[t]] + 1)
+            par = torch.tensor(pl, dtype=torch.int32, device="cuda")
+            depth = torch.tensor(dl, dtype=torch.int32, device="cuda")
+        scale = 1.0 / np.sqrt(D)
+        scratch = card.attn_scratch(T, Hq, Hk, D, S)
+        Ka, Va, Kb, Vb = K0.clone(), V0.clone(), K0.clone(), V0.clone()
+        q = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+        want, got = torch.zeros_like(q), torch.zeros_like(q)
+        card.norm_rope_kv(qkv, wq, wk, 1e-6, cos, sin, n0t, Ka, Va, q, Hq, Hk, D, depth=depth, centered=centered)
+        card.attn_decode(q, Ka, Va, want, n0t, Hq, Hk, D, scale, S, scratch, par=par)
+        card.attn_decode_qkv_rows(qkv, wq, wk, 1e-6, cos, sin, n0t, Kb, Vb, got, Hq, Hk, D, scale, S, scratch,
+                                  depth=depth, par=par, centered=centered)
+        torch.cuda.synchronize()
+        what = dict(G=G, Hk=Hk, T=T, n0=n0, cap=cap, norm=with_norm, centered=centered, tree=par is not None)
+        assert same(got, want) and same(Ka, Kb) and same(Va, Vb), what
+        assert bool(torch.isfinite(want.float()).all()), what
+        done += 1
+
+
 def test_attn_rows_from_the_fused_qkv_rows_only_where_it_fits(card):
     """shapes the fused pass does not take are named by the query and refused by the call: one row, more than 64
     (row, head) pairs a kv head, spans of 256 keys, 8 query heads a kv head"""
