@@ -416,7 +416,7 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
         s_k[lane * 2 + 1] = o[1];
         s_v[lane * 2] = (uint16_t)(vraw & 0xFFFFu);
         s_v[lane * 2 + 1] = (uint16_t)(vraw >> 16);
-        if (part == 0) {
+        if (part == 0 && n0 < cap) {  // a slot past the cache's end is never written (spans are rounded up past it)
             reinterpret_cast<uint32_t*>(K + (size_t)g * hs + (size_t)n0 * rs)[lane] = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
             reinterpret_cast<uint32_t*>(V + (size_t)g * hs + (size_t)n0 * rs)[lane] = vraw;
         }
@@ -659,13 +659,17 @@ size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, siz
 }
 
 // `work` is the caller's workspace, or nullptr for the library's own static array on the current device
+// `parts`: the caller's own three state arrays (part_m, part_l [T Hq S], part_acc [T Hq S D]) in place of one workspace;
+// the call then takes spans of `cap / S` keys exactly and only the kernel whose loads stay on live keys, so `cap` need
+// not be the cache's true capacity
 static int32_t attn_decode_any(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
                                const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
                                float scale, size_t cap, size_t S, float* work, bool own_scratch, void* stream,
-                               int64_t win = 0, const int32_t* tbl = nullptr) {
+                               int64_t win = 0, const int32_t* tbl = nullptr, float* const* parts = nullptr) {
     if (q == nullptr || K == nullptr || V == nullptr || att == nullptr || n0 == nullptr ||
-        (!own_scratch && work == nullptr))
+        (!own_scratch && work == nullptr && parts == nullptr))
         return ERR_NULL;
+    if (parts != nullptr && (parts[0] == nullptr || parts[1] == nullptr || parts[2] == nullptr)) return ERR_NULL;
     if (T == 0 || Hq == 0 || Hk == 0 || S == 0 || cap == 0 || T > 65535 || S > 1024 || Hq % Hk != 0 || hs <= 0 ||
         rs <= 0 || !(scale == scale))
         return ERR_DOMAIN;
@@ -697,9 +701,10 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
     // a span is a whole number of the workgroup's batches of keys (16 streams by 8 keys): a batch is the unit of its
     // work, and a span that ends inside one pays for all of it
     const int span = (int)(((cap + S - 1) / S + 127) / 128 * 128);
-    float* part_m = work;
-    float* part_l = work + T * Hq * S;
-    float* part_acc = work + 2 * T * Hq * S;
+    float* part_m = parts != nullptr ? parts[0] : work;
+    float* part_l = parts != nullptr ? parts[1] : work + T * Hq * S;
+    float* part_acc = parts != nullptr ? parts[2] : work + 2 * T * Hq * S;
+    if (parts != nullptr && (!al(part_m, 4) || !al(part_l, 4) || !al(part_acc, 16))) return ERR_DOMAIN;
     const float scale_log2 = scale * 1.4426950408889634f;
     const dim3 grid((unsigned)Hk, (unsigned)S, (unsigned)T);
     hipStream_t st = static_cast<hipStream_t>(stream);
@@ -721,7 +726,7 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
     // Several rows and spans of 128 keys: the matrix cores, every row of the pass that shares a kv head in one workgroup
     // (attn_mfma.hip). A pass of 8 rows over 4096 keys: 22.7 us a layer on the vector kernel below, which stays for
     // spans of 256 keys and behind the knob attn_mfma = 0.
-    if (attn_mfma_fits(T, G, span)) {
+    if (parts == nullptr && attn_mfma_fits(T, G, span)) {
         const int32_t rc = attn_decode_mfma(q, K, V, n0, par, T, Hq, Hk, (long long)hs, (long long)rs, scale_log2, part_m,
                                             part_l, part_acc, S, cap, (int)win, tbl, st);
         if (rc != OK) return rc;
@@ -734,7 +739,7 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
         return hip_status(hipGetLastError(), "attn_decode launch");
     }
     const int rows_knob = tuning("attn_rows_per_wg");
-    if (T >= 2 && (span == 128 || span == 256) && (G == 2 || G == 4) && rows_knob != 0) {
+    if (parts == nullptr && T >= 2 && (span == 128 || span == 256) && (G == 2 || G == 4) && rows_knob != 0) {
         int rpw = rows_knob > 0 ? rows_knob : 1;
         if (rpw > (int)T) rpw = (int)T;
         const dim3 rgrid((unsigned)Hk, (unsigned)S, (unsigned)((T + rpw - 1) / rpw));
@@ -776,6 +781,19 @@ int32_t btb_hip_attn_decode_win(const void* q, const void* K, const void* V, voi
                                 void* stream) {
     return attn_decode_any(q, K, V, att, n0, par, T, Hq, Hk, D, hs, rs, scale, cap, S, workspace, false, stream, win,
                            tbl);
+}
+
+int32_t btb_hip_attn_decode_parts(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
+                                  const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
+                                  float scale, size_t span, size_t S, int64_t win, const int32_t* tbl, float* part_m,
+                                  float* part_l, float* part_acc, void* stream) {
+    if (span == 0 || span % 128 != 0 || S == 0 || span > 0x7FFFFFFFull / (S ? S : 1)) {
+        set_error("attn_decode_parts: spans are a whole number of 128-key batches");
+        return ERR_DOMAIN;
+    }
+    float* const parts[3] = {part_m, part_l, part_acc};
+    return attn_decode_any(q, K, V, att, n0, par, T, Hq, Hk, D, hs, rs, scale, span * S, S, nullptr, false, stream, win,
+                           tbl, parts);
 }
 
 int32_t btb_hip_attn_decode_noalloc(const void* q, const void* K, const void* V, void* att, const int32_t* n0,

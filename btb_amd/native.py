@@ -17,6 +17,8 @@ from typing import Any, Sequence
 
 import torch
 
+from .card_launch import CardLaunch
+
 HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(HERE, "libbtb_hip.so")
 
@@ -74,6 +76,8 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_attn_scratch_floats": (_sz, [_sz, _sz, _sz, _sz, _sz]),
     "btb_hip_attn_decode": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
                                    ctypes.c_float, _sz, _sz, _vp, _vp]),
+    "btb_hip_attn_decode_parts": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
+                                         ctypes.c_float, _sz, _sz, ctypes.c_int64, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_attn_decode_noalloc": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64,
                                            ctypes.c_int64, ctypes.c_float, _sz, _sz, _vp]),
     "btb_hip_attn_decode_qkv": (_i32, [_vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
@@ -133,6 +137,11 @@ def _stream() -> ctypes.c_void_p:
     return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
 
 
+def _p(t: torch.Tensor) -> ctypes.c_void_p:
+    """a tensor's device address as a pointer argument of the C ABI"""
+    return ctypes.c_void_p(t.data_ptr())
+
+
 
 def _launch_table() -> dict[str, tuple[int, Any]]:
     """reference kernel name -> (its parameter count, parameters -> (entry point, its arguments less the stream))"""
@@ -162,13 +171,12 @@ def _launch_table() -> dict[str, tuple[int, Any]]:
             v[17])))
     # btb_attn_flash_d128(q, K, V, out, n0p, par, T, Hq, Hk, hs, rs, scale, part_m, part_l, part_acc, cnt, win, tbl) on
     # a grid (row tiles, key groups, kv heads): grid[1] key groups of 512 keys each reach the cache's capacity. The
-    # caller's partial-state arrays and arrival counter are not used (see HipCard._flash_work).
-    def flash(v, g, card):
-        T, Hq, S = int(v[6] or 1), int(v[7] or 1), max(int(g[1]), 1)
-        work = None if card is None else card._flash_work(T * Hq * S * 130)
-        return "btb_hip_attn_decode_win", (v[0], v[1], v[2], v[3], v[4], v[5], T, Hq, v[8], 128, v[9], v[10], v[11],
-                                           S * 512, S, v[16], v[17], work)
-    t["btb_attn_flash_d128"] = (18, flash)
+    # groups' states go into the caller's own part_m / part_l / part_acc (S T Hq and S T Hq D floats, the sizes the
+    # reference's card graph gives them), so the launch allocates nothing and a captured graph keeps its arrays; the
+    # arrival counter is left alone (the groups are folded by a second launch, not by the last arriver)
+    t["btb_attn_flash_d128"] = (18, lambda v, g, card: ("btb_hip_attn_decode_parts", (
+        v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], 128, v[9], v[10], v[11], 512, max(int(g[1]), 1), v[16],
+        v[17], v[12], v[13], v[14])))
     # btb_publish(n0, ids, out_tok, out_n0, out_ts)
     t["btb_publish"] = (5, lambda v, g, card: ("btb_hip_publish_only", (v[0], v[1], v[2], v[3], v[4])))
     # btb_mx4_widen(blocks, scales, seats, groups, out), grid.y seats
@@ -178,9 +186,12 @@ def _launch_table() -> dict[str, tuple[int, Any]]:
 
 _LAUNCH = _launch_table()
 
-class HipCard:
-    """The card's operators over torch tensors. `GEMV_ROWS` are the pass widths the reference's card graphs are
-    captured at (btb/engine/native.py:1918); any M up to 1024 is taken here."""
+class HipCard(CardLaunch):
+    """The card's operators over torch tensors: the reference's `_Cuda` (`CardLaunch` + `launch`,
+    btb/engine/native.py:1243) over this library. `launch` takes the reference's kernel names; `CardLaunch` adds the
+    typed launchers (`k.btb_add_rmsnorm(grid, block, ...)`, `k.btb_gemv_bf16(M, grid, block, ...)`) and
+    `ptr(role, tensor)`, which is all the reference's `_card_body` asks of its `k`. `GEMV_ROWS` are the pass widths the
+    reference's card graphs are captured at (btb/engine/native.py:1918); any M up to 1024 is taken here."""
 
     GEMV_ROWS = (1, 2, 4, 8, 16, 32)
 
@@ -202,10 +213,6 @@ class HipCard:
         if rc != OK:
             msg = self.lib.btb_hip_last_error().decode(errors="replace")
             raise HipError(f"[hip] {name} failed: {rc} {_CODES.get(rc, '?')} {msg}")
-
-    @staticmethod
-    def ptr(t: torch.Tensor) -> ctypes.c_void_p:
-        return ctypes.c_void_p(t.data_ptr())
 
     def set_tuning(self, key: str, value: int) -> None:
         self._call("btb_hip_set_tuning", key.encode(), int(value))
@@ -243,18 +250,8 @@ class HipCard:
         return {n: call([0] * count, (1, 1, 1), None)[0] for n, (count, call) in _LAUNCH.items()}
 
     def close(self) -> None:
-        """drops the card's own scratch (the library stays loaded for the process); may be called any number of times"""
-        self._flash_scratch = None
-
-    def _flash_work(self, floats: int) -> ctypes.c_void_p:
-        """the partial-state scratch behind `btb_attn_flash_d128` launched by name: the reference's caller passes
-        three arrays in its own layout (part_m / part_l / part_acc, [S, T, Hq(, D)]) and an arrival counter; this
-        library keeps one array in its own layout, owned by the card and grown on demand"""
-        cur = getattr(self, "_flash_scratch", None)
-        if cur is None or cur.numel() < floats:
-            cur = torch.empty(max(floats, 1), dtype=torch.float32, device="cuda")
-            self._flash_scratch = cur
-        return ctypes.c_void_p(cur.data_ptr())
+        """the reference's `_Cuda.close` unloads its module (btb/engine/native.py:1484-1492); the card here owns no
+        device memory and the library stays loaded for the process, so there is nothing to drop. Idempotent."""
 
     # -- bf16 matvec ------------------------------------------------------------------------------------------
 
@@ -271,7 +268,7 @@ class HipCard:
             self._need(y, torch.bfloat16, "y")
             if y.numel() != M * R:
                 raise ValueError(f"[hip] gemv: y holds {y.numel()} elements, the product has {M * R}")
-        self._call("btb_hip_gemv_bf16", self.ptr(w), self.ptr(x2), self.ptr(y), R, C, M, _stream())
+        self._call("btb_hip_gemv_bf16", _p(w), _p(x2), _p(y), R, C, M, _stream())
         return y
 
     def gemv_silu(self, w: torch.Tensor, gu: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
@@ -287,7 +284,7 @@ class HipCard:
             self._need(y, torch.bfloat16, "y")
             if y.numel() != M * R:
                 raise ValueError(f"[hip] gemv_silu: y holds {y.numel()} elements, the product has {M * R}")
-        self._call("btb_hip_gemv_silu_bf16", self.ptr(w), self.ptr(g2), self.ptr(y), R, C, M, _stream())
+        self._call("btb_hip_gemv_silu_bf16", _p(w), _p(g2), _p(y), R, C, M, _stream())
         return y
 
 
@@ -300,7 +297,7 @@ class HipCard:
         x2 = x.reshape(-1, C)
         M = int(x2.shape[0])
         m = self._out(m, M, R // 2, x.device, "gemv_glu_silu")
-        self._call("btb_hip_gemv_glu_silu_bf16", self.ptr(w), self.ptr(x2), self.ptr(m), R // 2, C, M, _stream())
+        self._call("btb_hip_gemv_glu_silu_bf16", _p(w), _p(x2), _p(m), R // 2, C, M, _stream())
         return m
 
     def gemv_norm(self, w: Any, h_in: torch.Tensor, y: torch.Tensor | None, norm_w: torch.Tensor, eps: float,
@@ -320,16 +317,16 @@ class HipCard:
             raise ValueError("[hip] gemv_norm: the rows, the norm weight and the output do not fit the matrix")
         if h_out is not None and h_out.data_ptr() == h_in.data_ptr():
             raise ValueError("[hip] gemv_norm: the new residual cannot be written over the one being read")
-        p = lambda t: None if t is None else self.ptr(t)
+        p = lambda t: None if t is None else _p(t)
         if isinstance(w, torch.Tensor):
             self._need(w, torch.bfloat16, "w")
-            self._call("btb_hip_gemv_bf16_norm", self.ptr(w), self.ptr(h_in), p(y), self.ptr(norm_w), float(eps),
-                       int(centered), p(h_out), self.ptr(out), R, C, M, int(glu), _stream())
+            self._call("btb_hip_gemv_bf16_norm", _p(w), _p(h_in), p(y), _p(norm_w), float(eps),
+                       int(centered), p(h_out), _p(out), R, C, M, int(glu), _stream())
         else:
             ne = int(w.esc_idx.numel())
-            self._call("btb_hip_gemv_p12_norm", self.ptr(w.lo), self.ptr(w.hi4), self.ptr(w.table),
-                       self.ptr(w.esc_idx) if ne else None, self.ptr(w.esc_val) if ne else None, ne, self.ptr(w.row_ptr),
-                       self.ptr(h_in), p(y), self.ptr(norm_w), float(eps), int(centered), p(h_out), self.ptr(out), R, C,
+            self._call("btb_hip_gemv_p12_norm", _p(w.lo), _p(w.hi4), _p(w.table),
+                       _p(w.esc_idx) if ne else None, _p(w.esc_val) if ne else None, ne, _p(w.row_ptr),
+                       _p(h_in), p(y), _p(norm_w), float(eps), int(centered), p(h_out), _p(out), R, C,
                        M, int(glu), _stream())
         return out
 
@@ -346,17 +343,17 @@ class HipCard:
         if table.dim() != 2 or table.shape[1] != C or norm_w.numel() != C or out.numel() != M * R \
                 or (h_out is not None and h_out.numel() != M * C):
             raise ValueError("[hip] gemv_embed_norm: the table, the norm weight and the outputs do not fit the matrix")
-        p = lambda t: None if t is None else self.ptr(t)
+        p = lambda t: None if t is None else _p(t)
         if isinstance(w, torch.Tensor):
             self._need(w, torch.bfloat16, "w")
-            self._call("btb_hip_gemv_bf16_embed_norm", self.ptr(w), self.ptr(table), self.ptr(ids), vocab,
-                       self.ptr(norm_w), float(eps), int(centered), p(h_out), self.ptr(out), R, C, M, _stream())
+            self._call("btb_hip_gemv_bf16_embed_norm", _p(w), _p(table), _p(ids), vocab,
+                       _p(norm_w), float(eps), int(centered), p(h_out), _p(out), R, C, M, _stream())
         else:
             ne = int(w.esc_idx.numel())
-            self._call("btb_hip_gemv_p12_embed_norm", self.ptr(w.lo), self.ptr(w.hi4), self.ptr(w.table),
-                       self.ptr(w.esc_idx) if ne else None, self.ptr(w.esc_val) if ne else None, ne, self.ptr(w.row_ptr),
-                       self.ptr(table), self.ptr(ids), vocab, self.ptr(norm_w), float(eps), int(centered), p(h_out),
-                       self.ptr(out), R, C, M, _stream())
+            self._call("btb_hip_gemv_p12_embed_norm", _p(w.lo), _p(w.hi4), _p(w.table),
+                       _p(w.esc_idx) if ne else None, _p(w.esc_val) if ne else None, ne, _p(w.row_ptr),
+                       _p(table), _p(ids), vocab, _p(norm_w), float(eps), int(centered), p(h_out),
+                       _p(out), R, C, M, _stream())
         return out
 
     # -- the stored forms ---------------------------------------------------------------------------------------
@@ -375,7 +372,7 @@ class HipCard:
         if esc_idx.numel() == 0:
             return
         flag = torch.zeros(1, dtype=torch.int32, device=esc_idx.device)
-        rc = self.lib.btb_hip_p12_check(self.ptr(esc_idx), esc_idx.numel(), int(n), self.ptr(flag), _stream())
+        rc = self.lib.btb_hip_p12_check(_p(esc_idx), esc_idx.numel(), int(n), _p(flag), _stream())
         if rc == ERR_DOMAIN:
             raise ValueError(f"[hip] pack12: {self.lib.btb_hip_last_error().decode(errors='replace')}")
         if rc != OK:
@@ -385,8 +382,8 @@ class HipCard:
         """int32 [rows + 1]: the first escape at or past each row's first weight (built once at upload)"""
         self._need(esc_idx, torch.int32, "esc_idx")
         out = torch.empty(rows + 1, dtype=torch.int32, device=esc_idx.device)
-        self._call("btb_hip_p12_row_ptr", self.ptr(esc_idx) if esc_idx.numel() else None, esc_idx.numel(), rows, cols,
-                   self.ptr(out), _stream())
+        self._call("btb_hip_p12_row_ptr", _p(esc_idx) if esc_idx.numel() else None, esc_idx.numel(), rows, cols,
+                   _p(out), _stream())
         return out
 
     def gemv_p12(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
@@ -397,9 +394,9 @@ class HipCard:
         M = int(x2.shape[0])
         y = self._out(y, M, R, x.device, "gemv_p12")
         ne = int(w.esc_idx.numel())
-        self._call("btb_hip_gemv_p12", self.ptr(w.lo), self.ptr(w.hi4), self.ptr(w.table),
-                   self.ptr(w.esc_idx) if ne else None, self.ptr(w.esc_val) if ne else None, ne, self.ptr(w.row_ptr),
-                   self.ptr(x2), self.ptr(y), R, C, M, _stream())
+        self._call("btb_hip_gemv_p12", _p(w.lo), _p(w.hi4), _p(w.table),
+                   _p(w.esc_idx) if ne else None, _p(w.esc_val) if ne else None, ne, _p(w.row_ptr),
+                   _p(x2), _p(y), R, C, M, _stream())
         return y
 
     def p12_widen(self, lo, hi4, table, esc_idx, esc_val, n: int, shape: Sequence[int],
@@ -417,8 +414,8 @@ class HipCard:
         if ne:
             self._need(esc_idx, torch.int32, "esc_idx")
             self._need(esc_val, torch.uint8, "esc_val")
-        self._call("btb_hip_p12_widen", self.ptr(lo), self.ptr(hi4), self.ptr(table), self.ptr(esc_idx) if ne else None,
-                   self.ptr(esc_val) if ne else None, ne, n, self.ptr(out), _stream())
+        self._call("btb_hip_p12_widen", _p(lo), _p(hi4), _p(table), _p(esc_idx) if ne else None,
+                   _p(esc_val) if ne else None, ne, n, _p(out), _stream())
         return out
 
     def gemv_fp8(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
@@ -431,7 +428,7 @@ class HipCard:
         x2 = x.reshape(-1, C)
         M = int(x2.shape[0])
         y = self._out(y, M, R, x.device, "gemv_fp8")
-        self._call("btb_hip_gemv_fp8", self.ptr(w.w), self.ptr(w.scales), sr, sc, self.ptr(x2), self.ptr(y), R, C, M,
+        self._call("btb_hip_gemv_fp8", _p(w.w), _p(w.scales), sr, sc, _p(x2), _p(y), R, C, M,
                    _stream())
         return y
 
@@ -440,7 +437,7 @@ class HipCard:
         a NaN the quiet NaN of its sign and upper payload: the crate's `round_bf16` with torch's NaN rule)"""
         self._need(x, torch.float32, "x")
         out = torch.empty(x.shape, dtype=torch.bfloat16, device=x.device)
-        self._call("btb_hip_round_bf16", self.ptr(x), self.ptr(out), int(x.numel()), _stream())
+        self._call("btb_hip_round_bf16", _p(x), _p(out), int(x.numel()), _stream())
         return out
 
     def fp8_widen(self, w: Any, dtype: torch.dtype = torch.bfloat16) -> torch.Tensor:
@@ -450,7 +447,7 @@ class HipCard:
         if dtype not in (torch.bfloat16, torch.float32):
             raise ValueError("[hip] fp8_widen writes bf16 or float32")
         out = torch.empty(R, C, dtype=dtype, device=w.w.device)
-        self._call("btb_hip_fp8_widen", self.ptr(w.w), self.ptr(w.scales), R, C, sr, sc, self.ptr(out),
+        self._call("btb_hip_fp8_widen", _p(w.w), _p(w.scales), R, C, sr, sc, _p(out),
                    int(dtype == torch.float32), _stream())
         return out
 
@@ -463,7 +460,7 @@ class HipCard:
         x2 = x.reshape(-1, C)
         M = int(x2.shape[0])
         y = self._out(y, M, R, x.device, "gemv_mx4")
-        self._call("btb_hip_gemv_mxfp4", self.ptr(w.blocks), self.ptr(w.scales), self.ptr(x2), self.ptr(y), R, C, M,
+        self._call("btb_hip_gemv_mxfp4", _p(w.blocks), _p(w.scales), _p(x2), _p(y), R, C, M,
                    _stream())
         return y
 
@@ -491,8 +488,8 @@ class HipCard:
         elif out.dtype != dtype or not out.is_contiguous() or out.numel() != n * groups * 32:
             raise ValueError(f"[hip] mx4_widen: out must be {n * groups * 32} contiguous {dtype}")
         if n:
-            self._call("btb_hip_mx4_widen", self.ptr(blocks), self.ptr(scales), None if seats is None else self.ptr(seats),
-                       n, groups, self.ptr(out), int(dtype == torch.float32), _stream())
+            self._call("btb_hip_mx4_widen", _p(blocks), _p(scales), None if seats is None else _p(seats),
+                       n, groups, _p(out), int(dtype == torch.float32), _stream())
         return out
 
 
@@ -516,23 +513,23 @@ class HipCard:
         self._need(w, torch.bfloat16, "w")
         R, C = (int(s) for s in w.shape)
         x2, b, y = self._rows_io(x, y, R, C, "gemv_lane16")
-        self._call("btb_hip_gemv_bf16_rows", self.ptr(w), R, C, self.ptr(x2), b, self.ptr(y), _stream())
+        self._call("btb_hip_gemv_bf16_rows", _p(w), R, C, _p(x2), b, _p(y), _stream())
         return y
 
     def gemv_lane16_p12(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
         R, C = w.shape
         x2, b, y = self._rows_io(x, y, R, C, "gemv_lane16_p12")
         ne = int(w.esc_idx.numel())
-        self._call("btb_hip_gemv_p12_rows", self.ptr(w.lo), self.ptr(w.hi4), self.ptr(w.table),
-                   self.ptr(w.esc_idx) if ne else None, self.ptr(w.esc_val) if ne else None, ne, R, C, self.ptr(x2), b,
-                   self.ptr(y), _stream())
+        self._call("btb_hip_gemv_p12_rows", _p(w.lo), _p(w.hi4), _p(w.table),
+                   _p(w.esc_idx) if ne else None, _p(w.esc_val) if ne else None, ne, R, C, _p(x2), b,
+                   _p(y), _stream())
         return y
 
     def gemv_lane16_mx4(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
         """the host's MXFP4 matvec to the bit (`_Cuda.gemv_lane16_mx4`, btb/engine/native.py:2367-2390)"""
         R, C = w.shape
         x2, b, y = self._rows_io(x, y, R, C, "gemv_lane16_mx4")
-        self._call("btb_hip_gemv_mxfp4_rows", self.ptr(w.blocks), self.ptr(w.scales), R, C, self.ptr(x2), b, self.ptr(y),
+        self._call("btb_hip_gemv_mxfp4_rows", _p(w.blocks), _p(w.scales), R, C, _p(x2), b, _p(y),
                    _stream())
         return y
 
@@ -544,14 +541,14 @@ class HipCard:
         if raw.numel() != rows * cols // 32 * 17:
             raise ValueError(f"[hip] gemv_lane16_mx4_ggml: {raw.numel()} bytes are not {rows} x {cols} weights in 17-byte blocks")
         x2, b, y = self._rows_io(x, y, rows, cols, "gemv_lane16_mx4_ggml")
-        self._call("btb_hip_gemv_mxfp4_ggml_rows", self.ptr(raw), rows, cols, self.ptr(x2), b, self.ptr(y), _stream())
+        self._call("btb_hip_gemv_mxfp4_ggml_rows", _p(raw), rows, cols, _p(x2), b, _p(y), _stream())
         return y
 
     def gemv_lane16_fp8(self, w: Any, x: torch.Tensor, y: torch.Tensor | None = None) -> torch.Tensor:
         R, C = w.shape
         sr, sc = w.grid
         x2, b, y = self._rows_io(x, y, R, C, "gemv_lane16_fp8")
-        self._call("btb_hip_gemv_fp8_rows", self.ptr(w.w), self.ptr(w.scales), R, C, sr, sc, self.ptr(x2), b, self.ptr(y),
+        self._call("btb_hip_gemv_fp8_rows", _p(w.w), _p(w.scales), R, C, sr, sc, _p(x2), b, _p(y),
                    _stream())
         return y
 
@@ -568,8 +565,8 @@ class HipCard:
         idx = torch.empty(T, k, dtype=torch.int32, device=logits.device)
         w = torch.empty(T, k, dtype=torch.bfloat16, device=logits.device)
         w32 = torch.empty(T, k, dtype=torch.float32, device=logits.device)
-        self._call("btb_hip_moe_route", self.ptr(logits), int(logits.dtype == torch.float32), ls, E, k, T, self.ptr(idx),
-                   self.ptr(w), self.ptr(w32), _stream())
+        self._call("btb_hip_moe_route", _p(logits), int(logits.dtype == torch.float32), ls, E, k, T, _p(idx),
+                   _p(w), _p(w32), _stream())
         return idx, w, w32
 
     def moe_group_picks(self, idx: torch.Tensor, num_experts: int):
@@ -584,8 +581,8 @@ class HipCard:
         token = torch.empty(T * k, dtype=torch.int32, device=dev)
         offs = torch.empty(int(num_experts), dtype=torch.int32, device=dev)
         counts = torch.empty(int(num_experts), dtype=torch.int32, device=dev)
-        self._call("btb_hip_moe_group_picks", self.ptr(idx), T, k, int(num_experts), self.ptr(slot), self.ptr(token),
-                   self.ptr(offs), self.ptr(counts), _stream())
+        self._call("btb_hip_moe_group_picks", _p(idx), T, k, int(num_experts), _p(slot), _p(token),
+                   _p(offs), _p(counts), _stream())
         return slot, token, offs, counts
 
     def moe_router(self, router: torch.Tensor, x: torch.Tensor, k: int):
@@ -603,8 +600,8 @@ class HipCard:
         idx = torch.empty(T, k, dtype=torch.int32, device=dev)
         w = torch.empty(T, k, dtype=torch.bfloat16, device=dev)
         w32 = torch.empty(T, k, dtype=torch.float32, device=dev)
-        self._call("btb_hip_moe_router_bf16", self.ptr(router), self.ptr(x), T, E, H, k, self.ptr(logits),
-                   self.ptr(logits16), self.ptr(idx), self.ptr(w), self.ptr(w32), _stream())
+        self._call("btb_hip_moe_router_bf16", _p(router), _p(x), T, E, H, k, _p(logits),
+                   _p(logits16), _p(idx), _p(w), _p(w32), _stream())
         return logits, logits16, idx, w, w32
 
     def moe_experts(self, gate_up: torch.Tensor, down: torch.Tensor, x: torch.Tensor, idx: torch.Tensor,
@@ -623,8 +620,8 @@ class HipCard:
             gu = torch.empty(T, k, I2, dtype=torch.bfloat16, device=x.device)
         if y is None:
             y = torch.empty(T, H, dtype=torch.bfloat16, device=x.device)
-        self._call("btb_hip_moe_experts_bf16", self.ptr(gate_up), self.ptr(down), self.ptr(x), self.ptr(idx), self.ptr(w),
-                   self.ptr(gu), self.ptr(y), T, k, E, H, I2 // 2, _stream())
+        self._call("btb_hip_moe_experts_bf16", _p(gate_up), _p(down), _p(x), _p(idx), _p(w),
+                   _p(gu), _p(y), T, k, E, H, I2 // 2, _stream())
         return y
 
 
@@ -635,7 +632,7 @@ class HipCard:
         self._need(ids, torch.int32, "ids")
         self._need(h, torch.bfloat16, "h")
         V, H = (int(s) for s in table.shape)
-        self._call("btb_hip_embed", self.ptr(table), self.ptr(ids), self.ptr(h), int(ids.numel()), H, V, _stream())
+        self._call("btb_hip_embed", _p(table), _p(ids), _p(h), int(ids.numel()), H, V, _stream())
         return h
 
     def add_rmsnorm(self, h: torch.Tensor, y: torch.Tensor | None, w: torch.Tensor, eps: float, x: torch.Tensor,
@@ -649,8 +646,8 @@ class HipCard:
         T = int(h.numel()) // H
         if h.numel() != T * H or x.numel() != T * H or (y is not None and y.numel() != T * H):
             raise ValueError("[hip] add_rmsnorm: h, y and x are [T, H] with H the weight's length")
-        self._call("btb_hip_add_rmsnorm", self.ptr(h), None if y is None else self.ptr(y), self.ptr(w), float(eps),
-                   self.ptr(x), T, H, int(bool(centered)), _stream())
+        self._call("btb_hip_add_rmsnorm", _p(h), None if y is None else _p(y), _p(w), float(eps),
+                   _p(x), T, H, int(bool(centered)), _stream())
         return x
 
     def norm_rope_kv(self, qkv: torch.Tensor, wq: torch.Tensor | None, wk: torch.Tensor | None, eps: float,
@@ -666,14 +663,14 @@ class HipCard:
         if K.dtype != torch.bfloat16 or V.dtype != torch.bfloat16 or K.stride(2) != 1 or K.stride() != V.stride():
             raise ValueError("[hip] norm_rope_kv: K and V are bf16 [Hk, cap, D] views with the same strides")
         T = int(qkv.numel()) // ((Hq + 2 * Hk) * D)
-        args = (self.ptr(qkv), None if wq is None else self.ptr(wq), None if wk is None else self.ptr(wk), float(eps),
-                self.ptr(cos), self.ptr(sin), self.ptr(n0), None if depth is None else self.ptr(depth), self.ptr(K),
-                self.ptr(V), self.ptr(q), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)), int(bool(centered)))
+        args = (_p(qkv), None if wq is None else _p(wq), None if wk is None else _p(wk), float(eps),
+                _p(cos), _p(sin), _p(n0), None if depth is None else _p(depth), _p(K),
+                _p(V), _p(q), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)), int(bool(centered)))
         if tbl is None:
             self._call("btb_hip_norm_rope_kv", *args, _stream())
         else:
             self._need(tbl, torch.int32, "tbl")
-            self._call("btb_hip_norm_rope_kv_tbl", *args, self.ptr(tbl), _stream())
+            self._call("btb_hip_norm_rope_kv_tbl", *args, _p(tbl), _stream())
 
     def attn_scratch(self, T: int, Hq: int, Hk: int, D: int, S: int, device: Any = "cuda") -> torch.Tensor:
         """the f32 scratch `attn_decode` leaves its spans' states in, at these sizes"""
@@ -706,14 +703,14 @@ class HipCard:
                 self._need(tbl, torch.int32, "tbl")
                 if tbl.numel() < int(K.shape[1]):
                     raise ValueError(f"[hip] attn_decode: tbl maps {tbl.numel()} slots, the cache has {int(K.shape[1])}")
-            self._call("btb_hip_attn_decode_win", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0),
-                       None if par is None else self.ptr(par), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)),
-                       float(scale), int(K.shape[1]), S, int(win), None if tbl is None else self.ptr(tbl),
-                       self.ptr(scratch), _stream())
+            self._call("btb_hip_attn_decode_win", _p(q), _p(K), _p(V), _p(att), _p(n0),
+                       None if par is None else _p(par), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)),
+                       float(scale), int(K.shape[1]), S, int(win), None if tbl is None else _p(tbl),
+                       _p(scratch), _stream())
             return
-        self._call("btb_hip_attn_decode", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0),
-                   None if par is None else self.ptr(par), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)),
-                   float(scale), int(K.shape[1]), S, self.ptr(scratch), _stream())
+        self._call("btb_hip_attn_decode", _p(q), _p(K), _p(V), _p(att), _p(n0),
+                   None if par is None else _p(par), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)),
+                   float(scale), int(K.shape[1]), S, _p(scratch), _stream())
 
     def attn_decode_noalloc(self, q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, att: torch.Tensor,
                             n0: torch.Tensor, Hq: int, Hk: int, D: int, scale: float, S: int,
@@ -732,8 +729,8 @@ class HipCard:
             self._need(par, torch.int32, "par")
             if par.numel() != T:
                 raise ValueError(f"[hip] attn_decode_noalloc: par names {par.numel()} rows, the pass has {T}")
-        self._call("btb_hip_attn_decode_noalloc", self.ptr(q), self.ptr(K), self.ptr(V), self.ptr(att), self.ptr(n0),
-                   None if par is None else self.ptr(par), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)),
+        self._call("btb_hip_attn_decode_noalloc", _p(q), _p(K), _p(V), _p(att), _p(n0),
+                   None if par is None else _p(par), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)),
                    float(scale), int(K.shape[1]), S, _stream())
 
     def attn_decode_qkv(self, qkv: torch.Tensor, wq: torch.Tensor | None, wk: torch.Tensor | None, eps: float,
@@ -760,10 +757,10 @@ class HipCard:
         need = int(self.lib.btb_hip_attn_scratch_floats(1, Hq, Hk, D, S))
         if scratch.numel() < need:
             raise ValueError(f"[hip] attn_decode_qkv: scratch holds {scratch.numel()} floats, {need} are needed")
-        p = lambda t: None if t is None else self.ptr(t)
-        self._call("btb_hip_attn_decode_qkv", self.ptr(qkv), p(wq), p(wk), float(eps), 1 if centered else 0,
-                   self.ptr(cos_t), self.ptr(sin_t), self.ptr(n0), self.ptr(K), self.ptr(V), self.ptr(att), Hq, Hk, D,
-                   int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S, self.ptr(scratch), _stream())
+        p = lambda t: None if t is None else _p(t)
+        self._call("btb_hip_attn_decode_qkv", _p(qkv), p(wq), p(wk), float(eps), 1 if centered else 0,
+                   _p(cos_t), _p(sin_t), _p(n0), _p(K), _p(V), _p(att), Hq, Hk, D,
+                   int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S, _p(scratch), _stream())
 
     def attn_rows_fused(self, T: int, Hq: int, Hk: int, D: int, cap: int, S: int) -> bool:
         """whether `attn_decode_qkv_rows` takes a pass of this shape"""
@@ -801,39 +798,39 @@ class HipCard:
         need = int(self.lib.btb_hip_attn_scratch_floats(T, Hq, Hk, D, S))
         if scratch.numel() < need:
             raise ValueError(f"[hip] attn_decode_qkv_rows: scratch holds {scratch.numel()} floats, {need} are needed")
-        p = lambda t: None if t is None else self.ptr(t)
-        self._call("btb_hip_attn_decode_qkv_rows", self.ptr(qkv), p(wq), p(wk), float(eps), 1 if centered else 0,
-                   self.ptr(cos_t), self.ptr(sin_t), self.ptr(n0), p(depth), p(par), self.ptr(K), self.ptr(V),
-                   self.ptr(att), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S,
-                   self.ptr(scratch), _stream())
+        p = lambda t: None if t is None else _p(t)
+        self._call("btb_hip_attn_decode_qkv_rows", _p(qkv), p(wq), p(wk), float(eps), 1 if centered else 0,
+                   _p(cos_t), _p(sin_t), _p(n0), p(depth), p(par), _p(K), _p(V),
+                   _p(att), T, Hq, Hk, D, int(K.stride(0)), int(K.stride(1)), float(scale), int(K.shape[1]), S,
+                   _p(scratch), _stream())
 
     def silu_mul(self, gu: torch.Tensor, m: torch.Tensor) -> torch.Tensor:
         self._need(gu, torch.bfloat16, "gu")
         self._need(m, torch.bfloat16, "m")
         I = int(gu.shape[-1]) // 2
-        self._call("btb_hip_silu_mul", self.ptr(gu), self.ptr(m), int(gu.numel()) // (2 * I), I, _stream())
+        self._call("btb_hip_silu_mul", _p(gu), _p(m), int(gu.numel()) // (2 * I), I, _stream())
         return m
 
     def argmax(self, logits: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
         self._need(logits, torch.bfloat16, "logits")
         self._need(out, torch.int32, "out")
         V = int(logits.shape[-1])
-        self._call("btb_hip_argmax", self.ptr(logits), self.ptr(out), int(logits.numel()) // V, V, _stream())
+        self._call("btb_hip_argmax", _p(logits), _p(out), int(logits.numel()) // V, V, _stream())
         return out
 
     def publish(self, n0: torch.Tensor, picked: torch.Tensor, next_ids: torch.Tensor | None = None,
                 out_tok: torch.Tensor | None = None, out_n0: torch.Tensor | None = None,
                 out_ts: torch.Tensor | None = None) -> None:
         """the step's end: next_ids = picked, n0 += 1, and the token / clock / length into pinned host tensors"""
-        p = lambda t: None if t is None else self.ptr(t)
-        self._call("btb_hip_publish", self.ptr(n0), self.ptr(picked), p(next_ids), p(out_tok), p(out_n0), p(out_ts),
+        p = lambda t: None if t is None else _p(t)
+        self._call("btb_hip_publish", _p(n0), _p(picked), p(next_ids), p(out_tok), p(out_n0), p(out_ts),
                    _stream())
 
     def publish_only(self, n0: torch.Tensor, ids: torch.Tensor, out_tok: torch.Tensor, out_n0: torch.Tensor | None = None,
                      out_ts: torch.Tensor | None = None) -> None:
         """the reference's `btb_publish`: token, clock and length into pinned host tensors, nothing else"""
-        p = lambda t: None if t is None else self.ptr(t)
-        self._call("btb_hip_publish_only", self.ptr(n0), self.ptr(ids), self.ptr(out_tok), p(out_n0), p(out_ts), _stream())
+        p = lambda t: None if t is None else _p(t)
+        self._call("btb_hip_publish_only", _p(n0), _p(ids), _p(out_tok), p(out_n0), p(out_ts), _stream())
 
     def argmax_publish(self, logits: torch.Tensor, picked: torch.Tensor, n0: torch.Tensor,
                        next_ids: torch.Tensor | None = None, out_tok: torch.Tensor | None = None,
@@ -845,8 +842,8 @@ class HipCard:
         V = int(logits.shape[-1])
         if logits.numel() != V:
             raise ValueError("[hip] argmax_publish: one row of logits")
-        p = lambda t: None if t is None else self.ptr(t)
-        self._call("btb_hip_argmax_publish", self.ptr(logits), V, self.ptr(picked), self.ptr(n0), p(next_ids),
+        p = lambda t: None if t is None else _p(t)
+        self._call("btb_hip_argmax_publish", _p(logits), V, _p(picked), _p(n0), p(next_ids),
                    p(out_tok), p(out_n0), p(out_ts), _stream())
 
     # -- the step as one persistent launch ------------------------------------------------------------------------

@@ -285,6 +285,18 @@ int32_t btb_hip_attn_decode_win(const void* q, const void* K, const void* V, voi
                                 float scale, size_t cap, size_t S, int64_t win, const int32_t* tbl, float* workspace,
                                 void* stream);
 
+/* btb_attn_flash_d128 with the reference kernel's own scratch arguments (native/cuda/btb_attn_flash.cuh:372-379): the
+ * spans' states go into the caller's three arrays - part_m and part_l of S * T * Hq floats, part_acc of S * T * Hq * 128,
+ * the sizes the reference's card graph allocates (btb/engine/cuda.py:1563-1583), in this library's own order - so a
+ * launch by the reference's kernel name allocates nothing and a captured graph keeps reading the arrays it was recorded
+ * with. `span` keys a span (a multiple of 128; the reference's key group is 512), S spans: S * span need not be the
+ * cache's capacity, only reach it - every load stays on a key the row sees. The bits are btb_hip_attn_decode_win's at
+ * cap = S * span on its general kernel; the reference's arrival counter is not needed (a second launch folds). */
+int32_t btb_hip_attn_decode_parts(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
+                                  const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
+                                  float scale, size_t span, size_t S, int64_t win, const int32_t* tbl, float* part_m,
+                                  float* part_l, float* part_acc, void* stream);
+
 /* btb_hip_attn_decode for callers that cannot allocate device memory or pass a workspace: code under hipGraph
  * capture, tight serving loops, harnesses that forbid hipMalloc. No counterpart in the reference. The spans' partial
  * states go into an array the library itself holds on every GPU it runs on (BTB_HIP_ATTN_NOALLOC_FLOATS floats =
@@ -302,7 +314,9 @@ int32_t btb_hip_attn_decode_noalloc(const void* q, const void* K, const void* V,
 /* The decode step's own attention (one row), straight from the fused qkv row [(Hq + 2 Hk) D] bf16: what
  * btb_hip_norm_rope_kv followed by btb_hip_attn_decode compute at T = 1, bit for bit, in one launch less - the
  * q / k norm and rope happen inside the attention workgroups (q never reaches memory), the workgroup whose key span
- * holds slot *n0 writes the new K / V row. Same scratch, spans and limits as btb_hip_attn_decode. Replaces the pair
+ * holds slot *n0 writes the new K / V row - unless *n0 >= cap: a cache that is already full is not written past
+ * (the keys the row then attends to are the cache's `cap` and its own, taken from the chip). Same scratch, spans and
+ * limits as btb_hip_attn_decode. Replaces the pair
  * btb_norm_rope_kv_d128 + btb_attn_flash_d128 of the reference's card step (btb/engine/cuda.py:1756-1790). */
 int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk, float eps, int32_t centered,
                                 const void* cos_t, const void* sin_t, const int32_t* n0, void* K, void* V, void* att,

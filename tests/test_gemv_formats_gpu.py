@@ -7,6 +7,8 @@ and the reference card's own bar of one bf16 ulp of the largest output.
 
 from __future__ import annotations
 
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -90,7 +92,7 @@ def test_format_refusals(card):
     x = torch.zeros(64, dtype=torch.bfloat16, device="cuda")
     y = torch.zeros(64, dtype=torch.bfloat16, device="cuda")
     s = torch.ones(16, dtype=torch.float32, device="cuda")
-    p = card.ptr
+    p = lambda t: card.ptr(ctypes.c_void_p, t)
     assert L.btb_hip_gemv_mxfp4(p(z), p(z), p(x), p(y), 4, 48, 1, None) == -6          # C % 32
     assert L.btb_hip_gemv_mxfp4(None, p(z), p(x), p(y), 4, 64, 1, None) == -1
     assert L.btb_hip_gemv_fp8(p(z), p(s), 3, 1, p(x), p(y), 4, 64, 1, None) == -6       # 3 does not divide 4

@@ -9,6 +9,8 @@ bf16 rounding flip: 2^-8 relative to the output. The reference's own card bar, o
 
 from __future__ import annotations
 
+import ctypes
+
 import numpy as np
 import pytest
 import torch
@@ -222,9 +224,9 @@ def test_refusals_launch_nothing(card):
         card.gemv(w, x, torch.empty(3, dtype=torch.bfloat16, device="cuda"))
     L = card.lib
     y = torch.full((1, 16), 7.0, dtype=torch.bfloat16, device="cuda")
-    assert L.btb_hip_gemv_bf16(None, card.ptr(x), card.ptr(y), 16, 64, 1, None) == -1
-    assert L.btb_hip_gemv_bf16(card.ptr(w), card.ptr(x), card.ptr(y), 0, 64, 1, None) == -6
-    assert L.btb_hip_gemv_bf16(card.ptr(w), card.ptr(x), card.ptr(y), 16, 60, 1, None) == -6  # C % 8
-    assert L.btb_hip_gemv_bf16(None, card.ptr(x), card.ptr(y), 0, 64, 1, None) == -1  # null before domain
+    assert L.btb_hip_gemv_bf16(None, card.ptr(ctypes.c_void_p, x), card.ptr(ctypes.c_void_p, y), 16, 64, 1, None) == -1
+    assert L.btb_hip_gemv_bf16(card.ptr(ctypes.c_void_p, w), card.ptr(ctypes.c_void_p, x), card.ptr(ctypes.c_void_p, y), 0, 64, 1, None) == -6
+    assert L.btb_hip_gemv_bf16(card.ptr(ctypes.c_void_p, w), card.ptr(ctypes.c_void_p, x), card.ptr(ctypes.c_void_p, y), 16, 60, 1, None) == -6  # C % 8
+    assert L.btb_hip_gemv_bf16(None, card.ptr(ctypes.c_void_p, x), card.ptr(ctypes.c_void_p, y), 0, 64, 1, None) == -1  # null before domain
     torch.cuda.synchronize()
     assert torch.all(y == 7.0)

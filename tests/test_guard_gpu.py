@@ -150,6 +150,28 @@ def test_attention_outputs_stay_inside(card, n0, T, S):
         assert torch.equal(att3.t, att.t)
 
 
+@pytest.mark.parametrize("n0", [100, 117, 127])
+def test_step_attention_writes_no_row_past_the_caches_end(card, n0):
+    """spans are whole 128-key batches, so a span can reach past the cache's last slot: a cache length at or past the
+    capacity (a caller that did not count its rows) must leave K and V - fenced - untouched"""
+    Hq, Hk, D, cap, S = 32, 8, 128, 100, 1
+    g = gen(925)
+    K = Fenced((Hk, cap, D), torch.bfloat16, torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda())
+    V = Fenced((Hk, cap, D), torch.bfloat16, torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda())
+    K0, V0 = K.t.clone(), V.t.clone()
+    qkv = fin(torch.randn(1, (Hq + 2 * Hk) * D, generator=g).to(torch.bfloat16))
+    wq = fin(torch.ones(D, dtype=torch.bfloat16))
+    cfg = StackConfig(layers=1, hidden=256, q_heads=Hq, kv_heads=Hk, head_dim=D, intermediate=256, vocab=256)
+    cos, sin = rope_tables(cfg, 128, "cuda")
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    scratch = Fenced((int(card.lib.btb_hip_attn_scratch_floats(1, Hq, Hk, D, S)),), torch.float32)
+    att = Fenced((1, Hq * D), torch.bfloat16)
+    card.attn_decode_qkv(qkv, wq, wq, 1e-6, cos, sin, n0t, K.t, V.t, att.t, Hq, Hk, D, D**-0.5, S, scratch.t)
+    for f, what in ((K, "K"), (V, "V"), (att, "att"), (scratch, "scratch")):
+        f.check(f"attn_decode_qkv past the end: {what}")
+    assert torch.equal(K.t, K0) and torch.equal(V.t, V0)
+
+
 @pytest.mark.parametrize("T", [1, 5])
 def test_moe_outputs_stay_inside(card, T):
     E, k, H, I = 16, 4, 2048, 768

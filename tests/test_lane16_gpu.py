@@ -119,8 +119,8 @@ def test_group_equals_single_calls_and_refusals(card):
     torch.cuda.synchronize()
     assert all(torch.equal(a, b) for a, b in zip(before, y))
     w0, x0, y0 = ws[0], x[0], y[0]
-    assert L.btb_hip_gemv_bf16_rows(card.ptr(w0), 12, 64, ctypes.c_void_p(x0.data_ptr() + 2), 2, card.ptr(y0), None) == -6
-    assert L.btb_hip_gemv_bf16_rows(None, 0, 64, card.ptr(x0), 2, card.ptr(y0), None) == -1
+    assert L.btb_hip_gemv_bf16_rows(card.ptr(ctypes.c_void_p, w0), 12, 64, ctypes.c_void_p(x0.data_ptr() + 2), 2, card.ptr(ctypes.c_void_p, y0), None) == -6
+    assert L.btb_hip_gemv_bf16_rows(None, 0, 64, card.ptr(ctypes.c_void_p, x0), 2, card.ptr(ctypes.c_void_p, y0), None) == -1
 
 
 @pytest.mark.parametrize("rows,cols", [(128, 2048), (67, 1100)])

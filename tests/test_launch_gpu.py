@@ -98,7 +98,8 @@ def test_launcher_refusals(card):
 def test_attention_rope_and_publish_kernels_by_name(card):
     """btb_norm_rope_kv_tbl_d128, btb_attn_flash_d128 and btb_publish with the reference's own parameter lists
     (btb/engine/card_launch.py:469-523, 2152-2212, 2334-2347): the typed wrappers' bits. The attention's partial-state
-    arrays and arrival counter are the caller's in the reference's layout and go unused here - the card keeps its own."""
+    arrays are the caller's, at the reference's sizes, and hold the key groups' states; its arrival counter is not
+    needed (a second launch folds the groups) and is left at zero."""
     import numpy as np
 
     from btb_amd.decode import StackConfig, rope_tables
@@ -135,12 +136,14 @@ def test_attention_rope_and_publish_kernels_by_name(card):
     a2 = torch.zeros_like(a1)
     card.attn_decode(q1, K1, V1, a1, n0t, Hq, Hk, D, scale, S, card.attn_scratch(T, Hq, Hk, D, S), par=par, win=300, tbl=tbl)
     part_m = torch.zeros(S * T * Hq, dtype=torch.float32, device="cuda")
+    part_l = torch.zeros(S * T * Hq, dtype=torch.float32, device="cuda")
     part_acc = torch.zeros(S * T * Hq * D, dtype=torch.float32, device="cuda")
     cnt = torch.zeros(T * Hq, dtype=torch.int32, device="cuda")
     card.launch("btb_attn_flash_d128", ((T * G + 7) // 8, S, Hk), (256, 1, 1),
                 [p(q1), p(K1), p(V1), p(a2), p(n0t), p(par), I(T), I(Hq), I(Hk), I(hs), I(rs), F(scale), p(part_m),
-                 p(part_m.clone()), p(part_acc), p(cnt), I(300), p(tbl)], shared=8192)
+                 p(part_l), p(part_acc), p(cnt), I(300), p(tbl)], shared=8192)
     assert torch.equal(a1, a2) and bool(a1.float().abs().sum() > 0)
+    assert int(cnt.abs().sum()) == 0 and bool(part_l.abs().sum() > 0)   # the states went into the caller's arrays
 
     ids = torch.tensor([4242], dtype=torch.int32, device="cuda")
     out_tok = torch.zeros(1, dtype=torch.int32).pin_memory()
