@@ -1,7 +1,7 @@
 """Benchmark of the decode hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode|decode_p12] [--no-cpu]
-    python bench.py --workload gemv_bf16|gemv_p12|gemv_fp8|gemv_mxfp4|moe [--m M]      (the other configs, one kernel each)
+    python bench.py --workload gemv_bf16|gemv_p12|gemv_fp8|gemv_mxfp4|moe|moe_mxfp4 [--m M]   (the other configs, one operator each)
     python bench.py --workload copy          (a plain 2^28-byte device copy: the scale of the FETCH_SIZE / WRITE_SIZE counters)
 
 A step is one decode step of a random-init Qwen3-4B-shaped dense stack (36 layers, hidden 2560, 32 query / 8 kv heads
@@ -112,11 +112,32 @@ def cpu_baseline(workload: str = "decode", m: int = 1, budget_s: float = 12.0) -
 
         per_call = None
         what = f"MoE layers: top-{k} of {E} experts, gate_up [{2 * I}x{H}] + down [{H}x{I}] bf16, {m} tokens"
+    elif workload == "moe_mxfp4":
+        from oracle import moe as omoe
+
+        E, k, H, I = 128, 8, 2048, 768
+        wr = (rng.integers(0x3A00, 0x3D00, (E, H), dtype=np.uint16) | (rng.integers(0, 2, (E, H), dtype=np.uint16) << 15))
+        gb = rng.integers(0, 256, (E, 2 * I, H // 32, 16), dtype=np.uint8)
+        gs = rng.integers(115, 123, (E, 2 * I, H // 32), dtype=np.uint8)
+        db = rng.integers(0, 256, (E, H, I // 32, 16), dtype=np.uint8)
+        ds = rng.integers(115, 123, (E, H, I // 32), dtype=np.uint8)
+        xs = [codecs.round_bf16(rng.standard_normal((m, H)).astype(np.float32)) for _ in range(16)]
+        distinct = []
+
+        def call(i, t):
+            x = xs[i % len(xs)]
+            _, w, picks = omoe.router(wr, x, k, "bf16")
+            omoe.experts_mx4(gb, gs, db, ds, x, picks, w, dt="bf16", oss=False)
+            distinct.append(len(set(picks.reshape(-1).tolist())))
+
+        per_call = None
+        what = (f"MoE layers: top-{k} of {E} experts, gate_up [{2 * I}x{H}] + down [{H}x{I}] MXFP4 as stored (random "
+                f"bytes), {m} tokens")
     else:
         raise ValueError(workload)
 
     call(0, 0)
-    if workload == "moe":
+    if workload in ("moe", "moe_mxfp4"):
         distinct.clear()
     t0 = time.perf_counter()
     calls = 0
@@ -124,8 +145,9 @@ def cpu_baseline(workload: str = "decode", m: int = 1, budget_s: float = 12.0) -
         call(calls, 0)
         calls += 1
     dt = time.perf_counter() - t0
-    if workload == "moe":
-        nbytes = sum(128 * 2048 * 2 + d * (2 * 768 * 2048 + 2048 * 768) * 2 for d in distinct)
+    if workload in ("moe", "moe_mxfp4"):
+        per_w = 2.0 if workload == "moe" else 17 / 32
+        nbytes = sum(128 * 2048 * 2 + d * (2 * 768 * 2048 + 2048 * 768) * per_w for d in distinct)
         return {"value": round(nbytes / dt / 1e9, 2), "unit": "GB/s", "cores": cores, "kind": "port", "isa": oracle.isa(),
                 "sample": f"{calls} {what} through the oracle's numpy + C layer, matvecs on all {cores} host threads, "
                           f"{dt:.1f} s; bytes = the router and every distinct picked expert"}
@@ -190,6 +212,7 @@ def kernel_workload(args: argparse.Namespace) -> int:
       gemv_fp8    C5a: fp8.quantize(N(0, 0.02) [18432, 7168], (128, 128))
       gemv_mxfp4  C5b: the same source through the MXFP4 encoder
       moe         C4: router [128, 2048] + top-8 of 128 experts (gate_up [1536, 2048], down [2048, 768]), M tokens
+      moe_mxfp4   the same layer with its expert stacks stored as MXFP4
     """
     import torch
 
@@ -208,7 +231,39 @@ def kernel_workload(args: argparse.Namespace) -> int:
         return torch.randn(*shape, generator=g, device=dev, dtype=torch.float32) * 0.02
 
     name = args.workload
-    if name == "moe":
+    if name == "moe_mxfp4":
+        # C4's layer with its experts stored as MXFP4 (what gpt-oss-style checkpoints ship): two layers' stacks and
+        # sixteen sets of rows, as below
+        from btb_amd.load import MxExperts
+        from btb_amd.moe import MxExpertsLayer
+
+        E, k, H, I, pool = 128, 8, 2048, 768, 16
+
+        def mx_layer():
+            gb, gs = mxfp4.quantize(normal(E * 2 * I, H))
+            db, ds = mxfp4.quantize(normal(E * H, I))
+            return MxExpertsLayer(card, MxExperts(gb.reshape(E, 2 * I, H // 32, 16), gs.reshape(E, 2 * I, H // 32),
+                                                  db.reshape(E, H, I // 32, 16), ds.reshape(E, H, I // 32)), oss=False)
+
+        sets = [(Router(card, normal(E, H).to(torch.bfloat16), k), mx_layer()) for _ in range(2)]
+        xs = [torch.randn(M, H, generator=g, device=dev).to(torch.bfloat16) for _ in range(pool)]
+        distinct = []
+
+        def call(i: int) -> None:
+            router, experts = sets[i % 2]
+            _, w, idx = router(xs[i])
+            experts(xs[i], idx, w)
+
+        for i in range(pool):
+            _, _, idx = sets[i % 2][0](xs[i])
+            distinct.append(int(torch.unique(idx).numel()))
+        per_expert = (2 * I * H + H * I) * 17 // 32
+        nbytes = [E * H * 2 + d * per_expert for d in distinct]
+        what = f"C4 with MXFP4 experts: top-{k} of {E}, gate_up [{2 * I}, {H}] + down [{H}, {I}] as stored, M={M} tokens"
+        extra = {"distinct_experts": distinct}
+        dtype = "mxfp4 expert weights widened to bf16 in registers, bf16 activations, f32 accumulate"
+        kernel = "the routed layer over MXFP4 stacks: router matvec + routing, gate/up with the SwiGLU fold, down with the weighted sum"
+    elif name == "moe":
         # two layers' stacks (3.6 GB) and sixteen sets of rows: every call routes to other experts, so a pass streams
         # 1.2 GB (one token) and more of distinct expert matrices - nothing comes back out of the 256 MB cache
         E, k, H, I, pool = 128, 8, 2048, 768, 16
@@ -401,7 +456,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="decode",
-                    choices=["decode", "decode_p12", "gemv_bf16", "gemv_p12", "gemv_fp8", "gemv_mxfp4", "moe", "copy"])
+                    choices=["decode", "decode_p12", "gemv_bf16", "gemv_p12", "gemv_fp8", "gemv_mxfp4", "moe", "moe_mxfp4", "copy"])
     ap.add_argument("--m", type=int, default=1, help="rows of x (tokens) for the single-operator workloads")
     ap.add_argument("--rows", type=int, default=1,
                     help="rows of a decode pass: 1 is the step the metric is quoted on, more a speculative verify pass")

@@ -186,18 +186,70 @@ __global__ void __launch_bounds__(256) moe_group_picks_kernel(const int32_t* __r
 }
 
 // ------------------------------------------------------------------------------------------------------------
+// the experts' stacks in their stored form, and the layer's middle
+// ------------------------------------------------------------------------------------------------------------
+
+// bf16: a = the weights [E, R, C]. MXFP4 (the checkpoint's layout, btb/mxfp4.py:4-29): a = blocks u8 [E, R, C / 32, 16],
+// b = scales u8 [E, R, C / 32]. An expert's matrix is a slice of the stack; nothing is widened ahead of the matvec.
+struct Stack {
+    const void* a;
+    const void* b;
+};
+template <class F>
+__device__ __forceinline__ typename F::Params expert_of(const Stack& s, int expert, int R, int units);
+template <>
+__device__ __forceinline__ FmtBf16::Params expert_of<FmtBf16>(const Stack& s, int expert, int R, int units) {
+    return FmtBf16::Params{static_cast<const uint4*>(s.a) + (size_t)expert * R * units};
+}
+template <>
+__device__ __forceinline__ FmtMx4::Params expert_of<FmtMx4>(const Stack& s, int expert, int R, int units) {
+    return FmtMx4::Params{static_cast<const uint8_t*>(s.a) + (size_t)expert * R * units * 16,
+                          static_cast<const uint8_t*>(s.b) + (size_t)expert * R * units};
+}
+
+// What becomes of an expert's gate and up sums (each already the rows' dtype: bf16(sum)).
+// OSS = false: the families that concatenate the halves - gate row r, up row I + r - and h = bf16(bf16(silu(g)) * u)
+// (`_silu_gate`, btb/engine/host.py:439-441). OSS = true: gpt-oss - the halves interleaved (gate row 2 r, up row
+// 2 r + 1), the expert's bias added to both, the gate clamped above and the up half on both sides, and
+// h = (up + 1) * (gate * sigmoid(alpha * gate)) with every operation rounded to the rows' dtype as torch rounds it
+// (`gpt_oss_gate`, host.py:443-451; `_act` adds the bias first, :414-419).
+struct Glu {
+    const uint16_t* bias;  // [E, 2I] bf16, or null
+    float alpha, limit;
+};
+template <bool OSS>
+__device__ __forceinline__ int glu_row(int r, int j, int I) {
+    return OSS ? 2 * r + j : r + j * I;
+}
+template <bool OSS>
+__device__ __forceinline__ uint16_t glu_out(float g, float u, const Glu& a, int expert, int r, int I) {
+    if (!OSS) return f32_bf16(bfround(g / (1.f + expf(-g))) * u);
+    if (a.bias != nullptr) {
+        const uint16_t* b = a.bias + (size_t)expert * 2 * I + 2 * r;
+        g = bfround(g + bf16_f32(b[0]));
+        u = bfround(u + bf16_f32(b[1]));
+    }
+    g = g > a.limit ? a.limit : g;  // a NaN stays a NaN, as in torch's clamp
+    u = u > a.limit ? a.limit : (u < -a.limit ? -a.limit : u);
+    const float t = bfround(g * a.alpha);
+    const float sg = bfround(1.f / (1.f + expf(-t)));
+    const float glu = bfround(g * sg);
+    const float up1 = bfround(u + 1.f);
+    return f32_bf16(up1 * glu);
+}
+
+// ------------------------------------------------------------------------------------------------------------
 // gate_up: the dense loop over (token, pick) pairs; blockIdx.y is the pair
 // ------------------------------------------------------------------------------------------------------------
 
 // A wave takes gate row r and up row I + r together (RPW = 2) and writes h[r] = bf16(bf16(silu(bf16(g))) * bf16(u)): the
 // pair's gu row is never stored, the down kernel finds its x ready.
-template <int LPR, int RPW, int U>
-__global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restrict__ stack, const uint16_t* __restrict__ x,
+template <class F, bool OSS, int LPR, int RPW, int U>
+__global__ void __launch_bounds__(256) moe_gate_up_kernel(Stack stack, const uint16_t* __restrict__ x,
                                                           const int32_t* __restrict__ idx, uint16_t* __restrict__ h,
-                                                          int R, int C, int k, int E) {
+                                                          int R, int C, int k, int E, Glu glu) {
     static_assert(RPW == 2, "gate and up");
     extern __shared__ __align__(16) uint32_t xs[];
-    using F = FmtBf16;
     constexpr int G = WAVE / LPR, ROWS = G;
     const int pair = blockIdx.y;
     const int token = pair / k;
@@ -210,28 +262,28 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
     const int I = R / 2;
     const int ntiles = (I + ROWS - 1) / ROWS;
     const int span = U * LPR;
-    F::Params p{stack + (size_t)expert * R * units};
+    const typename F::Params p = expert_of<F>(stack, expert, R, units);
     uint16_t* y = h + (size_t)pair * I;
 
     // the wave's first span of weights is requested right behind x's own loads, before anything waits for x: the
     // weights do not depend on x, and nothing about these loads is conditional (a wave past the last tile requests the
     // last tile's and drops them)
-    F::Raw first[U][RPW] = {};
+    typename F::Raw first[U][RPW] = {};
     stage_x<X_PLAIN>(xs, XArgs{x + (size_t)token * C, nullptr, nullptr, nullptr, 0.f, 0}, 1, C, [&] {
-        F::RowCtx c0[RPW];
+        typename F::RowCtx c0[RPW];
 #pragma unroll
         for (int j = 0; j < RPW; ++j)
-            c0[j] = F::row_ctx(p, (size_t)(min(min(wave, ntiles - 1) * ROWS + lane / LPR, I - 1) + j * I), units);
+            c0[j] = F::row_ctx(p, (size_t)glu_row<OSS>(min(min(wave, ntiles - 1) * ROWS + lane / LPR, I - 1), j, I), units);
         load_span_always<F, LPR, RPW, U>(first, c0, 0, sl, units);
     });
     const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
     for (int tile = wave; tile < ntiles; tile += nwaves) {
-        F::RowCtx ctx[RPW];
+        typename F::RowCtx ctx[RPW];
         int rows[RPW];
 #pragma unroll
         for (int j = 0; j < RPW; ++j) {
             rows[j] = tile * ROWS + lane / LPR;
-            ctx[j] = F::row_ctx(p, (size_t)(min(rows[j], I - 1) + j * I), units);
+            ctx[j] = F::row_ctx(p, (size_t)glu_row<OSS>(min(rows[j], I - 1), j, I), units);
         }
         float acc[RPW][1];
 #pragma unroll
@@ -242,7 +294,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
             k0 = span;
         }
         for (; k0 < units; k0 += span) {
-            F::Raw raw[U][RPW];
+            typename F::Raw raw[U][RPW];
             if (k0 + span <= units) {
                 load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
                 fma_span<F, 1, LPR, RPW, U, false>(raw, ctx, k0, sl, units, xs4, C / 8, acc);
@@ -253,7 +305,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
         }
         const float g = bfround(group_sum<LPR>(acc[0][0]));
         const float u = bfround(group_sum<LPR>(acc[1][0]));
-        if (sl == 0 && rows[0] < I) y[rows[0]] = f32_bf16(bfround(g / (1.f + expf(-g))) * u);
+        if (sl == 0 && rows[0] < I) y[rows[0]] = glu_out<OSS>(g, u, glu, expert, rows[0], I);
     }
 }
 
@@ -263,14 +315,12 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(const uint4* __restric
 // before asking memory for anything. A product is a row of x against a row of weights in the lane order above, so
 // each h row has the bits the kernel above gives it. n = T k <= GROUP_MAX_PAIRS.
 constexpr int GROUP_MAX_PAIRS = 256;
-template <int LPR, int RPW, int U, int MC>
-__global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* __restrict__ stack,
-                                                                  const uint16_t* __restrict__ x,
+template <class F, bool OSS, int LPR, int RPW, int U, int MC>
+__global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(Stack stack, const uint16_t* __restrict__ x,
                                                                   const int32_t* __restrict__ idx, uint16_t* __restrict__ h,
-                                                                  int R, int C, int k, int E, int n) {
+                                                                  int R, int C, int k, int E, int n, Glu glu) {
     static_assert(RPW == 2, "gate and up");
     extern __shared__ __align__(16) uint32_t xs[];  // [MC][C / 2]
-    using F = FmtBf16;
     constexpr int G = WAVE / LPR, ROWS = G;
     constexpr int NM = GROUP_MAX_PAIRS / WAVE;  // ballots that cover the pairs
     const int pair = blockIdx.y;
@@ -325,7 +375,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* _
     const int I = R / 2;
     const int ntiles = (I + ROWS - 1) / ROWS;
     const int span = U * LPR;
-    F::Params p{stack + (size_t)expert * R * units};
+    const typename F::Params p = expert_of<F>(stack, expert, R, units);
     const int per = C / 8;  // 16-byte pieces a row of x
     uint4* xd = reinterpret_cast<uint4*>(xs);
     const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
@@ -333,12 +383,13 @@ __global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* _
     // for before the rows of x are staged (it needs the expert only), as in the kernel above.
     auto pass = [&](auto mtag, int r0, int mc) {
         constexpr int M = decltype(mtag)::value;
-        F::Raw first[U][RPW] = {};
+        typename F::Raw first[U][RPW] = {};
         {
-            F::RowCtx c0[RPW];
+            typename F::RowCtx c0[RPW];
 #pragma unroll
             for (int j = 0; j < RPW; ++j)
-                c0[j] = F::row_ctx(p, (size_t)(min(min(wave, ntiles - 1) * ROWS + lane / LPR, I - 1) + j * I), units);
+                c0[j] = F::row_ctx(p, (size_t)glu_row<OSS>(min(min(wave, ntiles - 1) * ROWS + lane / LPR, I - 1), j, I),
+                                   units);
             load_span_always<F, LPR, RPW, U>(first, c0, 0, sl, units);
         }
         if (r0 != 0) __syncthreads();  // the previous pass has read its rows
@@ -355,12 +406,12 @@ __global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* _
         }
         __syncthreads();
         for (int tile = wave; tile < ntiles; tile += nwaves) {
-            F::RowCtx ctx[RPW];
+            typename F::RowCtx ctx[RPW];
             int rows[RPW];
 #pragma unroll
             for (int j = 0; j < RPW; ++j) {
                 rows[j] = tile * ROWS + lane / LPR;
-                ctx[j] = F::row_ctx(p, (size_t)(min(rows[j], I - 1) + j * I), units);
+                ctx[j] = F::row_ctx(p, (size_t)glu_row<OSS>(min(rows[j], I - 1), j, I), units);
             }
             float acc[RPW][M];
 #pragma unroll
@@ -373,7 +424,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* _
                 k0 = span;
             }
             for (; k0 < units; k0 += span) {
-                F::Raw raw[U][RPW];
+                typename F::Raw raw[U][RPW];
                 if (k0 + span <= units) {
                     load_span<F, LPR, RPW, U, false>(raw, ctx, k0, sl, units);
                     fma_span<F, M, LPR, RPW, U, false>(raw, ctx, k0, sl, units, xs4, C / 8, acc);
@@ -387,7 +438,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* _
                 const float g = bfround(group_sum<LPR>(acc[0][m]));
                 const float u = bfround(group_sum<LPR>(acc[1][m]));
                 if (sl == 0 && rows[0] < I && m < mc)
-                    h[(size_t)prs[m] * I + rows[0]] = f32_bf16(bfround(g / (1.f + expf(-g))) * u);
+                    h[(size_t)prs[m] * I + rows[0]] = glu_out<OSS>(g, u, glu, expert, rows[0], I);
             }
         }
     };
@@ -406,14 +457,16 @@ __global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(const uint4* _
 // down + weighted sum: blockIdx.y is the token; the k experts of a row are walked in ascending expert id
 // ------------------------------------------------------------------------------------------------------------
 
-template <int LPR, int RPW, int U, int KB>
-__global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__ stack, const uint16_t* __restrict__ h,
+// `bias` ([E, R] bf16 or null; gpt-oss): added to the expert's product after its rounding to the rows' dtype and before
+// the pick's weight, as `_down` adds it (btb/engine/host.py:427-432).
+template <class F, int LPR, int RPW, int U, int KB>
+__global__ void __launch_bounds__(256) moe_down_kernel(Stack stack, const uint16_t* __restrict__ h,
                                                        const int32_t* __restrict__ idx, const uint16_t* __restrict__ wts,
-                                                       uint16_t* __restrict__ y, int R, int C, int k, int E) {
+                                                       uint16_t* __restrict__ y, int R, int C, int k, int E,
+                                                       const uint16_t* __restrict__ bias) {
     extern __shared__ __align__(16) uint32_t hs[];  // [k][C / 2] the k experts' h rows, in ascending expert order
     __shared__ int s_expert[ROUTE_MAX_K];
     __shared__ float s_weight[ROUTE_MAX_K];
-    using F = FmtBf16;
     constexpr int G = WAVE / LPR, ROWS = G * RPW;
     const int token = blockIdx.y;
     const int units = C / F::UW;
@@ -456,13 +509,13 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__
 #pragma unroll
     for (int t = 0; t < PER; ++t) hv[t] = piece(min((int)threadIdx.x + t * 256, n - 1));
 
-    F::RowCtx ctx[KB][RPW];
-    F::Raw first[KB][U][RPW] = {};
+    typename F::RowCtx ctx[KB][RPW];
+    typename F::Raw first[KB][U][RPW] = {};
     auto request = [&](int tile, int q0, auto always) {
 #pragma unroll
         for (int b = 0; b < KB; ++b) {
             const int expert = s_expert[min(q0 + b, k - 1)] & 0xFFFFF;
-            F::Params p{stack + (size_t)expert * R * units};
+            const typename F::Params p = expert_of<F>(stack, expert, R, units);
 #pragma unroll
             for (int j = 0; j < RPW; ++j)
                 ctx[b][j] = F::row_ctx(p, (size_t)min(tile * ROWS + j * G + lane / LPR, R - 1), units);
@@ -500,15 +553,17 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__
                     const uint4* xq = hs4 + (size_t)q * (C / 8);
                     fma_span<F, 1, LPR, RPW, U, true>(first[b], ctx[b], 0, sl, units, xq, C / 8, acc);
                     for (int k0 = span; k0 < units; k0 += span) {
-                        F::Raw raw[U][RPW];
+                        typename F::Raw raw[U][RPW];
                         load_span<F, LPR, RPW, U, true>(raw, ctx[b], k0, sl, units);
                         fma_span<F, 1, LPR, RPW, U, true>(raw, ctx[b], k0, sl, units, xq, C / 8, acc);
                     }
                     const float wq = s_weight[q];
 #pragma unroll
                     for (int j = 0; j < RPW; ++j) {
-                        const float d = bfround(group_sum<LPR>(acc[j][0]));  // the expert's down product, as the row's dtype
-                        out[j] = bfround(out[j] + bfround(d * wq));          // times its weight, added in bf16
+                        float d = bfround(group_sum<LPR>(acc[j][0]));  // the expert's down product, as the row's dtype
+                        if (bias != nullptr)
+                            d = bfround(d + bf16_f32(bias[(size_t)(s_expert[q] & 0xFFFFF) * R + min(rows[j], R - 1)]));
+                        out[j] = bfround(out[j] + bfround(d * wq));    // times its weight, added in bf16
                     }
                 }
             }
@@ -521,15 +576,22 @@ __global__ void __launch_bounds__(256) moe_down_kernel(const uint4* __restrict__
 
 static bool al(const void* p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) == 0; }
 
+// lanes a row: enough that a lane's share of a row is a few units (one 16-byte load each)
 static int lanes_for(int units) {
     if (units % 64 == 0 || units >= 256) return 64;
     if (units % 32 == 0 || units >= 96) return 32;
     return 16;
 }
+// an MXFP4 unit is 32 weights, so rows hold few of them (64 in a 2048-wide row): fewer lanes a row, more rows a wave
+static int lanes_for_mx4(int units) {
+    if (units >= 256) return 64;
+    if (units >= 128) return 32;
+    return 16;
+}
 
-template <int LPR>
-static int32_t launch_gate_up(const void* stack, const void* x, const int32_t* idx, void* gu, int R, int C, int k, int E,
-                              int pairs, hipStream_t st) {
+template <class F, bool OSS, int LPR>
+static int32_t launch_gate_up(Stack stack, const void* x, const int32_t* idx, void* gu, int R, int C, int k, int E,
+                              int pairs, Glu glu, hipStream_t st) {
     constexpr int RPW = 2, U = 4, G = WAVE / LPR;
     const int ntiles = (R / 2 + G - 1) / G;
     const int grid = (ntiles + 3) / 4;
@@ -544,42 +606,67 @@ static int32_t launch_gate_up(const void* stack, const void* x, const int32_t* i
     const int grouped = tuning("moe_grouped");
     const bool wanted = grouped >= 0 ? grouped != 0 && pairs > k : pairs >= 8 * k;
     if (wanted && pairs <= GROUP_MAX_PAIRS && (size_t)MC * C * 2 <= (size_t)device_info().lds_bytes - 16 * 1024) {
-        auto kern = moe_gate_up_grouped_kernel<LPR, RPW, U, MC>;
+        auto kern = moe_gate_up_grouped_kernel<F, OSS, LPR, RPW, U, MC>;
         const size_t lds = (size_t)MC * C * 2;
         if (lds > 48 * 1024) {
             hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                                hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
             if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
         }
-        hipLaunchKernelGGL(kern, dim3(grid, pairs), dim3(256), lds, st, static_cast<const uint4*>(stack),
-                           static_cast<const uint16_t*>(x), idx, static_cast<uint16_t*>(gu), R, C, k, E, pairs);
+        hipLaunchKernelGGL(kern, dim3(grid, pairs), dim3(256), lds, st, stack, static_cast<const uint16_t*>(x), idx,
+                           static_cast<uint16_t*>(gu), R, C, k, E, pairs, glu);
         return hip_status(hipGetLastError(), "moe gate_up launch");
     }
-    hipLaunchKernelGGL((moe_gate_up_kernel<LPR, RPW, U>), dim3(grid, pairs), dim3(256), (size_t)C * 2, st,
-                       static_cast<const uint4*>(stack), static_cast<const uint16_t*>(x), idx,
-                       static_cast<uint16_t*>(gu), R, C, k, E);
+    hipLaunchKernelGGL((moe_gate_up_kernel<F, OSS, LPR, RPW, U>), dim3(grid, pairs), dim3(256), (size_t)C * 2, st, stack,
+                       static_cast<const uint16_t*>(x), idx, static_cast<uint16_t*>(gu), R, C, k, E, glu);
     return hip_status(hipGetLastError(), "moe gate_up launch");
 }
 
-template <int LPR>
-static int32_t launch_down(const void* stack, const void* gu, const int32_t* idx, const void* w, void* y, int R, int C,
-                           int k, int E, int T, hipStream_t st) {
+template <class F, int LPR>
+static int32_t launch_down(Stack stack, const void* gu, const int32_t* idx, const void* w, void* y, int R, int C, int k,
+                           int E, int T, const void* bias, hipStream_t st) {
     constexpr int RPW = 1, G = WAVE / LPR;
     const int ntiles = (R + G * RPW - 1) / (G * RPW);
     const int grid = (ntiles + 3) / 4;
     const size_t lds = (size_t)k * C * 2;
-    // a row of at most three units a lane (the 768-wide experts of the C4 shape): all eight picks' rows in one request
-    const bool shallow = C / FmtBf16::UW <= 3 * LPR;
-    auto kern = shallow ? moe_down_kernel<LPR, RPW, 3, 8> : moe_down_kernel<LPR, RPW, 4, 4>;
+    // a row of at most three units a lane (the 768-wide experts of the C4 shape: 96 bf16 units over 64 lanes, 24 MXFP4
+    // units over 16): all eight picks' rows in one request
+    const int upl = (C / F::UW + LPR - 1) / LPR;
+    auto kern = upl <= 2   ? moe_down_kernel<F, LPR, RPW, 2, 8>
+                : upl <= 3 ? moe_down_kernel<F, LPR, RPW, 3, 8>
+                           : moe_down_kernel<F, LPR, RPW, 4, 4>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
     }
-    hipLaunchKernelGGL(kern, dim3(grid, T), dim3(256), lds, st, static_cast<const uint4*>(stack),
-                       static_cast<const uint16_t*>(gu), idx, static_cast<const uint16_t*>(w),
-                       static_cast<uint16_t*>(y), R, C, k, E);
+    hipLaunchKernelGGL(kern, dim3(grid, T), dim3(256), lds, st, stack, static_cast<const uint16_t*>(gu), idx,
+                       static_cast<const uint16_t*>(w), static_cast<uint16_t*>(y), R, C, k, E,
+                       static_cast<const uint16_t*>(bias));
     return hip_status(hipGetLastError(), "moe down launch");
+}
+
+// the two launches of the experts over either stored form
+template <class F, bool OSS>
+static int32_t launch_experts(Stack gate_up, Stack down, const void* x, const int32_t* idx, const void* w, void* gu,
+                              void* y, size_t T, size_t k, size_t E, size_t H, size_t I, Glu glu, const void* dn_bias,
+                              hipStream_t st) {
+    const int R1 = (int)(2 * I), C1 = (int)H, R2 = (int)H, C2 = (int)I;
+    constexpr bool MX = std::is_same<F, FmtMx4>::value;
+    const int l1 = MX ? lanes_for_mx4(C1 / F::UW) : lanes_for(C1 / F::UW);
+    const int l2 = MX ? lanes_for_mx4(C2 / F::UW) : lanes_for(C2 / F::UW);
+    int32_t rc;
+    switch (l1) {
+        case 64: rc = launch_gate_up<F, OSS, 64>(gate_up, x, idx, gu, R1, C1, (int)k, (int)E, (int)(T * k), glu, st); break;
+        case 32: rc = launch_gate_up<F, OSS, 32>(gate_up, x, idx, gu, R1, C1, (int)k, (int)E, (int)(T * k), glu, st); break;
+        default: rc = launch_gate_up<F, OSS, 16>(gate_up, x, idx, gu, R1, C1, (int)k, (int)E, (int)(T * k), glu, st); break;
+    }
+    if (rc != OK) return rc;
+    switch (l2) {
+        case 64: return launch_down<F, 64>(down, gu, idx, w, y, R2, C2, (int)k, (int)E, (int)T, dn_bias, st);
+        case 32: return launch_down<F, 32>(down, gu, idx, w, y, R2, C2, (int)k, (int)E, (int)T, dn_bias, st);
+        default: return launch_down<F, 16>(down, gu, idx, w, y, R2, C2, (int)k, (int)E, (int)T, dn_bias, st);
+    }
 }
 
 }  // namespace btb
@@ -644,20 +731,39 @@ int32_t btb_hip_moe_experts_bf16(const void* gate_up, const void* down, const vo
         set_error("moe: the staged rows do not fit LDS");
         return ERR_DOMAIN;
     }
+    return launch_experts<FmtBf16, false>(Stack{gate_up, nullptr}, Stack{down, nullptr}, x, idx, w, gu, y, T, k, E, H, I,
+                                          Glu{nullptr, 0.f, 0.f}, nullptr, static_cast<hipStream_t>(stream));
+}
+
+int32_t btb_hip_moe_experts_mxfp4(const void* gu_blocks, const void* gu_scales, const void* dn_blocks,
+                                  const void* dn_scales, const void* gu_bias, const void* dn_bias, const void* x,
+                                  const int32_t* idx, const void* w, void* h, void* y, size_t T, size_t k, size_t E,
+                                  size_t H, size_t I, int32_t oss, float alpha, float limit, void* stream) {
+    if (gu_blocks == nullptr || gu_scales == nullptr || dn_blocks == nullptr || dn_scales == nullptr || x == nullptr ||
+        idx == nullptr || w == nullptr || h == nullptr || y == nullptr)
+        return ERR_NULL;
+    if (T == 0 || k == 0 || E == 0 || H == 0 || I == 0 || k > (size_t)ROUTE_MAX_K || T * k > 65535 || H % 32 != 0 ||
+        I % 32 != 0 || H > (1u << 20) || I > (1u << 20) || E > (1u << 20))
+        return ERR_DOMAIN;
+    if (!al(gu_blocks, 16) || !al(dn_blocks, 16) || !al(x, 16) || !al(h, 16) || !al(idx, 4) || !al(w, 2) || !al(y, 2) ||
+        !al(gu_bias, 2) || !al(dn_bias, 2))
+        return ERR_DOMAIN;
+    if (!oss && (gu_bias != nullptr || dn_bias != nullptr)) {
+        set_error("moe_experts_mxfp4: biases belong to the gpt-oss form (oss != 0)");
+        return ERR_DOMAIN;
+    }
+    if (oss && !(limit > 0.f && alpha == alpha)) return ERR_DOMAIN;
+    const DeviceInfo& dev = device_info();
+    if (k * I * 2 > (size_t)dev.lds_bytes || H * 2 > (size_t)dev.lds_bytes) {
+        set_error("moe: the staged rows do not fit LDS");
+        return ERR_DOMAIN;
+    }
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const int R1 = (int)(2 * I), C1 = (int)H, R2 = (int)H, C2 = (int)I;
-    int32_t rc;
-    switch (lanes_for(C1 / 8)) {
-        case 64: rc = launch_gate_up<64>(gate_up, x, idx, gu, R1, C1, (int)k, (int)E, (int)(T * k), st); break;
-        case 32: rc = launch_gate_up<32>(gate_up, x, idx, gu, R1, C1, (int)k, (int)E, (int)(T * k), st); break;
-        default: rc = launch_gate_up<16>(gate_up, x, idx, gu, R1, C1, (int)k, (int)E, (int)(T * k), st); break;
-    }
-    if (rc != OK) return rc;
-    switch (lanes_for(C2 / 8)) {
-        case 64: return launch_down<64>(down, gu, idx, w, y, R2, C2, (int)k, (int)E, (int)T, st);
-        case 32: return launch_down<32>(down, gu, idx, w, y, R2, C2, (int)k, (int)E, (int)T, st);
-        default: return launch_down<16>(down, gu, idx, w, y, R2, C2, (int)k, (int)E, (int)T, st);
-    }
+    const Stack gs{gu_blocks, gu_scales}, ds{dn_blocks, dn_scales};
+    if (oss)
+        return launch_experts<FmtMx4, true>(gs, ds, x, idx, w, h, y, T, k, E, H, I,
+                                            Glu{static_cast<const uint16_t*>(gu_bias), alpha, limit}, dn_bias, st);
+    return launch_experts<FmtMx4, false>(gs, ds, x, idx, w, h, y, T, k, E, H, I, Glu{nullptr, 0.f, 0.f}, nullptr, st);
 }
 
 }  // extern "C"

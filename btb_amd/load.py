@@ -207,10 +207,12 @@ class MxExperts:
     even rows); the rows are kept as stored. `gate_up(e)` / `down(e)` are expert e's matrices as `MxWeight` views
     (no copy) for `HipCard.gemv_mx4`; `widen` is `HipCard.mx4_widen` over a whole stack or the experts at `seats`."""
 
-    __slots__ = ("down_blocks", "down_scales", "experts", "gate_up_blocks", "gate_up_scales", "hidden", "intermediate")
+    __slots__ = ("down_bias", "down_blocks", "down_scales", "experts", "gate_up_bias", "gate_up_blocks", "gate_up_scales",
+                 "hidden", "intermediate")
 
     def __init__(self, gate_up_blocks: torch.Tensor, gate_up_scales: torch.Tensor, down_blocks: torch.Tensor,
-                 down_scales: torch.Tensor) -> None:
+                 down_scales: torch.Tensor, gate_up_bias: torch.Tensor | None = None,
+                 down_bias: torch.Tensor | None = None) -> None:
         for b, sc, what in ((gate_up_blocks, gate_up_scales, "gate_up"), (down_blocks, down_scales, "down")):
             if b.dtype != torch.uint8 or sc.dtype != torch.uint8 or b.dim() != 4 or b.shape[-1] != BLOCK_BYTES \
                     or tuple(b.shape[:-1]) != tuple(sc.shape):
@@ -225,6 +227,12 @@ class MxExperts:
         self.gate_up_blocks, self.gate_up_scales = gate_up_blocks.contiguous(), gate_up_scales.contiguous()
         self.down_blocks, self.down_scales = down_blocks.contiguous(), down_scales.contiguous()
         self.experts, self.hidden, self.intermediate = E, H, I
+        # gpt-oss's expert biases, bf16 as the checkpoint holds them: [E, 2I] (interleaved like the rows) and [E, H]
+        for b, shape, what in ((gate_up_bias, (E, 2 * I), "gate_up_bias"), (down_bias, (E, H), "down_bias")):
+            if b is not None and (tuple(b.shape) != shape or b.dtype != torch.bfloat16):
+                raise ValueError(f"[load] {what} is bf16 {shape}, got {tuple(b.shape)} {b.dtype}")
+        self.gate_up_bias = None if gate_up_bias is None else gate_up_bias.contiguous()
+        self.down_bias = None if down_bias is None else down_bias.contiguous()
 
     def gate_up(self, e: int) -> MxWeight:
         return MxWeight(self.gate_up_blocks[e].reshape(-1), self.gate_up_scales[e].reshape(-1), 2 * self.intermediate,
@@ -251,7 +259,8 @@ class MxExperts:
 
 def load_mx_experts(path: str | Store, layer: int, device: Any = "cuda",
                     prefix: str = "model.layers.{i}.mlp.experts.") -> MxExperts:
-    """layer `layer`'s MXFP4 expert stacks of a store, uploaded as stored (`<prefix>{gate_up,down}_proj_{blocks,scales}`)"""
+    """layer `layer`'s MXFP4 expert stacks of a store, uploaded as stored (`<prefix>{gate_up,down}_proj_{blocks,scales}`,
+    and `<prefix>{gate_up,down}_proj_bias` where the store holds them)"""
     store = path if isinstance(path, Store) else Store(path)
     base = prefix.format(i=int(layer))
     names = [base + n for n in ("gate_up_proj_blocks", "gate_up_proj_scales", "down_proj_blocks", "down_proj_scales")]
@@ -259,4 +268,6 @@ def load_mx_experts(path: str | Store, layer: int, device: Any = "cuda",
     if missing:
         raise KeyError(f"[load] not an MXFP4 expert layer: {missing[0]} is not in {store.path}")
     dev = torch.device(device)
-    return MxExperts(*(store.get(n).to(dev) for n in names))
+    biases = [store.get(base + n).to(torch.bfloat16).to(dev) if store.has(base + n) else None
+              for n in ("gate_up_proj_bias", "down_proj_bias")]
+    return MxExperts(*(store.get(n).to(dev) for n in names), *biases)

@@ -6,6 +6,12 @@ expert is resident in VRAM here, so there is no store, no wave and no host round
     experts = Experts(card, gate_up, down)           # bf16 stacks [E, 2I, H], [E, H, I]
     logits, weights, picks = router(x)               # x bf16 [T, H]
     y = experts(x, picks, weights)                   # bf16 [T, H], summed in ascending expert order
+
+MXFP4 expert stacks (gpt-oss's checkpoints, or any stack quantised the same way) stay as stored and go through the same
+two kernels with the widening in their registers:
+
+    experts = MxExpertsLayer(card, load_mx_experts(path, layer))          # gpt-oss: interleaved rows, biases, clamped gate
+    experts = MxExpertsLayer(card, MxExperts(...), oss=False)             # concatenated halves, SiLU
 """
 
 from __future__ import annotations
@@ -64,3 +70,30 @@ class Experts:
             self._gu = torch.empty(T, k, 2 * self.intermediate_dim, dtype=torch.bfloat16, device=x.device)
         return self.card.moe_experts(self.gate_up, self.down, x.contiguous(), top_k_index.to(torch.int32).contiguous(),
                                      top_k_weights.to(torch.bfloat16).contiguous(), out, self._gu[:T])
+
+
+class MxExpertsLayer:
+    """The layer's experts as MXFP4 stacks on the GPU, as the checkpoint stores them (`btb_amd.load.MxExperts`): the
+    reference's `_Experts` over `Native.gemv_mx4_group` (btb/engine/host.py:459-461, 508-569) with every expert
+    resident. `oss` (the default): gpt-oss's experts - gate and up rows interleaved, the experts' biases, the clamped
+    gate `(up + 1) * gate * sigmoid(alpha * gate)` (host.py:443-451); `oss=False`: concatenated halves and SiLU. Same
+    call and result as `Experts`."""
+
+    def __init__(self, card: Any, stacks: Any, oss: bool = True, alpha: float = 1.702, limit: float = 7.0) -> None:
+        if not oss and (stacks.gate_up_bias is not None or stacks.down_bias is not None):
+            raise ValueError("[moe] expert biases belong to the gpt-oss form")
+        self.card, self.stacks, self.oss, self.alpha, self.limit = card, stacks, bool(oss), float(alpha), float(limit)
+        self.num_experts, self.hidden_dim, self.intermediate_dim = stacks.experts, stacks.hidden, stacks.intermediate
+        self._h: torch.Tensor | None = None
+
+    def __call__(self, hidden_states: torch.Tensor, top_k_index: torch.Tensor, top_k_weights: torch.Tensor,
+                 out: torch.Tensor | None = None) -> torch.Tensor:
+        x = hidden_states.reshape(-1, self.hidden_dim)
+        if x.dtype != torch.bfloat16:
+            raise ValueError("[moe] the card's experts take bf16 rows")
+        T, k = (int(s) for s in top_k_index.shape)
+        if self._h is None or self._h.shape[0] < T or self._h.shape[1] != k:
+            self._h = torch.empty(T, k, self.intermediate_dim, dtype=torch.bfloat16, device=x.device)
+        return self.card.moe_experts_mx4(self.stacks, x.contiguous(), top_k_index.to(torch.int32).contiguous(),
+                                         top_k_weights.to(torch.bfloat16).contiguous(), out, self._h[:T], oss=self.oss,
+                                         alpha=self.alpha, limit=self.limit)

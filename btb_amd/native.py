@@ -64,6 +64,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_moe_group_picks": (_i32, [_vp, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_moe_router_bf16": (_i32, [_vp, _vp, _sz, _sz, _sz, _sz, _vp, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_moe_experts_bf16": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, _sz, _vp]),
+    "btb_hip_moe_experts_mxfp4": (_i32, [_vp] * 11 + [_sz] * 5 + [_i32, ctypes.c_float, ctypes.c_float, _vp]),
     "btb_hip_embed": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_add_rmsnorm": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _sz, _sz, _i32, _vp]),
     "btb_hip_norm_rope_kv": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
@@ -622,6 +623,41 @@ class HipCard(CardLaunch):
             y = torch.empty(T, H, dtype=torch.bfloat16, device=x.device)
         self._call("btb_hip_moe_experts_bf16", _p(gate_up), _p(down), _p(x), _p(idx), _p(w),
                    _p(gu), _p(y), T, k, E, H, I2 // 2, _stream())
+        return y
+
+    def moe_experts_mx4(self, ex: Any, x: torch.Tensor, idx: torch.Tensor, w: torch.Tensor,
+                        y: torch.Tensor | None = None, h: torch.Tensor | None = None, oss: bool = True,
+                        alpha: float = 1.702, limit: float = 7.0) -> torch.Tensor:
+        """y [T, H]: the routed experts of x [T, H] over a layer's MXFP4 stacks as stored (`MxExperts`: gate_up blocks
+        [E, 2I, H / 32, 16] + scales, down blocks [E, H, I / 32, 16] + scales, optional bf16 biases), picks idx int32
+        [T, k], weights w bf16 [T, k], summed in ascending expert order. `oss`: gpt-oss's experts (interleaved gate /
+        up rows, biases, the clamped gate with `alpha` and `limit`); else concatenated halves and SiLU."""
+        for t, what in ((ex.gate_up_blocks, "gate_up_blocks"), (ex.gate_up_scales, "gate_up_scales"),
+                        (ex.down_blocks, "down_blocks"), (ex.down_scales, "down_scales")):
+            self._need(t, torch.uint8, what)
+        for t, what in ((x, "x"), (w, "w")):
+            self._need(t, torch.bfloat16, what)
+        self._need(idx, torch.int32, "idx")
+        E, H, I = int(ex.experts), int(ex.hidden), int(ex.intermediate)
+        gb, db = getattr(ex, "gate_up_bias", None), getattr(ex, "down_bias", None)
+        for t, what, n in ((gb, "gate_up_bias", E * 2 * I), (db, "down_bias", E * H)):
+            if t is not None:
+                self._need(t, torch.bfloat16, what)
+                if t.numel() != n or not oss:
+                    raise ValueError(f"[hip] moe_experts_mx4: {what} holds {t.numel()} values; the gpt-oss form takes {n}")
+        if x.shape[-1] != H or idx.shape != w.shape or idx.dim() != 2:
+            raise ValueError(f"[hip] moe_experts_mx4: x {tuple(x.shape)}, idx {tuple(idx.shape)}, w {tuple(w.shape)} do "
+                             f"not fit a layer of hidden {H}")
+        T, k = (int(s) for s in idx.shape)
+        if h is None:
+            h = torch.empty(T, k, I, dtype=torch.bfloat16, device=x.device)
+        elif h.dtype != torch.bfloat16 or h.numel() < T * k * I or not h.is_contiguous():
+            raise ValueError(f"[hip] moe_experts_mx4: h is contiguous bf16 scratch of at least {T * k * I} values")
+        y = self._out(y, T, H, x.device, "moe_experts_mx4")
+        p = lambda t: None if t is None else _p(t)
+        self._call("btb_hip_moe_experts_mxfp4", _p(ex.gate_up_blocks), _p(ex.gate_up_scales), _p(ex.down_blocks),
+                   _p(ex.down_scales), p(gb), p(db), _p(x), _p(idx), _p(w), _p(h), _p(y), T, k, E, H, I, int(bool(oss)),
+                   float(alpha), float(limit), _stream())
         return y
 
 

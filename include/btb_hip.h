@@ -231,6 +231,21 @@ int32_t btb_hip_moe_router_bf16(const void* router, const void* x, size_t T, siz
 int32_t btb_hip_moe_experts_bf16(const void* gate_up, const void* down, const void* x, const int32_t* idx, const void* w,
                                  void* gu, void* y, size_t T, size_t k, size_t E, size_t H, size_t I, void* stream);
 
+/* btb_hip_moe_experts_bf16 over MXFP4 expert stacks as the checkpoint stores them (btb/mxfp4.py:4-29): gu_blocks u8
+ * [E, 2I, H / 32, 16] and gu_scales u8 [E, 2I, H / 32], dn_blocks u8 [E, H, I / 32, 16] and dn_scales u8 [E, H, I / 32];
+ * every weight fp4 * 2^(scale - 127), made in registers inside the matvec, no widened copy. The grouped device form of
+ * _Experts over `btb_gemv_mxfp4_group` (native/src/lib.rs:193-209; btb/engine/host.py:508-569, 906-967).
+ * oss == 0: the gate and up rows concatenated, h = bf16(bf16(silu(g)) * u), no biases (gu_bias, dn_bias NULL).
+ * oss != 0: gpt-oss's experts (host.py:414-451): gate row 2 r and up row 2 r + 1 interleaved; gu_bias bf16 [E, 2I]
+ * (or NULL) added to the rounded products; the gate clamped to <= limit and the up half to +-limit;
+ * h = (up + 1) * (gate * sigmoid(alpha * gate)), every operation rounded to bf16 as torch rounds it; dn_bias bf16
+ * [E, H] (or NULL) added to the expert's rounded down product before its weight. h [T, k, I] bf16 is scratch the
+ * caller owns. H and I multiples of 32; the other limits are btb_hip_moe_experts_bf16's. */
+int32_t btb_hip_moe_experts_mxfp4(const void* gu_blocks, const void* gu_scales, const void* dn_blocks,
+                                  const void* dn_scales, const void* gu_bias, const void* dn_bias, const void* x,
+                                  const int32_t* idx, const void* w, void* h, void* y, size_t T, size_t k, size_t E,
+                                  size_t H, size_t I, int32_t oss, float alpha, float limit, void* stream);
+
 /* ---- the decode step's kernels between the matvecs ---------------------------------------------------------- */
 
 /* h[t] = table[ids[t]]: the step's input row (the reference gathers it with torch before its graph). table

@@ -3,8 +3,8 @@
     python tests/golden/make_gpt_oss_experts.py [/root/reference]
 
 The reference keeps a four-layer gpt-oss store under tests/fixtures/tiny_gpt_oss (random MXFP4 bytes per expert:
-`mlp.experts.{gate_up,down}_proj_{blocks,scales}`, written by its tests/make_fixtures.py). Only those uint8 tensors, the
-router weights beside them and the config's shape fields are copied - through safetensors, nothing of the reference is
+`mlp.experts.{gate_up,down}_proj_{blocks,scales}` and the experts' bf16 biases, written by its tests/make_fixtures.py).
+Only those tensors, the router's weight and bias beside them and the config's shape fields are copied - through safetensors, nothing of the reference is
 run - into one shard with an index, which is all the MXFP4 store reader (btb_amd/load.py: `load_mx_experts`) needs.
 """
 
@@ -29,7 +29,8 @@ def main(ref: str) -> None:
     for shard in sorted(glob.glob(os.path.join(src, "*.safetensors"))):
         with safe_open(shard, framework="pt") as f:
             for k in f.keys():
-                if ".mlp.experts." in k and k.endswith(("_blocks", "_scales")) or k.endswith("mlp.router.weight"):
+                if ".mlp.experts." in k and k.endswith(("_blocks", "_scales", "_bias")) \
+                        or k.endswith(("mlp.router.weight", "mlp.router.bias")):
                     keep[k] = f.get_tensor(k).contiguous()
     name = "experts-00001-of-00001.safetensors"
     save_file(keep, os.path.join(out, name))
@@ -38,7 +39,7 @@ def main(ref: str) -> None:
     with open(os.path.join(src, "config.json")) as f:
         cfg = json.load(f)
     fields = ("model_type", "hidden_size", "intermediate_size", "num_hidden_layers", "num_local_experts",
-              "num_experts_per_tok", "experts_per_token")
+              "num_experts_per_tok", "experts_per_token", "swiglu_limit")
     with open(os.path.join(out, "config.json"), "w") as f:
         json.dump({k: cfg[k] for k in fields if k in cfg}, f, indent=1)
     print(f"{len(keep)} tensors -> {out}")

@@ -187,3 +187,145 @@ def test_rows_that_share_an_expert_go_through_it_together(card, layer_weights, T
     want = omoe.experts(bits16(gu), bits16(dn), x.float().cpu().numpy(), picks.cpu().numpy().astype(np.int64),
                         w.float().cpu().numpy(), "bf16")
     assert np.abs(y.float().cpu().numpy() - want).max() <= 1e-2 * np.abs(want).max()
+
+
+# -- MXFP4 expert stacks: the stored bytes through the same two kernels ------------------------------------------------
+
+
+def mx_stacks(seed: int, E_: int, I_: int, H_: int):
+    """N(0, 0.02) expert stacks quantised to MXFP4 (the repository's own encoder; what is checked is the layer over the
+    stored bytes, whatever made them)"""
+    from btb_amd import mxfp4
+    from btb_amd.load import MxExperts
+
+    g = gen(seed)
+    gu = torch.randn(E_ * 2 * I_, H_, generator=g) * 0.02
+    dn = torch.randn(E_ * H_, I_, generator=g) * 0.02
+    gb, gs = mxfp4.quantize(gu)
+    db, ds = mxfp4.quantize(dn)
+    return MxExperts(gb.reshape(E_, 2 * I_, H_ // 32, 16), gs.reshape(E_, 2 * I_, H_ // 32),
+                     db.reshape(E_, H_, I_ // 32, 16), ds.reshape(E_, H_, I_ // 32))
+
+
+def to_gpu(ex):
+    from btb_amd.load import MxExperts
+
+    mv = lambda t: None if t is None else t.cuda()
+    return MxExperts(ex.gate_up_blocks.cuda(), ex.gate_up_scales.cuda(), ex.down_blocks.cuda(), ex.down_scales.cuda(),
+                     mv(ex.gate_up_bias), mv(ex.down_bias))
+
+
+def oracle_mx(ex, x, picks, w, **kw):
+    f = lambda t: None if t is None else t.float().numpy()
+    return omoe.experts_mx4(ex.gate_up_blocks.numpy(), ex.gate_up_scales.numpy(), ex.down_blocks.numpy(),
+                            ex.down_scales.numpy(), x.float().numpy(), picks, w, dt="bf16", gu_bias=f(ex.gate_up_bias),
+                            dn_bias=f(ex.down_bias), **kw)
+
+
+@pytest.mark.parametrize("T", [1, 4, 8, 16])
+def test_mxfp4_moe_layer_matches_cpu_path(card, layer_weights, T):
+    """C4's layer with its experts stored as MXFP4 (concatenated halves, SiLU): the router's picks are the CPU's bit for
+    bit, the layer within 1e-2 of the CPU path over the same stored bytes (btb_gemv_mxfp4_rows per expert, the rows'
+    dtype chain of _Experts); 8 and 16 rows take the grouped gate/up kernel"""
+    from btb_amd.moe import MxExpertsLayer
+
+    wr = layer_weights[0]
+    ex = mx_stacks(540, E, I, H)
+    x = acts_bf16(T, H, seed=541 + T)
+    router = Router(card, wr.cuda(), K)
+    layer = MxExpertsLayer(card, to_gpu(ex), oss=False)
+    _, weights, picks = router(x.cuda())
+    y = layer(x.cuda(), picks, weights)
+    torch.cuda.synchronize()
+    _, ow, opicks = omoe.router(bits16(wr), x.float().numpy(), K, "bf16")
+    assert np.array_equal(picks.cpu().numpy().astype(np.int64), opicks)
+    want = oracle_mx(ex, x, opicks, weights.float().cpu().numpy(), oss=False)
+    got = y.float().cpu().numpy()
+    assert np.abs(want).max() > 0
+    assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max()
+    # the grouped gate/up kernel and the pair kernel: the same bits
+    card.set_tuning("moe_grouped", 0)
+    y0 = layer(x.cuda(), picks, weights).clone()
+    card.set_tuning("moe_grouped", 1)
+    y1 = layer(x.cuda(), picks, weights).clone()
+    card.set_tuning("moe_grouped", -1)
+    assert torch.equal(y0, y1) and torch.equal(y0, y)
+
+
+@pytest.mark.parametrize("layer,T", [(0, 1), (1, 3), (2, 8), (3, 16)])
+def test_gpt_oss_experts_on_the_reference_fixture(card, layer, T):
+    """the reference's tiny gpt-oss expert tensors as stored (interleaved gate / up rows, biases): the gpt-oss middle on
+    the GPU against the CPU path restated in oracle/moe.py (itself held to transformers' GptOssExperts in
+    tests/test_oracle_moe.py), picks drawn, weights a softmax over them; within 1e-2 of the largest output"""
+    import os
+
+    from btb_amd.load import load_mx_experts
+    from btb_amd.moe import MxExpertsLayer
+
+    from .helpers import GOLDEN
+
+    ex = load_mx_experts(os.path.join(GOLDEN, "tiny_gpt_oss"), layer, device="cpu")
+    assert ex.gate_up_bias is not None and ex.down_bias is not None and (ex.experts, ex.hidden, ex.intermediate) == (8, 64, 64)
+    g = gen(560 + layer)
+    k = 4
+    x = torch.randn(T, ex.hidden, generator=g).to(torch.bfloat16)
+    picks = torch.stack([torch.randperm(ex.experts, generator=g)[:k] for _ in range(T)])
+    w = torch.softmax(torch.randn(T, k, generator=g), dim=-1).to(torch.bfloat16)
+    y = MxExpertsLayer(card, to_gpu(ex))(x.cuda(), picks.to(torch.int32).cuda(), w.cuda())
+    want = oracle_mx(ex, x, picks.numpy(), w.float().numpy(), oss=True)
+    got = y.float().cpu().numpy()
+    assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max()
+    # the biases and the interleaving matter at this size: without them the result is far off
+    bare = oracle_mx(ex, x, picks.numpy(), w.float().numpy(), oss=False)
+    assert np.abs(bare - want).max() > 5e-2 * np.abs(want).max()
+
+
+def test_gpt_oss_experts_at_its_real_row_lengths(card):
+    """gpt-oss's 2880-wide rows (90 blocks: no power of two, a span's last units guarded), the clamps exercised by
+    large activations"""
+    from btb_amd.load import MxExperts
+    from btb_amd.moe import MxExpertsLayer
+
+    E_, H_, I_, k, T = 6, 2880, 2880, 4, 3
+    ex = mx_stacks(570, E_, I_, H_)
+    g = gen(571)
+    ex = MxExperts(ex.gate_up_blocks, ex.gate_up_scales, ex.down_blocks, ex.down_scales,
+                   (torch.randn(E_, 2 * I_, generator=g) * 0.5).to(torch.bfloat16),
+                   (torch.randn(E_, H_, generator=g) * 0.1).to(torch.bfloat16))
+    x = (torch.randn(T, H_, generator=g) * 6.0).to(torch.bfloat16)      # gate / up values past the limit of 7
+    picks = torch.stack([torch.randperm(E_, generator=g)[:k] for _ in range(T)])
+    w = torch.softmax(torch.randn(T, k, generator=g), dim=-1).to(torch.bfloat16)
+    y = MxExpertsLayer(card, to_gpu(ex))(x.cuda(), picks.to(torch.int32).cuda(), w.cuda())
+    want = oracle_mx(ex, x, picks.numpy(), w.float().numpy(), oss=True)
+    got = y.float().cpu().numpy()
+    assert np.abs(got - want).max() <= 1e-2 * np.abs(want).max()
+
+
+def test_mxfp4_experts_refusals(card):
+    from btb_amd.load import MxExperts
+    from btb_amd.moe import MxExpertsLayer
+
+    ex = to_gpu(mx_stacks(580, 4, 64, 64))
+    x = torch.zeros(2, 64, dtype=torch.bfloat16, device="cuda")
+    idx = torch.zeros(2, 2, dtype=torch.int32, device="cuda")
+    w = torch.ones(2, 2, dtype=torch.bfloat16, device="cuda")
+    with pytest.raises(ValueError):
+        card.moe_experts_mx4(ex, x[:, :32], idx, w)
+    with pytest.raises(ValueError):
+        card.moe_experts_mx4(ex, x, idx, w[:, :1])
+    biased = MxExperts(ex.gate_up_blocks, ex.gate_up_scales, ex.down_blocks, ex.down_scales,
+                       torch.zeros(4, 128, dtype=torch.bfloat16, device="cuda"), None)
+    with pytest.raises(ValueError):
+        MxExpertsLayer(card, biased, oss=False)
+    L = card.lib
+    p = lambda t: t.data_ptr()
+    h = torch.zeros(2, 2, 64, dtype=torch.bfloat16, device="cuda")
+    y = torch.zeros(2, 64, dtype=torch.bfloat16, device="cuda")
+    a = (p(ex.gate_up_blocks), p(ex.gate_up_scales), p(ex.down_blocks), p(ex.down_scales))
+    assert L.btb_hip_moe_experts_mxfp4(None, a[1], a[2], a[3], None, None, p(x), p(idx), p(w), p(h), p(y), 2, 2, 4, 64, 64,
+                                       0, 0.0, 0.0, None) == -1
+    assert L.btb_hip_moe_experts_mxfp4(*a, None, None, p(x), p(idx), p(w), p(h), p(y), 2, 2, 4, 48, 64, 0, 0.0, 0.0,
+                                       None) == -6          # H % 32
+    assert L.btb_hip_moe_experts_mxfp4(*a, p(y), None, p(x), p(idx), p(w), p(h), p(y), 2, 2, 4, 64, 64, 0, 0.0, 0.0,
+                                       None) == -6          # a bias without the gpt-oss form
+    assert bool((y == 0).all())

@@ -180,3 +180,87 @@ def test_group_picks_lists_an_experts_pairs_pick_major_then_row():
         assert n == len(p)
         assert pos[a : a + n].tolist() == p.tolist() and row[a : a + n].tolist() == r.tolist()
     assert int(counts.sum()) == T * k and offs[0] == 0
+
+
+# -- MXFP4 expert stacks, gpt-oss's middle ---------------------------------------------------------------------------
+
+
+def oss_fixture(layer: int = 0):
+    """the reference's tiny gpt-oss expert tensors (tests/golden/tiny_gpt_oss, copied as data): blocks, scales, biases"""
+    import os
+
+    from safetensors import safe_open
+
+    from .helpers import GOLDEN
+
+    base = f"model.layers.{layer}.mlp.experts."
+    with safe_open(os.path.join(GOLDEN, "tiny_gpt_oss", "experts-00001-of-00001.safetensors"), framework="pt") as f:
+        return {n: f.get_tensor(base + n) for n in ("gate_up_proj_blocks", "gate_up_proj_scales", "gate_up_proj_bias",
+                                                    "down_proj_blocks", "down_proj_scales", "down_proj_bias")}
+
+
+def oss_inputs(T, E, k, H, seed):
+    g = gen(seed)
+    x = torch.randn(T, H, generator=g).to(torch.bfloat16)
+    picks = torch.stack([torch.randperm(E, generator=g)[:k] for _ in range(T)]).numpy()
+    w = torch.softmax(torch.randn(T, k, generator=g), dim=-1).to(torch.bfloat16)
+    return x, picks, w
+
+
+def run_oracle_oss(t, x, picks, w, dt, **kw):
+    kw.setdefault("gu_bias", t["gate_up_proj_bias"].float().numpy())
+    kw.setdefault("dn_bias", t["down_proj_bias"].float().numpy())
+    return omoe.experts_mx4(t["gate_up_proj_blocks"].numpy(), t["gate_up_proj_scales"].numpy(),
+                            t["down_proj_blocks"].numpy(), t["down_proj_scales"].numpy(), x.float().numpy(), picks,
+                            w.float().numpy(), dt=dt, **kw)
+
+
+@pytest.mark.parametrize("layer,T", [(0, 1), (1, 5), (3, 8)])
+def test_gpt_oss_experts_agree_with_transformers_over_the_dequantised_stacks(layer, T):
+    """the f32 chain against transformers' GptOssExperts (a library here, not the reference) holding the same stacks
+    dequantised: interleaved halves, biases, clamps, (up + 1) * gate * sigmoid(alpha gate), the down bias before the
+    weight, the experts summed per row"""
+    tm = pytest.importorskip("transformers.models.gpt_oss.modeling_gpt_oss")
+    t = oss_fixture(layer)
+    E, I2, gh = t["gate_up_proj_scales"].shape
+    H, I, k = gh * 32, I2 // 2, 4
+    x, picks, w = oss_inputs(T, E, k, H, seed=950 + layer)
+    got = run_oracle_oss(t, x, picks, w, "f32")
+
+    from transformers import GptOssConfig
+
+    m = tm.GptOssExperts(GptOssConfig(intermediate_size=I, num_local_experts=E, hidden_size=H))
+    gu = torch.from_numpy(codecs.mxfp4_dequantize(t["gate_up_proj_blocks"].numpy(), t["gate_up_proj_scales"].numpy()))
+    dn = torch.from_numpy(codecs.mxfp4_dequantize(t["down_proj_blocks"].numpy(), t["down_proj_scales"].numpy()))
+    with torch.no_grad():
+        m.gate_up_proj.copy_(gu.reshape(E, 2 * I, H).transpose(1, 2))
+        m.down_proj.copy_(dn.reshape(E, H, I).transpose(1, 2))
+        m.gate_up_proj_bias.copy_(t["gate_up_proj_bias"].float())
+        m.down_proj_bias.copy_(t["down_proj_bias"].float())
+        want = m(x.float(), router_indices=torch.from_numpy(picks), routing_weights=w.float()).numpy()
+    assert np.abs(want).max() > 1e-3
+    assert np.abs(got - want).max() <= 1e-5 * np.abs(want).max()
+    # planted mistakes, each far past the bar: the halves concatenated, no clamp (limit huge moves nothing here, so a
+    # tiny limit stands in for "the clamp is applied"), up without its + 1 (alpha = 0 and the bias dropped differ too)
+    for wrong in (dict(oss=False, gu_bias=None, dn_bias=None), dict(limit=0.01), dict(alpha=0.0), dict(gu_bias=None),
+                  dict(dn_bias=None)):
+        bad = run_oracle_oss(t, x, picks, w, "f32", **wrong)
+        assert np.abs(bad - want).max() > 1e-3 * np.abs(want).max(), wrong
+
+
+def test_gpt_oss_gate_rounds_where_torch_rounds_it():
+    """the bf16 chain's rounding points: the same expression evaluated by torch on bf16 tensors, bit for bit, on
+    values that cross both clamps"""
+    g = gen(960)
+    gu = (torch.randn(64, 256, generator=g) * 4.0).to(torch.bfloat16)
+    alpha, limit = 1.702, 7.0
+    gate, up = gu[..., ::2], gu[..., 1::2]
+    gate = gate.clamp(min=None, max=limit)
+    up = up.clamp(min=-limit, max=limit)
+    want = (up + 1) * (gate * torch.sigmoid(gate * alpha))
+    assert want.dtype == torch.bfloat16 and bool((gu.float().abs() > limit).any())
+    got = omoe.gpt_oss_gate(gu.float().numpy(), alpha, limit, "bf16")
+    # torch's bf16 sigmoid and this one may differ in the last f32 bit before the rounding: a handful of bf16 flips
+    flips = np.count_nonzero(bits16(want) != bits16(torch.from_numpy(got).to(torch.bfloat16)))
+    assert flips <= want.numel() // 500, flips
+    assert np.abs(got - want.float().numpy()).max() <= 2.0**-7 * np.abs(want.float().numpy()).max()
