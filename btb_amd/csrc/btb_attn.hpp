@@ -1,6 +1,6 @@
 // Decode attention's shared pieces (head_dim 128): the q / k RMSNorm + rope of one head by one wave, and a key
 // stream's batch loads and online-softmax update - used by the stand-alone attention kernel that reads the fused qkv
-// row (glue.hip) and by the persistent step (step.hip).
+// row (glue.hip).
 #pragma once
 
 #include "btb_common.hpp"

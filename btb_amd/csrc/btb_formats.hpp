@@ -27,6 +27,7 @@ struct FmtBf16 {
         const uint4* row;
     };
     __device__ static __forceinline__ void prepare(Params&) {}
+    __device__ static __forceinline__ void prepare_finish(Params&) {}
     __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
         return RowCtx{p.w + r * (size_t)units};
     }
@@ -62,6 +63,8 @@ struct FmtP12 {
         const uint8_t* esc_val;
         const int32_t* row_ptr;  // [rows + 1] first escape at or past each row's start
         uint4 tbl;               // the table in registers: filled by prepare() on the device, not by the host
+        const uint16_t* pairs;   // [256] the pair table made at upload (FmtP12G), or null
+        uint32_t pair_reg;       // this thread's entry of it on its way to LDS (prepare -> prepare_finish)
     };
     struct Raw {
         uint4 lo;
@@ -84,6 +87,7 @@ struct FmtP12 {
     }
     // once per kernel (or phase), before any row_ctx: the table's 16 bytes are read here and only here
     __device__ static __forceinline__ void prepare(Params& p) { p.tbl = load_table(p.table); }
+    __device__ static __forceinline__ void prepare_finish(Params&) {}
     __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
         RowCtx c;
         c.lo = reinterpret_cast<const uint4*>(p.lo) + r * (size_t)units;
@@ -145,25 +149,31 @@ struct FmtP12 {
 };
 
 // The same form with the table lookups done in LDS: a 256-entry table of PAIRS - entry b holds the high bytes of the
-// two weights whose codes are byte b's nibbles - is built once a workgroup, and a byte of codes becomes its two high
-// bytes with one 16-bit LDS read where the in-register lookup takes two byte-permutes, a select and the nibble split
-// per four codes. Eight weights: 4 byte extractions, 4 LDS reads, 4 byte-permutes that zip high and low bytes (23
-// vector instructions before). prepare() must be followed by a workgroup barrier before the first widen (the
-// streaming kernel's x staging ends with one).
-struct FmtP12L : FmtP12 {
+// two weights whose codes are byte b's nibbles - and a byte of codes becomes its two high bytes with one 16-bit LDS
+// read where the in-register lookup takes two byte-permutes, a select and the nibble split per four codes. Eight
+// weights: 4 byte extractions, 4 LDS reads, 4 byte-permutes that zip high and low bytes (23 vector instructions
+// before). The table is made once, at upload (btb_hip_p12_pairs: 512 bytes beside row_ptr, slot 15 of the 16-byte
+// table taken as 0), and a workgroup of 256 threads brings it in with one 2-byte load a thread: prepare() asks for
+// it before anything else, prepare_finish() - called once the kernel's first weights have been requested - puts it
+// into LDS, and the workgroup barrier that ends the x staging makes it visible. Nothing of it sits on the way of the
+// weights: building the table in the kernel did (the plain forms lost 0.3 us a launch to it).
+struct FmtP12G : FmtP12 {
     __device__ static __forceinline__ uint16_t* pair_table() {
         __shared__ uint16_t pairs[256];
         return pairs;
     }
-    __device__ static __forceinline__ void prepare(Params& p) {
-        FmtP12::prepare(p);
-        uint16_t* t = pair_table();
-        const uint32_t d[4] = {p.tbl.x, p.tbl.y, p.tbl.z, p.tbl.w};
-        for (int b = threadIdx.x; b < 256; b += blockDim.x) {
-            const uint32_t lo = (d[(b & 15) >> 2] >> (8 * (b & 3))) & 0xFFu;
-            const uint32_t hi = (d[(b >> 4) >> 2] >> (8 * ((b >> 4) & 3))) & 0xFFu;
-            t[b] = (uint16_t)(lo | (hi << 8));
-        }
+    __device__ static __forceinline__ void prepare(Params& p) { p.pair_reg = p.pairs[threadIdx.x & 255]; }
+    __device__ static __forceinline__ void prepare_finish(Params& p) {
+        if (threadIdx.x < 256) pair_table()[threadIdx.x] = (uint16_t)p.pair_reg;
+    }
+    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
+        RowCtx c;
+        c.lo = reinterpret_cast<const uint4*>(p.lo) + r * (size_t)units;
+        c.hi4 = reinterpret_cast<const uint2*>(p.hi4) + r * (size_t)units;
+        c.table = make_uint4(0u, 0u, 0u, 0u);  // not read: the lookups go through LDS, an escape streams as slot 15 = 0
+        c.e0 = p.row_ptr[r];
+        c.e1 = p.row_ptr[r + 1];
+        return c;
     }
     // eight weights: codes c (weight k in nibble k), low bytes l0 (weights 0..3), l1 (4..7)
     __device__ static __forceinline__ void widen8(uint32_t c, uint32_t l0, uint32_t l1, uint32_t* w) {
@@ -210,6 +220,7 @@ struct FmtF8 {
         uint32_t magic;
     };
     __device__ static __forceinline__ void prepare(Params&) {}
+    __device__ static __forceinline__ void prepare_finish(Params&) {}
     __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
         return RowCtx{reinterpret_cast<const uint4*>(p.w) + r * (size_t)units, p.scales + (r / p.bm) * (size_t)p.sc,
                       p.upb, p.magic};
@@ -260,6 +271,7 @@ struct FmtMx4 {
         const uint8_t* srow;
     };
     __device__ static __forceinline__ void prepare(Params&) {}
+    __device__ static __forceinline__ void prepare_finish(Params&) {}
     __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
         return RowCtx{reinterpret_cast<const uint4*>(p.blocks) + r * (size_t)units, p.scales + r * (size_t)units};
     }

@@ -125,6 +125,7 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs x
             ctx[j] = F::row_ctx(p, (size_t)tile_row<LPR, RPW, EPI>(min(wave, ntiles - 1), j, lane, R, out_row), units);
         }
         load_span_always<F, LPR, RPW, U>(first, ctx, 0, lane % LPR, units);
+        F::prepare_finish(p);
     });
     const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
     if (wave >= ntiles) return;
@@ -162,7 +163,7 @@ static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void
     // Six workgroups' worth of waves a CU, measured best for every form (more, smaller workgroups than are resident
     // even out the grid's tail) but the pack12 form with the pair table, which does better cut for five - the head
     // matvec [151936 x 2560] takes 97 us instead of 113, the packed step 2.194 ms instead of 2.213.
-    if (per_cu <= 0) per_cu = std::is_same<F, FmtP12L>::value ? 5 : 6;
+    if (per_cu <= 0) per_cu = std::is_same<F, FmtP12G>::value ? 5 : 6;
     const int cap_waves = dev.cus * per_cu * 4;
     const int tiles_per_wave = (ntiles + cap_waves - 1) / cap_waves;
     const int waves = (ntiles + tiles_per_wave - 1) / tiles_per_wave;
@@ -349,9 +350,11 @@ static bool norm_on_mfma(const XArgs& xa, size_t R, size_t C, size_t M, bool glu
            mfma_lds_norm_fits((int)R, (int)C, (int)M) && al8(xa.x) && al8(xa.y) && al8(xa.norm_w) && al8(xa.h_out);
 }
 
-static int32_t p12_params(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
-                          size_t n_esc, const void* row_ptr, size_t R, size_t C, FmtP12::Params* p) {
+static int32_t p12_params(const void* lo, const void* hi4, const void* table, const void* pairs, const void* esc_idx,
+                          const void* esc_val, size_t n_esc, const void* row_ptr, size_t R, size_t C,
+                          FmtP12::Params* p) {
     if (lo == nullptr || hi4 == nullptr || table == nullptr || row_ptr == nullptr) return ERR_NULL;
+    if (reinterpret_cast<uintptr_t>(pairs) & 1u) return ERR_DOMAIN;
     if (n_esc > 0 && (esc_idx == nullptr || esc_val == nullptr)) return ERR_NULL;
     if (R * C > 0x7FFFFFFFull) return ERR_DOMAIN;  // the escape indices are int32
     if (!aligned16(lo) || (reinterpret_cast<uintptr_t>(hi4) & 7u) || (reinterpret_cast<uintptr_t>(row_ptr) & 3u) ||
@@ -360,7 +363,7 @@ static int32_t p12_params(const void* lo, const void* hi4, const void* table, co
     *p = FmtP12::Params{static_cast<const uint8_t*>(lo),      static_cast<const uint8_t*>(hi4),
                         static_cast<const uint8_t*>(table),   static_cast<const int32_t*>(esc_idx),
                         static_cast<const uint8_t*>(esc_val), static_cast<const int32_t*>(row_ptr),
-                        make_uint4(0, 0, 0, 0)};
+                        make_uint4(0, 0, 0, 0), static_cast<const uint16_t*>(pairs), 0u};
     return OK;
 }
 
@@ -457,16 +460,16 @@ int32_t btb_hip_gemv_bf16_embed_norm(const void* w, const void* table, const int
     return run_rows<FmtBf16, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, static_cast<hipStream_t>(stream));
 }
 
-int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
-                         size_t n_esc, const void* row_ptr, const void* x, void* y, size_t R, size_t C, size_t M,
-                         void* stream) {
+int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* pairs, const void* esc_idx,
+                         const void* esc_val, size_t n_esc, const void* row_ptr, const void* x, void* y, size_t R,
+                         size_t C, size_t M, void* stream) {
     if (x == nullptr || y == nullptr || lo == nullptr || hi4 == nullptr || table == nullptr || row_ptr == nullptr)
         return ERR_NULL;
     if (n_esc > 0 && (esc_idx == nullptr || esc_val == nullptr)) return ERR_NULL;
     int32_t rc = check_dims(R, C, M, FmtP12::UW);
     if (rc != OK) return rc;
     FmtP12::Params p;
-    rc = p12_params(lo, hi4, table, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
+    rc = p12_params(lo, hi4, table, pairs, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
     if (rc != OK) return rc;
     if (!aligned16(x) || !aligned2(y)) return ERR_DOMAIN;
     // the verify widths: the matrix cores. Weights straight into LDS, 16 rows of x a pass, where that kernel has a
@@ -494,16 +497,24 @@ int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, con
         }
         return OK;
     }
-    // the in-register lookup here, the pair table in LDS for the add + norm forms below: the table is built while the
-    // norm's staging waits for its sums anyway, where a plain x load is over before it is (measured: gate/up 19.2 ->
-    // 17.8 us, qkv 9.9 -> 9.3, head 116 -> 114 with the table; this plain [9728 x 2560] 9.85 -> 10.17)
-    if (tuning("p12_pair_table") > 0)
-        return run_rows<FmtP12L, X_PLAIN, E_PLAIN>(p, plain_x(x), y, R, C, M, static_cast<hipStream_t>(stream));
+    // The lookups through the pair table in LDS (the caller's, made at upload) where waves walk more than one tile - the
+    // kernel then streams, and the table's 1.5 vector instructions a weight beat the in-register lookup's 3.4 - and in
+    // registers where every wave has one tile or none: such a launch is one trip to memory and back, and the LDS
+    // lookups' own latency sits on it (measured with the table from upload, nothing built in the kernel: o
+    // [2560 x 4096] 6.35 against 5.62 us, the one-row [9728 x 2560] 10.5 against 9.9, down [2560 x 9728] level). The
+    // knob p12_pair_table forces either (1 / 0). The add + norm forms below always take the table: their staging
+    // waits for the norm's sums while it arrives.
+    const int knob = tuning("p12_pair_table");
+    const size_t tiles = R / (size_t)(WAVE / lanes_per_row((int)(C / FmtP12::UW)));
+    const bool streams = tiles > (size_t)device_info().cus * 5 * 4;
+    if (pairs != nullptr && (knob >= 0 ? knob != 0 : streams))
+        return run_rows<FmtP12G, X_PLAIN, E_PLAIN>(p, plain_x(x), y, R, C, M, static_cast<hipStream_t>(stream));
     return run_rows<FmtP12, X_PLAIN, E_PLAIN>(p, plain_x(x), y, R, C, M, static_cast<hipStream_t>(stream));
 }
 
-int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table, const void* esc_idx,
-                              const void* esc_val, size_t n_esc, const void* row_ptr, const void* h_in, const void* y,
+int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table, const void* pairs,
+                              const void* esc_idx, const void* esc_val, size_t n_esc, const void* row_ptr,
+                              const void* h_in, const void* y,
                               const void* norm_w, float eps, int32_t centered, void* h_out, void* out, size_t R,
                               size_t C, size_t M, int32_t glu, void* stream) {
     if (out == nullptr) return ERR_NULL;
@@ -511,7 +522,7 @@ int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table
     XArgs xa;
     int32_t rc = norm_args(h_in, y, norm_w, eps, centered, h_out, &xa);
     if (rc == ERR_NULL) return rc;
-    const int32_t rp = p12_params(lo, hi4, table, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
+    const int32_t rp = p12_params(lo, hi4, table, pairs, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
     if (rp == ERR_NULL) return rp;
     if (rc != OK) return rc;
     if (rp != OK) return rp;
@@ -519,15 +530,16 @@ int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table
     if (rc != OK) return rc;
     if (!aligned2(out) || (glu && R % 2 != 0)) return ERR_DOMAIN;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    if (tuning("p12_pair_table") != 0)
-        return glu ? run_rows<FmtP12L, X_ADDNORM, E_GLU>(p, xa, out, R, C, M, st)
-                   : run_rows<FmtP12L, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, st);
+    if (pairs != nullptr && tuning("p12_pair_table") != 0)
+        return glu ? run_rows<FmtP12G, X_ADDNORM, E_GLU>(p, xa, out, R, C, M, st)
+                   : run_rows<FmtP12G, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, st);
     return glu ? run_rows<FmtP12, X_ADDNORM, E_GLU>(p, xa, out, R, C, M, st)
                : run_rows<FmtP12, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, st);
 }
 
-int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void* table, const void* esc_idx,
-                                    const void* esc_val, size_t n_esc, const void* row_ptr, const void* embed,
+int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void* table, const void* pairs,
+                                    const void* esc_idx, const void* esc_val, size_t n_esc, const void* row_ptr,
+                                    const void* embed,
                                     const int32_t* ids, size_t vocab, const void* norm_w, float eps, int32_t centered,
                                     void* h_out, void* out, size_t R, size_t C, size_t M, void* stream) {
     if (out == nullptr) return ERR_NULL;
@@ -535,15 +547,15 @@ int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void*
     XArgs xa;
     int32_t rc = embed_args(embed, ids, vocab, norm_w, eps, centered, h_out, &xa);
     if (rc == ERR_NULL) return rc;
-    const int32_t rp = p12_params(lo, hi4, table, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
+    const int32_t rp = p12_params(lo, hi4, table, pairs, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
     if (rp == ERR_NULL) return rp;
     if (rc != OK) return rc;
     if (rp != OK) return rp;
     rc = check_dims(R, C, M, FmtP12::UW);
     if (rc != OK) return rc;
     if (!aligned2(out)) return ERR_DOMAIN;
-    if (tuning("p12_pair_table") != 0)
-        return run_rows<FmtP12L, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, static_cast<hipStream_t>(stream));
+    if (pairs != nullptr && tuning("p12_pair_table") != 0)
+        return run_rows<FmtP12G, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, static_cast<hipStream_t>(stream));
     return run_rows<FmtP12, X_ADDNORM, E_PLAIN>(p, xa, out, R, C, M, static_cast<hipStream_t>(stream));
 }
 

@@ -142,7 +142,24 @@ __global__ void __launch_bounds__(256) round_bf16_kernel(const float* __restrict
 }
 }  // namespace btb
 
+// entry b of the pair table: the high bytes of the two weights whose codes are byte b's nibbles (the earlier weight
+// the low nibble, its high byte the entry's low byte); slot 15 - the escape code - counts as 0 whatever the table says
+__global__ void __launch_bounds__(256) p12_pairs_kernel(const uint8_t* __restrict__ table, uint16_t* __restrict__ pairs) {
+    const uint32_t b = threadIdx.x;
+    const uint32_t c0 = b & 15u, c1 = b >> 4;
+    const uint32_t h0 = c0 == 15u ? 0u : table[c0], h1 = c1 == 15u ? 0u : table[c1];
+    pairs[b] = (uint16_t)(h0 | (h1 << 8));
+}
+
 extern "C" {
+
+int32_t btb_hip_p12_pairs(const void* table, void* pairs, void* stream) {
+    if (table == nullptr || pairs == nullptr) return ERR_NULL;
+    if (!al(pairs, 2)) return ERR_DOMAIN;
+    hipLaunchKernelGGL(p12_pairs_kernel, dim3(1), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const uint8_t*>(table), static_cast<uint16_t*>(pairs));
+    return hip_status(hipGetLastError(), "p12_pairs launch");
+}
 
 int32_t btb_hip_p12_row_ptr(const void* esc_idx, size_t n_esc, size_t rows, size_t cols, void* row_ptr, void* stream) {
     if (row_ptr == nullptr || (n_esc > 0 && esc_idx == nullptr)) return ERR_NULL;

@@ -102,8 +102,7 @@ class DecodeStep:
     (`Linear`), `embed` (bf16 [V, H]), `norm` and `head` (`Linear`)."""
 
     def __init__(self, card: Any, cfg: StackConfig, weights: dict[str, Any], cap: int, T: int = 1,
-                 attn_spans: int | None = None, fold_silu: bool | None = None, fused: bool | None = None,
-                 persistent: bool = False, workgroups: int | None = None, trace: bool = False) -> None:
+                 attn_spans: int | None = None, fold_silu: bool | None = None, fused: bool | None = None) -> None:
         dev = torch.device("cuda")
         self.card, self.cfg, self.w, self.cap, self.T = card, cfg, weights, int(cap), int(T)
         H, D, Hq, Hk, I = cfg.hidden, cfg.head_dim, cfg.q_heads, cfg.kv_heads, cfg.intermediate
@@ -175,73 +174,7 @@ class DecodeStep:
         # and its depth (the rope position past the cache), read by the kernels from these two device tensors
         self.par = torch.arange(-1, self.T - 1, dtype=torch.int32, device=dev) if self.T > 1 else None
         self.depth = torch.arange(self.T, dtype=torch.int32, device=dev) if self.T > 1 else None
-        self.persistent = bool(persistent)
         self._rows = 0  # the host's count of the cache's rows (n0 starts at 0 on the device too); reset() sets both
-        if self.persistent:
-            self._bind_persistent(workgroups, trace)
-
-    # -- the step as one persistent launch --------------------------------------------------------------------------
-
-    def _bind_persistent(self, workgroups: int | None, trace: bool = False) -> None:
-        """the argument block of `card.decode_step`: the layers' pointer table on the device, the buffers the phases
-        hand to one another, the barrier words. Two workgroups a CU unless told otherwise."""
-        from .native import StepArgs, StepLayer, StepMat
-
-        if self.T != 1:
-            raise ValueError("[decode] the persistent step takes one row")
-        cfg, w, dev = self.cfg, self.w, self.h.device
-        H, D, Hq, Hk, I = cfg.hidden, cfg.head_dim, cfg.q_heads, cfg.kv_heads, cfg.intermediate
-        if D != 128 or Hq != 4 * Hk:
-            raise ValueError("[decode] the persistent step is built for 4 query heads per kv head of 128 dims")
-        packed = [isinstance(w[f"layers.{i}.{k}"].w, P12Weight) for i in range(cfg.layers) for k in
-                  ("qkv", "o", "gu", "down")] + [isinstance(w["head"].w, P12Weight)]
-        if any(packed) != all(packed):
-            raise ValueError("[decode] the persistent step takes every linear in one stored form")
-        self.packed = all(packed)
-        ptr = lambda t: None if t is None else int(t.data_ptr())
-
-        def mat(lin: Linear) -> Any:
-            m = lin.w
-            if isinstance(m, P12Weight):
-                return StepMat(ptr(m.lo), ptr(m.hi4), ptr(m.table), ptr(m.esc_idx), ptr(m.esc_val), ptr(m.row_ptr))
-            return StepMat(ptr(m), None, None, None, None, None)
-
-        table = (StepLayer * cfg.layers)()
-        for i in range(cfg.layers):
-            L = f"layers.{i}."
-            table[i] = StepLayer(mat(w[L + "qkv"]), mat(w[L + "o"]), mat(w[L + "gu"]), mat(w[L + "down"]),
-                                 ptr(w[L + "ln1"]), ptr(w[L + "ln2"]), ptr(w.get(L + "wq")), ptr(w.get(L + "wk")),
-                                 ptr(self.kv[i, 0]), ptr(self.kv[i, 1]))
-        self._layer_table = torch.frombuffer(bytearray(bytes(table)), dtype=torch.uint8).to(dev)
-        self.workgroups = int(workgroups) if workgroups else 2 * int(self.card.sms)
-        self.part = torch.zeros(2 * Hq * self.S + Hq * self.S * D, dtype=torch.float32, device=dev)
-        self.cand_v = torch.zeros(4 * self.workgroups, dtype=torch.float32, device=dev)
-        self.cand_i = torch.zeros(4 * self.workgroups, dtype=torch.int32, device=dev)
-        self.sync = self.card.step_sync(dev)
-        K0 = self.kv[0, 0]
-        import numpy as np
-        a = StepArgs()
-        a.layers = ptr(self._layer_table)
-        a.nlayers, a.H, a.Hq, a.Hk, a.I, a.vocab = cfg.layers, H, Hq, Hk, I, cfg.vocab
-        a.S, a.span = self.S, ((self.cap + self.S - 1) // self.S + 127) // 128 * 128  # the library's rule for a span
-        a.hs, a.rs = int(K0.stride(0)), int(K0.stride(1))
-        a.eps = cfg.eps
-        a.scale_log2 = float(np.float32(self.scale) * np.float32(1.4426950408889634))
-        a.centered = 0
-        a.embed, a.norm_w, a.head = ptr(w["embed"]), ptr(w["norm"]), mat(w["head"])
-        a.cos_t, a.sin_t = ptr(self.cos), ptr(self.sin)
-        a.ids, a.picked, a.n0 = ptr(self.ids), ptr(self.picked), ptr(self.n0)
-        a.h_a, a.h_b, a.qkv, a.att, a.y, a.m = (ptr(t) for t in (self.h, self.h2, self.qkv, self.att, self.y, self.m))
-        a.logits, a.part, a.cand_v, a.cand_i, a.sync = (ptr(t) for t in (self.logits, self.part, self.cand_v,
-                                                                       self.cand_i, self.sync))
-        a.host_tok, a.host_n0, a.host_ts = ptr(self.host_tok), ptr(self.host_n0), ptr(self.host_ts)
-        self.trace = torch.zeros(2 * (5 * cfg.layers + 1), dtype=torch.int64, device=dev) if trace else None
-        a.trace = ptr(self.trace)
-        self._step_args = a
-
-    def barrier_timeouts(self) -> int:
-        """non-zero when a grid barrier of a persistent step gave up waiting (the step's results are then void)"""
-        return int(self.sync[64].item()) if self.persistent else 0
 
     # -- state ---------------------------------------------------------------------------------------------------
 
@@ -291,9 +224,7 @@ class DecodeStep:
     def body(self) -> None:
         if not torch.cuda.is_current_stream_capturing():  # a step being recorded runs nothing
             self._advance()
-        if self.persistent:
-            self.card.decode_step(self._step_args, self.packed, self.workgroups)
-        elif self.fused:
+        if self.fused:
             self._body_fused()
         else:
             self._body_plain()

@@ -39,11 +39,12 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_gemv_glu_silu_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_gemv_bf16_norm": (_i32, [_vp, _vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp, _sz, _sz, _sz, _i32, _vp]),
     "btb_hip_gemv_bf16_embed_norm": (_i32, [_vp, _vp, _vp, _sz, _vp, ctypes.c_float, _i32, _vp, _vp, _sz, _sz, _sz, _vp]),
-    "btb_hip_gemv_p12_embed_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _vp, ctypes.c_float, _i32,
-                                           _vp, _vp, _sz, _sz, _sz, _vp]),
-    "btb_hip_gemv_p12_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp,
-                                     _sz, _sz, _sz, _i32, _vp]),
-    "btb_hip_gemv_p12": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_gemv_p12_embed_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _vp, ctypes.c_float,
+                                           _i32, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_gemv_p12_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, ctypes.c_float, _i32, _vp,
+                                     _vp, _sz, _sz, _sz, _i32, _vp]),
+    "btb_hip_gemv_p12": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_p12_pairs": (_i32, [_vp, _vp, _vp]),
     "btb_hip_p12_row_ptr": (_i32, [_vp, _sz, _sz, _sz, _vp, _vp]),
     "btb_hip_p12_check": (_i32, [_vp, _sz, _sz, _vp, _vp]),
     "btb_hip_p12_widen": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _vp, _vp]),
@@ -91,31 +92,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_argmax": (_i32, [_vp, _vp, _sz, _sz, _vp]),
     "btb_hip_publish": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "btb_hip_argmax_publish": (_i32, [_vp, _sz, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
-    "btb_hip_step_sync_bytes": (_sz, []),
-    "btb_hip_decode_step": (_i32, [_vp, _i32, _i32, _vp]),
 }
-
-
-class StepMat(ctypes.Structure):
-    """btb_hip_step_mat: one matrix of the persistent step in its stored form"""
-    _fields_ = [(n, _vp) for n in ("w", "hi4", "table", "esc_idx", "esc_val", "row_ptr")]
-
-
-class StepLayer(ctypes.Structure):
-    """btb_hip_step_layer"""
-    _fields_ = [("qkv", StepMat), ("o", StepMat), ("gu", StepMat), ("down", StepMat)] + \
-               [(n, _vp) for n in ("ln1", "ln2", "wq", "wk", "K", "V")]
-
-
-class StepArgs(ctypes.Structure):
-    """btb_hip_step_args"""
-    _fields_ = [("layers", _vp)] + [(n, _i32) for n in ("nlayers", "H", "Hq", "Hk", "I", "vocab", "S", "span")] + \
-               [("hs", ctypes.c_int64), ("rs", ctypes.c_int64), ("eps", ctypes.c_float),
-                ("scale_log2", ctypes.c_float), ("centered", _i32), ("embed", _vp), ("norm_w", _vp),
-                ("head", StepMat)] + \
-               [(n, _vp) for n in ("cos_t", "sin_t", "ids", "picked", "n0", "h_a", "h_b", "qkv", "att", "y", "m",
-                                   "logits", "part", "cand_v", "cand_i", "sync", "host_tok", "host_n0", "host_ts",
-                                   "trace")]
 
 
 class HipError(RuntimeError):
@@ -325,7 +302,7 @@ class HipCard(CardLaunch):
                        int(centered), p(h_out), _p(out), R, C, M, int(glu), _stream())
         else:
             ne = int(w.esc_idx.numel())
-            self._call("btb_hip_gemv_p12_norm", _p(w.lo), _p(w.hi4), _p(w.table),
+            self._call("btb_hip_gemv_p12_norm", _p(w.lo), _p(w.hi4), _p(w.table), self._pairs(w),
                        _p(w.esc_idx) if ne else None, _p(w.esc_val) if ne else None, ne, _p(w.row_ptr),
                        _p(h_in), p(y), _p(norm_w), float(eps), int(centered), p(h_out), _p(out), R, C,
                        M, int(glu), _stream())
@@ -351,7 +328,7 @@ class HipCard(CardLaunch):
                        _p(norm_w), float(eps), int(centered), p(h_out), _p(out), R, C, M, _stream())
         else:
             ne = int(w.esc_idx.numel())
-            self._call("btb_hip_gemv_p12_embed_norm", _p(w.lo), _p(w.hi4), _p(w.table),
+            self._call("btb_hip_gemv_p12_embed_norm", _p(w.lo), _p(w.hi4), _p(w.table), self._pairs(w),
                        _p(w.esc_idx) if ne else None, _p(w.esc_val) if ne else None, ne, _p(w.row_ptr),
                        _p(table), _p(ids), vocab, _p(norm_w), float(eps), int(centered), p(h_out),
                        _p(out), R, C, M, _stream())
@@ -379,6 +356,21 @@ class HipCard(CardLaunch):
         if rc != OK:
             raise HipError(f"[hip] btb_hip_p12_check failed: {rc} {_CODES.get(rc, '?')}")
 
+    @staticmethod
+    def _pairs(w: Any) -> ctypes.c_void_p | None:
+        t = getattr(w, "pairs", None)
+        return None if t is None else _p(t)
+
+    def p12_pairs(self, table: torch.Tensor) -> torch.Tensor:
+        """int16 [256] (read as u16): the high bytes of the two weights each byte of codes stands for, the escape code
+        as 0 (built once at upload; the matvecs keep a copy in LDS)"""
+        self._need(table, torch.uint8, "table")
+        if table.numel() != 16:
+            raise ValueError("[hip] p12_pairs: the table holds 16 bytes")
+        out = torch.empty(256, dtype=torch.int16, device=table.device)
+        self._call("btb_hip_p12_pairs", _p(table), _p(out), _stream())
+        return out
+
     def p12_row_ptr(self, esc_idx: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
         """int32 [rows + 1]: the first escape at or past each row's first weight (built once at upload)"""
         self._need(esc_idx, torch.int32, "esc_idx")
@@ -395,7 +387,7 @@ class HipCard(CardLaunch):
         M = int(x2.shape[0])
         y = self._out(y, M, R, x.device, "gemv_p12")
         ne = int(w.esc_idx.numel())
-        self._call("btb_hip_gemv_p12", _p(w.lo), _p(w.hi4), _p(w.table),
+        self._call("btb_hip_gemv_p12", _p(w.lo), _p(w.hi4), _p(w.table), self._pairs(w),
                    _p(w.esc_idx) if ne else None, _p(w.esc_val) if ne else None, ne, _p(w.row_ptr),
                    _p(x2), _p(y), R, C, M, _stream())
         return y
@@ -881,17 +873,6 @@ class HipCard(CardLaunch):
         p = lambda t: None if t is None else _p(t)
         self._call("btb_hip_argmax_publish", _p(logits), V, _p(picked), _p(n0), p(next_ids),
                    p(out_tok), p(out_n0), p(out_ts), _stream())
-
-    # -- the step as one persistent launch ------------------------------------------------------------------------
-
-    def step_sync(self, device: Any = "cuda") -> torch.Tensor:
-        """the zeroed barrier words `decode_step` needs (one tensor per step object, reused by every step)"""
-        n = int(self.lib.btb_hip_step_sync_bytes())
-        return torch.zeros(n // 4, dtype=torch.int32, device=device)
-
-    def decode_step(self, args: StepArgs, packed: bool, workgroups: int) -> None:
-        """one decode step as one launch of `workgroups` resident workgroups (see btb_hip_decode_step)"""
-        self._call("btb_hip_decode_step", ctypes.byref(args), 1 if packed else 0, int(workgroups), _stream())
 
 
 class Native:

@@ -161,10 +161,14 @@ def check_escapes(esc_idx: torch.Tensor, esc_val: torch.Tensor, n: int) -> None:
 
 
 class P12Weight:
-    """One packed matrix on the GPU as the kernels read it; `shape` = (rows, cols). `row_ptr[r]` is the index of the
-    first escape at or past row r's first weight (int32 [rows + 1]), filled by the card at construction."""
+    """One packed matrix on the GPU as the kernels read it; `shape` = (rows, cols). Two arrays are made here, once, by
+    the card: `row_ptr[r]`, the index of the first escape at or past row r's first weight (int32 [rows + 1]), and
+    `pairs`, the 256 two-byte entries the matvecs look a byte of codes up in. The table is the matrix's own copy with
+    slot 15 - the escape code, which names no table entry - set to 0: a store that left another byte there (0x7F or
+    0xFF would make the streamed stand-in of an escaped weight inf or NaN, and its correction NaN) is as good as one
+    that wrote the 0 the packer writes."""
 
-    __slots__ = ("esc_idx", "esc_val", "hi4", "lo", "row_ptr", "shape", "table")
+    __slots__ = ("esc_idx", "esc_val", "hi4", "lo", "pairs", "row_ptr", "shape", "table")
 
     def __init__(self, lo, hi4, table, esc_idx, esc_val, rows: int, cols: int, card: Any) -> None:
         dev = lo.device
@@ -175,7 +179,9 @@ class P12Weight:
             raise ValueError(f"[pack12] [{rows}, {cols}] needs {n} low bytes, {(n + 1) // 2} code bytes and a "
                              f"16-byte table")
         check_size(n)
-        self.lo, self.hi4, self.table = lo.contiguous(), hi4.contiguous(), table.contiguous()
+        self.lo, self.hi4 = lo.contiguous(), hi4.contiguous()
+        self.table = table.to(torch.uint8).clone().contiguous()
+        self.table[15] = 0
         self.esc_idx = esc_idx.to(torch.int32).contiguous()
         self.esc_val = esc_val.to(torch.uint8).contiguous()
         self.shape = (int(rows), int(cols))
@@ -183,6 +189,7 @@ class P12Weight:
         check_escapes(self.esc_idx, self.esc_val, n)
         card.p12_check(self.esc_idx, n)
         self.row_ptr = card.p12_row_ptr(self.esc_idx, rows, cols)
+        self.pairs = card.p12_pairs(self.table)
 
     @classmethod
     def pack(cls, w: torch.Tensor, card: Any) -> "P12Weight":
@@ -191,7 +198,7 @@ class P12Weight:
 
     @property
     def nbytes(self) -> int:
-        return (self.lo.numel() + self.hi4.numel() + 16 + 5 * self.esc_idx.numel() + 4 * self.row_ptr.numel())
+        return (self.lo.numel() + self.hi4.numel() + 16 + 512 + 5 * self.esc_idx.numel() + 4 * self.row_ptr.numel())
 
     def __repr__(self) -> str:
         return f"P12Weight[{self.shape[0]}, {self.shape[1]}, {self.esc_idx.numel()} escapes]"

@@ -91,24 +91,33 @@ int32_t btb_hip_gemv_bf16_embed_norm(const void* w, const void* table, const int
 /* The matvec over a pack12 matrix (n = R * C weights): lo u8[n], hi4 u8[(n + 1) / 2] (weight 2k in the low nibble
  * of byte k), table u8[16], esc_idx i32[n_esc] strictly ascending, esc_val u8[n_esc] - the arrays of
  * btb_gemv_p12_rows (native/src/lib.rs:114-135), on the device, the list validated at upload by btb_hip_p12_check -
- * plus row_ptr i32[R + 1] from btb_hip_p12_row_ptr.
+ * plus two arrays made once at upload: row_ptr i32[R + 1] from btb_hip_p12_row_ptr and pairs u16[256] from
+ * btb_hip_p12_pairs (NULL: the table is looked up in registers instead, a slower kernel with the same bits).
  * x [M, C] bf16, y [M, R] bf16; C a multiple of 16, lo 16-byte and hi4 8-byte aligned. The reference has no card
  * kernel for this form (it widens a packed layer to bf16 before the card holds it: btb/engine/tiers.py:1200-1216). */
-int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* esc_idx, const void* esc_val,
-                         size_t n_esc, const void* row_ptr, const void* x, void* y, size_t R, size_t C, size_t M,
-                         void* stream);
+int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* pairs, const void* esc_idx,
+                         const void* esc_val, size_t n_esc, const void* row_ptr, const void* x, void* y, size_t R,
+                         size_t C, size_t M, void* stream);
 
 /* btb_hip_gemv_bf16_norm over a pack12 matrix (the arrays of btb_hip_gemv_p12). */
-int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table, const void* esc_idx,
-                              const void* esc_val, size_t n_esc, const void* row_ptr, const void* h_in, const void* y,
-                              const void* norm_w, float eps, int32_t centered, void* h_out, void* out, size_t R,
-                              size_t C, size_t M, int32_t glu, void* stream);
+int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table, const void* pairs,
+                              const void* esc_idx, const void* esc_val, size_t n_esc, const void* row_ptr,
+                              const void* h_in, const void* y, const void* norm_w, float eps, int32_t centered,
+                              void* h_out, void* out, size_t R, size_t C, size_t M, int32_t glu, void* stream);
 
 /* btb_hip_gemv_bf16_embed_norm over a pack12 matrix (`table` is the matrix's 16 high bytes, `embed` the embedding). */
-int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void* table, const void* esc_idx,
-                                    const void* esc_val, size_t n_esc, const void* row_ptr, const void* embed,
-                                    const int32_t* ids, size_t vocab, const void* norm_w, float eps, int32_t centered,
-                                    void* h_out, void* out, size_t R, size_t C, size_t M, void* stream);
+int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void* table, const void* pairs,
+                                    const void* esc_idx, const void* esc_val, size_t n_esc, const void* row_ptr,
+                                    const void* embed, const int32_t* ids, size_t vocab, const void* norm_w, float eps,
+                                    int32_t centered, void* h_out, void* out, size_t R, size_t C, size_t M,
+                                    void* stream);
+
+/* pairs[b] = table[b & 15] | table[b >> 4] << 8 for every byte b of codes, the escape code's slot 15 taken as 0: the
+ * high bytes of the two weights a byte of codes stands for, so that the matvec turns a byte of codes into two high
+ * bytes with one 2-byte read of its copy of these 512 bytes in LDS. Made once at upload, beside row_ptr; an escaped
+ * weight then streams as (0, low byte) and the escape list puts its true value in (the matrix should carry 0 in
+ * table[15], as the packer writes it: the kernels that look the table up in registers stream table[15] there). */
+int32_t btb_hip_p12_pairs(const void* table, void* pairs, void* stream);
 
 /* row_ptr[r] = how many escapes lie below weight r * cols, r = 0..rows: the per-row slices of the escape list the
  * matvec reads. Run once when a packed matrix is uploaded; replaces the per-call search of p12_cursors
@@ -378,83 +387,6 @@ int32_t btb_hip_publish(int32_t* n0, const int32_t* picked, int32_t* next_ids, i
  * clock into pinned host memory, then - after a system fence - the cache's length *n0; nothing on the device changes. */
 int32_t btb_hip_publish_only(const int32_t* n0, const int32_t* ids, int32_t* out_tok, int32_t* out_n0, int64_t* out_ts,
                              void* stream);
-
-/* ---- the whole decode step as one persistent launch ---------------------------------------------------------- */
-
-/* One matrix of the step in its stored form. bf16: w [R, C], the other fields NULL. pack12: the arguments of
- * btb_hip_gemv_p12 (w is `lo`). */
-typedef struct btb_hip_step_mat {
-    const void* w;
-    const void* hi4;
-    const void* table;
-    const void* esc_idx;
-    const void* esc_val;
-    const void* row_ptr;
-} btb_hip_step_mat;
-
-/* One layer: qkv [(Hq + 2 Hk) D, H], o [H, Hq D], gu [2 I, H] (gate rows then up rows), down [H, I]; the norm
- * weights ln1 / ln2 [H] and wq / wk [D] (NULL: no q/k norm) in bf16; the layer's caches (head g's slot j at
- * g * hs + j * rs elements). */
-typedef struct btb_hip_step_layer {
-    btb_hip_step_mat qkv, o, gu, down;
-    const void* ln1;
-    const void* ln2;
-    const void* wq;
-    const void* wk;
-    void* K;
-    void* V;
-} btb_hip_step_layer;
-
-/* Everything one step touches; every pointer is device memory except host_* (pinned host memory or NULL).
- * `layers` is a device array of nlayers btb_hip_step_layer. S key spans of `span` keys each cover the cache.
- * Buffers the step owns between its phases: h_a / h_b [H] (the residual, ping-pong), qkv [(Hq + 2 Hk) D], att
- * [Hq D], y [H], m [I], logits [vocab] in bf16; part: 2 Hq S + Hq S D floats; cand_v / cand_i: 4 * workgroups
- * floats / ints; sync: btb_hip_step_sync_bytes() bytes, zeroed once by the caller before the first step. */
-typedef struct btb_hip_step_args {
-    const btb_hip_step_layer* layers;
-    int32_t nlayers, H, Hq, Hk, I, vocab, S, span;
-    int64_t hs, rs;
-    float eps, scale_log2; /* scale_log2 = softmax scale * log2(e) */
-    int32_t centered;
-    const void* embed;     /* [vocab, H] bf16 */
-    const void* norm_w;    /* the final norm [H] */
-    btb_hip_step_mat head; /* [vocab, H] */
-    const void* cos_t;     /* rope tables [positions, D] bf16 */
-    const void* sin_t;
-    int32_t* ids;          /* in: the step's token; out: the picked one (the next step's input) */
-    int32_t* picked;
-    int32_t* n0;           /* in: rows the caches hold; out: + 1 */
-    void* h_a;
-    void* h_b;
-    void* qkv;
-    void* att;
-    void* y;
-    void* m;
-    void* logits;
-    float* part;
-    float* cand_v;
-    int32_t* cand_i;
-    uint32_t* sync;
-    int32_t* host_tok;
-    int32_t* host_n0;
-    int64_t* host_ts;
-    int64_t* trace;        /* NULL, or 2 * (5 nlayers + 1) device words: workgroup 0's clock (100 MHz) before and after
-                              every grid barrier, in order - the step's timeline by phase */
-} btb_hip_step_args;
-
-size_t btb_hip_step_sync_bytes(void);
-
-/* One decode step (M = 1, greedy pick) of a dense stack with 4 query heads per kv head of 128 dims, as ONE launch of
- * `workgroups` resident workgroups that walk the step's phases and meet at grid barriers: the arithmetic, rounding
- * points and summation orders of btb_hip_embed, btb_hip_gemv_bf16_norm (or _p12_norm, `packed` != 0),
- * btb_hip_norm_rope_kv, btb_hip_attn_decode, btb_hip_gemv_bf16, btb_hip_argmax and btb_hip_publish in the order
- * of the reference's _card_body (btb/engine/cuda.py:1722-1834), so logits and token are theirs bit for bit. The
- * reference replays those launches as a CUDA graph; this entry is that graph collapsed into one kernel. DOMAIN when
- * the grid would not be resident at once (the barriers need every workgroup running). A barrier that does not
- * complete within its bounded wait sets word 64 of `sync` and the step runs to its end with wrong results: read
- * that word after the step where a hang elsewhere on the GPU is possible, and zero `sync` before the next step. The
- * barrier words carry over from step to step: zero them as well before a step with a different `workgroups`. */
-int32_t btb_hip_decode_step(const btb_hip_step_args* args, int32_t packed, int32_t workgroups, void* stream);
 
 #ifdef __cplusplus
 }

@@ -23,8 +23,6 @@ pytestmark = pytest.mark.gpu
 
 CFG = StackConfig(layers=3, hidden=256, q_heads=4, kv_heads=2, head_dim=128, intermediate=512, vocab=1000)
 CAP, N0, TOKEN = 96, 40, 17
-# the persistent step's shape family: 4 query heads per kv head, every row length a multiple of 64 load units
-PCFG = StackConfig(layers=3, hidden=512, q_heads=8, kv_heads=2, head_dim=128, intermediate=1024, vocab=1000)
 
 
 def make_weights(card, packed: bool, CFG: StackConfig = CFG):
@@ -141,51 +139,6 @@ def test_graph_replays_equal_the_eager_step(card):
         toks.append(step.token())
     assert int(step.n0[0]) == N0 + 3 and toks[0] == want_tok
 
-
-@pytest.mark.parametrize("packed", [False, True])
-@pytest.mark.parametrize("spans,workgroups", [(1, 64), (3, 256), (3, None)])
-def test_persistent_step_changes_no_bit(card, packed, spans, workgroups):
-    """the step as one persistent launch (grid barriers between its phases) against the launch-per-operator graph:
-    the same logits, token, residual and cache rows bit for bit, over a run of steps that feed one another"""
-    _, dev, kv = make_weights(card, packed, PCFG)
-    ref = DecodeStep(card, PCFG, dev, CAP, attn_spans=spans)
-    one = DecodeStep(card, PCFG, dev, CAP, attn_spans=spans, persistent=True, workgroups=workgroups)
-    for s in (ref, one):
-        s.kv.copy_(kv.cuda())
-        s.reset(N0, TOKEN)
-    for i in range(4):
-        ref.body()
-        one.body()
-        torch.cuda.synchronize()
-        assert one.barrier_timeouts() == 0
-        assert torch.equal(ref.logits, one.logits), i
-        assert ref.token() == one.token() and int(one.host_n0[0]) == N0 + i + 1
-        assert int(one.n0[0]) == N0 + i + 1 and int(one.ids[0]) == one.token()
-        assert torch.equal(ref.kv, one.kv), i
-
-
-def test_persistent_step_replays_as_a_graph(card):
-    """the one-launch step captured and replayed, with eager work between the replays"""
-    _, dev, kv = make_weights(card, False, PCFG)
-    eager = DecodeStep(card, PCFG, dev, CAP)
-    eager.kv.copy_(kv.cuda())
-    eager.reset(N0, TOKEN)
-    eager.body()
-    torch.cuda.synchronize()
-    step = DecodeStep(card, PCFG, dev, CAP, persistent=True)
-    step.kv.copy_(kv.cuda())
-    step.reset(N0, TOKEN)
-    step.capture(warmup=1)
-    for rep in range(3):
-        step.kv.copy_(kv.cuda())
-        step.reset(N0, TOKEN)
-        step.replay()
-        torch.cuda.synchronize()
-        assert step.barrier_timeouts() == 0
-        assert torch.equal(step.logits, eager.logits) and step.token() == eager.token(), rep
-        junk = torch.randn(1 << 16, device="cuda").sum()
-        torch.cuda.synchronize()
-        assert torch.isfinite(junk)
 
 
 @pytest.mark.parametrize("fused", [False, True])

@@ -14,7 +14,7 @@ import pytest
 import torch
 
 import oracle
-from btb_amd import fp8, mxfp4
+from btb_amd import fp8, mxfp4, pack12
 from btb_amd.pack12 import P12Weight
 from oracle import codecs
 
@@ -97,8 +97,8 @@ def test_format_refusals(card):
     assert L.btb_hip_gemv_mxfp4(None, p(z), p(x), p(y), 4, 64, 1, None) == -1
     assert L.btb_hip_gemv_fp8(p(z), p(s), 3, 1, p(x), p(y), 4, 64, 1, None) == -6       # 3 does not divide 4
     assert L.btb_hip_gemv_fp8(p(z), p(s), 1, 8, p(x), p(y), 4, 64, 1, None) == -6       # 8-column blocks: not 16
-    assert L.btb_hip_gemv_p12(p(z), p(z), p(z), None, None, 2, p(s), p(x), p(y), 4, 64, 1, None) == -1
-    assert L.btb_hip_gemv_p12(p(z), p(z), p(z), None, None, 0, p(s), p(x), p(y), 4, 60, 1, None) == -6  # C % 16
+    assert L.btb_hip_gemv_p12(p(z), p(z), p(z), None, None, None, 2, p(s), p(x), p(y), 4, 64, 1, None) == -1
+    assert L.btb_hip_gemv_p12(p(z), p(z), p(z), None, None, None, 0, p(s), p(x), p(y), 4, 60, 1, None) == -6  # C % 16
 
 
 # ---- the verify widths (M >= 8): FP8 and MXFP4 widened into bf16 fragments for the matrix cores -------------------
@@ -407,3 +407,52 @@ def test_the_head_shape(card, packed):
     else:
         y = card.gemv(w.cuda(), x.cuda())
     check(y, ref)
+
+
+def test_pair_table_made_at_upload(card):
+    """pairs[b] = table[b & 15] | table[b >> 4] << 8 with the escape code's slot taken as 0, whatever byte the store
+    left in table[15]; the matrix's own table carries 0 there too"""
+    table = torch.arange(16, dtype=torch.uint8) * 7 + 33
+    table[15] = 0xFF
+    got = card.p12_pairs(table.cuda()).cpu().numpy().view(np.uint16)
+    t = table.numpy().astype(np.uint16).copy()
+    t[15] = 0
+    b = np.arange(256)
+    assert np.array_equal(got, t[b & 15] | (t[b >> 4] << 8))
+    w = weights_bf16(32, 64, seed=380)
+    lo, hi4, tb, ei, ev = (t_.cuda() for t_ in pack12.pack_bf16(w))
+    tb[15] = 0x7F
+    pw = P12Weight(lo, hi4, tb, ei, ev, 32, 64, card)
+    assert int(pw.table[15]) == 0 and int(tb[15]) == 0x7F and pw.pairs.numel() == 256   # its own copy, the caller's left
+
+
+@pytest.mark.parametrize("R,C", [(9728, 2560), (2560, 4096), (2560, 9728), (96, 272)])
+@pytest.mark.parametrize("M", [1, 4, 8, 16])
+def test_plain_packed_matvec_with_and_without_the_pair_table(card, R, C, M):
+    """the plain packed matvec looks its high bytes up in the pair table too (brought into LDS from the copy made at
+    upload); the in-register lookup (knob p12_pair_table = 0, or a caller without the table) gives the same bits. And a
+    store whose unused table slot 15 holds 0xFF - where the streamed stand-in of an escaped weight would be NaN - gives
+    the bits of the store that holds 0 there, at one row and at the matrix-core widths."""
+    w = weights_bf16(R, C, seed=381)
+    wb = bits16(w).copy().reshape(-1)
+    at = np.arange(0, wb.size, max(1, wb.size // 1009))          # forced escapes, low bytes >= 0x80 among them
+    wb[at] = (wb[at] & 0x00FF) | ((0x20 + np.arange(at.size) % 40).astype(np.uint16) << 8)
+    w = torch.from_numpy(wb.view(np.int16).reshape(R, C)).view(torch.bfloat16)
+    x = acts_bf16(M, C, seed=382).cuda()
+    lo, hi4, tb, ei, ev = (t_.cuda() for t_ in pack12.pack_bf16(w))
+    pw = P12Weight(lo, hi4, tb, ei, ev, R, C, card)
+    assert pw.esc_idx.numel() >= 500
+    y = card.gemv_p12(pw, x)
+    try:
+        card.set_tuning("p12_pair_table", 0)
+        y0 = card.gemv_p12(pw, x)
+        card.set_tuning("p12_pair_table", 1)
+        y1 = card.gemv_p12(pw, x)
+    finally:
+        card.set_tuning("p12_pair_table", -1)
+    assert torch.equal(y.view(torch.int16), y0.view(torch.int16)) and torch.equal(y.view(torch.int16), y1.view(torch.int16))
+    check(y, oracle.gemv_bf16(bits16(w), x.float().cpu().numpy(), threads=0))
+    foreign = tb.clone()
+    foreign[15] = 0xFF
+    yf = card.gemv_p12(P12Weight(lo, hi4, foreign, ei, ev, R, C, card), x)
+    assert torch.equal(yf.view(torch.int16), y.view(torch.int16)) and bool(torch.isfinite(yf.float()).all())
