@@ -202,7 +202,7 @@ def copy_workload() -> int:
     return 0
 
 
-def kernel_workload(args: argparse.Namespace) -> int:
+def kernel_workload(args: argparse.Namespace) -> dict:
     """The single-operator configs: one JSON line each, `value` the operator's HBM stream in GB/s. A step is one call
     over the next operand set of a pool larger than the last-level cache (256 MB), so nothing repeats from cache; the
     calls of one pass are replayed as a hipGraph and timed with device events.
@@ -350,7 +350,8 @@ def kernel_workload(args: argparse.Namespace) -> int:
     mean_bytes = sum(nbytes) / len(nbytes)
     gbs = mean_bytes / (us * 1e-6) / 1e9
     tr = traffic_entry(name, f"m{M}")
-    print(json.dumps({
+    del graph
+    return {
         "metric": "decode matvec HBM GB/s (% of peak), one operator", "value": round(gbs, 1), "unit": "GB/s",
         "n_gpus": 1, "steps": passes * pool, "warmup": args.warmup, "ms_per_step": round(us * 1e-3, 5),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype,
@@ -363,8 +364,7 @@ def kernel_workload(args: argparse.Namespace) -> int:
                      "traffic": None if tr is None else tr.get("bytes_per_launch"),
                      "traffic_source": None if tr is None else tr.get("source")},
         "cpu_baseline": None if args.no_cpu else cpu_baseline(name, M),
-    }))
-    return 0
+    }
 
 
 # ---------------------------------------------------------------------------------------------------------------
@@ -461,6 +461,8 @@ def main() -> int:
     ap.add_argument("--rows", type=int, default=1,
                     help="rows of a decode pass: 1 is the step the metric is quoted on, more a speculative verify pass")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="the default run: skip the other benchmark configurations it appends as `configs`")
     ap.add_argument("--tune", action="append", default=[], metavar="KNOB=VALUE",
                     help="set one of the library's tuning knobs before the run (repeatable); recorded in config")
     args = ap.parse_args()
@@ -470,14 +472,56 @@ def main() -> int:
     if args.workload == "copy":
         return copy_workload()
     if args.workload not in ("decode", "decode_p12"):
-        return kernel_workload(args)
+        print(json.dumps(kernel_workload(args)))
+        return 0
     if args.steps < 1 or args.warmup < 0 or args.steps + args.warmup > 480:
         print("bench.py: steps + warmup must stay within the cache's 480 spare rows", file=sys.stderr)
         return 2
     if not 1 <= args.rows <= 24:
         print("bench.py: a pass takes 1 to 24 rows here (the cache keeps 512 rows spare)", file=sys.stderr)
         return 2
+    line = decode_workload(args)
+    # the default run (the line the driver records) carries every other configuration of the benchmark beside the
+    # headline: each one its own workload of this file, timed the same way, without its CPU leg
+    if args.workload == "decode" and args.rows == 1 and not args.tune and not args.no_configs:
+        line["configs"] = other_configs(args)
+    print(json.dumps(line))
+    return 0
 
+
+def other_configs(args: argparse.Namespace) -> list[dict]:
+    """configs[0] and [2]..[4] of the benchmark, one compact record each: the workload, microseconds a step (one
+    operator call, or the whole packed decode step), achieved GB/s over its algorithmic bytes and the fraction of the
+    8 TB/s peak. A workload that fails is recorded with its error instead of ending the run."""
+    import gc
+
+    import torch
+
+    plan = [("gemv_bf16", 1), ("decode_p12", 1), ("moe", 1), ("moe", 4), ("moe", 8), ("moe_mxfp4", 1), ("moe_mxfp4", 4),
+            ("moe_mxfp4", 8), ("gemv_fp8", 1), ("gemv_fp8", 8), ("gemv_fp8", 16), ("gemv_mxfp4", 1), ("gemv_mxfp4", 8),
+            ("gemv_mxfp4", 16), ("gemv_p12", 1)]
+    name_of = {"gemv_bf16": "configs[0]", "decode_p12": "configs[2]", "moe": "configs[3]", "moe_mxfp4": "configs[3], MXFP4 experts",
+               "gemv_fp8": "configs[4a]", "gemv_mxfp4": "configs[4b]", "gemv_p12": "configs[0] in pack12"}
+    out = []
+    for workload, m in plan:
+        sub = argparse.Namespace(**{**vars(args), "workload": workload, "m": m, "no_cpu": True, "tune": [],
+                                    "steps": 100 if workload == "decode_p12" else 96, "warmup": 10 if workload == "decode_p12" else 32})
+        try:
+            d = decode_workload(sub) if workload == "decode_p12" else kernel_workload(sub)
+            rec = {"config": name_of[workload], "workload": d["config"]["workload"], "us_per_step": round(d["ms_per_step"] * 1e3, 2),
+                   "achieved": d["value"], "unit": "GB/s", "frac": d["hbm_frac"]}
+            if workload == "decode_p12":
+                rec["tokens_per_s"] = d["tokens_per_s"]
+        except Exception as e:  # noqa: BLE001 - the headline line must still be printed
+            rec = {"config": name_of[workload], "workload": f"{workload} M={m}", "error": f"{type(e).__name__}: {e}"[:200]}
+        out.append(rec)
+        gc.collect()
+        torch.cuda.empty_cache()
+    return out
+
+
+def decode_workload(args: argparse.Namespace) -> dict:
+    """the decode step (configs[1]; `decode_p12`: configs[2]) as one replayed hipGraph: the line's dict"""
     import torch
 
     from btb_amd.decode import QWEN3_4B, DecodeStep, random_stack
@@ -589,8 +633,8 @@ def main() -> int:
         "roofline": roofline,
         "cpu_baseline": None if args.no_cpu else cpu_baseline(args.workload, 1),
     }
-    print(json.dumps(line))
-    return 0
+    del step
+    return line
 
 
 if __name__ == "__main__":
