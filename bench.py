@@ -3,6 +3,7 @@
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload decode|decode_p12] [--no-cpu]
     python bench.py --workload gemv_bf16|gemv_p12|gemv_fp8|gemv_mxfp4|moe|moe_mxfp4 [--m M]   (the other configs, one operator each)
     python bench.py --workload copy          (a plain 2^28-byte device copy: the scale of the FETCH_SIZE / WRITE_SIZE counters)
+    python bench.py --workload ceiling       (the matvec's loads without the matvec: what the memory system gives such a kernel)
 
 A step is one decode step of a random-init Qwen3-4B-shaped dense stack (36 layers, hidden 2560, 32 query / 8 kv heads
 of 128, SwiGLU 9728, vocab 151936; weights ~N(0, 0.02) in bf16, seeded N(0, 1) K/V for a 4096-token context), M = 1
@@ -200,6 +201,51 @@ def copy_workload() -> int:
     torch.cuda.synchronize()
     print(json.dumps({"workload": "copy", "bytes": n, "copies": 3}))
     return 0
+
+
+def ceiling_workload(args: argparse.Namespace) -> dict:
+    """What the memory system gives a kernel with the streaming matvec's load structure and nothing else to do
+    (`btb_hip_stream_probe`): microseconds and TB/s at the sizes of the step's matrices, each over a pool of distinct
+    copies past the 256 MB last-level cache, replayed as a hipGraph and timed like every other workload here."""
+    import torch
+
+    from btb_amd.native import Native
+
+    card = Native.card_kernels()
+    out = []
+    for what, rows in (("o-sized [4096 x 2560]", 4096), ("qkv [6144 x 2560]", 6144), ("C1 / down-sized [9728 x 2560]", 9728),
+                       ("gate/up [19456 x 2560]", 19456), ("head [151936 x 2560]", 151936)):
+        nbytes = rows * 5120
+        pool = max(3, -(-1_200_000_000 // nbytes))
+        mats = [torch.empty(rows, 2560, dtype=torch.bfloat16, device="cuda").fill_(0.01 * (i + 1)) for i in range(pool)]
+        side = torch.cuda.Stream()
+        with torch.cuda.stream(side):
+            for m in mats:
+                card.stream_probe(m)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph):
+            for m in mats:
+                card.stream_probe(m)
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = max(2, 2000 // pool // max(1, rows // 4096))
+        e0.record(torch.cuda.current_stream())
+        for _ in range(reps):
+            graph.replay()
+        e1.record(torch.cuda.current_stream())
+        torch.cuda.synchronize()
+        us = e0.elapsed_time(e1) * 1e3 / (reps * pool)
+        out.append({"matrix": what, "bytes": nbytes, "us": round(us, 2), "achieved": round(nbytes / us / 1e3, 1), "unit": "GB/s",
+                    "frac_of_8TBs": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4)})
+        del graph, mats
+        torch.cuda.empty_cache()
+    return {"metric": "streaming ceiling: the matvec's loads without the matvec, HBM GB/s", "unit": "GB/s",
+            "value": out[-2]["achieved"], "n_gpus": 1, "higher_is_better": True, "data": "constant-filled matrices",
+            "config": {"workload": "btb_hip_stream_probe over bf16 [R, 2560] matrices, pools past the last-level cache"},
+            "sizes": out}
 
 
 def kernel_workload(args: argparse.Namespace) -> dict:
@@ -456,7 +502,8 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=100)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="decode",
-                    choices=["decode", "decode_p12", "gemv_bf16", "gemv_p12", "gemv_fp8", "gemv_mxfp4", "moe", "moe_mxfp4", "copy"])
+                    choices=["decode", "decode_p12", "gemv_bf16", "gemv_p12", "gemv_fp8", "gemv_mxfp4", "moe", "moe_mxfp4", "copy",
+                             "ceiling"])
     ap.add_argument("--m", type=int, default=1, help="rows of x (tokens) for the single-operator workloads")
     ap.add_argument("--rows", type=int, default=1,
                     help="rows of a decode pass: 1 is the step the metric is quoted on, more a speculative verify pass")
@@ -471,6 +518,9 @@ def main() -> int:
         return 2
     if args.workload == "copy":
         return copy_workload()
+    if args.workload == "ceiling":
+        print(json.dumps(ceiling_workload(args)))
+        return 0
     if args.workload not in ("decode", "decode_p12"):
         print(json.dumps(kernel_workload(args)))
         return 0

@@ -76,10 +76,8 @@ static Knob g_knobs[] = {
     {"p12_pair_table", {-1}},
     {"moe_wgs_per_cu", {-1}},
     {"moe_grouped", {-1}},
-    {"moe_fused_router", {-1}},
     {"attn_split", {-1}},
     {"attn_heads_per_wg", {-1}},
-    {"attn_rows_per_wg", {-1}},
     {"attn_mfma", {-1}},
     {"attn_rows_fused", {-1}},
 };

@@ -1,5 +1,4 @@
-// The routing of one row of router logits by one wave, shared by the routing kernel (moe.hip) and by the router
-// matvec whose last workgroup routes the rows it has just finished (lane16.hip).
+// The routing of one row of router logits by one wave (the routing kernels of moe.hip).
 #pragma once
 
 #include <type_traits>
@@ -8,12 +7,8 @@
 
 namespace btb {
 
-template <bool F32, bool COHERENT = false>
+template <bool F32>
 __device__ __forceinline__ float logit_at(const void* base, size_t i) {
-    if constexpr (COHERENT) {
-        static_assert(F32, "the fused router's logits are f32");
-        return __hip_atomic_load(static_cast<const float*>(base) + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
     return F32 ? static_cast<const float*>(base)[i] : bf16_f32(static_cast<const uint16_t*>(base)[i]);
 }
 
@@ -50,9 +45,9 @@ __device__ __forceinline__ unsigned long long wave_max_u64(unsigned long long v)
     return best;
 }
 
-// one wave routes row t, whose logits start at logits[base]; COHERENT: the logits were written by other workgroups of
+// one wave routes row t, whose logits start at logits[base]
 // this launch and are read past the first-level cache
-template <bool F32, int P, bool COHERENT>
+template <bool F32, int P>
 __device__ __forceinline__ void route_row_reg(const void* __restrict__ logits, size_t base, int t, int lane, int E, int k,
                                               int32_t* __restrict__ idx, uint16_t* __restrict__ w,
                                               float* __restrict__ w32, uint16_t* __restrict__ logits16) {
@@ -60,7 +55,7 @@ __device__ __forceinline__ void route_row_reg(const void* __restrict__ logits, s
 #pragma unroll
     for (int s = 0; s < P; ++s) {
         const int e = lane + WAVE * s;
-        lv[s] = e < E ? logit_at<F32, COHERENT>(logits, base + e) : bits_f32(0xff800000u);
+        lv[s] = e < E ? logit_at<F32>(logits, base + e) : bits_f32(0xff800000u);
     }
     if (logits16 != nullptr) {
 #pragma unroll

@@ -289,66 +289,65 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
 }
 
 // The same for a pass of several rows and short spans: a workgroup takes one kv head, one span of NBT batches of keys
-// (128 NBT keys) and `rows_per_wg` of the pass's rows (one, as launched: see the launcher). The span's K and V rows are
-// all asked for at once and stay in registers; each row in turn brings its G query heads, folds the span's batches
-// into a fresh state and leaves its partial state. A row's arithmetic is attn_decode_kernel's at the same span length:
-// a key the row does not see scores -inf there and here, and weighs 0.
+// (128 NBT keys) and one of the pass's rows. The span's K and V rows are all asked for at once and stay in registers; the
+// row brings its G query heads, folds the span's batches into a fresh state and leaves its partial state. A row's
+// arithmetic is attn_decode_kernel's at the same span length: a key the row does not see scores -inf there and here,
+// and weighs 0. (Several rows of a pass sharing a workgroup's keys was built and measured: it loses - the rows run one
+// after another, each with its own fold of the 16 streams, which costs more than the other rows' workgroups reading
+// the same keys out of L2; 8 rows over 4096 keys: 3.67 ms a pass with one row a workgroup, 3.71 with two, 4.23 with
+// eight.)
 template <int G, int NBT>
 __global__ void __launch_bounds__(256) attn_decode_rows_kernel(
     const uint16_t* __restrict__ q, const uint16_t* __restrict__ K, const uint16_t* __restrict__ V,
     const int32_t* __restrict__ n0p, const int32_t* __restrict__ par, int T, int Hq, int Hk, long long hs, long long rs,
-    float scale_log2, float* __restrict__ part_m, float* __restrict__ part_l, float* __restrict__ part_acc,
-    int rows_per_wg, int win, const int32_t* __restrict__ tbl) {
+    float scale_log2, float* __restrict__ part_m, float* __restrict__ part_l, float* __restrict__ part_acc, int win,
+    const int32_t* __restrict__ tbl) {
     constexpr int D = ATT_D, SPAN = 16 * KB * NBT;
     __shared__ float s_m[16][G], s_l[16][G];
     __shared__ __align__(16) float s_acc[16][G][D];
     __shared__ __align__(16) float s_x[16][XCH];  // the streams' exchange areas
-    const int g = blockIdx.x, sp = blockIdx.y, S = gridDim.y;
-    const int t0 = blockIdx.z * rows_per_wg, t1 = min(T, t0 + rows_per_wg);
+    const int g = blockIdx.x, sp = blockIdx.y, S = gridDim.y, t = blockIdx.z;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int sub = lane >> 4, dl = lane & 15;
     const int grp = wv * 4 + sub;
     const int n0 = *n0p;
-    // the keys any of the workgroup's rows may see end at n_max (a chain's last row, or the whole pass for a tree)
-    const int n_max = par != nullptr ? n0 + T : n0 + t1;
+    // the keys the row may see end at n_max (a chain's row t, or the whole pass for a tree)
+    const int n_max = par != nullptr ? n0 + T : n0 + t + 1;
     const int k_begin = sp * SPAN, k_lim = min(n_max, k_begin + SPAN);
     const uint16_t* Kh = K + (size_t)g * hs + dl * 8;
     const uint16_t* Vh = V + (size_t)g * hs + dl * 8;
     KeyBatch kb[NBT];
 #pragma unroll
     for (int nb = 0; nb < NBT; ++nb) load_keys(kb[nb], Kh, Vh, rs, k_begin + grp + nb * 16 * KB, max(k_lim, 1), -1, tbl);
-    for (int t = t0; t < t1; ++t) {
-        const RowView rv = row_view(par, t, T, n0, win);
-        const int k_end = min(rv.n, k_begin + SPAN);
-        uint32_t qp[G][4];
+    const RowView rv = row_view(par, t, T, n0, win);
+    const int k_end = min(rv.n, k_begin + SPAN);
+    uint32_t qp[G][4];
 #pragma unroll
-        for (int j = 0; j < G; ++j) {
-            const uint4 raw = *reinterpret_cast<const uint4*>(q + ((size_t)t * Hq + (size_t)g * G + j) * D + dl * 8);
-            qp[j][0] = raw.x;
-            qp[j][1] = raw.y;
-            qp[j][2] = raw.z;
-            qp[j][3] = raw.w;
-        }
-        AttnState<G> st;
-        st.init();
-#pragma unroll
-        for (int nb = 0; nb < NBT; ++nb) {
-            const int key0 = k_begin + grp + nb * 16 * KB;
-            if (key0 < k_end)
-                use_keys<G>(kb[nb], key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, st, &s_x[grp][0], rv.tree_base,
-                            rv.tree_mask, rv.k_first);
-        }
-        const size_t prow = ((size_t)t * Hk + g) * S + sp;
-        fold_streams<G>(st, grp, dl, &s_x[grp][0], &s_m[0][0], &s_l[0][0], &s_acc[0][0][0], threadIdx.x,
-                        [&](int j, int d, float M, float L, float A) {
-                            part_acc[(prow * G + j) * D + d] = A;
-                            if (d == 0) {
-                                part_m[prow * G + j] = M;
-                                part_l[prow * G + j] = L;
-                            }
-                        });
-        __syncthreads();  // the fold's LDS is the next row's
+    for (int j = 0; j < G; ++j) {
+        const uint4 raw = *reinterpret_cast<const uint4*>(q + ((size_t)t * Hq + (size_t)g * G + j) * D + dl * 8);
+        qp[j][0] = raw.x;
+        qp[j][1] = raw.y;
+        qp[j][2] = raw.z;
+        qp[j][3] = raw.w;
     }
+    AttnState<G> st;
+    st.init();
+#pragma unroll
+    for (int nb = 0; nb < NBT; ++nb) {
+        const int key0 = k_begin + grp + nb * 16 * KB;
+        if (key0 < k_end)
+            use_keys<G>(kb[nb], key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, st, &s_x[grp][0], rv.tree_base,
+                        rv.tree_mask, rv.k_first);
+    }
+    const size_t prow = ((size_t)t * Hk + g) * S + sp;
+    fold_streams<G>(st, grp, dl, &s_x[grp][0], &s_m[0][0], &s_l[0][0], &s_acc[0][0][0], threadIdx.x,
+                    [&](int j, int d, float M, float L, float A) {
+                        part_acc[(prow * G + j) * D + d] = A;
+                        if (d == 0) {
+                            part_m[prow * G + j] = M;
+                            part_l[prow * G + j] = L;
+                        }
+                    });
 }
 
 // The step's own form (one row): the kernel reads the fused qkv row itself. A workgroup takes GW of a kv head's query
@@ -717,15 +716,10 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
                        tbl);                                                                                         \
     hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,       \
                        (int)Hk, (int)S, part_m, part_l, part_acc)
-    // Several rows and spans of one or two batches of keys: the span's keys are asked for at once and kept in registers.
-    // Rows a workgroup takes: one. Sharing a workgroup's keys among several rows (knob attn_rows_per_wg) was measured
-    // and loses - a pass of 8 rows over 4096 keys, 36 spans: 3.67 ms with one row a workgroup, 3.71 with two, 3.83
-    // with four, 4.23 with eight: the rows of a workgroup run one after another, each with its own fold of the 16
-    // streams, which costs more than the other rows' workgroups reading the same keys out of L2 (the keys leave memory
-    // once either way). Against attn_decode_kernel at its best span count the pass takes 3.67 instead of 3.83 ms.
     // Several rows and spans of 128 keys: the matrix cores, every row of the pass that shares a kv head in one workgroup
-    // (attn_mfma.hip). A pass of 8 rows over 4096 keys: 22.7 us a layer on the vector kernel below, which stays for
-    // spans of 256 keys and behind the knob attn_mfma = 0.
+    // (attn_mfma.hip). A pass of 8 rows over 4096 keys: 22.7 us a layer on the vector kernel below (spans of one or two
+    // batches of keys, asked for at once and kept in registers, a workgroup a row), which stays for spans of 256 keys
+    // and behind the knob attn_mfma = 0.
     if (parts == nullptr && attn_mfma_fits(T, G, span)) {
         const int32_t rc = attn_decode_mfma(q, K, V, n0, par, T, Hq, Hk, (long long)hs, (long long)rs, scale_log2, part_m,
                                             part_l, part_acc, S, cap, (int)win, tbl, st);
@@ -738,15 +732,12 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
                                (int)Hk, (int)S, part_m, part_l, part_acc);
         return hip_status(hipGetLastError(), "attn_decode launch");
     }
-    const int rows_knob = tuning("attn_rows_per_wg");
-    if (parts == nullptr && T >= 2 && (span == 128 || span == 256) && (G == 2 || G == 4) && rows_knob != 0) {
-        int rpw = rows_knob > 0 ? rows_knob : 1;
-        if (rpw > (int)T) rpw = (int)T;
-        const dim3 rgrid((unsigned)Hk, (unsigned)S, (unsigned)((T + rpw - 1) / rpw));
+    if (parts == nullptr && T >= 2 && (span == 128 || span == 256) && (G == 2 || G == 4)) {
+        const dim3 rgrid((unsigned)Hk, (unsigned)S, (unsigned)T);
 #define ATTR(GG, NB)                                                                                                  \
     hipLaunchKernelGGL((attn_decode_rows_kernel<GG, NB>), rgrid, dim3(256), 0, st, static_cast<const uint16_t*>(q),   \
                        static_cast<const uint16_t*>(K), static_cast<const uint16_t*>(V), n0, par, (int)T, (int)Hq,    \
-                       (int)Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, rpw, (int)win, tbl); \
+                       (int)Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, (int)win, tbl);      \
     hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,        \
                        (int)Hk, (int)S, part_m, part_l, part_acc)
         if (G == 4 && span == 128) { ATTR(4, 1); }

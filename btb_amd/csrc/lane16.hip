@@ -131,20 +131,6 @@ __global__ void __launch_bounds__(256) lane16_kernel(W w, const XT* __restrict__
     }
 }
 
-// What the router's matvec does when its rows are done: the last workgroup of a pass to finish routes the pass's rows
-// of x (moe.hip's routing of f32 logits, one wave a row), so logits and picks come out of one launch. "Last" is by a
-// ticket a pass, counted in g_route_tickets and set back to zero by the workgroup that takes the last one, so every
-// launch finds zeros; launches that overlap on one GPU would share the tickets and must not (streams are the caller's).
-struct RouteTail {
-    int32_t* idx = nullptr;  // nullptr: a plain matvec
-    uint16_t* w = nullptr;
-    float* w32 = nullptr;
-    uint16_t* logits16 = nullptr;
-    int k = 0;
-};
-constexpr int ROUTE_TICKETS = 1024;
-static __device__ unsigned int g_route_tickets[ROUTE_TICKETS];
-
 // bf16 rows 128 columns wide a step: the group's sixteen lanes bring 256 contiguous bytes in with one 16-byte load each
 // and hand them round through a slab of LDS the group owns, where lane j then finds its columns j, j + 16, ... - one
 // request a lane for eight of its columns instead of eight. x is staged once a workgroup, as f32. The sums are the same
@@ -153,7 +139,7 @@ static __device__ unsigned int g_route_tickets[ROUTE_TICKETS];
 template <int B, int NB, class XT>
 __global__ void __launch_bounds__(256) lane16_bf16_wide_kernel(const uint16_t* __restrict__ w, const XT* __restrict__ x,
                                                                float* __restrict__ y, size_t rows, size_t cols, size_t b0,
-                                                               size_t btotal, RouteTail rt) {
+                                                               size_t btotal) {
     extern __shared__ __align__(16) unsigned char smem[];
     constexpr int BP = B == 3 ? 4 : B;  // a column's B values of x side by side, one LDS read
     float* xs = reinterpret_cast<float*>(smem);           // [cols][BP]
@@ -223,37 +209,12 @@ __global__ void __launch_bounds__(256) lane16_bf16_wide_kernel(const uint16_t* _
         const float s = group_sum<16>(acc[i]);
         if (j == 0 && live && b0 + i < btotal) y[(b0 + i) * rows + r] = s;
     }
-    if (rt.idx == nullptr) return;
-    // the routing of the pass's rows, by the workgroup that finishes last: its sums above are visible to the device
-    // before its ticket is taken, and the others' are read past this CU's first-level cache
-    int* s_last = reinterpret_cast<int*>(slabs + 16 * NB * 256);  // a word past the slabs (launch_wide leaves 16 bytes)
-    __threadfence();
-    __syncthreads();
-    if (tid == 0) {
-        const unsigned int t = atomicAdd(&g_route_tickets[blockIdx.y], 1u);
-        *s_last = t == gridDim.x - 1;
-        if (*s_last) g_route_tickets[blockIdx.y] = 0u;
-    }
-    __syncthreads();
-    if (!*s_last) return;
-    __threadfence();
-    const int wv = tid / WAVE, lane = tid & (WAVE - 1);
-    if (wv < B && b0 + wv < btotal) {
-        const int t = (int)(b0 + wv), E = (int)rows;
-        const size_t base = (size_t)t * rows;
-        if (E <= WAVE)
-            route_row_reg<true, 1, true>(y, base, t, lane, E, rt.k, rt.idx, rt.w, rt.w32, rt.logits16);
-        else if (E <= 2 * WAVE)
-            route_row_reg<true, 2, true>(y, base, t, lane, E, rt.k, rt.idx, rt.w, rt.w32, rt.logits16);
-        else
-            route_row_reg<true, 4, true>(y, base, t, lane, E, rt.k, rt.idx, rt.w, rt.w32, rt.logits16);
-    }
 }
 
 template <int B, int NB, class XT>
 static bool launch_wide(const uint16_t* w, const XT* x, float* y, size_t rows, size_t cols, size_t b0, size_t b,
-                        unsigned passes, hipStream_t st, const RouteTail& rt = RouteTail{}) {
-    const size_t lds = (size_t)(B == 3 ? 4 : B) * cols * 4 + 16 * NB * 256 + 16;  // x, the slabs, the tail's flag
+                        unsigned passes, hipStream_t st) {
+    const size_t lds = (size_t)(B == 3 ? 4 : B) * cols * 4 + 16 * NB * 256;  // x, the slabs
     if (lds > (size_t)device_info().lds_bytes) return false;
     auto kern = lane16_bf16_wide_kernel<B, NB, XT>;
     static bool raised = false;  // per instance; the attribute is the function's, set before its first large launch
@@ -263,7 +224,7 @@ static bool launch_wide(const uint16_t* w, const XT* x, float* y, size_t rows, s
             return false;
         raised = true;
     }
-    hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 15) / 16), passes), dim3(256), lds, st, w, x, y, rows, cols, b0, b, rt);
+    hipLaunchKernelGGL(kern, dim3((unsigned)((rows + 15) / 16), passes), dim3(256), lds, st, w, x, y, rows, cols, b0, b);
     return true;
 }
 
@@ -337,31 +298,6 @@ int32_t lane16_bf16_rows16(const uint16_t* w, size_t rows, size_t cols, const ui
                            hipStream_t st) {
     if (!shape_ok(rows, cols, b)) return ERR_DOMAIN;
     return launch_lane16(W16Bf16{w}, x, y, rows, cols, b, st);
-}
-
-// The same logits and, out of the same launch, their routing (btb_route.hpp): idx i32 [b, k], wts bf16 [b, k], w32 and
-// logits16 optional. Returns ERR_UNSUPPORTED, having launched nothing, for the shapes this form does not take (rows not
-// a multiple of 128 columns or not 16-byte aligned, more than 256 experts, more passes than tickets) and unless the knob
-// moe_fused_router asks for it: the caller then uses the matvec and the routing kernel one after the other. Off by
-// default because it is no faster: inside a graph the routing kernel's launch costs less than the tail's fence,
-// ticket and barrier cost every workgroup of the matvec (Qwen3-30B-A3B router, one row: 29.4 us a layer against 27.5).
-int32_t lane16_bf16_router16(const uint16_t* w, size_t rows, size_t cols, const uint16_t* x, size_t b, float* y,
-                             int32_t* idx, uint16_t* wts, float* w32, uint16_t* logits16, int k, hipStream_t st) {
-    if (!shape_ok(rows, cols, b)) return ERR_DOMAIN;
-    const size_t passes = b == 1 ? 1 : (b + 3) / 4;
-    if (cols % 128 != 0 || ((reinterpret_cast<uintptr_t>(w) | reinterpret_cast<uintptr_t>(x)) & 15) != 0 ||
-        rows > 4 * WAVE || passes > (size_t)ROUTE_TICKETS || tuning("moe_fused_router") <= 0)
-        return ERR_UNSUPPORTED;
-    RouteTail rt;
-    rt.idx = idx;
-    rt.w = wts;
-    rt.w32 = w32;
-    rt.logits16 = logits16;
-    rt.k = k;
-    const bool done = b == 1 ? launch_wide<1, 16>(w, x, y, rows, cols, 0, b, 1, st, rt)
-                             : launch_wide<4, 4>(w, x, y, rows, cols, 0, b, (unsigned)passes, st, rt);
-    if (!done) return ERR_UNSUPPORTED;
-    return hip_status(hipGetLastError(), "router launch");
 }
 
 }  // namespace btb

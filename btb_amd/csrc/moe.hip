@@ -26,8 +26,6 @@ namespace btb {
 
 int32_t lane16_bf16_rows16(const uint16_t* w, size_t rows, size_t cols, const uint16_t* x, size_t b, float* y,
                            hipStream_t st);  // lane16.hip
-int32_t lane16_bf16_router16(const uint16_t* w, size_t rows, size_t cols, const uint16_t* x, size_t b, float* y,
-                             int32_t* idx, uint16_t* wts, float* w32, uint16_t* logits16, int k, hipStream_t st);
 
 constexpr int ROUTE_MAX_K = 32;  // the reference's ROUTE_MAX_K (native/cuda/btb_kernels.cu:859)
 
@@ -109,7 +107,7 @@ template <bool F32, int P>
 __global__ void __launch_bounds__(64) moe_route_reg_kernel(const void* __restrict__ logits, size_t ls, int E, int k,
                                                            int32_t* __restrict__ idx, uint16_t* __restrict__ w,
                                                            float* __restrict__ w32, uint16_t* __restrict__ logits16) {
-    route_row_reg<F32, P, false>(logits, (size_t)blockIdx.x * ls, (int)blockIdx.x, (int)threadIdx.x, E, k, idx, w, w32,
+    route_row_reg<F32, P>(logits, (size_t)blockIdx.x * ls, (int)blockIdx.x, (int)threadIdx.x, E, k, idx, w, w32,
                                  logits16);
 }
 
@@ -705,12 +703,8 @@ int32_t btb_hip_moe_router_bf16(const void* router, const void* x, size_t T, siz
     if (!al(router, 2) || !al(x, 2) || !al(logits, 4) || !al(logits16, 2) || !al(idx, 4) || !al(w, 2) || !al(w32, 4))
         return ERR_DOMAIN;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    // one launch where the matvec's last workgroup can route (up to 256 experts, rows of whole 128-column steps)
-    int32_t rc = lane16_bf16_router16(static_cast<const uint16_t*>(router), E, H, static_cast<const uint16_t*>(x), T,
-                                      logits, idx, static_cast<uint16_t*>(w), w32, static_cast<uint16_t*>(logits16),
-                                      (int)k, st);
-    if (rc != ERR_UNSUPPORTED) return rc;
-    rc = lane16_bf16_rows16(static_cast<const uint16_t*>(router), E, H, static_cast<const uint16_t*>(x), T, logits, st);
+    const int32_t rc =
+        lane16_bf16_rows16(static_cast<const uint16_t*>(router), E, H, static_cast<const uint16_t*>(x), T, logits, st);
     if (rc != OK) return rc;
     return launch_route<true>(logits, E, (int)E, (int)k, (int)T, idx, static_cast<uint16_t*>(w), w32,
                               static_cast<uint16_t*>(logits16), st);

@@ -34,6 +34,7 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_sms": (_i32, []),
     "btb_hip_last_error": (ctypes.c_char_p, []),
     "btb_hip_set_tuning": (_i32, [ctypes.c_char_p, _i32]),
+    "btb_hip_stream_probe": (_i32, [_vp, _sz, _vp, _vp]),
     "btb_hip_gemv_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_gemv_silu_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_gemv_glu_silu_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
@@ -191,6 +192,13 @@ class HipCard(CardLaunch):
         if rc != OK:
             msg = self.lib.btb_hip_last_error().decode(errors="replace")
             raise HipError(f"[hip] {name} failed: {rc} {_CODES.get(rc, '?')} {msg}")
+
+    def stream_probe(self, a: torch.Tensor) -> None:
+        """the streaming matvec's loads over a bf16 [R, 2560] matrix, without the matvec (a measurement aid)"""
+        self._need(a, torch.bfloat16, "a")
+        if a.dim() != 2 or a.shape[1] != 2560 or a.shape[0] % 2:
+            raise ValueError("[hip] stream_probe reads a bf16 [R, 2560] matrix, R even")
+        self._call("btb_hip_stream_probe", _p(a), int(a.shape[0]), None, _stream())
 
     def set_tuning(self, key: str, value: int) -> None:
         self._call("btb_hip_set_tuning", key.encode(), int(value))

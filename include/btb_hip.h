@@ -52,6 +52,15 @@ const char* btb_hip_last_error(void);
  * BTB_ERR_DOMAIN. For measurement only: no knob changes any result bit. No counterpart in the reference. */
 int32_t btb_hip_set_tuning(const char* key, int32_t value);
 
+/* A measurement aid: the streaming matvec's loads without the matvec. Reads a [rows, 2560] bf16-shaped matrix (rows
+ * even, 5120 bytes a row, 16-byte aligned) the way btb_hip_gemv_bf16_norm's gate/up form does - a wave a pair of rows
+ * half the matrix apart, ten 16-byte non-temporal loads a lane in flight, the streaming kernel's grid - folds what
+ * arrives with a few integer instructions and writes nothing (`sink`, a device word or NULL, is never written in
+ * practice). bytes / time of this launch is what the memory system gives a kernel of the matvec's load structure at
+ * this size: the practical ceiling beside the data sheet's 8 TB/s (`bench.py --workload ceiling`). No counterpart in
+ * the reference. */
+int32_t btb_hip_stream_probe(const void* a, size_t rows, uint32_t* sink, void* stream);
+
 /* ---- card operators: bf16 activations in, f32 accumulate, bf16 out ------------------------------------- */
 
 /* y[m][r] = bf16(sum_c w[r][c] * x[m][c]).  w [R, C] bf16 row-major, x [M, C] bf16, y [M, R] bf16; C a multiple

@@ -5,8 +5,8 @@
   mxfp4    btb/mxfp4.py:41, 102-124 (table, dequantize, scale factors)
 
 The MXFP4 *encoder* has no counterpart in the reference (it only ever decodes checkpoints or draws random bytes:
-tests/helpers.py:305-316); `mxfp4_encode` follows the OCP MX rule and its parity is unpinned - only the decode of
-what it writes is pinned.
+tests/helpers.py:305-316), so no reference result exists for it to match; `mxfp4_encode` follows the OCP MX rule and
+is held to that rule by an exhaustive nearest-value search in exact arithmetic (tests/test_codecs.py).
 """
 
 from __future__ import annotations
@@ -203,7 +203,10 @@ def mxfp4_dequantize(blocks: np.ndarray, scales: np.ndarray) -> np.ndarray:
 def mxfp4_encode(t: np.ndarray):
     """f32 [rows, K] to (blocks [rows, K/32, 16], scales [rows, K/32]) by the OCP MX rule: the block's shared
     exponent is floor(log2(amax)) - 2, elements round to the nearest e2m1 value (ties to the even code) and
-    saturate at 6. No counterpart in the reference: parity unpinned."""
+    saturate at 6. No counterpart in the reference (it reads MXFP4 checkpoints and never writes one), so there is
+    no reference result to be in parity with; the rule itself is pinned by tests/test_codecs.py: every element against
+    an exhaustive nearest-value search in exact rationals over the grid's midpoints, their neighbours and the
+    saturation edge, the scale byte against the exponent rule."""
     t = np.asarray(t, dtype=np.float32)
     rows, K = t.shape
     if K % 32:

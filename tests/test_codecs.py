@@ -151,9 +151,9 @@ def test_mxfp4_dequantize_matches_transformers():
 
 
 def test_mxfp4_encoder_round_trip_and_agreement():
-    """the encoder has no counterpart in the reference (parity unpinned); what is checked: the two restatements
-    agree, every representable matrix survives encode -> decode, and the error stays within the rule's bound: half
-    the widest grid gap, or the saturation of a block's peak (below 8 units) at 6"""
+    """the encoder has no counterpart in the reference; beside the brute-force test below: the two restatements
+    agree on N(0, 0.02) weights, every representable matrix survives encode -> decode, and the error stays within the
+    rule's bound: half the widest grid gap, or the saturation of a block's peak (below 8 units) at 6"""
     w = weights_bf16(16, 256, 41).float()
     pb, ps = mxfp4.quantize(w)
     ob, os_ = codecs.mxfp4_encode(w.numpy())
@@ -163,6 +163,58 @@ def test_mxfp4_encoder_round_trip_and_agreement():
     assert torch.equal(mxfp4.dequantize(pb2, ps2), deq)
     unit = mxfp4.scale_factors(ps)[..., None]
     assert torch.all((deq - w).abs().reshape(16, 8, 32) <= 2.0 * unit)
+
+
+def _nearest_e2m1(v: float, scale_byte: int) -> int:
+    """the code of the e2m1 value nearest to v / 2^(scale - 127), by exhaustive search in exact arithmetic: ties go to
+    the code with an even mantissa bit (0, 1, 2, 4: codes 0, 2, 4, 6), magnitudes past 6 saturate at 6; the sign bit is
+    v's (a negative zero keeps it)"""
+    import math
+    from fractions import Fraction
+
+    a = abs(Fraction(float(v))) / Fraction(2) ** (scale_byte - 127)
+    mags = [Fraction(x) for x in (0, 0.5, 1, 1.5, 2, 3, 4, 6)]
+    best = min(range(8), key=lambda c: (abs(mags[c] - a), c & 1))   # nearest, then the even code
+    return best | (8 if math.copysign(1.0, float(v)) < 0 else 0)
+
+
+def test_mxfp4_encoder_is_the_ocp_rule_by_brute_force():
+    """The reference has no MXFP4 encoder (it reads checkpoints; its tests draw random bytes), so there is nothing to
+    be in parity with; what fixes an encoder is the OCP MX rule itself: shared exponent floor(log2(amax)) - 2, elements
+    to the NEAREST e2m1 value, ties to even, saturation at 6. Every element of blocks built around the grid's exact
+    midpoints, their neighbours one f32 step either side, the saturation edge, zeros and negative zeros is held to an
+    exhaustive nearest-value search in exact rationals; the scale byte is held to the exponent rule on powers of two
+    and just below them. An encoder that rounds toward zero (or ties away from even) fails on the midpoints."""
+    rng = np.random.default_rng(7)
+    mids = np.array([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0], np.float32)
+    rows = []
+    want_scale = []
+    for k in (-20, -9, -3, 0, 5):                        # the block's unit 2^k: its peak fixes the shared exponent
+        unit = np.float32(2.0) ** np.float32(k)
+        for peak in (4.0, 5.9, 6.0, 7.999):             # floor(log2(peak * unit)) - 2 == k for each of these
+            v = np.concatenate([mids, np.nextafter(mids, np.float32(0)), np.nextafter(mids, np.float32(9)),
+                                [0.0, -0.0, 0.1, 6.0, 6.5, 7.5]]).astype(np.float32)
+            v = np.concatenate([v, -v[:4]])[:31]
+            v = np.concatenate([v, np.zeros(31 - v.size, np.float32), [np.float32(peak)]]).astype(np.float32)
+            sign = np.where(rng.random(32) < 0.5, np.float32(-1), np.float32(1))
+            sign[-1] = 1
+            rows.append((v * sign * unit).astype(np.float32))
+            want_scale.append(127 + k)
+    rows.append(np.zeros(32, np.float32))                # an all-zero block: scale byte 127, every code a zero
+    want_scale.append(127)
+    t = np.stack(rows)
+    ob, os_ = codecs.mxfp4_encode(t)
+    pb, ps = mxfp4.quantize(torch.from_numpy(t))
+    assert np.array_equal(ob, pb.numpy()) and np.array_equal(os_, ps.numpy())
+    assert os_.reshape(-1).tolist() == want_scale
+    codes = np.stack([ob & 0x0F, ob >> 4], axis=-1).reshape(len(rows), 32)
+    want = np.array([[_nearest_e2m1(x, sb) for x in row] for row, sb in zip(t, want_scale)], np.uint8)
+    assert np.array_equal(codes, want)
+    # the test's own teeth: an encoder that truncates toward zero differs from the search on these very inputs
+    mags = np.array([0, 0.5, 1, 1.5, 2, 3, 4, 6], np.float64)
+    scaled = np.abs(t.astype(np.float64)) / np.exp2(np.array(want_scale, np.float64) - 127)[:, None]
+    trunc = (np.searchsorted(mags, np.minimum(scaled, 6.0), side="right") - 1).astype(np.uint8)
+    assert np.count_nonzero(trunc != (want & 7)) > 50
 
 
 # -- a damaged 12-bit store is refused before it reaches a kernel -----------------------------------------------------

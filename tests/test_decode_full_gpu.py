@@ -100,7 +100,7 @@ def test_each_full_shape_layer_alone_against_the_cpu_path(card, packed):
     """Every one of the 36 full-shape layers on its own, at the tight bar: the layer is handed the CPU path's own
     input - the residual and the pending block output as the oracle's step had them at that depth (teacher forcing) -
     runs the step's launches (add + norm + qkv, attention over the 4096-key cache, o, add + norm + gate/up + SwiGLU,
-    down) and must leave the oracle's residual and block output within 3e-2 of the largest value, with no drift from
+    down) and must leave the oracle's residual and block output within 1e-2 of the largest value (measured: 7e-3 at worst), with no drift from
     the layers before it to lean on. Both stored forms: bf16, and the same weights at 12 bits a weight."""
     cfg = QWEN3_4B
     Hq, Hk, D, H, I = cfg.q_heads, cfg.kv_heads, cfg.head_dim, cfg.hidden, cfg.intermediate
@@ -136,8 +136,8 @@ def test_each_full_shape_layer_alone_against_the_cpu_path(card, packed):
         eh = _rel(ha.float().cpu().numpy(), h_want)[0]
         ey = _rel(step.y.float().cpu().numpy(), y_want)[0]
         worst_h, worst_y = max(worst_h, eh), max(worst_y, ey)
-        assert eh <= 3e-2 and ey <= 3e-2, (i, eh, ey)
+        assert eh <= 1e-2 and ey <= 1e-2, (i, eh, ey)
         # the layer's new key and value rows are the oracle's too
         krow = step.kv[i, :, :, N0].float().cpu().numpy()
-        assert np.abs(krow - okv[i, :, :, N0]).max() <= 3e-2 * np.abs(okv[i, :, :, N0]).max(), i
+        assert np.abs(krow - okv[i, :, :, N0]).max() <= 1e-2 * np.abs(okv[i, :, :, N0]).max(), i
     print(f"teacher-forced layers ({'pack12' if packed else 'bf16'}): worst residual {worst_h:.2e}, worst block output {worst_y:.2e}")

@@ -144,7 +144,7 @@ def test_attn_decode_over_a_tree_of_rows(card, n0, T, Hq, Hk, S, seed):
 def test_attn_short_spans_kept_in_registers(card, n0, T, Hq, Hk, S, tree, win):
     """a pass of several rows whose spans are one or two batches of keys (128 / 256) takes the kernel that asks for a
     span's keys at once: against f64 attention over the keys each row sees, the bits of the general kernel at the same
-    span count (knob attn_rows_per_wg = 0), and the same bits however many rows a workgroup takes"""
+    span count"""
     D = 128
     cap = n0 + T + 3
     span = -(-(-(-cap // S)) // 128) * 128
@@ -158,20 +158,24 @@ def test_attn_short_spans_kept_in_registers(card, n0, T, Hq, Hk, S, tree, win):
     scratch = card.attn_scratch(T, Hq, Hk, D, S)
     n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
     scale = 1.0 / np.sqrt(D)
-    outs = {}
     card.set_tuning("attn_mfma", 0)  # the vector-ALU kernels: the matrix-core form has a test of its own below
     try:
-        for knob in (-1, 0, 2, 3, T):
-            card.set_tuning("attn_rows_per_wg", knob)
-            att = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
-            card.attn_decode(q.cuda(), K.cuda(), V.cuda(), att, n0t, Hq, Hk, D, scale, S, scratch, par=part, win=win)
-            outs[knob] = att.clone()
+        att = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+        card.attn_decode(q.cuda(), K.cuda(), V.cuda(), att, n0t, Hq, Hk, D, scale, S, scratch, par=part, win=win)
     finally:
-        card.set_tuning("attn_rows_per_wg", -1)
         card.set_tuning("attn_mfma", -1)
-    for knob, a in outs.items():
-        assert torch.equal(a, outs[-1]), knob
-    got = outs[-1].float().cpu().numpy()
+    # the general kernel at the same span count (what a launch by the reference's kernel name takes): the same bits
+    pm = torch.zeros(S * T * Hq, dtype=torch.float32, device="cuda")
+    pl, pa = torch.zeros_like(pm), torch.zeros(S * T * Hq * D, dtype=torch.float32, device="cuda")
+    general = torch.zeros_like(att)
+    Kc, Vc = K.cuda(), V.cuda()
+    p_ = lambda t: None if t is None else t.data_ptr()
+    assert card.lib.btb_hip_attn_decode_parts(p_(q.cuda().contiguous()), p_(Kc), p_(Vc), p_(general), p_(n0t), p_(part), T,
+                                              Hq, Hk, D, int(Kc.stride(0)), int(Kc.stride(1)), float(scale), span, S,
+                                              int(win), None, p_(pm), p_(pl), p_(pa), None) == 0
+    torch.cuda.synchronize()
+    assert torch.equal(att, general)
+    got = att.float().cpu().numpy()
     for t in range(T):
         if par is None:
             slots = list(range(n0 + t + 1))            # slot = position in a chain
