@@ -32,6 +32,9 @@ SPEC: dict[str, tuple[str, str]] = {
     "btb_attn_flash": ("D", "q:Query:p K:KCache:p V:VCache:p out:AttnOut:p n0p:PrefixLen:p par:TreeParents:p T:Rows:i "
                             "Hq:QHeads:i Hk:KvHeads:i hs:CacheHeadStride:i rs:CacheRowStride:i scale:AttnScale:f "
                             "part_m:PartMax:p part_l:PartSum:p part_acc:PartAcc:p cnt:Arrivals:p win:Window:i tbl:RowMap:p"),
+    "btb_attn_flash_rows": ("D", "q:Query:p K:KCache:p V:VCache:p out:AttnOut:p rw:RowsLayout:p T:Rows:i Hq:QHeads:i "
+                                 "Hk:KvHeads:i hs:CacheHeadStride:i rs:CacheRowStride:i scale:AttnScale:f part_m:PartMax:p "
+                                 "part_l:PartSum:p part_acc:PartAcc:p cnt:Arrivals:p win:Window:i"),
     "btb_gemv_bf16": ("M", "w:Weight:p x:MatIn:p y:MatOut:p R:OutDim:i C:InDim:i"),
     "btb_gemv_silu_bf16": ("M", "w:Weight:p gu:GateUp:p y:MatOut:p R:OutDim:i C:InDim:i"),
     "btb_gemv_lane16_f32": ("M", "w:Weight:p x:MatInF32:p y:MatOutF32:p R:OutDim:i C:InDim:i"),
@@ -47,6 +50,9 @@ SPEC: dict[str, tuple[str, str]] = {
     "btb_norm_rope_kv": ("D", "qkv:Qkv:p wq:QNorm:p wk:KNorm:p eps:NormEps:f cos_t:RopeCos:p sin_t:RopeSin:p "
                               "n0p:PrefixLen:p depth:Depths:p K:KCache:p V:VCache:p qo:Query:p T:Rows:i Hq:QHeads:i "
                               "Hk:KvHeads:i hs:CacheHeadStride:i rs:CacheRowStride:i centered:NormCentered:i"),
+    "btb_norm_rope_kv_rows": ("D", "qkv:Qkv:p wq:QNorm:p wk:KNorm:p eps:NormEps:f cos_t:RopeCos:p sin_t:RopeSin:p "
+                                   "rw:RowsLayout:p K:KCache:p V:VCache:p qo:Query:p T:Rows:i Hq:QHeads:i Hk:KvHeads:i "
+                                   "hs:CacheHeadStride:i rs:CacheRowStride:i centered:NormCentered:i"),
     "btb_norm_rope_kv_tbl": ("D", "qkv:Qkv:p wq:QNorm:p wk:KNorm:p eps:NormEps:f cos_t:RopeCos:p sin_t:RopeSin:p "
                                   "n0p:PrefixLen:p depth:Depths:p K:KCache:p V:VCache:p qo:Query:p T:Rows:i Hq:QHeads:i "
                                   "Hk:KvHeads:i hs:CacheHeadStride:i rs:CacheRowStride:i centered:NormCentered:i "
@@ -73,7 +79,7 @@ def kernel_names(family: str) -> tuple[str, ...]:
 # every kernel name this path serves, a family's at each of its instantiations (the reference's `KERNELS`, :207-425,
 # less the kernels of other paths; the attention is built for head_dim 128 only)
 KERNELS: tuple[str, ...] = tuple(n for fam in SPEC for n in kernel_names(fam)
-                                 if not (fam == "btb_attn_flash" and n != "btb_attn_flash_d128"))
+                                 if not (fam.startswith("btb_attn_flash") and not n.endswith("_d128")))
 
 # the roles: what a parameter is, as a type of its own over int (the reference's btb/kinds.py, from
 # native/cuda/btb_roles.cuh) - `ptr(Query, q)` is q's card address typed as the attention's query rows

@@ -65,20 +65,37 @@ __device__ __forceinline__ void head_norm_rope(const uint16_t* src, const uint16
     head_finish(in, wn != nullptr, eps, centered, lane, out);
 }
 
+// A pass whose T rows are T sequences of their own, a token each (a fork's rows, which share one prefix, or a batch's,
+// which lie end to end) - the reference's rows layout (native/cuda/btb_kernels.cu:232-249): one int32 array on the
+// device, [base, steps, W, then (col, off, len) a row]. Row t's keys in logical order are its prefix - len cache
+// slots from off - and then its own steps, step i at slot base + i * W + col; it stands at position len + steps.
+// len < 0: a padding row, for which nothing is computed.
+struct SeqPlace {
+    int base, step, W, col, off, len;
+    __device__ __forceinline__ void read(const int32_t* rw, int t) {
+        base = rw[0], step = rw[1], W = rw[2];
+        col = rw[3 + 3 * t], off = rw[4 + 3 * t], len = rw[5 + 3 * t];
+    }
+    __device__ __forceinline__ int slot(int j) const { return j < len ? off + j : base + (j - len) * W + col; }
+};
+
 // one batch of a key stream: eight keys sixteen apart, their K and V rows (this lane's 8 dims) requested together
 constexpr int KB = 8;
 struct KeyBatch {
     uint4 k[KB], v[KB];
 };
 __device__ __forceinline__ void load_keys(KeyBatch& kb, const uint16_t* Kh, const uint16_t* Vh, long long rs, int key0,
-                                          int k_end, int n0, const int32_t* tbl = nullptr) {
+                                          int k_end, int n0, const int32_t* tbl = nullptr,
+                                          const SeqPlace* seq = nullptr) {
 #pragma unroll
     for (int b = 0; b < KB; ++b) {
         const int key = min(key0 + 16 * b, k_end - 1);  // a key past the span's end is loaded again, not used
         // slot n0 is this step's own row: it is taken from LDS, the cache's copy may not have landed yet
         int safe = key == n0 ? max(n0 - 1, 0) : key;
-        // the cache's row map (the reference's `tbl`, native/cuda/btb_attn_flash.cuh:34): logical slot -> cache row
+        // the cache's row map (the reference's `tbl`, native/cuda/btb_attn_flash.cuh:34): logical slot -> cache row;
+        // or the row's own sequence: logical key -> cache slot
         if (tbl != nullptr) safe = tbl[safe];
+        if (seq != nullptr) safe = seq->slot(safe);
         kb.k[b] = *reinterpret_cast<const uint4*>(Kh + (size_t)safe * rs);
         kb.v[b] = *reinterpret_cast<const uint4*>(Vh + (size_t)safe * rs);
     }

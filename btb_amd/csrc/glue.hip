@@ -158,13 +158,23 @@ __global__ void __launch_bounds__(64) norm_rope_kv_kernel(const uint16_t* __rest
                                                           const int32_t* __restrict__ depth, uint16_t* __restrict__ K,
                                                           uint16_t* __restrict__ V, uint16_t* __restrict__ qo, int Hq,
                                                           int Hk, long long hs, long long rs, int centered,
-                                                          const int32_t* __restrict__ tbl) {
+                                                          const int32_t* __restrict__ tbl,
+                                                          const int32_t* __restrict__ rw) {
     constexpr int E = D / 64;
     const int head = blockIdx.x, t = blockIdx.y, lane = threadIdx.x;
-    const int n0 = *n0p;
-    int slot = n0 + t;
+    int slot, pos;
+    if (rw != nullptr) {  // row t is a sequence of its own: it stands past its prefix and steps, at its step's slot
+        SeqPlace sq;
+        sq.read(rw, t);
+        if (sq.len < 0) return;
+        pos = sq.len + sq.step;
+        slot = sq.slot(pos);
+    } else {
+        const int n0 = *n0p;
+        slot = n0 + t;
+        pos = n0 + (depth != nullptr ? depth[t] : t);
+    }
     if (tbl != nullptr) slot = tbl[slot];  // the cache's row map: the row lands where the attention's walk reads it
-    const int pos = n0 + (depth != nullptr ? depth[t] : t);
     const int width = (Hq + 2 * Hk) * D;
     const uint16_t* src = qkv + (size_t)t * width + (size_t)head * D + lane * E;
     if (head >= Hq + Hk) {
@@ -235,7 +245,8 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
                                                           const int32_t* __restrict__ par, int T, int Hq, int Hk, long long hs,
                                                           long long rs, float scale_log2, float* __restrict__ part_m,
                                                           float* __restrict__ part_l, float* __restrict__ part_acc,
-                                                          int span, int win, const int32_t* __restrict__ tbl) {
+                                                          int span, int win, const int32_t* __restrict__ tbl,
+                                                          const int32_t* __restrict__ rw) {
     constexpr int D = ATT_D;
     __shared__ float s_m[16][G], s_l[16][G];
     __shared__ __align__(16) float s_acc[16][G][D];
@@ -244,8 +255,22 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int sub = lane >> 4, dl = lane & 15;   // the lane's key within a quad of keys, its 8 dims
     const int grp = wv * 4 + sub;                // one of the workgroup's 16 key streams
-    const int n0 = *n0p;
-    const RowView rv = row_view(par, t, T, n0, win);
+    SeqPlace sq;
+    const SeqPlace* seq = nullptr;
+    RowView rv;
+    if (rw != nullptr) {
+        // row t is a sequence of its own: its keys, in logical order, are its prefix and its own steps up to this one
+        sq.read(rw, t);
+        if (sq.len < 0) return;  // a padding row: no state is left, and the merge leaves its output alone
+        seq = &sq;
+        const int last = sq.len + sq.step;
+        rv.n = last + 1;
+        rv.tree_base = -1;
+        rv.tree_mask = 0u;
+        rv.k_first = win > 0 ? max(last + 1 - win, 0) : 0;
+    } else {
+        rv = row_view(par, t, T, *n0p, win);
+    }
     const int tree_base = rv.tree_base, n = rv.n, k_first = rv.k_first;
     const uint32_t tree_mask = rv.tree_mask;
     const int k_begin = sp * span, k_end = min(n, k_begin + span);
@@ -268,10 +293,10 @@ __global__ void __launch_bounds__(256) attn_decode_kernel(const uint16_t* __rest
     // is folded in (past the span's end they fall on its last key again, unused), so a span of several batches - a
     // pass of many rows takes long spans - pays the trip to memory once
     KeyBatch kb;
-    load_keys(kb, Kh, Vh, rs, k_begin + grp, max(k_end, 1), -1, tbl);
+    load_keys(kb, Kh, Vh, rs, k_begin + grp, max(k_end, 1), -1, tbl, seq);
     for (int key0 = k_begin + grp; key0 < k_end; key0 += 16 * KB) {
         KeyBatch nx;
-        load_keys(nx, Kh, Vh, rs, key0 + 16 * KB, k_end, -1, tbl);
+        load_keys(nx, Kh, Vh, rs, key0 + 16 * KB, k_end, -1, tbl, seq);
         use_keys<G>(kb, key0, k_end, -1, nullptr, nullptr, dl, qp, scale_log2, st, &s_x[grp][0], tree_base, tree_mask,
                     k_first);
         kb = nx;
@@ -455,9 +480,11 @@ template <int G>
 __global__ void __launch_bounds__(256) attn_merge_kernel(uint16_t* __restrict__ att, int Hq, int Hk, int S,
                                                          const float* __restrict__ part_m,
                                                          const float* __restrict__ part_l,
-                                                         const float* __restrict__ part_acc) {
+                                                         const float* __restrict__ part_acc,
+                                                         const int32_t* __restrict__ rw) {
     extern __shared__ float f_m[];  // [S][G] maxima / factors, then [S][G] sums
     const int g = blockIdx.x, t = blockIdx.y;
+    if (rw != nullptr && rw[5 + 3 * t] < 0) return;  // a padding row of a pass of sequences: its output is left alone
     merge_spans<G, false>(att + (size_t)t * Hq * ATT_D, g, S, ((size_t)t * Hk + g) * S, part_m, part_l, part_acc, f_m,
                           threadIdx.x);
 }
@@ -608,12 +635,12 @@ int32_t btb_hip_add_rmsnorm(void* h, const void* y, const void* w, float eps, vo
 static int32_t norm_rope_kv_any(const void* qkv, const void* wq, const void* wk, float eps, const void* cos_t,
                                 const void* sin_t, const int32_t* n0, const int32_t* depth, void* K, void* V, void* q,
                                 size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered,
-                                const int32_t* tbl, void* stream) {
-    if (qkv == nullptr || cos_t == nullptr || sin_t == nullptr || n0 == nullptr || K == nullptr || V == nullptr ||
-        q == nullptr)
+                                const int32_t* tbl, void* stream, const int32_t* rw = nullptr) {
+    if (qkv == nullptr || cos_t == nullptr || sin_t == nullptr || (n0 == nullptr && rw == nullptr) || K == nullptr ||
+        V == nullptr || q == nullptr)
         return ERR_NULL;
     if (T == 0 || Hq == 0 || Hk == 0 || T > 65535 || Hq + 2 * Hk > 0x7FFFFFFFull || hs <= 0 || rs <= 0 ||
-        !(eps >= 0.f) || !al(tbl, 4))
+        !(eps >= 0.f) || !al(tbl, 4) || !al(rw, 4))
         return ERR_DOMAIN;
     if (D != 64 && D != 128 && D != 256) return ERR_DOMAIN;
     const dim3 grid((unsigned)(Hq + 2 * Hk), (unsigned)T);
@@ -623,7 +650,7 @@ static int32_t norm_rope_kv_any(const void* qkv, const void* wq, const void* wk,
                        static_cast<const uint16_t*>(wq), static_cast<const uint16_t*>(wk), eps,                      \
                        static_cast<const uint16_t*>(cos_t), static_cast<const uint16_t*>(sin_t), n0, depth,          \
                        static_cast<uint16_t*>(K), static_cast<uint16_t*>(V), static_cast<uint16_t*>(q), (int)Hq,      \
-                       (int)Hk, (long long)hs, (long long)rs, centered, tbl)
+                       (int)Hk, (long long)hs, (long long)rs, centered, tbl, rw)
     if (D == 64)
         NRK(64);
     else if (D == 128)
@@ -651,6 +678,14 @@ int32_t btb_hip_norm_rope_kv_tbl(const void* qkv, const void* wq, const void* wk
                             stream);
 }
 
+int32_t btb_hip_norm_rope_kv_seqs(const void* qkv, const void* wq, const void* wk, float eps, const void* cos_t,
+                                  const void* sin_t, const int32_t* rw, void* K, void* V, void* q, size_t T, size_t Hq,
+                                  size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered, void* stream) {
+    if (rw == nullptr) return ERR_NULL;
+    return norm_rope_kv_any(qkv, wq, wk, eps, cos_t, sin_t, nullptr, nullptr, K, V, q, T, Hq, Hk, D, hs, rs, centered,
+                            nullptr, stream, rw);
+}
+
 size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, size_t S) {
     // part_m and part_l [T, Hk, S, G], part_acc [T, Hk, S, G, D]: Hk * G = Hq
     (void)Hk;
@@ -664,10 +699,12 @@ size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, siz
 static int32_t attn_decode_any(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
                                const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs,
                                float scale, size_t cap, size_t S, float* work, bool own_scratch, void* stream,
-                               int64_t win = 0, const int32_t* tbl = nullptr, float* const* parts = nullptr) {
-    if (q == nullptr || K == nullptr || V == nullptr || att == nullptr || n0 == nullptr ||
+                               int64_t win = 0, const int32_t* tbl = nullptr, float* const* parts = nullptr,
+                               const int32_t* rw = nullptr) {
+    if (q == nullptr || K == nullptr || V == nullptr || att == nullptr || (n0 == nullptr && rw == nullptr) ||
         (!own_scratch && work == nullptr && parts == nullptr))
         return ERR_NULL;
+    if (rw != nullptr && (parts == nullptr || par != nullptr || tbl != nullptr || !al(rw, 4))) return ERR_DOMAIN;
     if (parts != nullptr && (parts[0] == nullptr || parts[1] == nullptr || parts[2] == nullptr)) return ERR_NULL;
     if (T == 0 || Hq == 0 || Hk == 0 || S == 0 || cap == 0 || T > 65535 || S > 1024 || Hq % Hk != 0 || hs <= 0 ||
         rs <= 0 || !(scale == scale))
@@ -713,9 +750,9 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
     hipLaunchKernelGGL(attn_decode_kernel<GG>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(q),              \
                        static_cast<const uint16_t*>(K), static_cast<const uint16_t*>(V), n0, par, (int)T, (int)Hq,   \
                        (int)Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, span, (int)win,   \
-                       tbl);                                                                                         \
+                       tbl, rw);                                                                                    \
     hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,       \
-                       (int)Hk, (int)S, part_m, part_l, part_acc)
+                       (int)Hk, (int)S, part_m, part_l, part_acc, rw)
     // Several rows and spans of 128 keys: the matrix cores, every row of the pass that shares a kv head in one workgroup
     // (attn_mfma.hip). A pass of 8 rows over 4096 keys: 22.7 us a layer on the vector kernel below (spans of one or two
     // batches of keys, asked for at once and kept in registers, a workgroup a row), which stays for spans of 256 keys
@@ -726,10 +763,10 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
         if (rc != OK) return rc;
         if (G == 4)
             hipLaunchKernelGGL(attn_merge_kernel<4>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
-                               (int)Hk, (int)S, part_m, part_l, part_acc);
+                               (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr));
         else
             hipLaunchKernelGGL(attn_merge_kernel<2>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
-                               (int)Hk, (int)S, part_m, part_l, part_acc);
+                               (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr));
         return hip_status(hipGetLastError(), "attn_decode launch");
     }
     if (parts == nullptr && T >= 2 && (span == 128 || span == 256) && (G == 2 || G == 4)) {
@@ -739,7 +776,7 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
                        static_cast<const uint16_t*>(K), static_cast<const uint16_t*>(V), n0, par, (int)T, (int)Hq,    \
                        (int)Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, (int)win, tbl);      \
     hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,        \
-                       (int)Hk, (int)S, part_m, part_l, part_acc)
+                       (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr))
         if (G == 4 && span == 128) { ATTR(4, 1); }
         else if (G == 4) { ATTR(4, 2); }
         else if (span == 128) { ATTR(2, 1); }
@@ -785,6 +822,19 @@ int32_t btb_hip_attn_decode_parts(const void* q, const void* K, const void* V, v
     float* const parts[3] = {part_m, part_l, part_acc};
     return attn_decode_any(q, K, V, att, n0, par, T, Hq, Hk, D, hs, rs, scale, span * S, S, nullptr, false, stream, win,
                            tbl, parts);
+}
+
+int32_t btb_hip_attn_decode_seqs(const void* q, const void* K, const void* V, void* att, const int32_t* rw, size_t T,
+                                 size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t span,
+                                 size_t S, int64_t win, float* part_m, float* part_l, float* part_acc, void* stream) {
+    if (rw == nullptr) return ERR_NULL;
+    if (span == 0 || span % 128 != 0 || S == 0 || span > 0x7FFFFFFFull / (S ? S : 1)) {
+        set_error("attn_decode_seqs: spans are a whole number of 128-key batches");
+        return ERR_DOMAIN;
+    }
+    float* const parts[3] = {part_m, part_l, part_acc};
+    return attn_decode_any(q, K, V, att, nullptr, nullptr, T, Hq, Hk, D, hs, rs, scale, span * S, S, nullptr, false,
+                           stream, win, nullptr, parts, rw);
 }
 
 int32_t btb_hip_attn_decode_noalloc(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
@@ -838,7 +888,7 @@ int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk,
                        (long long)rs, scale_log2, part_m, part_l, part_acc, span, (int)cap)
 #define MERGE(GG)                                                                                                    \
     hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,       \
-                       (int)Hk, (int)S, part_m, part_l, part_acc)
+                       (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr))
     if (G != 1 && G != 2 && G != 4 && G != 8) {
         set_error("attn_decode_qkv: 1, 2, 4 or 8 query heads per kv head");
         return ERR_DOMAIN;
@@ -907,10 +957,10 @@ int32_t btb_hip_attn_decode_qkv_rows(const void* qkv, const void* wq, const void
     const size_t mlds = 2 * S * G * sizeof(float);
     if (G == 4)
         hipLaunchKernelGGL(attn_merge_kernel<4>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
-                           (int)Hk, (int)S, part_m, part_l, part_acc);
+                           (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr));
     else
         hipLaunchKernelGGL(attn_merge_kernel<2>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
-                           (int)Hk, (int)S, part_m, part_l, part_acc);
+                           (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr));
     return hip_status(hipGetLastError(), "attn_decode_qkv_rows launch");
 }
 

@@ -71,6 +71,8 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_add_rmsnorm": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _sz, _sz, _i32, _vp]),
     "btb_hip_norm_rope_kv": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
                                     _sz, ctypes.c_int64, ctypes.c_int64, _i32, _vp]),
+    "btb_hip_norm_rope_kv_seqs": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz,
+                                         ctypes.c_int64, ctypes.c_int64, _i32, _vp]),
     "btb_hip_norm_rope_kv_tbl": (_i32, [_vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
                                         _sz, ctypes.c_int64, ctypes.c_int64, _i32, _vp, _vp]),
     "btb_hip_attn_decode_win": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
@@ -81,6 +83,8 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
                                    ctypes.c_float, _sz, _sz, _vp, _vp]),
     "btb_hip_attn_decode_parts": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
                                          ctypes.c_float, _sz, _sz, ctypes.c_int64, _vp, _vp, _vp, _vp, _vp]),
+    "btb_hip_attn_decode_seqs": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64, ctypes.c_int64,
+                                        ctypes.c_float, _sz, _sz, ctypes.c_int64, _vp, _vp, _vp, _vp]),
     "btb_hip_attn_decode_noalloc": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _sz, ctypes.c_int64,
                                            ctypes.c_int64, ctypes.c_float, _sz, _sz, _vp]),
     "btb_hip_attn_decode_qkv": (_i32, [_vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp, _vp, _vp, _vp, _vp, _sz, _sz, _sz,
@@ -156,6 +160,15 @@ def _launch_table() -> dict[str, tuple[int, Any]]:
     t["btb_attn_flash_d128"] = (18, lambda v, g, card: ("btb_hip_attn_decode_parts", (
         v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], 128, v[9], v[10], v[11], 512, max(int(g[1]), 1), v[16],
         v[17], v[12], v[13], v[14])))
+    # the same pair for a pass whose rows are sequences of their own (`rw`, the rows layout):
+    # btb_norm_rope_kv_rows_d{D}(qkv, wq, wk, eps, cos, sin, rw, K, V, q, T, Hq, Hk, hs, rs, centered) and
+    # btb_attn_flash_rows_d128(q, K, V, out, rw, T, Hq, Hk, hs, rs, scale, part_m, part_l, part_acc, cnt, win)
+    for D in (64, 128, 256):
+        t[f"btb_norm_rope_kv_rows_d{D}"] = (16, lambda v, g, card, D=D: ("btb_hip_norm_rope_kv_seqs", (
+            v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], v[8], v[9], v[10], v[11], v[12], D, v[13], v[14], v[15])))
+    t["btb_attn_flash_rows_d128"] = (16, lambda v, g, card: ("btb_hip_attn_decode_seqs", (
+        v[0], v[1], v[2], v[3], v[4], v[5], v[6], v[7], 128, v[8], v[9], v[10], 512, max(int(g[1]), 1), v[15], v[11],
+        v[12], v[13])))
     # btb_publish(n0, ids, out_tok, out_n0, out_ts)
     t["btb_publish"] = (5, lambda v, g, card: ("btb_hip_publish_only", (v[0], v[1], v[2], v[3], v[4])))
     # btb_mx4_widen(blocks, scales, seats, groups, out), grid.y seats
@@ -707,6 +720,58 @@ class HipCard(CardLaunch):
         else:
             self._need(tbl, torch.int32, "tbl")
             self._call("btb_hip_norm_rope_kv_tbl", *args, _p(tbl), _stream())
+
+    @staticmethod
+    def rows_layout(base: int, steps: int, W: int, rows: Sequence[tuple[int, int, int]], pad_to: int = 0,
+                    device: Any = "cuda") -> torch.Tensor:
+        """The layout of a pass whose rows are sequences of their own (the reference fills the same array before a
+        rows step, btb/engine/cuda.py:3457-3464): int32 [base, steps, W, then (col, off, len) a row] - row t's prefix is
+        `len` cache slots from `off`, its own step i lies at slot base + i * W + col. Rows past `rows` up to `pad_to`
+        are padding (len -1), which the kernels skip."""
+        lay = [int(base), int(steps), int(W)]
+        for col, off, n in rows:
+            lay += [int(col), int(off), int(n)]
+        lay += [0, 0, -1] * max(0, int(pad_to) - len(rows))
+        return torch.tensor(lay, dtype=torch.int32, device=device)
+
+    def norm_rope_kv_seqs(self, qkv: torch.Tensor, wq: torch.Tensor | None, wk: torch.Tensor | None, eps: float,
+                          cos: torch.Tensor, sin: torch.Tensor, rw: torch.Tensor, K: torch.Tensor, V: torch.Tensor,
+                          q: torch.Tensor, Hq: int, Hk: int, D: int, centered: bool = False) -> None:
+        """`norm_rope_kv` for a pass whose rows are sequences of their own, laid out by `rw` (`rows_layout`): row t is
+        roped at its own position len + steps and written to its step's slot (`btb_norm_rope_kv_rows_d{D}`)"""
+        for t, what in ((qkv, "qkv"), (cos, "cos"), (sin, "sin"), (q, "q")):
+            self._need(t, torch.bfloat16, what)
+        self._need(rw, torch.int32, "rw")
+        if K.dtype != torch.bfloat16 or V.dtype != torch.bfloat16 or K.stride(2) != 1 or K.stride() != V.stride():
+            raise ValueError("[hip] norm_rope_kv_seqs: K and V are bf16 [Hk, cap, D] views with the same strides")
+        T = int(qkv.numel()) // ((Hq + 2 * Hk) * D)
+        if rw.numel() < 3 + 3 * T:
+            raise ValueError(f"[hip] norm_rope_kv_seqs: the layout holds {rw.numel()} words, {T} rows take {3 + 3 * T}")
+        self._call("btb_hip_norm_rope_kv_seqs", _p(qkv), None if wq is None else _p(wq), None if wk is None else _p(wk),
+                   float(eps), _p(cos), _p(sin), _p(rw), _p(K), _p(V), _p(q), T, Hq, Hk, D, int(K.stride(0)),
+                   int(K.stride(1)), int(bool(centered)), _stream())
+
+    def attn_decode_seqs(self, q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, att: torch.Tensor, rw: torch.Tensor,
+                         Hq: int, Hk: int, D: int, scale: float, span: int, S: int, part_m: torch.Tensor,
+                         part_l: torch.Tensor, part_acc: torch.Tensor, win: int = 0) -> None:
+        """decode attention for a pass whose rows are sequences of their own (`rw`): row t over its own prefix and
+        steps, in S spans of `span` keys; the spans' states go into the caller's three arrays
+        (`btb_attn_flash_rows_d128`)"""
+        for t, what in ((q, "q"), (att, "att")):
+            self._need(t, torch.bfloat16, what)
+        self._need(rw, torch.int32, "rw")
+        for t, what in ((part_m, "part_m"), (part_l, "part_l"), (part_acc, "part_acc")):
+            self._need(t, torch.float32, what)
+        if K.dtype != torch.bfloat16 or V.dtype != torch.bfloat16 or K.stride(2) != 1 or K.stride() != V.stride():
+            raise ValueError("[hip] attn_decode_seqs: K and V are bf16 [Hk, cap, D] views with the same strides")
+        T = int(q.numel()) // (Hq * D)
+        if q.numel() != T * Hq * D or att.numel() != T * Hq * D or rw.numel() < 3 + 3 * T:
+            raise ValueError("[hip] attn_decode_seqs: q and att are [T, Hq D], the layout holds 3 + 3 T words")
+        if part_m.numel() < T * Hq * S or part_l.numel() < T * Hq * S or part_acc.numel() < T * Hq * S * D:
+            raise ValueError(f"[hip] attn_decode_seqs: part_m / part_l hold T Hq S = {T * Hq * S} floats, part_acc D times that")
+        self._call("btb_hip_attn_decode_seqs", _p(q), _p(K), _p(V), _p(att), _p(rw), T, Hq, Hk, D, int(K.stride(0)),
+                   int(K.stride(1)), float(scale), int(span), int(S), int(win), _p(part_m), _p(part_l), _p(part_acc),
+                   _stream())
 
     def attn_scratch(self, T: int, Hq: int, Hk: int, D: int, S: int, device: Any = "cuda") -> torch.Tensor:
         """the f32 scratch `attn_decode` leaves its spans' states in, at these sizes"""

@@ -292,6 +292,17 @@ int32_t btb_hip_norm_rope_kv_tbl(const void* qkv, const void* wq, const void* wk
                                  size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered,
                                  const int32_t* tbl, void* stream);
 
+/* The same for a pass whose T rows are T sequences of their own, a token each - a fork's rows, which share one
+ * prefix, or a batch's, whose prefixes lie end to end in the cache. rw is the reference's rows layout, int32 on the
+ * device: [base, steps, W, then (col, off, len) a row]. Row t's keys in logical order are its prefix (len cache slots
+ * from off) and then its own steps, step i at slot base + i * W + col; the row stands at position len + steps and is
+ * written to that step's slot. A row with len < 0 is padding: nothing is read or written for it. The layout is
+ * trusted as the reference's kernel trusts it: every slot it names must lie inside the cache. Replaces
+ * btb_norm_rope_kv_rows_d{D} (native/cuda/btb_kernels.cu:232-249, 339-346). */
+int32_t btb_hip_norm_rope_kv_seqs(const void* qkv, const void* wq, const void* wk, float eps, const void* cos_t,
+                                  const void* sin_t, const int32_t* rw, void* K, void* V, void* q, size_t T, size_t Hq,
+                                  size_t Hk, size_t D, int64_t hs, int64_t rs, int32_t centered, void* stream);
+
 /* floats of scratch btb_hip_attn_decode needs for T rows and S key spans */
 size_t btb_hip_attn_scratch_floats(size_t T, size_t Hq, size_t Hk, size_t D, size_t S);
 
@@ -339,6 +350,17 @@ int32_t btb_hip_attn_decode_parts(const void* q, const void* K, const void* V, v
  * looked up once, by btb_hip_init or by the first call there. Every call on a GPU shares that GPU's array: calls that
  * overlap on one GPU (two streams, two threads) race on it - serialise them or use btb_hip_attn_decode. Nothing in
  * the array needs clearing between calls: every state a call reads, it has written first. */
+/* Decode attention for a pass of T sequences a token each (rw: the rows layout of btb_hip_norm_rope_kv_seqs). Row t
+ * attends to its own sequence's len + steps + 1 keys, walked in logical order in S spans of `span` keys (a multiple
+ * of 128), under a window of `win` keys when win > 0: the partition, the arithmetic and so the bits are those of
+ * btb_hip_attn_decode_parts at T = 1 over a cache that holds that sequence alone, whatever rows step beside it. The
+ * spans' states go into the caller's part_m, part_l (T Hq S floats each) and part_acc (T Hq S D floats); a padding
+ * row's output is left as it was. head_dim 128. Replaces btb_attn_flash_rows_d128
+ * (native/cuda/btb_attn_flash.cuh:395-404, 663-672; btb/engine/cuda.py:1752-1756). */
+int32_t btb_hip_attn_decode_seqs(const void* q, const void* K, const void* V, void* att, const int32_t* rw, size_t T,
+                                 size_t Hq, size_t Hk, size_t D, int64_t hs, int64_t rs, float scale, size_t span,
+                                 size_t S, int64_t win, float* part_m, float* part_l, float* part_acc, void* stream);
+
 #define BTB_HIP_ATTN_NOALLOC_FLOATS ((size_t)1 << 20)
 int32_t btb_hip_attn_decode_noalloc(const void* q, const void* K, const void* V, void* att, const int32_t* n0,
                                     const int32_t* par, size_t T, size_t Hq, size_t Hk, size_t D, int64_t hs,

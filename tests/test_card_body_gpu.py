@@ -64,8 +64,9 @@ def buffers(cfg, T: int, mma: bool, tail: bool = True) -> dict:
     }
 
 
-def card_body(k, cfg, W, g, arena, tables, row_map=None, fused=False):
-    """one pass over `g`'s buffers: every layer and the tail, each kernel by its reference name"""
+def card_body(k, cfg, W, g, arena, tables, row_map=None, fused=False, rows=None):
+    """one pass over `g`'s buffers: every layer and the tail, each kernel by its reference name. `rows`: the pass's
+    rows are sequences of their own, laid out by that int32 array (the reference's `rows` mode, cuda.py:1736-1756)"""
     T, M, mma = g["T"], g["M"], g["mma"]
     H, Hq, Hk, D, I = cfg.hidden, cfg.q_heads, cfg.kv_heads, cfg.head_dim, cfg.intermediate
     G, S = Hq // Hk, g["S"]
@@ -76,6 +77,7 @@ def card_body(k, cfg, W, g, arena, tables, row_map=None, fused=False):
     part_acc, cnt = k.ptr(cl.PartAcc, g["part_acc"]), k.ptr(cl.Arrivals, g["cnt"])
     q, att = k.ptr(cl.Query, g["q"]), k.ptr(cl.AttnOut, g["att"])
     tbl = k.ptr(cl.RowMap, row_map)
+    layout = k.ptr(cl.RowsLayout, rows)
     t_rows, q_heads, kv_heads = cl.Rows(T), cl.QHeads(Hq), cl.KvHeads(Hk)
     cen = cl.NormCentered(0)
     h, x, hidden, row = k.ptr(cl.Residual, g["h"]), k.ptr(cl.Normed, g["x"]), cl.Hidden(H), (T, 1, 1)
@@ -103,14 +105,21 @@ def card_body(k, cfg, W, g, arena, tables, row_map=None, fused=False):
         matvec(W[L + "qkv"].w, g["x"], g["qkv"], (Hq + 2 * Hk) * D, H)
         qkv, wq, wk = k.ptr(cl.Qkv, g["qkv"]), k.ptr(cl.QNorm, W[L + "wq"]), k.ptr(cl.KNorm, W[L + "wk"])
         nrk_grid = (Hq + 2 * Hk, T, 1)
-        if paged:
+        if rows is not None:
+            k.btb_norm_rope_kv_rows(D, nrk_grid, (32, 1, 1), qkv, wq, wk, eps, cos, sin, layout, K, V, q, t_rows,
+                                    q_heads, kv_heads, hs, rs, cen)
+        elif paged:
             k.btb_norm_rope_kv_tbl(D, nrk_grid, (32, 1, 1), qkv, wq, wk, eps, cos, sin, n0p, depth, K, V, q, t_rows,
                                    q_heads, kv_heads, hs, rs, cen, tbl)
         else:
             k.btb_norm_rope_kv(D, nrk_grid, (32, 1, 1), qkv, wq, wk, eps, cos, sin, n0p, depth, K, V, q, t_rows,
                                q_heads, kv_heads, hs, rs, cen)
-        k.btb_attn_flash(D, attn_grid, attn_block, q, K, V, att, n0p, par, t_rows, q_heads, kv_heads, hs, rs, scale,
-                         part_m, part_l, part_acc, cnt, win, tbl)
+        if rows is not None:
+            k.btb_attn_flash_rows(D, (T * ((G + 7) // 8), S, Hk), attn_block, q, K, V, att, layout, t_rows, q_heads,
+                                  kv_heads, hs, rs, scale, part_m, part_l, part_acc, cnt, win)
+        else:
+            k.btb_attn_flash(D, attn_grid, attn_block, q, K, V, att, n0p, par, t_rows, q_heads, kv_heads, hs, rs,
+                             scale, part_m, part_l, part_acc, cnt, win, tbl)
         matvec(W[L + "o"].w, g["att"], g["y"], H, Hq * D)
         k.btb_add_rmsnorm(row, (256, 1, 1), h, k.ptr(cl.BlockOut, g["y"]), k.ptr(cl.NormWeight, W[L + "ln2"]), eps, x,
                           hidden, cen)
@@ -139,9 +148,9 @@ class Pass:
     """a pass graph as the reference keeps it: buffers made once, the body run eagerly as a warm-up, then captured; a
     pass = the inputs written into the static buffers, then a replay"""
 
-    def __init__(self, k, cfg, W, arena, tables, T, mma, row_map=None, fused=False, capture=True):
+    def __init__(self, k, cfg, W, arena, tables, T, mma, row_map=None, fused=False, capture=True, rows=None):
         self.k, self.cfg, self.W, self.g = k, cfg, W, buffers(cfg, T, mma)
-        self.run = lambda: card_body(k, cfg, W, self.g, arena, tables, row_map, fused)
+        self.run = lambda: card_body(k, cfg, W, self.g, arena, tables, row_map, fused, rows)
         self.graph = None
         if capture:
             side = torch.cuda.Stream()
@@ -261,6 +270,45 @@ def test_the_verify_pass_by_kernel_names_reproduces_the_receipts(card, tiny, rec
     for i in range(cfg.layers):
         assert worst(at(arena[i, 0])[:, :rows].float().cpu().numpy(), r["keys"][i][0][0]) <= 2e-2, i
         assert worst(at(arena[i, 1])[:, :rows].float().cpu().numpy(), r["keys"][i][1][0]) <= 2e-2, i
+
+
+def test_a_pass_of_forked_rows_by_kernel_names(card, tiny, receipts):
+    """the reference's rows mode: four forks of the prompt, a token each, stepped twice as one captured pass of four
+    rows (`btb_norm_rope_kv_rows`, `btb_attn_flash_rows`; the layout array rewritten between the replays, as the
+    reference rewrites it, cuda.py:3457-3464; a fifth, padding row behind them). Every fork's logits are the bits of
+    that sequence stepped alone through the one-row graph over a cache of its own, and the fork that follows the
+    receipts' greedy path picks the receipts' tokens"""
+    cfg, W = tiny
+    r = receipts["bf16"]
+    tables = rope_tables(cfg, CAP, "cuda")
+    n, B, T, base, Wd = len(PROMPT), 4, 5, 512, 4
+    forks = [[r["greedy"][0], r["greedy"][1]], [9, 33], [r["greedy"][0], 71], [200, 200]]
+    # each fork alone: the prompt, then its two tokens, through the one-row step
+    alone = []
+    A1, arena1 = new_arena(cfg)
+    step = Pass(card, cfg, W, arena1, tables, T=1, mma=False)
+    for toks in forks:
+        A1.zero_()
+        for n0, tok in enumerate(PROMPT):
+            step([tok], n0)
+        alone.append([step([tok], n + d)[0].copy() for d, tok in enumerate(toks)])
+    # the forks as rows of one pass over one arena: the prompt's rows once, every fork's steps in stretches of Wd slots
+    A, arena = new_arena(cfg)
+    rw = torch.zeros(3 + 3 * T, dtype=torch.int32, device="cuda")
+    rows = Pass(card, cfg, W, arena, tables, T=T, mma=False, rows=rw)
+    A.zero_()
+    A[:, :, :n] = A1[:, :, :n]                                   # the shared prefix (any fork's: the prompt's rows)
+    for d in range(2):
+        rw.copy_(card.rows_layout(base, d, Wd, [(c, 0, n) for c in range(B)], pad_to=T))
+        logits = rows([f[d] for f in forks] + [0], 0)
+        for t in range(B):
+            assert np.array_equal(logits[t], alone[t][d]), (d, t)
+        assert int(np.argmax(logits[0])) == r["greedy"][d + 1]
+    # the forks' rows lie where the layout says, and nowhere else
+    live = torch.zeros(CAP, dtype=torch.bool, device="cuda")
+    live[:n] = True
+    live[base : base + 2 * Wd] = True
+    assert not bool(A[:, :, ~live].any()) and bool(A[:, :, base : base + 2 * Wd].any())
 
 
 def test_card_launch_surface(card):
