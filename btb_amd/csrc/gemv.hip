@@ -301,7 +301,8 @@ int32_t gemv_mfma_dl_mxfp4(const void* blocks, const void* scales, const void* x
                            hipStream_t st);
 // and for pack12 rows of the lengths it has shapes for
 bool mfma_dl_fits_p12(int R, int C, int M);
-int32_t gemv_mfma_dl_p12(const uint8_t* lo, const uint8_t* hi4, const uint8_t* table, const int32_t* esc_idx,
+int32_t gemv_mfma_dl_p12(const uint8_t* lo, const uint8_t* hi4, const uint8_t* table, const uint16_t* pairs,
+                         const int32_t* esc_idx,
                          const uint8_t* esc_val, const int32_t* row_ptr, const void* x, void* y, int R, int C, int M,
                          hipStream_t st);
 
@@ -480,7 +481,7 @@ int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, con
         uint16_t* yp = static_cast<uint16_t*>(y);
         for (size_t m0 = 0; m0 < M; m0 += 16) {
             const int mm = (int)(M - m0 < 16 ? M - m0 : 16);
-            rc = gemv_mfma_dl_p12(p.lo, p.hi4, p.table, p.esc_idx, p.esc_val, p.row_ptr, xp + m0 * C, yp + m0 * R, (int)R,
+            rc = gemv_mfma_dl_p12(p.lo, p.hi4, p.table, p.pairs, p.esc_idx, p.esc_val, p.row_ptr, xp + m0 * C, yp + m0 * R, (int)R,
                                   (int)C, mm, static_cast<hipStream_t>(stream));
             if (rc != OK) return rc;
         }

@@ -235,11 +235,16 @@ struct DlMx4 : DlNoTail {
 // half. A fragment is eight low bytes and eight codes zipped through the 16-entry table of high bytes, which the
 // lanes keep in four registers. The escapes - weights whose high byte is not in the table; the matrix cores multiply
 // the table's last entry in their place - are not this wave's business: see escape_wave below.
-template <int SBS_>
+// PAIRS: the high bytes come out of the 256-entry pair table (btb_hip_p12_pairs: entry b = the high bytes of the two
+// weights whose codes are byte b's nibbles, slot 15 taken as 0), which the escape wave - the one wave here whose loads
+// are ordinary ones - brings into LDS before the first tile: eight weights are then four 2-byte LDS reads and four
+// byte-permutes in place of the in-register lookup's two dozen instructions.
+template <int SBS_, bool PAIRS_>
 struct DlP12 {
     static_assert(SBS_ == 4 || SBS_ == 8, "a sub-block's codes are one or two load instructions");
     static constexpr int STEPB = 32;
     static constexpr bool TAIL = true;
+    static constexpr bool PAIRS = PAIRS_;
     struct Mat {
         const uint8_t* w;  // lo
         const uint8_t* codes;
@@ -247,6 +252,7 @@ struct DlP12 {
         const int32_t* esc_idx;
         const uint8_t* esc_val;
         const int32_t* row_ptr;
+        const uint16_t* pairs;
     };
     struct Ctx {
         uint4 tbl;
@@ -254,7 +260,13 @@ struct DlP12 {
     // the table's sixteen bytes (4-byte aligned: the host checks), read before the kernel stores anything
     __device__ static __forceinline__ Ctx make_ctx(const Mat& m) {
         const u32x4 t = *reinterpret_cast<const u32x4*>(m.table);
-        return Ctx{make_uint4(t.x, t.y, t.z, t.w)};
+        // with the pair table an escape streams as slot 15 = 0, whatever the 16-byte table holds there
+        return Ctx{make_uint4(t.x, t.y, t.z, PAIRS ? (t.w & 0x00FFFFFFu) : t.w)};
+    }
+    // one wave brings the pair table in: four entries a lane
+    __device__ static __forceinline__ void stage_pairs(const Mat& m, int lane) {
+        const u32x2 v = reinterpret_cast<const u32x2*>(m.pairs)[lane];
+        reinterpret_cast<u32x2*>(FmtP12G::pair_table())[lane] = v;
     }
     __host__ __device__ static constexpr int scale_bytes(int sbs) { return sbs == 4 ? 1024 : 2 * (1024 + 128); }
     __host__ __device__ static constexpr int aux_loads(int sbs) { return sbs == 4 ? 1 : 2; }
@@ -289,7 +301,10 @@ struct DlP12 {
     __device__ static __forceinline__ bf16x8 frag(const uint8_t* p, const uint32_t (&ew)[N], int t, const Ctx& ctx) {
         const uint2 l = *reinterpret_cast<const uint2*>(p);
         uint32_t w[4];
-        FmtP12::widen8(ctx.tbl, ew[t], l.x, l.y, w);
+        if constexpr (PAIRS)
+            FmtP12G::widen8(ew[t], l.x, l.y, w);
+        else
+            FmtP12::widen8(ctx.tbl, ew[t], l.x, l.y, w);
         return __builtin_bit_cast(bf16x8, make_uint4(w[0], w[1], w[2], w[3]));
     }
 };
@@ -408,6 +423,12 @@ __device__ __forceinline__ void escape_wave(const typename DF::Mat& mat, const t
 }
 
 // ---- the kernel ---------------------------------------------------------------------------------------------------
+
+// whether a form brings a table into LDS before the first tile (pack12 with its pair table)
+template <class DF, class = void>
+struct dl_pairs : std::false_type {};
+template <class DF>
+struct dl_pairs<DF, std::enable_if_t<DF::PAIRS>> : std::true_type {};
 
 // The loads of one sub-block into `slot` (tile `tile`, the wave's steps step0 .. step0 + SBS - 1: GB column blocks).
 // `slot` is a __restrict__ parameter on purpose, here and in sub_block below: the compiler orders an LDS read behind
@@ -541,6 +562,10 @@ __global__ void __launch_bounds__((KS + (DF::TAIL ? 1 : 0)) * 64)
     const int nt = first < ntiles ? (ntiles - first + grid - 1) / grid : 0;  // this workgroup's tiles
     if constexpr (DF::TAIL) {
         if (wv == KS) {
+            if constexpr (dl_pairs<DF>::value) {  // the pair table into LDS; the streaming waves wait below
+                DF::stage_pairs(mat, lane);
+                asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+            }
             escape_wave<DF, KS>(mat, ctx, reinterpret_cast<const uint16_t*>(x), C, M, first, grid, nt, lane, esc, part);
             return;
         }
@@ -585,6 +610,8 @@ __global__ void __launch_bounds__((KS + (DF::TAIL ? 1 : 0)) * 64)
             __builtin_amdgcn_sched_barrier(0);
         }
     }
+    // the pair table is in LDS once the escape wave has arrived (a barrier for LDS traffic only: the loads above stay out)
+    if constexpr (dl_pairs<DF>::value) asm volatile("s_barrier" ::: "memory");
     // One body of the tile loop: TPB tiles. FIRST: the kernel's first body, whose first tile's waits let the parts of x
     // asked for behind a sub-block's own stay outstanding.
     auto body = [&](int k0, auto first_tag) {
@@ -631,7 +658,8 @@ static int32_t launch_dl(const typename DF::Mat& mat, const void* x, void* y, in
     const int nsteps = C / 32;
     // a row: whole sub-blocks, every wave a first one, only the waves' last ones missing
     const bool row_ok = C % 32 == 0 && nsteps % SBS == 0 && nsteps > KS * (MAXSB - 1) * SBS && nsteps <= KS * SPW;
-    if (lds > (size_t)device_info().lds_bytes || !row_ok || R % 16 != 0 || M < 1 || M > 16) {
+    constexpr size_t fixed = dl_pairs<DF>::value ? 512 : 0;  // the pair table, a static array beside the dynamic ones
+    if (lds + fixed > (size_t)device_info().lds_bytes || !row_ok || R % 16 != 0 || M < 1 || M > 16) {
         set_error("gemv_mfma_dl: a shape this kernel does not take");
         return ERR_DOMAIN;
     }
@@ -706,15 +734,25 @@ bool mfma_dl_fits_p12(int R, int C, int M) {
     const int cls = row_class(C, 4, 8);
     return pass_ok(R, M) && cls >= 1;
 }
-int32_t gemv_mfma_dl_p12(const uint8_t* lo, const uint8_t* hi4, const uint8_t* table, const int32_t* esc_idx,
-                         const uint8_t* esc_val, const int32_t* row_ptr, const void* x, void* y, int R, int C, int M,
-                         hipStream_t st) {
+int32_t gemv_mfma_dl_p12(const uint8_t* lo, const uint8_t* hi4, const uint8_t* table, const uint16_t* pairs,
+                         const int32_t* esc_idx, const uint8_t* esc_val, const int32_t* row_ptr, const void* x, void* y,
+                         int R, int C, int M, hipStream_t st) {
+    // the pair table (made at upload) where the caller has one and it can be read eight bytes a lane
+    const bool tab = pairs != nullptr && (reinterpret_cast<uintptr_t>(pairs) & 7u) == 0 && tuning("p12_pair_table") != 0;
+#define P12DL(SB, KS, SPW, GB, NB)                                                                                    \
+    return tab ? launch_dl<DlP12<SB, true>, KS, SPW, GB, NB>(                                                         \
+                     DlP12<SB, true>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr, pairs}, x, y, R, C, M, st)       \
+               : launch_dl<DlP12<SB, false>, KS, SPW, GB, NB>(                                                        \
+                     DlP12<SB, false>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr, pairs}, x, y, R, C, M, st)
     switch (row_class(C, 4, 8)) {
-        case 1: return launch_dl<DlP12<4>, 10, 8, 1, 4>(DlP12<4>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr}, x, y, R, C, M, st);
-        case 2: return launch_dl<DlP12<4>, 8, 16, 1, 4>(DlP12<4>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr}, x, y, R, C, M, st);
-        case 3: return launch_dl<DlP12<8>, 7, 48, 2, 3>(DlP12<8>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr}, x, y, R, C, M, st);
+        case 1: P12DL(4, 10, 8, 1, 4);
+        case 2: P12DL(4, 8, 16, 1, 4);
+        case 3:  // its rings and partial tiles leave 112 bytes of the CU's LDS: no room for the table
+            return launch_dl<DlP12<8, false>, 7, 48, 2, 3>(
+                DlP12<8, false>::Mat{lo, hi4, table, esc_idx, esc_val, row_ptr, pairs}, x, y, R, C, M, st);
         default: set_error("gemv_mfma_dl: a row length this kernel has no shape for"); return ERR_DOMAIN;
     }
+#undef P12DL
 }
 
 }  // namespace btb
