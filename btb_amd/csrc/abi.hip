@@ -60,11 +60,7 @@ struct Knob {
 };
 static Knob g_knobs[] = {
     {"gemv_wgs_per_cu", {-1}},
-    {"gemv_variant", {-1}},
     {"gemv_no_mfma", {-1}},
-    {"gemv_short_span", {-1}},
-    {"gemv_glu_split", {-1}},
-    {"gemv_stretch", {-1}},
     {"mfma_wgs_per_cu", {-1}},
     {"mfma_classic", {-1}},
     {"mfma_lds", {-1}},
@@ -76,7 +72,6 @@ static Knob g_knobs[] = {
     {"p12_pair_table", {-1}},
     {"moe_wgs_per_cu", {-1}},
     {"moe_grouped", {-1}},
-    {"attn_split", {-1}},
     {"attn_heads_per_wg", {-1}},
     {"attn_mfma", {-1}},
     {"attn_rows_fused", {-1}},

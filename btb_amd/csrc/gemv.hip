@@ -186,44 +186,42 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
     // waves resident: one row by four (pack12, MXFP4), two rows by two (FP8, whose two rows share a scale fetch
     // pattern). Neither choice changes a result bit (a lane's units stay in ascending order).
     constexpr bool WIDENS = sizeof(typename F::Raw) != 16;  // everything but plain bf16
-    // One row of x (the decode step proper): where a slightly longer span saves a whole round trip to memory - a row of
-    // 5 units a lane read as 5, not 4 + 1; 19 as 10 + 9, not 8 + 8 + 3 - the span is stretched to 5 (10 for one bf16
-    // row a wave). A lane's units stay in ascending order, so no result bit changes.
+    // One bf16 row of x (the decode step proper): where a slightly longer span saves a whole round trip to memory - a
+    // row of 5 units a lane read as 5, not 4 + 1; 19 as 10 + 9, not 8 + 8 + 3 - the span is stretched to 5 (10 for one
+    // row a wave). Measured a gain for bf16 and a loss for the forms that widen, which keep their spans.
     const int per_lane = (C / F::UW + LPR - 1) / LPR;
     auto fewer = [per_lane](int u_new, int u_base) { return (per_lane + u_new - 1) / u_new < (per_lane + u_base - 1) / u_base; };
-    const int stretch_knob = tuning("gemv_stretch");  // measured: a gain for bf16, a loss for the forms that widen
-    const bool stretch = M == 1 && (stretch_knob >= 0 ? stretch_knob == 1 : !WIDENS);
     if constexpr (EPI == E_GLU) {
-        // a widening form whose rows take at most 32 lanes: gate and up side by side, one row a lane
         if constexpr (WIDENS && LPR <= 32) {
-            if (tuning("gemv_glu_split") != 0) {
-                if constexpr (M == 1 && F::TWO_ROWS == false) {
-                    if (stretch && fewer(5, 4)) return launch_variant<F, M, LPR, 1, 5, XMODE, E_GLU_SPLIT>(p, xa, y, R, C, st);
-                }
-                return launch_variant<F, M, LPR, 1, 4, XMODE, E_GLU_SPLIT>(p, xa, y, R, C, st);
+            // a widening form whose rows take at most 32 lanes: gate and up side by side, one row a lane
+            return launch_variant<F, M, LPR, 1, 4, XMODE, E_GLU_SPLIT>(p, xa, y, R, C, st);
+        } else if constexpr (WIDENS) {
+            return launch_variant<F, M, LPR, 2, 2, XMODE, E_GLU>(p, xa, y, R, C, st);
+        } else {
+            if constexpr (M == 1) {
+                if (fewer(5, 4)) return launch_variant<F, M, LPR, 2, 5, XMODE, E_GLU>(p, xa, y, R, C, st);
             }
+            return launch_variant<F, M, LPR, 2, (M <= 2 ? 4 : 2), XMODE, E_GLU>(p, xa, y, R, C, st);
         }
-        if constexpr (M == 1 && !WIDENS) {
-            if (stretch && fewer(5, 4)) return launch_variant<F, M, LPR, 2, 5, XMODE, E_GLU>(p, xa, y, R, C, st);
+    } else if constexpr (WIDENS) {
+        if constexpr (F::TWO_ROWS)
+            return launch_variant<F, M, LPR, 2, 2, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+        else
+            return launch_variant<F, M, LPR, 1, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+    } else {
+        const bool tall = R >= 4096 * (WAVE / LPR);
+        if constexpr (M <= 2) {
+            if constexpr (M == 1) {
+                if (tall && fewer(5, 4)) return launch_variant<F, M, LPR, 2, 5, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+                if (!tall && fewer(10, 8)) return launch_variant<F, M, LPR, 1, 10, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+            }
+            if (tall) return launch_variant<F, M, LPR, 2, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+            return launch_variant<F, M, LPR, 1, 8, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+        } else {
+            if (tall) return launch_variant<F, M, LPR, 2, 2, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+            return launch_variant<F, M, LPR, 1, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
         }
-        return launch_variant<F, M, LPR, 2, (M <= 2 && !WIDENS ? 4 : 2), XMODE, E_GLU>(p, xa, y, R, C, st);
     }
-    const int v = tuning("gemv_variant");
-    const int shorter = tuning("gemv_short_span");
-    const bool tall = v >= 0 ? (v == 1) : (WIDENS ? F::TWO_ROWS : R >= 4096 * (WAVE / LPR));
-    if (M <= 2 && (shorter >= 0 ? shorter == 0 : !WIDENS)) {
-        if constexpr (M == 1 && !WIDENS) {
-            if (stretch && tall && fewer(5, 4)) return launch_variant<F, M, LPR, 2, 5, XMODE, E_PLAIN>(p, xa, y, R, C, st);
-            if (stretch && !tall && fewer(10, 8)) return launch_variant<F, M, LPR, 1, 10, XMODE, E_PLAIN>(p, xa, y, R, C, st);
-        }
-        if (tall) return launch_variant<F, M, LPR, 2, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
-        return launch_variant<F, M, LPR, 1, 8, XMODE, E_PLAIN>(p, xa, y, R, C, st);
-    }
-    if constexpr (M == 1 && WIDENS && F::TWO_ROWS == false) {
-        if (stretch && !tall && fewer(5, 4)) return launch_variant<F, M, LPR, 1, 5, XMODE, E_PLAIN>(p, xa, y, R, C, st);
-    }
-    if (tall) return launch_variant<F, M, LPR, 2, 2, XMODE, E_PLAIN>(p, xa, y, R, C, st);
-    return launch_variant<F, M, LPR, 1, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
 }
 
 template <class F, int M, int XMODE, int EPI>
