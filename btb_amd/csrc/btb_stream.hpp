@@ -238,15 +238,10 @@ __device__ __forceinline__ float dot2(uint32_t w, uint32_t x, float acc) {
 }
 
 template <class F, int M, int RPW>
-__device__ __forceinline__ void fma_unit(const typename F::RowCtx (&ctx)[RPW], const typename F::Raw (&raw)[RPW],
-                                         int unit, const uint4* xs4, int xrow4, float (&acc)[RPW][M]) {
+__device__ __forceinline__ void fma_unit_x(const typename F::RowCtx (&ctx)[RPW], const typename F::Raw (&raw)[RPW],
+                                           int unit, const uint4 (&xv)[F::UW / 8][M], float (&acc)[RPW][M]) {
     constexpr int UW = F::UW;
     constexpr int H = UW / 8;
-    uint4 xv[H][M];
-#pragma unroll
-    for (int h = 0; h < H; ++h)
-#pragma unroll
-        for (int m = 0; m < M; ++m) xv[h][m] = xs4[m * xrow4 + unit * H + h];
 #pragma unroll
     for (int j = 0; j < RPW; ++j) {
         uint32_t w[UW / 2];
@@ -263,6 +258,17 @@ __device__ __forceinline__ void fma_unit(const typename F::RowCtx (&ctx)[RPW], c
                 acc[j][m] = a;
             }
     }
+}
+template <class F, int M, int RPW>
+__device__ __forceinline__ void fma_unit(const typename F::RowCtx (&ctx)[RPW], const typename F::Raw (&raw)[RPW],
+                                         int unit, const uint4* xs4, int xrow4, float (&acc)[RPW][M]) {
+    constexpr int H = F::UW / 8;
+    uint4 xv[H][M];
+#pragma unroll
+    for (int h = 0; h < H; ++h)
+#pragma unroll
+        for (int m = 0; m < M; ++m) xv[h][m] = xs4[m * xrow4 + unit * H + h];
+    fma_unit_x<F, M, RPW>(ctx, raw, unit, xv, acc);
 }
 
 // what a finished pair of row sums becomes. E_PLAIN: y[m][r] = bf16(sum). E_GLU: the matrix is [2I, C], gate rows then
@@ -330,13 +336,34 @@ template <class F, int M, int LPR, int RPW, int U, bool GUARD>
 __device__ __forceinline__ void fma_span(const typename F::Raw (&raw)[U][RPW], const typename F::RowCtx (&ctx)[RPW],
                                          int k0, int sl, int units, const uint4* xs4, int xrow4,
                                          float (&acc)[RPW][M]) {
+    if constexpr (M == 1) {
+        // One row of x: the span's x values are all asked of LDS before the first product, so their trips overlap one
+        // another (and, for a span still on its way from memory, the weights' flight) instead of standing one behind
+        // the other between the products. A unit past the row's end reads the row's last unit (and is not used).
+        constexpr int H = F::UW / 8;
+        uint4 xv[U][H][1];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-        const int unit = k0 + u * LPR + sl;
-        if (!GUARD || unit < units) fma_unit<F, M, RPW>(ctx, raw[u], unit, xs4, xrow4, acc);
-        // one unit's widening and products at a time: without the fence the scheduler hoists every unit's widening
-        // ahead of the first product and the live registers cost the kernel its occupancy
+        for (int u = 0; u < U; ++u) {
+            const int unit = GUARD ? min(k0 + u * LPR + sl, units - 1) : k0 + u * LPR + sl;
+#pragma unroll
+            for (int h = 0; h < H; ++h) xv[u][h][0] = xs4[unit * H + h];
+        }
         __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int unit = k0 + u * LPR + sl;
+            if (!GUARD || unit < units) fma_unit_x<F, 1, RPW>(ctx, raw[u], unit, xv[u], acc);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    } else {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int unit = k0 + u * LPR + sl;
+            if (!GUARD || unit < units) fma_unit<F, M, RPW>(ctx, raw[u], unit, xs4, xrow4, acc);
+            // one unit's widening and products at a time: without the fence the scheduler hoists every unit's
+            // widening ahead of the first product and the live registers cost the kernel its occupancy
+            __builtin_amdgcn_sched_barrier(0);
+        }
     }
 }
 

@@ -52,7 +52,10 @@ __device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typ
 
     int k0 = 0;
     if (PRIMED) {
-        fma_span<F, M, LPR, RPW, U, true>(first, ctx, 0, sl, units, xs4, xrow4, acc);
+        if (span <= units)  // uniform: the first span is a full one, nothing in it to guard
+            fma_span<F, M, LPR, RPW, U, false>(first, ctx, 0, sl, units, xs4, xrow4, acc);
+        else
+            fma_span<F, M, LPR, RPW, U, true>(first, ctx, 0, sl, units, xs4, xrow4, acc);
         k0 = span;
     }
     for (; k0 < units; k0 += span) {
