@@ -416,6 +416,21 @@ __global__ void __launch_bounds__(256) attn_decode_qkv_kernel(const uint16_t* __
 
     const int n0 = *n0p;
     const int k_end = min(n0 + 1, k_begin + span);
+    if (k_begin > n0) {
+        // A span past the row's keys (spans are cut from the cache's capacity, not from its length): the state the fold
+        // below would leave - no maximum, no sum, zeros - written at once; the workgroup prepares no head, waits for no
+        // key and leaves its CU to the workgroups that have work.
+        const size_t prow = (size_t)g * gridDim.y + sp;
+        for (int o = threadIdx.x; o < GW * D; o += 256) {
+            const int j = o / D, d = o - j * D;
+            part_acc[((prow * Gt) + j0 + j) * D + d] = 0.f;
+            if (d == 0) {
+                part_m[prow * Gt + j0 + j] = bits_f32(0xff800000u);
+                part_l[prow * Gt + j0 + j] = 0.f;
+            }
+        }
+        return;
+    }
     constexpr int NQ = (GW + 3) / 4;  // query heads a wave prepares
     HeadIn qin[NQ];
 #pragma unroll
