@@ -336,23 +336,31 @@ template <class F, int M, int LPR, int RPW, int U, bool GUARD>
 __device__ __forceinline__ void fma_span(const typename F::Raw (&raw)[U][RPW], const typename F::RowCtx (&ctx)[RPW],
                                          int k0, int sl, int units, const uint4* xs4, int xrow4,
                                          float (&acc)[RPW][M]) {
-    if constexpr (M == 1) {
-        // One row of x: the span's x values are all asked of LDS before the first product, so their trips overlap one
-        // another (and, for a span still on its way from memory, the weights' flight) instead of standing one behind
-        // the other between the products. A unit past the row's end reads the row's last unit (and is not used).
-        constexpr int H = F::UW / 8;
-        uint4 xv[U][H][1];
+    constexpr int H = F::UW / 8;
+    constexpr bool WIDENS = sizeof(typename F::Raw) != 16;  // everything but plain bf16
+    if constexpr (!WIDENS && (M == 1 || (M <= 3 && U * H * M <= 8))) {
+        // bf16, one row of x (or two or three, where that is at most 32 registers): the span's x values are all asked
+        // of LDS before the first product, so their trips overlap one another (and, for a span still on its way from
+        // memory, the weights' flight) instead of standing one behind the other between the products. A unit past the
+        // row's end reads the row's last unit (and is not used). Measured: the one-row bf16 step 2.150 -> 2.115 ms,
+        // a pass of two rows 0.6 % faster. At four rows the registers cost more than the overlap returns (bf16
+        // [9728 x 2560] 11.8 -> 12.6 us, the grouped MoE gate/up 109 -> 124 us a layer at 8 tokens), and so they do
+        // for the forms that widen in registers at any width (one row: pack12 9.75 -> 11.2 us, FP8 26.7 -> 28.2, the
+        // packed step 2.14 -> 2.27 ms).
+        uint4 xv[U][H][M];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int unit = GUARD ? min(k0 + u * LPR + sl, units - 1) : k0 + u * LPR + sl;
 #pragma unroll
-            for (int h = 0; h < H; ++h) xv[u][h][0] = xs4[unit * H + h];
+            for (int h = 0; h < H; ++h)
+#pragma unroll
+                for (int m = 0; m < M; ++m) xv[u][h][m] = xs4[m * xrow4 + unit * H + h];
         }
         __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int u = 0; u < U; ++u) {
             const int unit = k0 + u * LPR + sl;
-            if (!GUARD || unit < units) fma_unit_x<F, 1, RPW>(ctx, raw[u], unit, xv[u], acc);
+            if (!GUARD || unit < units) fma_unit_x<F, M, RPW>(ctx, raw[u], unit, xv[u], acc);
             __builtin_amdgcn_sched_barrier(0);
         }
     } else {
