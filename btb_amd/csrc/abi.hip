@@ -70,7 +70,6 @@ static Knob g_knobs[] = {
     {"mfma_direct", {-1}},
     {"mfma_direct_grid", {-1}},
     {"p12_pair_table", {-1}},
-    {"moe_wgs_per_cu", {-1}},
     {"moe_grouped", {-1}},
     {"attn_heads_per_wg", {-1}},
     {"attn_mfma", {-1}},

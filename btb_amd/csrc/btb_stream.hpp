@@ -301,9 +301,6 @@ __device__ __forceinline__ int tile_row(int tile, int j, int lane, int R, int& o
     return min(out_row, R - 1);  // a row past the end reads the last row again (no divergence) and is not written
 }
 
-// where the kernel reads x from: LDS (staged once per workgroup) or straight from global memory through the caches
-enum XSrc { XS_LDS = 0, XS_GLOBAL = 1 };
-
 // the loads of one span: U units of each of the RPW rows; a unit past the row's end is not loaded
 template <class F, int LPR, int RPW, int U, bool GUARD>
 __device__ __forceinline__ void load_span(typename F::Raw (&raw)[U][RPW], const typename F::RowCtx (&ctx)[RPW], int k0,
