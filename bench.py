@@ -209,6 +209,7 @@ def ceiling_workload(args: argparse.Namespace) -> dict:
     copies past the 256 MB last-level cache, replayed as a hipGraph and timed like every other workload here."""
     import torch
 
+    from btb_amd.decode import recording
     from btb_amd.native import Native
 
     card = Native.card_kernels()
@@ -224,7 +225,7 @@ def ceiling_workload(args: argparse.Namespace) -> dict:
                 card.stream_probe(m)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph):
+        with recording(graph):
             for m in mats:
                 card.stream_probe(m)
         for _ in range(3):
@@ -263,6 +264,7 @@ def kernel_workload(args: argparse.Namespace) -> dict:
     import torch
 
     from btb_amd import fp8, mxfp4
+    from btb_amd.decode import recording
     from btb_amd.moe import Experts, Router
     from btb_amd.native import Native
     from btb_amd.pack12 import P12Weight
@@ -378,7 +380,7 @@ def kernel_workload(args: argparse.Namespace) -> dict:
             call(i)
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(graph):
+    with recording(graph):
         for i in range(pool):
             call(i)
     passes = max(1, (args.steps + pool - 1) // pool)
@@ -475,6 +477,8 @@ def step_classes(step, card) -> list[dict]:
 def time_region(torch, fn, launches: int, reps: int) -> float:
     """average microseconds per launch of `fn`'s launches, replayed as a hipGraph `reps` times between two device
     events recorded on the stream the graph runs on"""
+    from btb_amd.decode import recording
+
     side = torch.cuda.Stream()
     side.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(side):
@@ -482,7 +486,7 @@ def time_region(torch, fn, launches: int, reps: int) -> float:
     torch.cuda.current_stream().wait_stream(side)
     torch.cuda.synchronize()
     g = torch.cuda.CUDAGraph()
-    with torch.cuda.graph(g):
+    with recording(g):
         fn()
     g.replay()
     torch.cuda.synchronize()

@@ -14,6 +14,8 @@ memory.
 
 from __future__ import annotations
 
+import contextlib
+import gc
 import math
 from dataclasses import dataclass
 from typing import Any
@@ -23,6 +25,23 @@ import torch
 from .fp8 import F8Weight
 from .mxfp4 import MxWeight
 from .pack12 import P12Weight
+
+
+@contextlib.contextmanager
+def recording(graph: torch.cuda.CUDAGraph):
+    """`torch.cuda.graph(graph)` with Python's cyclic collector held off while the stream records. A collection that
+    runs in the middle of a recording can drop an older graph or device tensors that a dead reference cycle still
+    held, and the runtime does not take a graph destroyed or device memory released while a stream records: the
+    process aborts. So what is already dead is collected before the recording starts, and nothing is while it runs."""
+    gc.collect()
+    was_on = gc.isenabled()
+    gc.disable()
+    try:
+        with torch.cuda.graph(graph):
+            yield graph
+    finally:
+        if was_on:
+            gc.enable()
 
 
 @dataclass(frozen=True)
@@ -320,7 +339,7 @@ class DecodeStep:
         torch.cuda.current_stream().wait_stream(side)
         torch.cuda.synchronize()
         g = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(g):
+        with recording(g):
             self.body()
         self.graph = g
         return g

@@ -17,6 +17,7 @@ tests/test_oracle_decode.py) and the greedy tokens must be the receipts'.
 
 from __future__ import annotations
 
+import functools
 import os
 
 import numpy as np
@@ -24,7 +25,7 @@ import pytest
 import torch
 
 from btb_amd import card_launch as cl
-from btb_amd.decode import rope_tables
+from btb_amd.decode import recording, rope_tables
 from btb_amd.load import load_stack
 
 from .helpers import GOLDEN
@@ -150,7 +151,7 @@ class Pass:
 
     def __init__(self, k, cfg, W, arena, tables, T, mma, row_map=None, fused=False, capture=True, rows=None):
         self.k, self.cfg, self.W, self.g = k, cfg, W, buffers(cfg, T, mma)
-        self.run = lambda: card_body(k, cfg, W, self.g, arena, tables, row_map, fused, rows)
+        self.run = functools.partial(card_body, k, cfg, W, self.g, arena, tables, row_map, fused, rows)
         self.graph = None
         if capture:
             side = torch.cuda.Stream()
@@ -161,7 +162,7 @@ class Pass:
             torch.cuda.current_stream().wait_stream(side)
             torch.cuda.synchronize()
             self.graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(self.graph):
+            with recording(self.graph):
                 self.run()
 
     def __call__(self, tokens, n0, par=None):
