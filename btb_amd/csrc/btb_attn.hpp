@@ -394,7 +394,7 @@ template <int G, bool DEV>
 __device__ __forceinline__ void merge_spans(uint16_t* out, int g, int S, size_t base, const float* part_m,
                                             const float* part_l, const float* part_acc, float* lds, int tid) {
     constexpr int NOUT = G >= 2 ? G / 2 : 1;  // outputs a thread makes: (j, d) = ((tid + 256 q) / 128, tid % 128)
-    constexpr int MS = NOUT <= 2 ? 40 : 20;   // spans a pass (a 4096-key cache is 33 to 36 spans: one pass)
+    constexpr int MS = NOUT <= 2 ? 40 : 20;  // spans a pass (a 4096-key cache is 33 to 36 spans: one pass)
     const float ninf = bits_f32(0xff800000u);
     auto ld = [](const float* p) { return DEV ? ld_dev(p) : *p; };
     float* f_m = lds;          // [S][G] maxima, then the factors
@@ -479,6 +479,41 @@ __device__ __forceinline__ void merge_spans(uint16_t* out, int g, int S, size_t 
                 *dst = o;
         }
     }
+}
+
+// The same fold for a few spans (S <= MS <= 32), with nothing shared between waves: a workgroup of 128 threads takes
+// one query head. A thread asks for its output's partial values of every span at once, and lane s of its wave for span
+// s's maximum and sum - one trip to memory, no LDS, no barrier. Lane s makes span s's factor; every lane reads it back
+// by lane number. The operations and their order are merge_spans': the same bits.
+template <int GS, int MS>
+__device__ __forceinline__ void merge_spans_few(uint16_t* out, int g, int j, int S, size_t base, const float* part_m,
+                                                const float* part_l, const float* part_acc, int d) {
+    const float ninf = bits_f32(0xff800000u);
+    const int lane = d & 63, last = S - 1;
+    const size_t sl = (base + min(lane, last)) * GS + j;
+    const float m = part_m[sl], l = part_l[sl];
+    float v[MS];
+#pragma unroll
+    for (int s2 = 0; s2 < MS; ++s2)  // past the last span: it again, unused
+        v[s2] = part_acc[((base + min(s2, last)) * GS + j) * AD + d];
+    float M = lane < S ? m : ninf;  // the spans' maximum, in every lane that holds a span
+    M = fmaxf(M, dpp_f32<0xB1>(M));
+    M = fmaxf(M, dpp_f32<0x4E>(M));
+    M = fmaxf(M, dpp_f32<0x141>(M));
+    M = fmaxf(M, dpp_f32<0x140>(M));
+    M = fmaxf(M, __shfl_xor(M, 16, WAVE));
+    // No branch on S below: with one, the compiler moves each load into its span's branch, a trip to memory a span.
+    // A span past the last adds a zero to the sum and leaves the output's value as it is (its factor and its partial
+    // value are made zero).
+    const float fac = (lane >= S || m == ninf) ? 0.f : __builtin_amdgcn_exp2f(m - M);
+    const float lsc = l * fac;
+    float A = 0.f, L = 0.f;
+#pragma unroll
+    for (int s2 = 0; s2 < MS; ++s2) {
+        L += bits_f32((uint32_t)__builtin_amdgcn_readlane((int)f32_bits(lsc), s2));
+        A = fmaf(s2 < S ? v[s2] : 0.f, bits_f32((uint32_t)__builtin_amdgcn_readlane((int)f32_bits(fac), s2)), A);
+    }
+    out[((size_t)g * GS + j) * AD + d] = f32_bf16(A * (1.f / L));
 }
 
 // What row t of a pass sees. A chain of rows (par null): the cache's keys and the pass's rows up to itself. A tree

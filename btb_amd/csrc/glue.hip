@@ -504,6 +504,41 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(uint16_t* __restrict__ 
                           threadIdx.x);
 }
 
+// the fold of a few spans (up to MERGE_FEW: the step's 18 are such): one workgroup of 128 per (row, query head)
+constexpr int MERGE_FEW = 20;
+template <int G, bool SEQS>
+__global__ void __launch_bounds__(128) attn_merge_few_kernel(uint16_t* __restrict__ att, int Hq, int Hk, int S,
+                                                             const float* __restrict__ part_m,
+                                                             const float* __restrict__ part_l,
+                                                             const float* __restrict__ part_acc,
+                                                             const int32_t* __restrict__ rw) {
+    const int g = blockIdx.x / G, j = blockIdx.x % G, t = blockIdx.y;
+    // SEQS: a pass of sequences, whose padding rows are skipped. A kernel of its own, so that the others do not read
+    // rw's pointer ahead of everything else (a trip for the kernel's arguments of its own: the step's pair of launches
+    // 12.1 -> 15.6 us a layer with it).
+    if constexpr (SEQS) {
+        if (rw[5 + 3 * t] < 0) return;
+    }
+    merge_spans_few<G, MERGE_FEW>(att + (size_t)t * Hq * ATT_D, g, j, S, ((size_t)t * Hk + g) * S, part_m, part_l,
+                                  part_acc, threadIdx.x);
+}
+
+// The fold behind every attention kernel here. Up to MERGE_FEW spans: the fold that shares nothing (the step's pair of
+// launches 13.7 -> 12.1 us a layer against the general fold); more: the general one. The same bits either way.
+template <int G>
+void launch_merge(hipStream_t st, void* att, size_t T, size_t Hq, size_t Hk, size_t S, const float* part_m,
+                  const float* part_l, const float* part_acc, const int32_t* rw) {
+    if (S <= (size_t)MERGE_FEW && rw == nullptr)
+        hipLaunchKernelGGL((attn_merge_few_kernel<G, false>), dim3((unsigned)(Hk * G), (unsigned)T), dim3(128), 0, st,
+                           static_cast<uint16_t*>(att), (int)Hq, (int)Hk, (int)S, part_m, part_l, part_acc, rw);
+    else if (S <= (size_t)MERGE_FEW)
+        hipLaunchKernelGGL((attn_merge_few_kernel<G, true>), dim3((unsigned)(Hk * G), (unsigned)T), dim3(128), 0, st,
+                           static_cast<uint16_t*>(att), (int)Hq, (int)Hk, (int)S, part_m, part_l, part_acc, rw);
+    else
+        hipLaunchKernelGGL(attn_merge_kernel<G>, dim3((unsigned)Hk, (unsigned)T), dim3(256), 2 * S * G * sizeof(float),
+                           st, static_cast<uint16_t*>(att), (int)Hq, (int)Hk, (int)S, part_m, part_l, part_acc, rw);
+}
+
 __global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ m,
                                                        size_t T, size_t I) {
     const size_t n = T * I;
@@ -759,15 +794,12 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
     const float scale_log2 = scale * 1.4426950408889634f;
     const dim3 grid((unsigned)Hk, (unsigned)S, (unsigned)T);
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const dim3 mgrid((unsigned)Hk, (unsigned)T);
-    const size_t mlds = 2 * S * G * sizeof(float);
 #define ATT(GG)                                                                                                      \
     hipLaunchKernelGGL(attn_decode_kernel<GG>, grid, dim3(256), 0, st, static_cast<const uint16_t*>(q),              \
                        static_cast<const uint16_t*>(K), static_cast<const uint16_t*>(V), n0, par, (int)T, (int)Hq,   \
                        (int)Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, span, (int)win,   \
                        tbl, rw);                                                                                    \
-    hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,       \
-                       (int)Hk, (int)S, part_m, part_l, part_acc, rw)
+    launch_merge<GG>(st, att, T, Hq, Hk, S, part_m, part_l, part_acc, rw)
     // Several rows and spans of 128 keys: the matrix cores, every row of the pass that shares a kv head in one workgroup
     // (attn_mfma.hip). A pass of 8 rows over 4096 keys: 22.7 us a layer on the vector kernel below (spans of one or two
     // batches of keys, asked for at once and kept in registers, a workgroup a row), which stays for spans of 256 keys
@@ -776,12 +808,8 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
         const int32_t rc = attn_decode_mfma(q, K, V, n0, par, T, Hq, Hk, (long long)hs, (long long)rs, scale_log2, part_m,
                                             part_l, part_acc, S, cap, (int)win, tbl, st);
         if (rc != OK) return rc;
-        if (G == 4)
-            hipLaunchKernelGGL(attn_merge_kernel<4>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
-                               (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr));
-        else
-            hipLaunchKernelGGL(attn_merge_kernel<2>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
-                               (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr));
+        if (G == 4) launch_merge<4>(st, att, T, Hq, Hk, S, part_m, part_l, part_acc, nullptr);
+        else launch_merge<2>(st, att, T, Hq, Hk, S, part_m, part_l, part_acc, nullptr);
         return hip_status(hipGetLastError(), "attn_decode launch");
     }
     if (parts == nullptr && T >= 2 && (span == 128 || span == 256) && (G == 2 || G == 4)) {
@@ -790,8 +818,7 @@ static int32_t attn_decode_any(const void* q, const void* K, const void* V, void
     hipLaunchKernelGGL((attn_decode_rows_kernel<GG, NB>), rgrid, dim3(256), 0, st, static_cast<const uint16_t*>(q),   \
                        static_cast<const uint16_t*>(K), static_cast<const uint16_t*>(V), n0, par, (int)T, (int)Hq,    \
                        (int)Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, (int)win, tbl);      \
-    hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,        \
-                       (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr))
+    launch_merge<GG>(st, att, T, Hq, Hk, S, part_m, part_l, part_acc, nullptr)
         if (G == 4 && span == 128) { ATTR(4, 1); }
         else if (G == 4) { ATTR(4, 2); }
         else if (span == 128) { ATTR(2, 1); }
@@ -886,8 +913,6 @@ int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk,
     float* part_acc = workspace + 2 * Hq * S;
     const float scale_log2 = scale * 1.4426950408889634f;
     hipStream_t st = static_cast<hipStream_t>(stream);
-    const dim3 mgrid((unsigned)Hk, 1);
-    const size_t mlds = 2 * S * G * sizeof(float);
     // query heads a workgroup takes: all G of its kv head, or fewer (the workgroups of one kv head are Hk apart in
     // the grid, which on this GPU - workgroups dealt to its eight dies in turn - keeps them on one die when Hk is 8)
     // Measured on MI355X (Qwen3-4B shape, 4096 keys of 4608 slots, whole step): two heads a workgroup and 18 spans (of
@@ -901,9 +926,7 @@ int32_t btb_hip_attn_decode_qkv(const void* qkv, const void* wq, const void* wk,
                        static_cast<const uint16_t*>(cos_t), static_cast<const uint16_t*>(sin_t), n0,                 \
                        static_cast<uint16_t*>(K), static_cast<uint16_t*>(V), (int)Hq, (int)Hk, (long long)hs,        \
                        (long long)rs, scale_log2, part_m, part_l, part_acc, span, (int)cap)
-#define MERGE(GG)                                                                                                    \
-    hipLaunchKernelGGL(attn_merge_kernel<GG>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,       \
-                       (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr))
+#define MERGE(GG) launch_merge<GG>(st, att, 1, Hq, Hk, S, part_m, part_l, part_acc, nullptr)
     if (G != 1 && G != 2 && G != 4 && G != 8) {
         set_error("attn_decode_qkv: 1, 2, 4 or 8 query heads per kv head");
         return ERR_DOMAIN;
@@ -968,14 +991,8 @@ int32_t btb_hip_attn_decode_qkv_rows(const void* qkv, const void* wq, const void
                                             Hk, (long long)hs, (long long)rs, scale_log2, part_m, part_l, part_acc, S, cap,
                                             st);
     if (rc != OK) return rc;
-    const dim3 mgrid((unsigned)Hk, (unsigned)T);
-    const size_t mlds = 2 * S * G * sizeof(float);
-    if (G == 4)
-        hipLaunchKernelGGL(attn_merge_kernel<4>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
-                           (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr));
-    else
-        hipLaunchKernelGGL(attn_merge_kernel<2>, mgrid, dim3(256), mlds, st, static_cast<uint16_t*>(att), (int)Hq,
-                           (int)Hk, (int)S, part_m, part_l, part_acc, static_cast<const int32_t*>(nullptr));
+    if (G == 4) launch_merge<4>(st, att, T, Hq, Hk, S, part_m, part_l, part_acc, nullptr);
+    else launch_merge<2>(st, att, T, Hq, Hk, S, part_m, part_l, part_acc, nullptr);
     return hip_status(hipGetLastError(), "attn_decode_qkv_rows launch");
 }
 
