@@ -72,6 +72,7 @@ static Knob g_knobs[] = {
     {"p12_pair_table", {-1}},
     {"moe_grouped", {-1}},
     {"attn_heads_per_wg", {-1}},
+    {"attn_merge_few", {-1}},
     {"attn_mfma", {-1}},
     {"attn_rows_fused", {-1}},
 };

@@ -481,7 +481,7 @@ __device__ __forceinline__ void merge_spans(uint16_t* out, int g, int S, size_t 
     }
 }
 
-// The same fold for a few spans (S <= MS <= 32), with nothing shared between waves: a workgroup of 128 threads takes
+// The same fold for a few spans (S <= MS <= 64), with nothing shared between waves: a workgroup of 128 threads takes
 // one query head. A thread asks for its output's partial values of every span at once, and lane s of its wave for span
 // s's maximum and sum - one trip to memory, no LDS, no barrier. Lane s makes span s's factor; every lane reads it back
 // by lane number. The operations and their order are merge_spans': the same bits.
@@ -502,6 +502,7 @@ __device__ __forceinline__ void merge_spans_few(uint16_t* out, int g, int j, int
     M = fmaxf(M, dpp_f32<0x141>(M));
     M = fmaxf(M, dpp_f32<0x140>(M));
     M = fmaxf(M, __shfl_xor(M, 16, WAVE));
+    if (MS > 32) M = fmaxf(M, __shfl_xor(M, 32, WAVE));
     // No branch on S below: with one, the compiler moves each load into its span's branch, a trip to memory a span.
     // A span past the last adds a zero to the sum and leaves the output's value as it is (its factor and its partial
     // value are made zero).

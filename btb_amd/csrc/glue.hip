@@ -506,7 +506,7 @@ __global__ void __launch_bounds__(256) attn_merge_kernel(uint16_t* __restrict__ 
 
 // the fold of a few spans (up to MERGE_FEW: the step's 18 are such): one workgroup of 128 per (row, query head)
 constexpr int MERGE_FEW = 20;
-template <int G, bool SEQS>
+template <int G, bool SEQS, int MS>
 __global__ void __launch_bounds__(128) attn_merge_few_kernel(uint16_t* __restrict__ att, int Hq, int Hk, int S,
                                                              const float* __restrict__ part_m,
                                                              const float* __restrict__ part_l,
@@ -519,24 +519,29 @@ __global__ void __launch_bounds__(128) attn_merge_few_kernel(uint16_t* __restric
     if constexpr (SEQS) {
         if (rw[5 + 3 * t] < 0) return;
     }
-    merge_spans_few<G, MERGE_FEW>(att + (size_t)t * Hq * ATT_D, g, j, S, ((size_t)t * Hk + g) * S, part_m, part_l,
+    merge_spans_few<G, MS>(att + (size_t)t * Hq * ATT_D, g, j, S, ((size_t)t * Hk + g) * S, part_m, part_l,
                                   part_acc, threadIdx.x);
 }
 
-// The fold behind every attention kernel here. Up to MERGE_FEW spans: the fold that shares nothing (the step's pair of
-// launches 13.7 -> 12.1 us a layer against the general fold); more: the general one. The same bits either way.
+// The fold behind every attention kernel here. Up to 2 * MERGE_FEW spans: the fold that shares nothing, built for 20
+// and for 40 spans (the step's pair of launches 13.6 -> 11.75 us a layer against the general fold at 18 spans; a pass
+// of 4 / 8 rows over 36 spans 2.95 / 2.96 -> 2.86 / 2.91 ms); more: the general one. The same bits either way.
 template <int G>
 void launch_merge(hipStream_t st, void* att, size_t T, size_t Hq, size_t Hk, size_t S, const float* part_m,
                   const float* part_l, const float* part_acc, const int32_t* rw) {
-    if (S <= (size_t)MERGE_FEW && rw == nullptr)
-        hipLaunchKernelGGL((attn_merge_few_kernel<G, false>), dim3((unsigned)(Hk * G), (unsigned)T), dim3(128), 0, st,
-                           static_cast<uint16_t*>(att), (int)Hq, (int)Hk, (int)S, part_m, part_l, part_acc, rw);
-    else if (S <= (size_t)MERGE_FEW)
-        hipLaunchKernelGGL((attn_merge_few_kernel<G, true>), dim3((unsigned)(Hk * G), (unsigned)T), dim3(128), 0, st,
-                           static_cast<uint16_t*>(att), (int)Hq, (int)Hk, (int)S, part_m, part_l, part_acc, rw);
+    size_t S_few = MERGE_FEW;
+#define FEW(SEQS, MS)                                                                                               \
+    hipLaunchKernelGGL((attn_merge_few_kernel<G, SEQS, MS>), dim3((unsigned)(Hk * G), (unsigned)T), dim3(128), 0, st, \
+                       static_cast<uint16_t*>(att), (int)Hq, (int)Hk, (int)S, part_m, part_l, part_acc, rw)
+    if (tuning("attn_merge_few") == 0) S_few = 0;  // 0: the general fold whatever the count (the tests compare the two)
+    if (S <= S_few && rw == nullptr) FEW(false, MERGE_FEW);
+    else if (S <= S_few) FEW(true, MERGE_FEW);
+    else if (S <= 2 * S_few && rw == nullptr) FEW(false, 2 * MERGE_FEW);
+    else if (S <= 2 * S_few) FEW(true, 2 * MERGE_FEW);
     else
         hipLaunchKernelGGL(attn_merge_kernel<G>, dim3((unsigned)Hk, (unsigned)T), dim3(256), 2 * S * G * sizeof(float),
                            st, static_cast<uint16_t*>(att), (int)Hq, (int)Hk, (int)S, part_m, part_l, part_acc, rw);
+#undef FEW
 }
 
 __global__ void __launch_bounds__(256) silu_mul_kernel(const uint16_t* __restrict__ gu, uint16_t* __restrict__ m,

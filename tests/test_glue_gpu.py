@@ -95,6 +95,35 @@ def test_attn_decode_against_f64(card, n0, T, Hq, Hk, S):
         assert worst <= 2.0**-7, worst
 
 
+@pytest.mark.parametrize("Hq,Hk", [(8, 8), (8, 4), (16, 4), (8, 1)])
+@pytest.mark.parametrize("n0,T,S", [(700, 1, 1), (700, 1, 2), (2400, 1, 19), (2559, 1, 20), (2600, 3, 21), (300, 2, 20),
+                                     (4990, 1, 39), (5000, 2, 40), (5200, 1, 41), (90, 1, 40)])
+def test_the_fold_of_a_few_spans_gives_the_general_folds_bits(card, n0, T, Hq, Hk, S):
+    """up to 40 spans are folded by a kernel that shares nothing between its waves; the knob attn_merge_few = 0 sends
+    every count through the general fold: the same output bits, at the counts on both sides of each limit, with spans
+    past the row's keys (no maximum, no sum) and for every number of query heads a kv head"""
+    D = 128
+    cap = n0 + T + 3
+    g = gen(7000 + n0 + S + Hq)
+    K = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda()
+    V = torch.randn(Hk, cap, D, generator=g).to(torch.bfloat16).cuda()
+    q = torch.randn(T, Hq * D, generator=g).to(torch.bfloat16).cuda()
+    scratch = card.attn_scratch(T, Hq, Hk, D, S)
+    n0t = torch.tensor([n0], dtype=torch.int32, device="cuda")
+    outs = []
+    try:
+        for knob in (0, -1):
+            card.set_tuning("attn_merge_few", knob)
+            att = torch.zeros(T, Hq * D, dtype=torch.bfloat16, device="cuda")
+            card.attn_decode(q, K, V, att, n0t, Hq, Hk, D, 1.0 / np.sqrt(D), S, scratch)
+            torch.cuda.synchronize()
+            outs.append(att)
+    finally:
+        card.set_tuning("attn_merge_few", -1)
+    assert torch.equal(outs[0], outs[1])
+    assert bool(outs[0].float().abs().sum() > 0)
+
+
 @pytest.mark.parametrize("n0,T,Hq,Hk,S,seed", [(300, 8, 32, 8, 5, 0), (0, 5, 8, 2, 1, 1), (63, 32, 16, 2, 7, 2),
                                                 (1000, 16, 8, 1, 16, 3)])
 def test_attn_decode_over_a_tree_of_rows(card, n0, T, Hq, Hk, S, seed):
