@@ -42,7 +42,7 @@ __device__ __forceinline__ void head_finish(const HeadIn& in, bool has_wn, float
     float v[2] = {bf16lo_f32(in.raw), bf16hi_f32(in.raw)};
     if (has_wn) {
         float ss = fmaf(v[1], v[1], fmaf(v[0], v[0], 0.f));
-        ss = group_sum<64>(ss);
+        ss = wave_sum(ss);
         const float rstd = rsqrtf(ss / (float)AD + eps);
         const float w2[2] = {bf16lo_f32(in.wn), bf16hi_f32(in.wn)};
 #pragma unroll
@@ -501,8 +501,11 @@ __device__ __forceinline__ void merge_spans_few(uint16_t* out, int g, int j, int
     M = fmaxf(M, dpp_f32<0x4E>(M));
     M = fmaxf(M, dpp_f32<0x141>(M));
     M = fmaxf(M, dpp_f32<0x140>(M));
-    M = fmaxf(M, __shfl_xor(M, 16, WAVE));
-    if (MS > 32) M = fmaxf(M, __shfl_xor(M, 32, WAVE));
+    {   // across the rows of 16 lanes: their last lanes' values as scalars (no trip through the LDS unit)
+        auto row = [&](int l) { return bits_f32((uint32_t)__builtin_amdgcn_readlane((int)f32_bits(M), l)); };
+        const float lo = fmaxf(row(15), row(31));
+        M = MS > 32 ? fmaxf(lo, fmaxf(row(47), row(63))) : lo;
+    }
     // No branch on S below: with one, the compiler moves each load into its span's branch, a trip to memory a span.
     // A span past the last adds a zero to the sum and leaves the output's value as it is (its factor and its partial
     // value are made zero).

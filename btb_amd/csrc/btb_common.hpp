@@ -112,4 +112,31 @@ __device__ __forceinline__ float group_sum(float v) {
     return v;
 }
 
+// The same sum, the same bits (the same pairs are added, some the other way round), for a caller that needs it in one
+// lane only: the group's LAST lane. The steps across rows of 16 are row broadcasts on the vector ALU (lane 15 of a row
+// into the next row, lane 31 into the upper half) in place of two exchanges through the LDS unit, which a wave's
+// last tile has nothing to hide behind. Other lanes end up with partial sums.
+template <int LANES>
+__device__ __forceinline__ float group_sum_last(float v) {
+    v += dpp_f32<0xB1>(v);
+    v += dpp_f32<0x4E>(v);
+    v += dpp_f32<0x141>(v);
+    v += dpp_f32<0x140>(v);
+    if (LANES >= 32) v += dpp_f32<0x142, 0xA>(v);  // row_bcast:15 into rows 1 and 3 (the others add 0)
+    if (LANES >= 64) v += dpp_f32<0x143, 0xC>(v);  // row_bcast:31 into rows 2 and 3
+    return v;
+}
+// the whole wave's sum in every lane: the last lane's, handed round as a scalar. The same bits as group_sum<64>
+// (there every lane ends with the same pairs added, some the other way round).
+__device__ __forceinline__ float wave_sum(float v) {
+    v = group_sum_last<64>(v);
+    return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+// a value of the last lane of the lower neighbouring group of LANES lanes (16 or 32), in the lanes of the upper one
+template <int LANES>
+__device__ __forceinline__ float from_lower_group(float v) {
+    static_assert(LANES == 16 || LANES == 32, "groups of 16 or 32 lanes");
+    return LANES == 16 ? dpp_f32<0x142, 0xA>(v) : dpp_f32<0x143, 0xC>(v);
+}
+
 }  // namespace btb

@@ -75,8 +75,7 @@ __device__ __forceinline__ void route_row_reg(const void* __restrict__ logits, s
         pr[s] = e < E ? expf(lv[s] - m) : 0.f;
         if (e < E) sum_p += pr[s];
     }
-    sum_p = group_sum<64>(sum_p);
-    sum_p = __shfl(sum_p, 0, WAVE);
+    sum_p = wave_sum(sum_p);
     unsigned long long key[P];
 #pragma unroll
     for (int s = 0; s < P; ++s) {

@@ -40,9 +40,9 @@ __device__ __forceinline__ uint32_t silu_pair(uint32_t g2, uint32_t u2) {
 
 // sum over a 256-thread block in a fixed order: each wave's DPP tree, then waves 0..3 in order
 __device__ __forceinline__ float block_sum256(float v, float* red) {
-    v = group_sum<64>(v);
+    v = group_sum_last<64>(v);
     const int wv = threadIdx.x >> 6;
-    if ((threadIdx.x & 63) == 0) red[wv] = v;
+    if ((threadIdx.x & 63) == 63) red[wv] = v;
     __syncthreads();
     const float s = ((red[0] + red[1]) + red[2]) + red[3];
     __syncthreads();

@@ -71,30 +71,32 @@ __device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typ
 #pragma unroll
     for (int j = 0; j < RPW; ++j)
         F::template tail<M>(p, ctx[j], (size_t)rows[j], sl, LPR, C, reinterpret_cast<const uint32_t*>(xs4), acc[j]);
+    // the row's sum is needed by the one lane that stores it: the group's last (group_sum_last)
+    constexpr int LAST = LPR - 1;
     if constexpr (EPI == E_GLU) {
 #pragma unroll
         for (int m = 0; m < M; ++m) {
-            const float g = bfround(group_sum<LPR>(acc[0][m]));
-            const float u = bfround(group_sum<LPR>(acc[RPW - 1][m]));
+            const float g = bfround(group_sum_last<LPR>(acc[0][m]));
+            const float u = bfround(group_sum_last<LPR>(acc[RPW - 1][m]));
             const float sg = bfround(g / (1.f + expf(-g)));
-            if (sl == 0 && outs[0] < Rout) y[(size_t)m * Rout + outs[0]] = f32_bf16(sg * u);
+            if (sl == LAST && outs[0] < Rout) y[(size_t)m * Rout + outs[0]] = f32_bf16(sg * u);
         }
-    } else if (EPI == E_GLU_SPLIT) {
+    } else if constexpr (EPI == E_GLU_SPLIT) {
 #pragma unroll
         for (int m = 0; m < M; ++m) {
-            const float mine = group_sum<LPR>(acc[0][m]);
-            const float other = __shfl_xor(mine, LPR, WAVE);  // the neighbouring row group's sum: the up row's
-            const float g = bfround(mine), u = bfround(other);
+            // the gate row's group is the lower neighbour of the up row's: the up group's last lane takes the gate's sum
+            const float mine = group_sum_last<LPR>(acc[0][m]);
+            const float g = bfround(from_lower_group<LPR>(mine)), u = bfround(mine);
             const float sg = bfround(g / (1.f + expf(-g)));
-            if (sl == 0 && ((lane / LPR) & 1) == 0 && outs[0] < Rout) y[(size_t)m * Rout + outs[0]] = f32_bf16(sg * u);
+            if (sl == LAST && ((lane / LPR) & 1) == 1 && outs[0] < Rout) y[(size_t)m * Rout + outs[0]] = f32_bf16(sg * u);
         }
     } else {
 #pragma unroll
         for (int j = 0; j < RPW; ++j)
 #pragma unroll
             for (int m = 0; m < M; ++m) {
-                const float s = group_sum<LPR>(acc[j][m]);
-                if (sl == 0 && outs[j] < R) y[(size_t)m * R + outs[j]] = f32_bf16(s);
+                const float s = group_sum_last<LPR>(acc[j][m]);
+                if (sl == LAST && outs[j] < R) y[(size_t)m * R + outs[j]] = f32_bf16(s);
             }
     }
 }

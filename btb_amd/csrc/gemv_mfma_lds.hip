@@ -495,8 +495,8 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
                         if (writer) reinterpret_cast<uint2*>(xa.h_out + (size_t)m * C)[i] = hb;
                     }
                 }
-                ss = group_sum<64>(ss);
-                if (lane == 0) red[m * 4 + (wv & 3)] = ss;
+                ss = group_sum_last<64>(ss);
+                if (lane == 63) red[m * 4 + (wv & 3)] = ss;
             }
         }
         __syncthreads();

@@ -192,7 +192,7 @@ __global__ void __launch_bounds__(64) norm_rope_kv_kernel(const uint16_t* __rest
         float ss = 0.f;
 #pragma unroll
         for (int e = 0; e < E; ++e) ss = fmaf(v[e], v[e], ss);
-        ss = group_sum<64>(ss);
+        ss = wave_sum(ss);
         const float rstd = rsqrtf(ss / (float)D + eps);
 #pragma unroll
         for (int e = 0; e < E; ++e) {

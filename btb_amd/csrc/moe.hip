@@ -64,8 +64,7 @@ __global__ void __launch_bounds__(64) moe_route_kernel(const void* __restrict__ 
         pr[e] = p;
         s += p;
     }
-    s = group_sum<64>(s);
-    s = __shfl(s, 0, WAVE);
+    s = wave_sum(s);
     for (int e = lane; e < E; e += WAVE) pr[e] = pr[e] / s;
     __syncthreads();
     // k rounds of the maximum; probabilities are >= 0, so -1 is below every live one and a pick is marked -2. A row of
@@ -301,9 +300,9 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(Stack stack, const uin
                 fma_span<F, 1, LPR, RPW, U, true>(raw, ctx, k0, sl, units, xs4, C / 8, acc);
             }
         }
-        const float g = bfround(group_sum<LPR>(acc[0][0]));
-        const float u = bfround(group_sum<LPR>(acc[1][0]));
-        if (sl == 0 && rows[0] < I) y[rows[0]] = glu_out<OSS>(g, u, glu, expert, rows[0], I);
+        const float g = bfround(group_sum_last<LPR>(acc[0][0]));  // in the group's last lane: the one that stores
+        const float u = bfround(group_sum_last<LPR>(acc[1][0]));
+        if (sl == LPR - 1 && rows[0] < I) y[rows[0]] = glu_out<OSS>(g, u, glu, expert, rows[0], I);
     }
 }
 
@@ -433,9 +432,9 @@ __global__ void __launch_bounds__(256) moe_gate_up_grouped_kernel(Stack stack, c
             }
 #pragma unroll
             for (int m = 0; m < M; ++m) {
-                const float g = bfround(group_sum<LPR>(acc[0][m]));
-                const float u = bfround(group_sum<LPR>(acc[1][m]));
-                if (sl == 0 && rows[0] < I && m < mc)
+                const float g = bfround(group_sum_last<LPR>(acc[0][m]));
+                const float u = bfround(group_sum_last<LPR>(acc[1][m]));
+                if (sl == LPR - 1 && rows[0] < I && m < mc)
                     h[(size_t)prs[m] * I + rows[0]] = glu_out<OSS>(g, u, glu, expert, rows[0], I);
             }
         }
@@ -558,7 +557,8 @@ __global__ void __launch_bounds__(256) moe_down_kernel(Stack stack, const uint16
                     const float wq = s_weight[q];
 #pragma unroll
                     for (int j = 0; j < RPW; ++j) {
-                        float d = bfround(group_sum<LPR>(acc[j][0]));  // the expert's down product, as the row's dtype
+                        // the expert's down product, as the row's dtype (in the group's last lane, which stores)
+                        float d = bfround(group_sum_last<LPR>(acc[j][0]));
                         if (bias != nullptr)
                             d = bfround(d + bf16_f32(bias[(size_t)(s_expert[q] & 0xFFFFF) * R + min(rows[j], R - 1)]));
                         out[j] = bfround(out[j] + bfround(d * wq));    // times its weight, added in bf16
@@ -568,7 +568,7 @@ __global__ void __launch_bounds__(256) moe_down_kernel(Stack stack, const uint16
         }
 #pragma unroll
         for (int j = 0; j < RPW; ++j)
-            if (sl == 0 && rows[j] < R) y[(size_t)token * R + rows[j]] = f32_bf16(out[j]);
+            if (sl == LPR - 1 && rows[j] < R) y[(size_t)token * R + rows[j]] = f32_bf16(out[j]);
     }
 }
 
