@@ -58,8 +58,9 @@ __host__ __device__ constexpr size_t stage_lds_bytes(int xmode, int M, int C) {
 // Leaves the rows in xs (a barrier included). 256 threads. `after_issue` is called once, right after the first loads
 // of the staging have been issued and before anything waits for them: the caller requests its first weights there,
 // so they travel while the staging's own (short) round trip and arithmetic run.
-// MR: the number of rows where the caller knows it at compile time (M is then MR), 0 otherwise.
-template <int XMODE, int MR = 0, class AfterIssue>
+// MR: the number of rows where the caller knows it at compile time (M is then MR), 0 otherwise. KEEP: the one-row
+// add + norm keeps its words in registers across the sum (see there).
+template <int XMODE, int MR = 0, bool KEEP = false, class AfterIssue>
 __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C, AfterIssue after_issue) {
     const int tid = threadIdx.x, nt = blockDim.x;
     if (XMODE == X_PLAIN) {
@@ -100,6 +101,61 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
         uint2* wkeep = rows4 + (size_t)M * n4;
         constexpr int PER = 3;  // words a thread holds at once: rows up to 3072 wide take one pass
         const bool writer = blockIdx.x == 0 && blockIdx.y == 0 && a.h_out != nullptr;
+        if (KEEP && MR == 1 && n4 <= PER * 256) {
+            // One row, one pass (the decode step's own launches): the thread's words stay in registers between the
+            // sum of squares and the scaling - nothing of them goes to LDS and comes back - and the one sum needs
+            // one barrier, not two (its four partial sums are not written again). The arithmetic, its order and the
+            // stores are the loop's below. Taken by the forms that widen in registers (the packed step 2.063 ->
+            // 2.054 ms); the bf16 kernels lose by it (qkv 7.40 -> 7.50 us, the step 2.026 -> 2.035 ms) and keep the
+            // loop.
+            uint2 hv[PER], yv[PER], wv[PER];
+            size_t hrow = 0;
+            if (a.ids != nullptr) hrow = (size_t)min(max(a.ids[0], 0), a.vocab - 1);
+            const uint2* hs = reinterpret_cast<const uint2*>(a.x + hrow * C);
+            const uint2* ys = a.y == nullptr ? hs : reinterpret_cast<const uint2*>(a.y);
+            const uint2* ws = reinterpret_cast<const uint2*>(a.norm_w);
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                const int i = min(q * 256 + tid, n4 - 1);
+                hv[q] = hs[i];
+                yv[q] = ys[i];
+                wv[q] = ws[i];
+            }
+            after_issue();
+            const bool has_y = a.y != nullptr;
+            float f[PER][4];
+            float ss = 0.f;
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                const bool live = q * 256 + tid < n4;
+                const float h4[4] = {bf16lo_f32(hv[q].x), bf16hi_f32(hv[q].x), bf16lo_f32(hv[q].y), bf16hi_f32(hv[q].y)};
+                const float g[4] = {bf16lo_f32(yv[q].x), bf16hi_f32(yv[q].x), bf16lo_f32(yv[q].y), bf16hi_f32(yv[q].y)};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const float sum = bfround(h4[e] + g[e]);
+                    f[q][e] = has_y ? sum : h4[e];
+                    const float sq = fmaf(f[q][e], f[q][e], ss);
+                    ss = live ? sq : ss;
+                }
+                if (writer)
+                    reinterpret_cast<uint2*>(a.h_out)[min(q * 256 + tid, n4 - 1)] =
+                        make_uint2(f32x2_bf16(f[q][0], f[q][1]), f32x2_bf16(f[q][2], f[q][3]));
+            }
+            ss = group_sum_last<64>(ss);
+            if ((tid & 63) == 63) red[tid >> 6] = ss;
+            __syncthreads();
+            const float rstd = rsqrtf((((red[0] + red[1]) + red[2]) + red[3]) / (float)C + a.eps);
+#pragma unroll
+            for (int q = 0; q < PER; ++q) {
+                const float g[4] = {bf16lo_f32(wv[q].x), bf16hi_f32(wv[q].x), bf16lo_f32(wv[q].y), bf16hi_f32(wv[q].y)};
+                float o[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) o[e] = f[q][e] * rstd * (a.centered ? 1.f + g[e] : g[e]);
+                rows4[min(q * 256 + tid, n4 - 1)] = make_uint2(f32x2_bf16(o[0], o[1]), f32x2_bf16(o[2], o[3]));
+            }
+            __syncthreads();
+            return;
+        }
         if (MR > 1 && n4 <= PER * 256) {
             // Several rows, each one pass: every row's words are requested before anything waits - and before the
             // caller's first weights, which travel behind them. Row by row (the loop below) a row's loads queue
@@ -223,7 +279,7 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
 
 template <int XMODE>
 __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C) {
-    stage_x<XMODE, 0>(xs, a, M, C, [] {});
+    stage_x<XMODE, 0, false>(xs, a, M, C, [] {});
 }
 
 // ------------------------------------------------------------------------------------------------------------

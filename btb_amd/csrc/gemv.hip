@@ -120,7 +120,7 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs x
     F::prepare(p);
 
     typename F::Raw first[U][RPW] = {};
-    stage_x<XMODE, M>(xs, xa, M, C, [&] {
+    stage_x<XMODE, M, sizeof(typename F::Raw) != 16>(xs, xa, M, C, [&] {
         // a wave with no tile requests the last tile's span and drops it: nothing here is conditional (see
         // load_span_always)
         typename F::RowCtx ctx[RPW];
