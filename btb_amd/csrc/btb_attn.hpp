@@ -52,7 +52,7 @@ __device__ __forceinline__ void head_finish(const HeadIn& in, bool has_wn, float
     const float c2[2] = {bf16lo_f32(in.cs), bf16hi_f32(in.cs)}, s2[2] = {bf16lo_f32(in.sn), bf16hi_f32(in.sn)};
 #pragma unroll
     for (int e = 0; e < 2; ++e) {
-        const float rot = __shfl_xor(v[e], 32, WAVE);
+        const float rot = xor32(v[e]);
         const float qc = bfround(v[e] * c2[e]);
         out[e] = f32_bf16(fmaf(sgn * rot, s2[e], qc));
     }

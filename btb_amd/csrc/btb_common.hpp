@@ -132,6 +132,13 @@ __device__ __forceinline__ float wave_sum(float v) {
     v = group_sum_last<64>(v);
     return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
+// lane l ^ 32's value, on the vector ALU: v_permlane32_swap of a register with itself leaves the lower half's values
+// in both halves of one result and the upper half's in both halves of the other. (__shfl_xor goes through the LDS unit.)
+__device__ __forceinline__ float xor32(float v) {
+    const int i = __builtin_bit_cast(int, v);
+    const auto r = __builtin_amdgcn_permlane32_swap(i, i, false, false);
+    return __builtin_bit_cast(float, (threadIdx.x & 32) ? r[0] : r[1]);
+}
 // a value of the last lane of the lower neighbouring group of LANES lanes (16 or 32), in the lanes of the upper one
 template <int LANES>
 __device__ __forceinline__ float from_lower_group(float v) {

@@ -624,8 +624,7 @@ __global__ void __launch_bounds__(KS * 64) gemv_mfma_lds(typename MF::Mat mat, c
             const int m = wv * 16 + li;
             if (half) {
                 // lanes of row groups 0, 1 hold gate sums, the lanes 32 further on the up sums of the same outputs
-                const f32x4 up = f32x4{__shfl_xor(s.x, 32, WAVE), __shfl_xor(s.y, 32, WAVE), __shfl_xor(s.z, 32, WAVE),
-                                       __shfl_xor(s.w, 32, WAVE)};
+                const f32x4 up = f32x4{xor32(s.x), xor32(s.y), xor32(s.z), xor32(s.w)};
                 if (m < M && lg < 2) {
                     // the arithmetic of the stand-alone fold over the two rounded outputs (silu_pair)
                     auto fold = [](float g, float u) {

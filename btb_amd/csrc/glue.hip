@@ -208,7 +208,7 @@ __global__ void __launch_bounds__(64) norm_rope_kv_kernel(const uint16_t* __rest
                          : (K + (size_t)(head - Hq) * hs + (size_t)slot * rs + lane * E);
 #pragma unroll
     for (int e = 0; e < E; ++e) {
-        const float rot = __shfl_xor(v[e], 32, WAVE);
+        const float rot = xor32(v[e]);
         const float qc = bfround(v[e] * bf16_f32(cp[e]));
         dst[e] = f32_bf16(fmaf(sgn * rot, bf16_f32(sp[e]), qc));
     }
