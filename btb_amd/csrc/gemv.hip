@@ -27,10 +27,11 @@ namespace btb {
 
 
 // one tile of gemv_stream: its RPW rows' sums over the M rows of x, written out. PRIMED: the tile's first span is
-// already in `first` (requested before x was staged).
+// already in `first` (requested before x was staged) and its rows' contexts in `first_ctx`.
 template <class F, int M, int LPR, int RPW, int U, int EPI, bool PRIMED>
-__device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typename F::Raw (&first)[U][RPW], int tile,
-                                          const uint4* xs4, uint16_t* __restrict__ y, int R, int C, int lane) {
+__device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typename F::Raw (&first)[U][RPW],
+                                          const typename F::RowCtx (&first_ctx)[RPW], int tile, const uint4* xs4,
+                                          uint16_t* __restrict__ y, int R, int C, int lane) {
     const int Rout = EPI == E_PLAIN ? R : R / 2;
     const int units = C / F::UW;         // units per row
     const int sl = lane % LPR;           // the lane's place among its row's lanes
@@ -42,7 +43,9 @@ __device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typ
 #pragma unroll
     for (int j = 0; j < RPW; ++j) {
         rows[j] = tile_row<LPR, RPW, EPI>(tile, j, lane, R, outs[j]);
-        ctx[j] = F::row_ctx(p, (size_t)rows[j], units);
+        // PRIMED: the rows' contexts were made where the span was requested - what a context asks of memory (pack12: the
+        // row's slice of the escape list) was asked for ahead of the weights, not after the staging's barrier
+        ctx[j] = PRIMED ? first_ctx[j] : F::row_ctx(p, (size_t)rows[j], units);
     }
     float acc[RPW][M];
 #pragma unroll
@@ -120,23 +123,24 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs x
     F::prepare(p);
 
     typename F::Raw first[U][RPW] = {};
+    typename F::RowCtx first_ctx[RPW];
     stage_x<XMODE, M, sizeof(typename F::Raw) != 16>(xs, xa, M, C, [&] {
         // a wave with no tile requests the last tile's span and drops it: nothing here is conditional (see
         // load_span_always)
-        typename F::RowCtx ctx[RPW];
 #pragma unroll
         for (int j = 0; j < RPW; ++j) {
             int out_row;
-            ctx[j] = F::row_ctx(p, (size_t)tile_row<LPR, RPW, EPI>(min(wave, ntiles - 1), j, lane, R, out_row), units);
+            first_ctx[j] =
+                F::row_ctx(p, (size_t)tile_row<LPR, RPW, EPI>(min(wave, ntiles - 1), j, lane, R, out_row), units);
         }
-        load_span_always<F, LPR, RPW, U>(first, ctx, 0, lane % LPR, units);
+        load_span_always<F, LPR, RPW, U>(first, first_ctx, 0, lane % LPR, units);
         F::prepare_finish(p);
     });
     const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
     if (wave >= ntiles) return;
-    gemv_tile<F, M, LPR, RPW, U, EPI, true>(p, first, wave, xs4, y, R, C, lane);
+    gemv_tile<F, M, LPR, RPW, U, EPI, true>(p, first, first_ctx, wave, xs4, y, R, C, lane);
     for (int tile = wave + nwaves; tile < ntiles; tile += nwaves)
-        gemv_tile<F, M, LPR, RPW, U, EPI, false>(p, first, tile, xs4, y, R, C, lane);
+        gemv_tile<F, M, LPR, RPW, U, EPI, false>(p, first, first_ctx, tile, xs4, y, R, C, lane);
 }
 
 // ------------------------------------------------------------------------------------------------------------
