@@ -28,7 +28,7 @@ struct FmtBf16 {
     };
     __device__ static __forceinline__ void prepare(Params&) {}
     __device__ static __forceinline__ void prepare_finish(Params&) {}
-    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
+    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units, int sl = 0) {
         return RowCtx{p.w + r * (size_t)units};
     }
     __device__ static __forceinline__ Raw load(const RowCtx& c, int unit) { return Raw{load_stream16(c.row + unit)}; }
@@ -65,6 +65,7 @@ struct FmtP12 {
         uint4 tbl;               // the table in registers: filled by prepare() on the device, not by the host
         const uint16_t* pairs;   // [256] the pair table made at upload (FmtP12G), or null
         uint32_t pair_reg;       // this thread's entry of it on its way to LDS (prepare -> prepare_finish)
+        const uint32_t* row_esc; // [rows][4] every row's first four escapes, a word each, made at upload, or null
     };
     struct Raw {
         uint4 lo;
@@ -74,8 +75,24 @@ struct FmtP12 {
         const uint4* lo;
         const uint2* hi4;
         uint4 table;
-        int e0, e1;  // the row's escapes: [e0, e1) of the list
+        int e0, e1;  // the row's escapes: [e0, e1) of the list; where the matrix has the rows' words: the lane's word
     };
+    // A row's words (row_esc, made at upload: btb_hip_p12_row_esc): its first ROW_ESC_SLOTS escapes, one a word - low
+    // byte in bits 0..7, true high byte in 8..15, column in 16..30 (ROW_ESC_NONE: no such escape) - and in bit 31 of
+    // every word of the row: the row has more escapes than words.
+    static constexpr uint32_t ROW_ESC_NONE = 0x7FFFu;
+    static constexpr int ROW_ESC_SLOTS = 4;
+    // The part of a row's context that comes out of memory: the lane's word of the row's words where the matrix has
+    // them (lane sl of the row's lanes: word min(sl, 3)), else the row's slice of the list. Two 4-byte loads from
+    // addresses chosen without a branch: a branch here makes the compiler wait for what was loaded before it, ahead
+    // of the row's weights.
+    __device__ static __forceinline__ void row_escapes(const Params& p, size_t r, int sl, RowCtx& c) {
+        const bool words = p.row_esc != nullptr;
+        const int32_t* base = words ? reinterpret_cast<const int32_t*>(p.row_esc) : p.row_ptr;
+        const size_t at = words ? r * ROW_ESC_SLOTS + (size_t)min(sl, ROW_ESC_SLOTS - 1) : r;
+        c.e0 = base[at];
+        c.e1 = base[words ? at : at + 1];
+    }
     // the table's 16 bytes as four registers, entry k in byte k
     __device__ static __forceinline__ uint4 load_table(const uint8_t* t) {
         uint32_t d[4];
@@ -88,13 +105,12 @@ struct FmtP12 {
     // once per kernel (or phase), before any row_ctx: the table's 16 bytes are read here and only here
     __device__ static __forceinline__ void prepare(Params& p) { p.tbl = load_table(p.table); }
     __device__ static __forceinline__ void prepare_finish(Params&) {}
-    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
+    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units, int sl = 0) {
         RowCtx c;
         c.lo = reinterpret_cast<const uint4*>(p.lo) + r * (size_t)units;
         c.hi4 = reinterpret_cast<const uint2*>(p.hi4) + r * (size_t)units;
         c.table = p.tbl;
-        c.e0 = p.row_ptr[r];
-        c.e1 = p.row_ptr[r + 1];
+        row_escapes(p, r, sl, c);
         return c;
     }
     __device__ static __forceinline__ Raw load(const RowCtx& c, int unit) {
@@ -127,23 +143,43 @@ struct FmtP12 {
         widen8(c.table, r.codes.x, r.lo.x, r.lo.y, w);
         widen8(c.table, r.codes.y, r.lo.z, r.lo.w, w + 4);
     }
-    // the row's escapes, spread over the row's lanes: the streamed term out, the true term in
+    // The row's escapes, spread over the row's lanes (escape k of the row: lane k % lpr, in list order): the streamed
+    // term out, the true term in. Out of the list that is three round trips one behind the other - the row's slice,
+    // its entries, the low bytes they name - at the end of a tile, where a wave has nothing left to hide them behind:
+    // a tenth of the packed decode step, and a launch ends with its slowest wave, so it is not enough to spare most
+    // rows the walk. Hence the rows' words: a row's first four escapes stand in four words of the row's own, whose
+    // address the row number gives, and lane k < 4 asks for word k ahead of the row's weights - it has all it needs
+    // when the products are done. Only a row with more than four escapes (one in six thousand of a N(0, 0.02) matrix
+    // 2560 wide) walks the list, from its fifth entry on.
+    template <int M>
+    __device__ static __forceinline__ void esc_term(const RowCtx& c, int C, const uint32_t* xs, float (&acc)[M], int col,
+                                                    uint32_t val, uint32_t lo) {
+        const uint32_t t15 = c.table.w >> 24;
+        const uint16_t* x16 = reinterpret_cast<const uint16_t*>(xs);
+        const float streamed = bits_f32((t15 << 24) | (lo << 16));
+        const float truth = bits_f32((val << 24) | (lo << 16));
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            const float xv = bf16_f32(x16[(size_t)m * C + col]);
+            acc[m] = fmaf(truth, xv, fmaf(-streamed, xv, acc[m]));
+        }
+    }
     template <int M>
     __device__ static __forceinline__ void tail(const Params& p, const RowCtx& c, size_t r, int sl, int lpr, int C,
                                                 const uint32_t* xs, float (&acc)[M]) {
-        const uint32_t t15 = c.table.w >> 24;
-        const uint16_t* x16 = reinterpret_cast<const uint16_t*>(xs);
-        for (int e = c.e0 + sl; e < c.e1; e += lpr) {
+        int e0 = c.e0, e1 = c.e1, from = sl;
+        if (p.row_esc != nullptr) {  // uniform
+            const uint32_t rec = (uint32_t)c.e0, col = (rec >> 16) & 0x7FFFu;
+            if (sl < ROW_ESC_SLOTS && col != ROW_ESC_NONE)
+                esc_term<M>(c, C, xs, acc, (int)col, (rec >> 8) & 0xFFu, rec & 0xFFu);
+            if ((rec >> 31) == 0u) return;
+            e0 = p.row_ptr[r];
+            e1 = p.row_ptr[r + 1];
+            from = sl < ROW_ESC_SLOTS ? sl + lpr : sl;  // the first four are done
+        }
+        for (int e = e0 + from; e < e1; e += lpr) {
             const size_t i = (size_t)p.esc_idx[e];
-            const uint32_t lo = p.lo[i];
-            const float streamed = bits_f32((t15 << 24) | (lo << 16));
-            const float truth = bits_f32(((uint32_t)p.esc_val[e] << 24) | (lo << 16));
-            const int col = (int)(i - r * (size_t)C);
-#pragma unroll
-            for (int m = 0; m < M; ++m) {
-                const float xv = bf16_f32(x16[(size_t)m * C + col]);
-                acc[m] = fmaf(truth, xv, fmaf(-streamed, xv, acc[m]));
-            }
+            esc_term<M>(c, C, xs, acc, (int)(i - r * (size_t)C), (uint32_t)p.esc_val[e], (uint32_t)p.lo[i]);
         }
     }
 };
@@ -166,13 +202,12 @@ struct FmtP12G : FmtP12 {
     __device__ static __forceinline__ void prepare_finish(Params& p) {
         if (threadIdx.x < 256) pair_table()[threadIdx.x] = (uint16_t)p.pair_reg;
     }
-    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
+    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units, int sl = 0) {
         RowCtx c;
         c.lo = reinterpret_cast<const uint4*>(p.lo) + r * (size_t)units;
         c.hi4 = reinterpret_cast<const uint2*>(p.hi4) + r * (size_t)units;
         c.table = make_uint4(0u, 0u, 0u, 0u);  // not read: the lookups go through LDS, an escape streams as slot 15 = 0
-        c.e0 = p.row_ptr[r];
-        c.e1 = p.row_ptr[r + 1];
+        row_escapes(p, r, sl, c);
         return c;
     }
     // eight weights: codes c (weight k in nibble k), low bytes l0 (weights 0..3), l1 (4..7)
@@ -221,7 +256,7 @@ struct FmtF8 {
     };
     __device__ static __forceinline__ void prepare(Params&) {}
     __device__ static __forceinline__ void prepare_finish(Params&) {}
-    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
+    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units, int sl = 0) {
         return RowCtx{reinterpret_cast<const uint4*>(p.w) + r * (size_t)units, p.scales + (r / p.bm) * (size_t)p.sc,
                       p.upb, p.magic};
     }
@@ -272,7 +307,7 @@ struct FmtMx4 {
     };
     __device__ static __forceinline__ void prepare(Params&) {}
     __device__ static __forceinline__ void prepare_finish(Params&) {}
-    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units) {
+    __device__ static __forceinline__ RowCtx row_ctx(const Params& p, size_t r, int units, int sl = 0) {
         return RowCtx{reinterpret_cast<const uint4*>(p.blocks) + r * (size_t)units, p.scales + r * (size_t)units};
     }
     __device__ static __forceinline__ Raw load(const RowCtx& c, int unit) {

@@ -45,7 +45,7 @@ __device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typ
         rows[j] = tile_row<LPR, RPW, EPI>(tile, j, lane, R, outs[j]);
         // PRIMED: the rows' contexts were made where the span was requested - what a context asks of memory (pack12: the
         // row's slice of the escape list) was asked for ahead of the weights, not after the staging's barrier
-        ctx[j] = PRIMED ? first_ctx[j] : F::row_ctx(p, (size_t)rows[j], units);
+        ctx[j] = PRIMED ? first_ctx[j] : F::row_ctx(p, (size_t)rows[j], units, sl);
     }
     float acc[RPW][M];
 #pragma unroll
@@ -131,7 +131,8 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs x
         for (int j = 0; j < RPW; ++j) {
             int out_row;
             first_ctx[j] =
-                F::row_ctx(p, (size_t)tile_row<LPR, RPW, EPI>(min(wave, ntiles - 1), j, lane, R, out_row), units);
+                F::row_ctx(p, (size_t)tile_row<LPR, RPW, EPI>(min(wave, ntiles - 1), j, lane, R, out_row), units,
+                           lane % LPR);
         }
         load_span_always<F, LPR, RPW, U>(first, first_ctx, 0, lane % LPR, units);
         F::prepare_finish(p);
@@ -359,19 +360,21 @@ static bool norm_on_mfma(const XArgs& xa, size_t R, size_t C, size_t M, bool glu
 }
 
 static int32_t p12_params(const void* lo, const void* hi4, const void* table, const void* pairs, const void* esc_idx,
-                          const void* esc_val, size_t n_esc, const void* row_ptr, size_t R, size_t C,
-                          FmtP12::Params* p) {
+                          const void* esc_val, size_t n_esc, const void* row_ptr, const void* row_esc, size_t R,
+                          size_t C, FmtP12::Params* p) {
     if (lo == nullptr || hi4 == nullptr || table == nullptr || row_ptr == nullptr) return ERR_NULL;
     if (reinterpret_cast<uintptr_t>(pairs) & 1u) return ERR_DOMAIN;
     if (n_esc > 0 && (esc_idx == nullptr || esc_val == nullptr)) return ERR_NULL;
     if (R * C > 0x7FFFFFFFull) return ERR_DOMAIN;  // the escape indices are int32
     if (!aligned16(lo) || (reinterpret_cast<uintptr_t>(hi4) & 7u) || (reinterpret_cast<uintptr_t>(row_ptr) & 3u) ||
-        (reinterpret_cast<uintptr_t>(esc_idx) & 3u))
+        (reinterpret_cast<uintptr_t>(esc_idx) & 3u) || (reinterpret_cast<uintptr_t>(row_esc) & 3u))
         return ERR_DOMAIN;
+    if (row_esc != nullptr && C > FmtP12::ROW_ESC_NONE) return ERR_DOMAIN;  // a word's column field
     *p = FmtP12::Params{static_cast<const uint8_t*>(lo),      static_cast<const uint8_t*>(hi4),
                         static_cast<const uint8_t*>(table),   static_cast<const int32_t*>(esc_idx),
                         static_cast<const uint8_t*>(esc_val), static_cast<const int32_t*>(row_ptr),
-                        make_uint4(0, 0, 0, 0), static_cast<const uint16_t*>(pairs), 0u};
+                        make_uint4(0, 0, 0, 0), static_cast<const uint16_t*>(pairs), 0u,
+                        static_cast<const uint32_t*>(row_esc)};
     return OK;
 }
 
@@ -469,15 +472,15 @@ int32_t btb_hip_gemv_bf16_embed_norm(const void* w, const void* table, const int
 }
 
 int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* pairs, const void* esc_idx,
-                         const void* esc_val, size_t n_esc, const void* row_ptr, const void* x, void* y, size_t R,
-                         size_t C, size_t M, void* stream) {
+                         const void* esc_val, size_t n_esc, const void* row_ptr, const void* row_esc, const void* x,
+                         void* y, size_t R, size_t C, size_t M, void* stream) {
     if (x == nullptr || y == nullptr || lo == nullptr || hi4 == nullptr || table == nullptr || row_ptr == nullptr)
         return ERR_NULL;
     if (n_esc > 0 && (esc_idx == nullptr || esc_val == nullptr)) return ERR_NULL;
     int32_t rc = check_dims(R, C, M, FmtP12::UW);
     if (rc != OK) return rc;
     FmtP12::Params p;
-    rc = p12_params(lo, hi4, table, pairs, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
+    rc = p12_params(lo, hi4, table, pairs, esc_idx, esc_val, n_esc, row_ptr, row_esc, R, C, &p);
     if (rc != OK) return rc;
     if (!aligned16(x) || !aligned2(y)) return ERR_DOMAIN;
     // the verify widths: the matrix cores. Weights straight into LDS, 16 rows of x a pass, where that kernel has a
@@ -522,7 +525,7 @@ int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, con
 
 int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table, const void* pairs,
                               const void* esc_idx, const void* esc_val, size_t n_esc, const void* row_ptr,
-                              const void* h_in, const void* y,
+                              const void* row_esc, const void* h_in, const void* y,
                               const void* norm_w, float eps, int32_t centered, void* h_out, void* out, size_t R,
                               size_t C, size_t M, int32_t glu, void* stream) {
     if (out == nullptr) return ERR_NULL;
@@ -530,7 +533,7 @@ int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table
     XArgs xa;
     int32_t rc = norm_args(h_in, y, norm_w, eps, centered, h_out, &xa);
     if (rc == ERR_NULL) return rc;
-    const int32_t rp = p12_params(lo, hi4, table, pairs, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
+    const int32_t rp = p12_params(lo, hi4, table, pairs, esc_idx, esc_val, n_esc, row_ptr, row_esc, R, C, &p);
     if (rp == ERR_NULL) return rp;
     if (rc != OK) return rc;
     if (rp != OK) return rp;
@@ -547,7 +550,7 @@ int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table
 
 int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void* table, const void* pairs,
                                     const void* esc_idx, const void* esc_val, size_t n_esc, const void* row_ptr,
-                                    const void* embed,
+                                    const void* row_esc, const void* embed,
                                     const int32_t* ids, size_t vocab, const void* norm_w, float eps, int32_t centered,
                                     void* h_out, void* out, size_t R, size_t C, size_t M, void* stream) {
     if (out == nullptr) return ERR_NULL;
@@ -555,7 +558,7 @@ int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void*
     XArgs xa;
     int32_t rc = embed_args(embed, ids, vocab, norm_w, eps, centered, h_out, &xa);
     if (rc == ERR_NULL) return rc;
-    const int32_t rp = p12_params(lo, hi4, table, pairs, esc_idx, esc_val, n_esc, row_ptr, R, C, &p);
+    const int32_t rp = p12_params(lo, hi4, table, pairs, esc_idx, esc_val, n_esc, row_ptr, row_esc, R, C, &p);
     if (rp == ERR_NULL) return rp;
     if (rc != OK) return rc;
     if (rp != OK) return rp;

@@ -153,6 +153,38 @@ __global__ void __launch_bounds__(256) p12_pairs_kernel(const uint8_t* __restric
 
 extern "C" {
 
+// a row's first four escapes as four words of the row's own (FmtP12::row_escapes reads them, FmtP12::tail uses them)
+__global__ void __launch_bounds__(256) p12_row_esc_kernel(const uint8_t* __restrict__ lo, const int32_t* __restrict__ esc_idx,
+                                                          const uint8_t* __restrict__ esc_val,
+                                                          const int32_t* __restrict__ row_ptr, int rows, int cols,
+                                                          uint32_t* __restrict__ out) {
+    const int r = blockIdx.x * 256 + threadIdx.x;
+    if (r >= rows) return;
+    const int e0 = row_ptr[r], e1 = row_ptr[r + 1];
+    const uint32_t more = e1 - e0 > FmtP12::ROW_ESC_SLOTS ? 0x80000000u : 0u;
+    for (int k = 0; k < FmtP12::ROW_ESC_SLOTS; ++k) {
+        uint32_t w = FmtP12::ROW_ESC_NONE << 16;
+        if (e0 + k < e1) {
+            const size_t i = (size_t)esc_idx[e0 + k];
+            w = (uint32_t)lo[i] | ((uint32_t)esc_val[e0 + k] << 8) | ((uint32_t)(i - (size_t)r * cols) << 16);
+        }
+        out[(size_t)r * FmtP12::ROW_ESC_SLOTS + k] = w | more;
+    }
+}
+
+int32_t btb_hip_p12_row_esc(const void* lo, const void* esc_idx, const void* esc_val, size_t n_esc, const void* row_ptr,
+                            size_t rows, size_t cols, void* row_esc, void* stream) {
+    if (lo == nullptr || row_ptr == nullptr || row_esc == nullptr) return ERR_NULL;
+    if (n_esc > 0 && (esc_idx == nullptr || esc_val == nullptr)) return ERR_NULL;
+    if (rows == 0 || cols == 0 || cols > FmtP12::ROW_ESC_NONE || rows * cols > 0x7FFFFFFFull) return ERR_DOMAIN;
+    if (!al(esc_idx, 4) || !al(row_ptr, 4) || !al(row_esc, 4)) return ERR_DOMAIN;
+    hipLaunchKernelGGL(p12_row_esc_kernel, dim3((unsigned)((rows + 255) / 256)), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), static_cast<const uint8_t*>(lo),
+                       static_cast<const int32_t*>(esc_idx), static_cast<const uint8_t*>(esc_val),
+                       static_cast<const int32_t*>(row_ptr), (int)rows, (int)cols, static_cast<uint32_t*>(row_esc));
+    return hip_status(hipGetLastError(), "p12_row_esc launch");
+}
+
 int32_t btb_hip_p12_pairs(const void* table, void* pairs, void* stream) {
     if (table == nullptr || pairs == nullptr) return ERR_NULL;
     if (!al(pairs, 2)) return ERR_DOMAIN;
@@ -204,7 +236,7 @@ int32_t btb_hip_p12_widen(const void* lo, const void* hi4, const void* table, co
     hipStream_t st = static_cast<hipStream_t>(stream);
     FmtP12::Params p{static_cast<const uint8_t*>(lo),      static_cast<const uint8_t*>(hi4),
                      static_cast<const uint8_t*>(table),   static_cast<const int32_t*>(esc_idx),
-                     static_cast<const uint8_t*>(esc_val), nullptr, make_uint4(0, 0, 0, 0)};
+                     static_cast<const uint8_t*>(esc_val), nullptr, make_uint4(0, 0, 0, 0), nullptr, 0u, nullptr};
     const size_t threads = n / FmtP12::UW + 1;
     hipLaunchKernelGGL(p12_widen_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, st, p, n,
                        static_cast<uint16_t*>(out));

@@ -40,12 +40,13 @@ SIGNATURES: dict[str, tuple[Any, list[Any]]] = {
     "btb_hip_gemv_glu_silu_bf16": (_i32, [_vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_gemv_bf16_norm": (_i32, [_vp, _vp, _vp, _vp, ctypes.c_float, _i32, _vp, _vp, _sz, _sz, _sz, _i32, _vp]),
     "btb_hip_gemv_bf16_embed_norm": (_i32, [_vp, _vp, _vp, _sz, _vp, ctypes.c_float, _i32, _vp, _vp, _sz, _sz, _sz, _vp]),
-    "btb_hip_gemv_p12_embed_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _vp, ctypes.c_float,
+    "btb_hip_gemv_p12_embed_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _vp, ctypes.c_float,
                                            _i32, _vp, _vp, _sz, _sz, _sz, _vp]),
-    "btb_hip_gemv_p12_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, ctypes.c_float, _i32, _vp,
+    "btb_hip_gemv_p12_norm": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _i32, _vp,
                                      _vp, _sz, _sz, _sz, _i32, _vp]),
-    "btb_hip_gemv_p12": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
+    "btb_hip_gemv_p12": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp, _sz, _vp, _vp, _vp, _vp, _sz, _sz, _sz, _vp]),
     "btb_hip_p12_pairs": (_i32, [_vp, _vp, _vp]),
+    "btb_hip_p12_row_esc": (_i32, [_vp, _vp, _vp, _sz, _vp, _sz, _sz, _vp, _vp]),
     "btb_hip_p12_row_ptr": (_i32, [_vp, _sz, _sz, _sz, _vp, _vp]),
     "btb_hip_p12_check": (_i32, [_vp, _sz, _sz, _vp, _vp]),
     "btb_hip_p12_widen": (_i32, [_vp, _vp, _vp, _vp, _vp, _sz, _sz, _vp, _vp]),
@@ -325,7 +326,7 @@ class HipCard(CardLaunch):
             ne = int(w.esc_idx.numel())
             self._call("btb_hip_gemv_p12_norm", _p(w.lo), _p(w.hi4), _p(w.table), self._pairs(w),
                        _p(w.esc_idx) if ne else None, _p(w.esc_val) if ne else None, ne, _p(w.row_ptr),
-                       _p(h_in), p(y), _p(norm_w), float(eps), int(centered), p(h_out), _p(out), R, C,
+                       self._row_esc(w), _p(h_in), p(y), _p(norm_w), float(eps), int(centered), p(h_out), _p(out), R, C,
                        M, int(glu), _stream())
         return out
 
@@ -351,7 +352,7 @@ class HipCard(CardLaunch):
             ne = int(w.esc_idx.numel())
             self._call("btb_hip_gemv_p12_embed_norm", _p(w.lo), _p(w.hi4), _p(w.table), self._pairs(w),
                        _p(w.esc_idx) if ne else None, _p(w.esc_val) if ne else None, ne, _p(w.row_ptr),
-                       _p(table), _p(ids), vocab, _p(norm_w), float(eps), int(centered), p(h_out),
+                       self._row_esc(w), _p(table), _p(ids), vocab, _p(norm_w), float(eps), int(centered), p(h_out),
                        _p(out), R, C, M, _stream())
         return out
 
@@ -382,6 +383,31 @@ class HipCard(CardLaunch):
         t = getattr(w, "pairs", None)
         return None if t is None else _p(t)
 
+    @staticmethod
+    def _row_esc(w: Any) -> ctypes.c_void_p | None:
+        t = getattr(w, "row_esc", None)
+        return None if t is None else _p(t)
+
+    def p12_row_esc(self, lo: torch.Tensor, esc_idx: torch.Tensor, esc_val: torch.Tensor, row_ptr: torch.Tensor,
+                    rows: int, cols: int) -> torch.Tensor | None:
+        """int32 [rows, 4] (read as u32): every row's first four escapes, a word each (low byte, true high byte,
+        column; bit 31: the row has more), which the matvecs ask for ahead of the row's weights (built once at upload).
+        None for rows wider than 32767, whose columns a word cannot hold: the matvecs then walk the list."""
+        if cols > 0x7FFF:
+            return None
+        self._need(lo, torch.uint8, "lo")
+        self._need(esc_idx, torch.int32, "esc_idx")
+        self._need(esc_val, torch.uint8, "esc_val")
+        self._need(row_ptr, torch.int32, "row_ptr")
+        if row_ptr.numel() != rows + 1 or lo.numel() != rows * cols or esc_val.numel() != esc_idx.numel():
+            raise ValueError("[hip] p12_row_esc: lo holds rows * cols bytes, row_ptr rows + 1 entries, the list's two "
+                             "arrays one entry an escape")
+        out = torch.empty(rows, 4, dtype=torch.int32, device=lo.device)
+        ne = int(esc_idx.numel())
+        self._call("btb_hip_p12_row_esc", _p(lo), _p(esc_idx) if ne else None, _p(esc_val) if ne else None, ne,
+                   _p(row_ptr), rows, cols, _p(out), _stream())
+        return out
+
     def p12_pairs(self, table: torch.Tensor) -> torch.Tensor:
         """int16 [256] (read as u16): the high bytes of the two weights each byte of codes stands for, the escape code
         as 0 (built once at upload; the matvecs keep a copy in LDS)"""
@@ -410,7 +436,7 @@ class HipCard(CardLaunch):
         ne = int(w.esc_idx.numel())
         self._call("btb_hip_gemv_p12", _p(w.lo), _p(w.hi4), _p(w.table), self._pairs(w),
                    _p(w.esc_idx) if ne else None, _p(w.esc_val) if ne else None, ne, _p(w.row_ptr),
-                   _p(x2), _p(y), R, C, M, _stream())
+                   self._row_esc(w), _p(x2), _p(y), R, C, M, _stream())
         return y
 
     def p12_widen(self, lo, hi4, table, esc_idx, esc_val, n: int, shape: Sequence[int],

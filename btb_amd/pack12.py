@@ -161,14 +161,15 @@ def check_escapes(esc_idx: torch.Tensor, esc_val: torch.Tensor, n: int) -> None:
 
 
 class P12Weight:
-    """One packed matrix on the GPU as the kernels read it; `shape` = (rows, cols). Two arrays are made here, once, by
-    the card: `row_ptr[r]`, the index of the first escape at or past row r's first weight (int32 [rows + 1]), and
-    `pairs`, the 256 two-byte entries the matvecs look a byte of codes up in. The table is the matrix's own copy with
+    """One packed matrix on the GPU as the kernels read it; `shape` = (rows, cols). Three arrays are made here, once, by
+    the card: `row_ptr[r]`, the index of the first escape at or past row r's first weight (int32 [rows + 1]), `pairs`,
+    the 256 two-byte entries the matvecs look a byte of codes up in, and `row_esc`, every row's first four escapes as
+    four words of the row's own (None for rows wider than 32767). The table is the matrix's own copy with
     slot 15 - the escape code, which names no table entry - set to 0: a store that left another byte there (0x7F or
     0xFF would make the streamed stand-in of an escaped weight inf or NaN, and its correction NaN) is as good as one
     that wrote the 0 the packer writes."""
 
-    __slots__ = ("esc_idx", "esc_val", "hi4", "lo", "pairs", "row_ptr", "shape", "table")
+    __slots__ = ("esc_idx", "esc_val", "hi4", "lo", "pairs", "row_esc", "row_ptr", "shape", "table")
 
     def __init__(self, lo, hi4, table, esc_idx, esc_val, rows: int, cols: int, card: Any) -> None:
         dev = lo.device
@@ -190,6 +191,7 @@ class P12Weight:
         card.p12_check(self.esc_idx, n)
         self.row_ptr = card.p12_row_ptr(self.esc_idx, rows, cols)
         self.pairs = card.p12_pairs(self.table)
+        self.row_esc = card.p12_row_esc(self.lo, self.esc_idx, self.esc_val, self.row_ptr, rows, cols)
 
     @classmethod
     def pack(cls, w: torch.Tensor, card: Any) -> "P12Weight":
@@ -198,7 +200,8 @@ class P12Weight:
 
     @property
     def nbytes(self) -> int:
-        return (self.lo.numel() + self.hi4.numel() + 16 + 512 + 5 * self.esc_idx.numel() + 4 * self.row_ptr.numel())
+        return (self.lo.numel() + self.hi4.numel() + 16 + 512 + 5 * self.esc_idx.numel() + 4 * self.row_ptr.numel()
+                + (0 if self.row_esc is None else 4 * self.row_esc.numel()))
 
     def __repr__(self) -> str:
         return f"P12Weight[{self.shape[0]}, {self.shape[1]}, {self.esc_idx.numel()} escapes]"

@@ -100,26 +100,29 @@ int32_t btb_hip_gemv_bf16_embed_norm(const void* w, const void* table, const int
 /* The matvec over a pack12 matrix (n = R * C weights): lo u8[n], hi4 u8[(n + 1) / 2] (weight 2k in the low nibble
  * of byte k), table u8[16], esc_idx i32[n_esc] strictly ascending, esc_val u8[n_esc] - the arrays of
  * btb_gemv_p12_rows (native/src/lib.rs:114-135), on the device, the list validated at upload by btb_hip_p12_check -
- * plus two arrays made once at upload: row_ptr i32[R + 1] from btb_hip_p12_row_ptr and pairs u16[256] from
- * btb_hip_p12_pairs (NULL: the table is looked up in registers instead, a slower kernel with the same bits).
+ * plus three arrays made once at upload: row_ptr i32[R + 1] from btb_hip_p12_row_ptr, pairs u16[256] from
+ * btb_hip_p12_pairs (NULL: the table is looked up in registers instead, a slower kernel with the same bits) and
+ * row_esc u32[4 R] from btb_hip_p12_row_esc (NULL: every escape is fetched through the list at the end of its row's
+ * tile, slower with the same bits; with it C <= 32767).
  * x [M, C] bf16, y [M, R] bf16; C a multiple of 16, lo 16-byte and hi4 8-byte aligned. The reference has no card
  * kernel for this form (it widens a packed layer to bf16 before the card holds it: btb/engine/tiers.py:1200-1216). */
 int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* pairs, const void* esc_idx,
-                         const void* esc_val, size_t n_esc, const void* row_ptr, const void* x, void* y, size_t R,
-                         size_t C, size_t M, void* stream);
+                         const void* esc_val, size_t n_esc, const void* row_ptr, const void* row_esc, const void* x,
+                         void* y, size_t R, size_t C, size_t M, void* stream);
 
 /* btb_hip_gemv_bf16_norm over a pack12 matrix (the arrays of btb_hip_gemv_p12). */
 int32_t btb_hip_gemv_p12_norm(const void* lo, const void* hi4, const void* table, const void* pairs,
                               const void* esc_idx, const void* esc_val, size_t n_esc, const void* row_ptr,
-                              const void* h_in, const void* y, const void* norm_w, float eps, int32_t centered,
-                              void* h_out, void* out, size_t R, size_t C, size_t M, int32_t glu, void* stream);
+                              const void* row_esc, const void* h_in, const void* y, const void* norm_w, float eps,
+                              int32_t centered, void* h_out, void* out, size_t R, size_t C, size_t M, int32_t glu,
+                              void* stream);
 
 /* btb_hip_gemv_bf16_embed_norm over a pack12 matrix (`table` is the matrix's 16 high bytes, `embed` the embedding). */
 int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void* table, const void* pairs,
                                     const void* esc_idx, const void* esc_val, size_t n_esc, const void* row_ptr,
-                                    const void* embed, const int32_t* ids, size_t vocab, const void* norm_w, float eps,
-                                    int32_t centered, void* h_out, void* out, size_t R, size_t C, size_t M,
-                                    void* stream);
+                                    const void* row_esc, const void* embed, const int32_t* ids, size_t vocab,
+                                    const void* norm_w, float eps, int32_t centered, void* h_out, void* out, size_t R,
+                                    size_t C, size_t M, void* stream);
 
 /* pairs[b] = table[b & 15] | table[b >> 4] << 8 for every byte b of codes, the escape code's slot 15 taken as 0: the
  * high bytes of the two weights a byte of codes stands for, so that the matvec turns a byte of codes into two high
@@ -127,6 +130,14 @@ int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void*
  * weight then streams as (0, low byte) and the escape list puts its true value in (the matrix should carry 0 in
  * table[15], as the packer writes it: the kernels that look the table up in registers stream table[15] there). */
 int32_t btb_hip_p12_pairs(const void* table, void* pairs, void* stream);
+
+/* row_esc[4 r + k] = row r's escape k (k = 0..3) as one word: the weight's low byte in bits 0..7, its true high byte
+ * in 8..15, its column in 16..30 (0x7FFF: the row has no such escape); bit 31 of all four words: the row has more
+ * than four. The matvec asks for a row's words ahead of the row's weights, so an escape costs it no trip to memory of
+ * its own at the end of the row (the list does: its slice, its entries, the low bytes they name). Made once at upload
+ * from the list, the low bytes and row_ptr; cols <= 32767 (BTB_ERR_DOMAIN beyond). No counterpart in the reference. */
+int32_t btb_hip_p12_row_esc(const void* lo, const void* esc_idx, const void* esc_val, size_t n_esc, const void* row_ptr,
+                            size_t rows, size_t cols, void* row_esc, void* stream);
 
 /* row_ptr[r] = how many escapes lie below weight r * cols, r = 0..rows: the per-row slices of the escape list the
  * matvec reads. Run once when a packed matrix is uploaded; replaces the per-call search of p12_cursors

@@ -97,8 +97,8 @@ def test_format_refusals(card):
     assert L.btb_hip_gemv_mxfp4(None, p(z), p(x), p(y), 4, 64, 1, None) == -1
     assert L.btb_hip_gemv_fp8(p(z), p(s), 3, 1, p(x), p(y), 4, 64, 1, None) == -6       # 3 does not divide 4
     assert L.btb_hip_gemv_fp8(p(z), p(s), 1, 8, p(x), p(y), 4, 64, 1, None) == -6       # 8-column blocks: not 16
-    assert L.btb_hip_gemv_p12(p(z), p(z), p(z), None, None, None, 2, p(s), p(x), p(y), 4, 64, 1, None) == -1
-    assert L.btb_hip_gemv_p12(p(z), p(z), p(z), None, None, None, 0, p(s), p(x), p(y), 4, 60, 1, None) == -6  # C % 16
+    assert L.btb_hip_gemv_p12(p(z), p(z), p(z), None, None, None, 2, p(s), None, p(x), p(y), 4, 64, 1, None) == -1
+    assert L.btb_hip_gemv_p12(p(z), p(z), p(z), None, None, None, 0, p(s), None, p(x), p(y), 4, 60, 1, None) == -6  # C % 16
 
 
 # ---- the verify widths (M >= 8): FP8 and MXFP4 widened into bf16 fragments for the matrix cores -------------------
@@ -424,6 +424,81 @@ def test_pair_table_made_at_upload(card):
     tb[15] = 0x7F
     pw = P12Weight(lo, hi4, tb, ei, ev, 32, 64, card)
     assert int(pw.table[15]) == 0 and int(tb[15]) == 0x7F and pw.pairs.numel() == 256   # its own copy, the caller's left
+
+
+def escapes_in_rows(R, C, counts, seed):
+    """a bf16 matrix whose row r holds counts[r % len(counts)] forced escapes (rare high bytes, low bytes of both
+    halves) at scattered columns"""
+    w = weights_bf16(R, C, seed=seed)
+    wb = bits16(w).copy()
+    rng = np.random.default_rng(seed)
+    for r in range(R):
+        k = counts[r % len(counts)]
+        if k:
+            cols = np.sort(rng.choice(C, size=k, replace=False))
+            wb[r, cols] = (wb[r, cols] & 0x00FF) | ((0x20 + (np.arange(k) + r) % 40).astype(np.uint16) << 8)
+    return torch.from_numpy(wb.view(np.int16)).view(torch.bfloat16)
+
+
+def test_rows_words_made_at_upload(card):
+    """row_esc[r, k] = row r's escape k as (low byte, true high byte << 8, column << 16), 0x7FFF for the column where
+    the row has no such escape, bit 31 of all four words where it has more than four; rows too wide for a word's
+    column field get none"""
+    R, C = 48, 272
+    w = escapes_in_rows(R, C, [0, 1, 2, 4, 5, 9, 0, 3], seed=390)
+    lo, hi4, tb, ei, ev = (t_.cuda() for t_ in pack12.pack_bf16(w))
+    pw = P12Weight(lo, hi4, tb, ei, ev, R, C, card)
+    got = pw.row_esc.cpu().numpy().view(np.uint32)
+    idx, val, lob = ei.cpu().numpy().astype(np.int64), ev.cpu().numpy(), lo.cpu().numpy().reshape(-1)
+    want = np.zeros((R, 4), dtype=np.uint32)
+    for r in range(R):
+        mine = np.flatnonzero((idx >= r * C) & (idx < (r + 1) * C))
+        for k in range(4):
+            if k < mine.size:
+                e = mine[k]
+                want[r, k] = int(lob[idx[e]]) | (int(val[e]) << 8) | (int(idx[e] - r * C) << 16)
+            else:
+                want[r, k] = 0x7FFF << 16
+        if mine.size > 4:
+            want[r] |= 0x80000000
+    assert np.array_equal(got, want)
+    assert (got[:, 0] >> 31).sum() > 0 and ((got[:, 0] >> 16) & 0x7FFF == 0x7FFF).sum() > 0   # both kinds of row met
+    assert card.p12_row_esc(lo, ei, ev, pw.row_ptr, R, 40000) is None          # a column a word cannot hold
+    L, p_ = card.lib, (lambda t: t.data_ptr())
+    out = torch.empty(4 * R, dtype=torch.int32, device="cuda")
+    assert L.btb_hip_p12_row_esc(p_(lo), p_(ei), p_(ev), ei.numel(), p_(pw.row_ptr), 1, 0x8000, p_(out), None) == -6
+    assert L.btb_hip_p12_row_esc(None, p_(ei), p_(ev), ei.numel(), p_(pw.row_ptr), R, C, p_(out), None) == -1
+
+
+@pytest.mark.parametrize("R,C", [(2560, 4096), (6144, 2560), (96, 272), (2560, 9728), (64, 1024)])
+@pytest.mark.parametrize("M", [1, 2, 4])
+def test_packed_matvec_with_the_rows_words_and_through_the_list(card, R, C, M):
+    """a row's first four escapes come out of the row's own words, asked for ahead of its weights; a caller without
+    them (row_esc NULL) walks the list: the same bits - with rows of none, one, four, five and forty escapes, the plain
+    matvec, the one with the residual add + norm folded in and its gate / up form - and the oracle's values"""
+    w = escapes_in_rows(R, C, [0, 1, 0, 4, 5, 2, 40, 0, 1, 3, 0, 17], seed=391 + M)
+    x = acts_bf16(M, C, seed=392).cuda()
+    lo, hi4, tb, ei, ev = (t_.cuda() for t_ in pack12.pack_bf16(w))
+    pw = P12Weight(lo, hi4, tb, ei, ev, R, C, card)
+    assert pw.row_esc is not None and pw.esc_idx.numel() > R
+    h = acts_bf16(M, C, seed=393).cuda()
+    nw = (1.0 + 0.1 * torch.randn(C, generator=torch.Generator().manual_seed(394))).to(torch.bfloat16).cuda()
+    def run():
+        y = card.gemv_p12(pw, x)
+        h2 = torch.empty_like(h)
+        yn = card.gemv_norm(pw, h, x, nw, 1e-6, h2, torch.empty(M, R, dtype=torch.bfloat16, device="cuda"))
+        yg = card.gemv_norm(pw, h, x, nw, 1e-6, torch.empty_like(h),
+                            torch.empty(M, R // 2, dtype=torch.bfloat16, device="cuda"), glu=True)
+        return y, yn, h2, yg
+    with_words = run()
+    words, pw.row_esc = pw.row_esc, None
+    try:
+        through_list = run()
+    finally:
+        pw.row_esc = words
+    for a, b in zip(with_words, through_list):
+        assert torch.equal(a.view(torch.int16), b.view(torch.int16))
+    check(with_words[0], oracle.gemv_bf16(bits16(w), x.float().cpu().numpy(), threads=0))
 
 
 @pytest.mark.parametrize("R,C", [(9728, 2560), (2560, 4096), (2560, 9728), (96, 272)])
