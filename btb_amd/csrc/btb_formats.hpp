@@ -77,19 +77,24 @@ struct FmtP12 {
         uint4 table;
         int e0, e1;  // the row's escapes: [e0, e1) of the list; where the matrix has the rows' words: the lane's word
     };
-    // A row's words (row_esc, made at upload: btb_hip_p12_row_esc): its first ROW_ESC_SLOTS escapes, one a word - low
-    // byte in bits 0..7, true high byte in 8..15, column in 16..30 (ROW_ESC_NONE: no such escape) - and in bit 31 of
-    // every word of the row: the row has more escapes than words.
+    // A row's words (row_esc, made at upload: btb_hip_p12_row_esc): its first row_esc_slots(C) escapes, one a word -
+    // low byte in bits 0..7, true high byte in 8..15, column in 16..30 (ROW_ESC_NONE: no such escape) - and in bit 31 of
+    // every word of the row: the row has more escapes than words. Eight words a row up to 4096 columns, sixteen beyond:
+    // a launch ends with its slowest wave, so what counts is that next to no row of a launch has more (at 0.02 % of
+    // the weights escaped a row of 2560 holds more than four once in six thousand rows - three rows of every gate/up
+    // launch - and more than eight once in 10^8; a row of 9728 more than eight once in five thousand, more than
+    // sixteen never).
     static constexpr uint32_t ROW_ESC_NONE = 0x7FFFu;
-    static constexpr int ROW_ESC_SLOTS = 4;
+    __host__ __device__ static constexpr int row_esc_slots(int C) { return C <= 4096 ? 8 : 16; }
     // The part of a row's context that comes out of memory: the lane's word of the row's words where the matrix has
-    // them (lane sl of the row's lanes: word min(sl, 3)), else the row's slice of the list. Two 4-byte loads from
-    // addresses chosen without a branch: a branch here makes the compiler wait for what was loaded before it, ahead
-    // of the row's weights.
-    __device__ static __forceinline__ void row_escapes(const Params& p, size_t r, int sl, RowCtx& c) {
+    // them (lane sl of the row's lanes: word min(sl, slots - 1)), else the row's slice of the list. Two 4-byte loads
+    // from addresses chosen without a branch: a branch here makes the compiler wait for what was loaded before it,
+    // ahead of the row's weights.
+    __device__ static __forceinline__ void row_escapes(const Params& p, size_t r, int units, int sl, RowCtx& c) {
         const bool words = p.row_esc != nullptr;
+        const int slots = row_esc_slots(units * UW);
         const int32_t* base = words ? reinterpret_cast<const int32_t*>(p.row_esc) : p.row_ptr;
-        const size_t at = words ? r * ROW_ESC_SLOTS + (size_t)min(sl, ROW_ESC_SLOTS - 1) : r;
+        const size_t at = words ? r * (size_t)slots + (size_t)min(sl, slots - 1) : r;
         c.e0 = base[at];
         c.e1 = base[words ? at : at + 1];
     }
@@ -110,7 +115,7 @@ struct FmtP12 {
         c.lo = reinterpret_cast<const uint4*>(p.lo) + r * (size_t)units;
         c.hi4 = reinterpret_cast<const uint2*>(p.hi4) + r * (size_t)units;
         c.table = p.tbl;
-        row_escapes(p, r, sl, c);
+        row_escapes(p, r, units, sl, c);
         return c;
     }
     __device__ static __forceinline__ Raw load(const RowCtx& c, int unit) {
@@ -147,10 +152,10 @@ struct FmtP12 {
     // term out, the true term in. Out of the list that is three round trips one behind the other - the row's slice,
     // its entries, the low bytes they name - at the end of a tile, where a wave has nothing left to hide them behind:
     // a tenth of the packed decode step, and a launch ends with its slowest wave, so it is not enough to spare most
-    // rows the walk. Hence the rows' words: a row's first four escapes stand in four words of the row's own, whose
-    // address the row number gives, and lane k < 4 asks for word k ahead of the row's weights - it has all it needs
-    // when the products are done. Only a row with more than four escapes (one in six thousand of a N(0, 0.02) matrix
-    // 2560 wide) walks the list, from its fifth entry on.
+    // rows the walk. Hence the rows' words: a row's first eight (or sixteen) escapes stand in words of the row's own,
+    // whose address the row number gives, and lane k asks for word k ahead of the row's weights - it has all it needs
+    // when the products are done. Only a row with more escapes than words walks the list, from the first entry that
+    // has no word on.
     template <int M>
     __device__ static __forceinline__ void esc_term(const RowCtx& c, int C, const uint32_t* xs, float (&acc)[M], int col,
                                                     uint32_t val, uint32_t lo) {
@@ -170,12 +175,13 @@ struct FmtP12 {
         int e0 = c.e0, e1 = c.e1, from = sl;
         if (p.row_esc != nullptr) {  // uniform
             const uint32_t rec = (uint32_t)c.e0, col = (rec >> 16) & 0x7FFFu;
-            if (sl < ROW_ESC_SLOTS && col != ROW_ESC_NONE)
+            const int slots = row_esc_slots(C);
+            if (sl < slots && col != ROW_ESC_NONE)
                 esc_term<M>(c, C, xs, acc, (int)col, (rec >> 8) & 0xFFu, rec & 0xFFu);
             if ((rec >> 31) == 0u) return;
             e0 = p.row_ptr[r];
             e1 = p.row_ptr[r + 1];
-            from = sl < ROW_ESC_SLOTS ? sl + lpr : sl;  // the first four are done
+            from = sl < slots ? sl + lpr : sl;  // those with a word are done
         }
         for (int e = e0 + from; e < e1; e += lpr) {
             const size_t i = (size_t)p.esc_idx[e];
@@ -207,7 +213,7 @@ struct FmtP12G : FmtP12 {
         c.lo = reinterpret_cast<const uint4*>(p.lo) + r * (size_t)units;
         c.hi4 = reinterpret_cast<const uint2*>(p.hi4) + r * (size_t)units;
         c.table = make_uint4(0u, 0u, 0u, 0u);  // not read: the lookups go through LDS, an escape streams as slot 15 = 0
-        row_escapes(p, r, sl, c);
+        row_escapes(p, r, units, sl, c);
         return c;
     }
     // eight weights: codes c (weight k in nibble k), low bytes l0 (weights 0..3), l1 (4..7)

@@ -153,7 +153,7 @@ __global__ void __launch_bounds__(256) p12_pairs_kernel(const uint8_t* __restric
 
 extern "C" {
 
-// a row's first four escapes as four words of the row's own (FmtP12::row_escapes reads them, FmtP12::tail uses them)
+// a row's first 8 or 16 escapes as words of the row's own (FmtP12::row_escapes reads them, FmtP12::tail uses them)
 __global__ void __launch_bounds__(256) p12_row_esc_kernel(const uint8_t* __restrict__ lo, const int32_t* __restrict__ esc_idx,
                                                           const uint8_t* __restrict__ esc_val,
                                                           const int32_t* __restrict__ row_ptr, int rows, int cols,
@@ -161,14 +161,15 @@ __global__ void __launch_bounds__(256) p12_row_esc_kernel(const uint8_t* __restr
     const int r = blockIdx.x * 256 + threadIdx.x;
     if (r >= rows) return;
     const int e0 = row_ptr[r], e1 = row_ptr[r + 1];
-    const uint32_t more = e1 - e0 > FmtP12::ROW_ESC_SLOTS ? 0x80000000u : 0u;
-    for (int k = 0; k < FmtP12::ROW_ESC_SLOTS; ++k) {
+    const int slots = FmtP12::row_esc_slots(cols);
+    const uint32_t more = e1 - e0 > slots ? 0x80000000u : 0u;
+    for (int k = 0; k < slots; ++k) {
         uint32_t w = FmtP12::ROW_ESC_NONE << 16;
         if (e0 + k < e1) {
             const size_t i = (size_t)esc_idx[e0 + k];
             w = (uint32_t)lo[i] | ((uint32_t)esc_val[e0 + k] << 8) | ((uint32_t)(i - (size_t)r * cols) << 16);
         }
-        out[(size_t)r * FmtP12::ROW_ESC_SLOTS + k] = w | more;
+        out[(size_t)r * slots + k] = w | more;
     }
 }
 

@@ -390,9 +390,10 @@ class HipCard(CardLaunch):
 
     def p12_row_esc(self, lo: torch.Tensor, esc_idx: torch.Tensor, esc_val: torch.Tensor, row_ptr: torch.Tensor,
                     rows: int, cols: int) -> torch.Tensor | None:
-        """int32 [rows, 4] (read as u32): every row's first four escapes, a word each (low byte, true high byte,
-        column; bit 31: the row has more), which the matvecs ask for ahead of the row's weights (built once at upload).
-        None for rows wider than 32767, whose columns a word cannot hold: the matvecs then walk the list."""
+        """int32 [rows, S] (read as u32; S = 8 up to 4096 columns, else 16): every row's first S escapes, a word each
+        (low byte, true high byte, column; bit 31: the row has more), which the matvecs ask for ahead of the row's
+        weights (built once at upload). None for rows wider than 32767, whose columns a word cannot hold: the matvecs
+        then walk the list."""
         if cols > 0x7FFF:
             return None
         self._need(lo, torch.uint8, "lo")
@@ -402,7 +403,7 @@ class HipCard(CardLaunch):
         if row_ptr.numel() != rows + 1 or lo.numel() != rows * cols or esc_val.numel() != esc_idx.numel():
             raise ValueError("[hip] p12_row_esc: lo holds rows * cols bytes, row_ptr rows + 1 entries, the list's two "
                              "arrays one entry an escape")
-        out = torch.empty(rows, 4, dtype=torch.int32, device=lo.device)
+        out = torch.empty(rows, 8 if cols <= 4096 else 16, dtype=torch.int32, device=lo.device)
         ne = int(esc_idx.numel())
         self._call("btb_hip_p12_row_esc", _p(lo), _p(esc_idx) if ne else None, _p(esc_val) if ne else None, ne,
                    _p(row_ptr), rows, cols, _p(out), _stream())

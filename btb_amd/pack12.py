@@ -163,8 +163,8 @@ def check_escapes(esc_idx: torch.Tensor, esc_val: torch.Tensor, n: int) -> None:
 class P12Weight:
     """One packed matrix on the GPU as the kernels read it; `shape` = (rows, cols). Three arrays are made here, once, by
     the card: `row_ptr[r]`, the index of the first escape at or past row r's first weight (int32 [rows + 1]), `pairs`,
-    the 256 two-byte entries the matvecs look a byte of codes up in, and `row_esc`, every row's first four escapes as
-    four words of the row's own (None for rows wider than 32767). The table is the matrix's own copy with
+    the 256 two-byte entries the matvecs look a byte of codes up in, and `row_esc`, every row's first 8 (16 beyond 4096
+    columns) escapes as words of the row's own (None for rows wider than 32767). The table is the matrix's own copy with
     slot 15 - the escape code, which names no table entry - set to 0: a store that left another byte there (0x7F or
     0xFF would make the streamed stand-in of an escaped weight inf or NaN, and its correction NaN) is as good as one
     that wrote the 0 the packer writes."""

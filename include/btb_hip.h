@@ -102,8 +102,8 @@ int32_t btb_hip_gemv_bf16_embed_norm(const void* w, const void* table, const int
  * btb_gemv_p12_rows (native/src/lib.rs:114-135), on the device, the list validated at upload by btb_hip_p12_check -
  * plus three arrays made once at upload: row_ptr i32[R + 1] from btb_hip_p12_row_ptr, pairs u16[256] from
  * btb_hip_p12_pairs (NULL: the table is looked up in registers instead, a slower kernel with the same bits) and
- * row_esc u32[4 R] from btb_hip_p12_row_esc (NULL: every escape is fetched through the list at the end of its row's
- * tile, slower with the same bits; with it C <= 32767).
+ * row_esc u32[S R] from btb_hip_p12_row_esc (S = 8 words a row up to 4096 columns, 16 beyond; NULL: every escape is
+ * fetched through the list at the end of its row's tile, slower with the same bits; with it C <= 32767).
  * x [M, C] bf16, y [M, R] bf16; C a multiple of 16, lo 16-byte and hi4 8-byte aligned. The reference has no card
  * kernel for this form (it widens a packed layer to bf16 before the card holds it: btb/engine/tiers.py:1200-1216). */
 int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, const void* pairs, const void* esc_idx,
@@ -131,9 +131,9 @@ int32_t btb_hip_gemv_p12_embed_norm(const void* lo, const void* hi4, const void*
  * table[15], as the packer writes it: the kernels that look the table up in registers stream table[15] there). */
 int32_t btb_hip_p12_pairs(const void* table, void* pairs, void* stream);
 
-/* row_esc[4 r + k] = row r's escape k (k = 0..3) as one word: the weight's low byte in bits 0..7, its true high byte
- * in 8..15, its column in 16..30 (0x7FFF: the row has no such escape); bit 31 of all four words: the row has more
- * than four. The matvec asks for a row's words ahead of the row's weights, so an escape costs it no trip to memory of
+/* row_esc[S r + k] = row r's escape k (k < S; S = 8 where cols <= 4096, else 16) as one word: the weight's low byte
+ * in bits 0..7, its true high byte in 8..15, its column in 16..30 (0x7FFF: the row has no such escape); bit 31 of all
+ * the row's words: the row has more than S. The matvec asks for a row's words ahead of the row's weights, so an escape costs it no trip to memory of
  * its own at the end of the row (the list does: its slice, its entries, the low bytes they name). Made once at upload
  * from the list, the low bytes and row_ptr; cols <= 32767 (BTB_ERR_DOMAIN beyond). No counterpart in the reference. */
 int32_t btb_hip_p12_row_esc(const void* lo, const void* esc_idx, const void* esc_val, size_t n_esc, const void* row_ptr,

@@ -440,32 +440,33 @@ def escapes_in_rows(R, C, counts, seed):
     return torch.from_numpy(wb.view(np.int16)).view(torch.bfloat16)
 
 
-def test_rows_words_made_at_upload(card):
+@pytest.mark.parametrize("R,C,S", [(48, 272, 8), (40, 4096, 8), (24, 4112, 16)])
+def test_rows_words_made_at_upload(card, R, C, S):
     """row_esc[r, k] = row r's escape k as (low byte, true high byte << 8, column << 16), 0x7FFF for the column where
-    the row has no such escape, bit 31 of all four words where it has more than four; rows too wide for a word's
-    column field get none"""
-    R, C = 48, 272
-    w = escapes_in_rows(R, C, [0, 1, 2, 4, 5, 9, 0, 3], seed=390)
+    the row has no such escape, bit 31 of all the row's words where it has more than words (8 a row up to 4096
+    columns, 16 beyond); rows too wide for a word's column field get none"""
+    w = escapes_in_rows(R, C, [0, 1, 2, 8, 9, 17, 0, 3, 16, 20], seed=390)
     lo, hi4, tb, ei, ev = (t_.cuda() for t_ in pack12.pack_bf16(w))
     pw = P12Weight(lo, hi4, tb, ei, ev, R, C, card)
     got = pw.row_esc.cpu().numpy().view(np.uint32)
     idx, val, lob = ei.cpu().numpy().astype(np.int64), ev.cpu().numpy(), lo.cpu().numpy().reshape(-1)
-    want = np.zeros((R, 4), dtype=np.uint32)
+    assert got.shape == (R, S)
+    want = np.zeros((R, S), dtype=np.uint32)
     for r in range(R):
         mine = np.flatnonzero((idx >= r * C) & (idx < (r + 1) * C))
-        for k in range(4):
+        for k in range(S):
             if k < mine.size:
                 e = mine[k]
                 want[r, k] = int(lob[idx[e]]) | (int(val[e]) << 8) | (int(idx[e] - r * C) << 16)
             else:
                 want[r, k] = 0x7FFF << 16
-        if mine.size > 4:
+        if mine.size > S:
             want[r] |= 0x80000000
     assert np.array_equal(got, want)
     assert (got[:, 0] >> 31).sum() > 0 and ((got[:, 0] >> 16) & 0x7FFF == 0x7FFF).sum() > 0   # both kinds of row met
     assert card.p12_row_esc(lo, ei, ev, pw.row_ptr, R, 40000) is None          # a column a word cannot hold
     L, p_ = card.lib, (lambda t: t.data_ptr())
-    out = torch.empty(4 * R, dtype=torch.int32, device="cuda")
+    out = torch.empty(16 * R, dtype=torch.int32, device="cuda")
     assert L.btb_hip_p12_row_esc(p_(lo), p_(ei), p_(ev), ei.numel(), p_(pw.row_ptr), 1, 0x8000, p_(out), None) == -6
     assert L.btb_hip_p12_row_esc(None, p_(ei), p_(ev), ei.numel(), p_(pw.row_ptr), R, C, p_(out), None) == -1
 
@@ -474,9 +475,9 @@ def test_rows_words_made_at_upload(card):
 @pytest.mark.parametrize("M", [1, 2, 4])
 def test_packed_matvec_with_the_rows_words_and_through_the_list(card, R, C, M):
     """a row's first four escapes come out of the row's own words, asked for ahead of its weights; a caller without
-    them (row_esc NULL) walks the list: the same bits - with rows of none, one, four, five and forty escapes, the plain
+    them (row_esc NULL) walks the list: the same bits - with rows of none, one, eight, nine, sixteen and forty escapes, the plain
     matvec, the one with the residual add + norm folded in and its gate / up form - and the oracle's values"""
-    w = escapes_in_rows(R, C, [0, 1, 0, 4, 5, 2, 40, 0, 1, 3, 0, 17], seed=391 + M)
+    w = escapes_in_rows(R, C, [0, 1, 0, 8, 9, 2, 40, 0, 1, 3, 16, 17], seed=391 + M)
     x = acts_bf16(M, C, seed=392).cuda()
     lo, hi4, tb, ei, ev = (t_.cuda() for t_ in pack12.pack_bf16(w))
     pw = P12Weight(lo, hi4, tb, ei, ev, R, C, card)
