@@ -523,8 +523,8 @@ __global__ void __launch_bounds__(128) attn_merge_few_kernel(uint16_t* __restric
                                   part_acc, threadIdx.x);
 }
 
-// The fold behind every attention kernel here. Up to 2 * MERGE_FEW spans: the fold that shares nothing, built for 20
-// and for 40 spans (the step's pair of launches 13.6 -> 11.75 us a layer against the general fold at 18 spans; a pass
+// The fold behind every attention kernel here. Up to 64 spans: the fold that shares nothing, built for 20, 40 and 64
+// spans (the step's pair of launches 13.6 -> 11.75 us a layer against the general fold at 18 spans; a pass
 // of 4 / 8 rows over 36 spans 2.95 / 2.96 -> 2.86 / 2.91 ms); more: the general one. The same bits either way.
 template <int G>
 void launch_merge(hipStream_t st, void* att, size_t T, size_t Hq, size_t Hk, size_t S, const float* part_m,
@@ -538,6 +538,8 @@ void launch_merge(hipStream_t st, void* att, size_t T, size_t Hq, size_t Hk, siz
     else if (S <= S_few) FEW(true, MERGE_FEW);
     else if (S <= 2 * S_few && rw == nullptr) FEW(false, 2 * MERGE_FEW);
     else if (S <= 2 * S_few) FEW(true, 2 * MERGE_FEW);
+    else if (S_few != 0 && S <= 64 && rw == nullptr) FEW(false, 64);  // a lane a span: as many as a wave has lanes
+    else if (S_few != 0 && S <= 64) FEW(true, 64);
     else
         hipLaunchKernelGGL(attn_merge_kernel<G>, dim3((unsigned)Hk, (unsigned)T), dim3(256), 2 * S * G * sizeof(float),
                            st, static_cast<uint16_t*>(att), (int)Hq, (int)Hk, (int)S, part_m, part_l, part_acc, rw);

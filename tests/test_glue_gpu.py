@@ -97,9 +97,10 @@ def test_attn_decode_against_f64(card, n0, T, Hq, Hk, S):
 
 @pytest.mark.parametrize("Hq,Hk", [(8, 8), (8, 4), (16, 4), (8, 1)])
 @pytest.mark.parametrize("n0,T,S", [(700, 1, 1), (700, 1, 2), (2400, 1, 19), (2559, 1, 20), (2600, 3, 21), (300, 2, 20),
-                                     (4990, 1, 39), (5000, 2, 40), (5200, 1, 41), (90, 1, 40)])
+                                     (4990, 1, 39), (5000, 2, 40), (5200, 1, 41), (90, 1, 40), (8000, 1, 63),
+                                     (8100, 2, 64), (8300, 1, 65), (300, 1, 64)])
 def test_the_fold_of_a_few_spans_gives_the_general_folds_bits(card, n0, T, Hq, Hk, S):
-    """up to 40 spans are folded by a kernel that shares nothing between its waves; the knob attn_merge_few = 0 sends
+    """up to 64 spans are folded by a kernel that shares nothing between its waves (built for 20, 40 and 64); the knob attn_merge_few = 0 sends
     every count through the general fold: the same output bits, at the counts on both sides of each limit, with spans
     past the row's keys (no maximum, no sum) and for every number of query heads a kv head"""
     D = 128
