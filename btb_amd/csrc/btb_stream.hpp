@@ -60,6 +60,9 @@ __host__ __device__ constexpr size_t stage_lds_bytes(int xmode, int M, int C) {
 // so they travel while the staging's own (short) round trip and arithmetic run.
 // MR: the number of rows where the caller knows it at compile time (M is then MR), 0 otherwise. KEEP: the one-row
 // add + norm keeps its words in registers across the sum (see there).
+// a scheduling barrier that only loads and stores of global memory may not cross (ALU and LDS instructions may)
+constexpr int VMEM_STAYS = 0x38F;
+
 template <int XMODE, int MR = 0, bool KEEP = false, class AfterIssue>
 __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C, AfterIssue after_issue) {
     const int tid = threadIdx.x, nt = blockDim.x;
@@ -69,13 +72,18 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
         // exactly and does not take in the weights requested behind them. The stores are unconditional as well (a
         // load whose only use sits in a branch is moved into it, behind the weights): the repeated piece is written
         // to its own place again
-        const uint4* src = reinterpret_cast<const uint4*>(a.x);
-        uint4* dst = reinterpret_cast<uint4*>(xs);
+        // (the pieces wait in an array of compiler vectors: an array of HIP's uint4 structs goes to scratch memory once
+        // the scheduling barrier below stands between its writes and its reads)
+        const u32x4* src = reinterpret_cast<const u32x4*>(a.x);
+        u32x4* dst = reinterpret_cast<u32x4*>(xs);
         const int n = M * C / 8;
         constexpr int PER = 5;
-        uint4 v[PER];
+        u32x4 v[PER];
 #pragma unroll
         for (int q = 0; q < PER; ++q) v[q] = src[min(tid + q * 256, n - 1)];
+        // the caller's weights stay behind these loads: moved ahead of them by the scheduler, the staging below waited
+        // for weights out of HBM where it needs x out of L2 (loads come back in order)
+        __builtin_amdgcn_sched_barrier(VMEM_STAYS);
         after_issue();
 #pragma unroll
         for (int q = 0; q < PER; ++q) dst[min(tid + q * 256, n - 1)] = v[q];
