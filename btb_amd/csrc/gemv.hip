@@ -508,17 +508,13 @@ int32_t btb_hip_gemv_p12(const void* lo, const void* hi4, const void* table, con
         }
         return OK;
     }
-    // The lookups through the pair table in LDS (the caller's, made at upload) where waves walk more than one tile - the
-    // kernel then streams, and the table's 1.5 vector instructions a weight beat the in-register lookup's 3.4 - and in
-    // registers where every wave has one tile or none: such a launch is one trip to memory and back, and the LDS
-    // lookups' own latency sits on it (measured with the table from upload, nothing built in the kernel: o
-    // [2560 x 4096] 6.35 against 5.62 us, the one-row [9728 x 2560] 10.5 against 9.9, down [2560 x 9728] level). The
-    // knob p12_pair_table forces either (1 / 0). The add + norm forms below always take the table: their staging
-    // waits for the norm's sums while it arrives.
+    // The lookups go through the pair table in LDS where the caller has one (made at upload; 1.5 vector instructions
+    // a weight against the in-register lookup's 3.4). While an escape still cost a launch three trips to memory at
+    // its end, a launch of one tile a wave did better with the lookup in registers (o [2560 x 4096] 5.62 against
+    // 6.35 us); with the rows' words the table wins or draws at every shape of the step (down [2560 x 9728] 9.3
+    // against 9.6 us, o level). The knob p12_pair_table forces either (1 / 0).
     const int knob = tuning("p12_pair_table");
-    const size_t tiles = R / (size_t)(WAVE / lanes_per_row((int)(C / FmtP12::UW)));
-    const bool streams = tiles > (size_t)device_info().cus * 5 * 4;
-    if (pairs != nullptr && (knob >= 0 ? knob != 0 : streams))
+    if (pairs != nullptr && knob != 0)
         return run_rows<FmtP12G, X_PLAIN, E_PLAIN>(p, plain_x(x), y, R, C, M, static_cast<hipStream_t>(stream));
     return run_rows<FmtP12, X_PLAIN, E_PLAIN>(p, plain_x(x), y, R, C, M, static_cast<hipStream_t>(stream));
 }
