@@ -175,9 +175,18 @@ static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void
     // matvec [151936 x 2560] takes 97 us instead of 113, the packed step 2.194 ms instead of 2.213.
     if (per_cu <= 0) per_cu = std::is_same<F, FmtP12G>::value ? 5 : 6;
     const int cap_waves = dev.cus * per_cu * 4;
-    const int tiles_per_wave = (ntiles + cap_waves - 1) / cap_waves;
-    const int waves = (ntiles + tiles_per_wave - 1) / tiles_per_wave;
-    int grid = (waves + 3) / 4;
+    // ... and of the counts from there to two more, the one whose workgroups fill the CUs' turns most evenly (when it
+    // gains a twentieth or more): a launch ends with its fullest CU, and the forms that widen are bound by what a CU
+    // computes (MXFP4 [18432 x 7168]: 1152 workgroups of 2 tiles a wave, 4.5 a CU, 15.7 us; 768 of 3, 3 a CU, 14.4).
+    auto grid_of = [&](int tpw) { return ((ntiles + tpw - 1) / tpw + 3) / 4; };
+    auto evenness = [&](int g) { return (double)g / (double)(((g + dev.cus - 1) / dev.cus) * dev.cus); };
+    int tiles_per_wave = (ntiles + cap_waves - 1) / cap_waves;
+    if (tuning("gemv_even_grid") != 0) {
+        const int base = tiles_per_wave;
+        for (int t = base + 1; t <= base + 2; ++t)
+            if (evenness(grid_of(t)) >= evenness(grid_of(tiles_per_wave)) + 0.04) tiles_per_wave = t;
+    }
+    int grid = grid_of(tiles_per_wave);
     if (grid < 1) grid = 1;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
