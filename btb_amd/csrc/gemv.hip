@@ -223,9 +223,21 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
             return launch_variant<F, M, LPR, 2, (M <= 2 ? 4 : 2), XMODE, E_GLU>(p, xa, y, R, C, st);
         }
     } else if constexpr (WIDENS) {
-        if constexpr (F::TWO_ROWS)
+        if constexpr (F::TWO_ROWS) {
+            if constexpr (M == 1 && XMODE == X_PLAIN) {
+                // One row of x over FP8: a lane's 5 to 8 units of a row asked for at once, one row a wave - one trip to
+                // memory for the row instead of three or four spans of two units ([18432 x 7168], 7 units a lane:
+                // 26.3 -> 24.4 us; two rows by four units 25.1, by three 25.4, one row by four 27.2).
+                switch (per_lane) {
+                    case 5: return launch_variant<F, M, LPR, 1, 5, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+                    case 6: return launch_variant<F, M, LPR, 1, 6, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+                    case 7: return launch_variant<F, M, LPR, 1, 7, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+                    case 8: return launch_variant<F, M, LPR, 1, 8, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+                    default: break;
+                }
+            }
             return launch_variant<F, M, LPR, 2, 2, XMODE, E_PLAIN>(p, xa, y, R, C, st);
-        else
+        } else
             return launch_variant<F, M, LPR, 1, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
     } else {
         const bool tall = R >= 4096 * (WAVE / LPR);
