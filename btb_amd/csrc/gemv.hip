@@ -213,6 +213,9 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
     if constexpr (EPI == E_GLU) {
         if constexpr (WIDENS && LPR <= 32) {
             // a widening form whose rows take at most 32 lanes: gate and up side by side, one row a lane
+            if constexpr (M == 1 && std::is_base_of<FmtP12, F>::value) {
+                if (per_lane == 5) return launch_variant<F, M, LPR, 1, 5, XMODE, E_GLU_SPLIT>(p, xa, y, R, C, st);
+            }
             return launch_variant<F, M, LPR, 1, 4, XMODE, E_GLU_SPLIT>(p, xa, y, R, C, st);
         } else if constexpr (WIDENS) {
             return launch_variant<F, M, LPR, 2, 2, XMODE, E_GLU>(p, xa, y, R, C, st);
@@ -237,8 +240,15 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
                 }
             }
             return launch_variant<F, M, LPR, 2, 2, XMODE, E_PLAIN>(p, xa, y, R, C, st);
-        } else
+        } else {
+            // one row of x over pack12 rows of five units a lane (2560 columns): the five at once, one trip for the row
+            // where four and one were two (the one-row [9728 x 2560] 8.8 -> 8.3 us, qkv + norm 7.3 -> 6.9; rows of four
+            // or ten units a lane lose by it: o 5.06 -> 5.22, down 9.3 -> 9.4)
+            if constexpr (M == 1 && std::is_base_of<FmtP12, F>::value) {
+                if (per_lane == 5) return launch_variant<F, M, LPR, 1, 5, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+            }
             return launch_variant<F, M, LPR, 1, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
+        }
     } else {
         const bool tall = R >= 4096 * (WAVE / LPR);
         if constexpr (M <= 2) {
