@@ -171,9 +171,11 @@ static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void
     auto kern = gemv_stream<F, M, LPR, RPW, U, XMODE, EPI>;
     int per_cu = tuning("gemv_wgs_per_cu");
     // Six workgroups' worth of waves a CU, measured best for every form (more, smaller workgroups than are resident
-    // even out the grid's tail) but the pack12 form with the pair table, which does better cut for five - the head
-    // matvec [151936 x 2560] takes 97 us instead of 113, the packed step 2.194 ms instead of 2.213.
-    if (per_cu <= 0) per_cu = std::is_same<F, FmtP12G>::value ? 5 : 6;
+    // even out the grid's tail) but the pack12 form with the pair table, which does better with fewer: cut for five the
+    // head matvec [151936 x 2560] took 97 us instead of 113, and its gate/up form cut for four (since its rows of five units a
+    // lane come in one trip) takes 15.4 us instead of 16.3, the packed step 1.912 ms instead of 1.926 (the plain one-row
+    // [9728 x 2560] loses by four: 8.25 -> 9.15 us).
+    if (per_cu <= 0) per_cu = std::is_same<F, FmtP12G>::value ? (EPI == E_PLAIN ? 5 : 4) : 6;
     const int cap_waves = dev.cus * per_cu * 4;
     // ... and of the counts from there to two more, the one whose workgroups fill the CUs' turns most evenly (when it
     // gains a twentieth or more): a launch ends with its fullest CU, and the forms that widen are bound by what a CU
