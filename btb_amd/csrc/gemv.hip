@@ -170,12 +170,13 @@ static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void
     const int ntiles = (Rout + ROWS - 1) / ROWS;
     auto kern = gemv_stream<F, M, LPR, RPW, U, XMODE, EPI>;
     int per_cu = tuning("gemv_wgs_per_cu");
-    // Six workgroups' worth of waves a CU, measured best for every form (more, smaller workgroups than are resident
-    // even out the grid's tail) but the pack12 form with the pair table, which does better with fewer: cut for five the
-    // head matvec [151936 x 2560] took 97 us instead of 113, and its gate/up form cut for four (since its rows of five units a
-    // lane come in one trip) takes 15.4 us instead of 16.3, the packed step 1.912 ms instead of 1.926 (the plain one-row
-    // [9728 x 2560] loses by four: 8.25 -> 9.15 us).
-    if (per_cu <= 0) per_cu = std::is_same<F, FmtP12G>::value ? (EPI == E_PLAIN ? 5 : 4) : 6;
+    // Six workgroups' worth of waves a CU, measured best for the plain forms (more, smaller workgroups than are resident
+    // even out the grid's tail), five for the pack12 form with the pair table (the head matvec [151936 x 2560] 97 us
+    // instead of 113), and four for the gate / up forms at one or two rows of x, whose waves then walk three tiles
+    // instead of two: bf16 gate/up 17.55 -> 17.0 us and the step 2.022 -> 2.004 ms, packed 16.3 -> 15.5 us and
+    // 1.928 -> 1.914 ms; at three rows the pass loses by it (2.58 -> 2.67 ms), and so does the plain one-row packed
+    // [9728 x 2560] (8.25 -> 9.15 us).
+    if (per_cu <= 0) per_cu = (EPI != E_PLAIN && M <= 2) ? 4 : std::is_same<F, FmtP12G>::value ? 5 : 6;
     const int cap_waves = dev.cus * per_cu * 4;
     // ... and of the counts from there to two more, the one whose workgroups fill the CUs' turns most evenly (when it
     // gains a twentieth or more): a launch ends with its fullest CU, and the forms that widen are bound by what a CU
