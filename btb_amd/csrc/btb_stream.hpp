@@ -63,8 +63,10 @@ __host__ __device__ constexpr size_t stage_lds_bytes(int xmode, int M, int C) {
 // a scheduling barrier that only loads and stores of global memory may not cross (ALU and LDS instructions may)
 constexpr int VMEM_STAYS = 0x38F;
 
-template <int XMODE, int MR = 0, bool KEEP = false, class AfterIssue>
+// NT: the workgroup's threads (256; 320 for the plain copy, where five waves a workgroup fill the CUs evenly).
+template <int XMODE, int MR = 0, bool KEEP = false, int NT = 256, class AfterIssue>
 __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C, AfterIssue after_issue) {
+    static_assert(NT == 256 || XMODE == X_PLAIN, "only the plain copy is written for other workgroup sizes");
     const int tid = threadIdx.x, nt = blockDim.x;
     if (XMODE == X_PLAIN) {
         // the first five 16-byte pieces a thread copies (rows up to 10240 values) are requested together and
@@ -77,17 +79,17 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
         const u32x4* src = reinterpret_cast<const u32x4*>(a.x);
         u32x4* dst = reinterpret_cast<u32x4*>(xs);
         const int n = M * C / 8;
-        constexpr int PER = 5;
+        constexpr int PER = 1280 / NT;  // rows up to 10240 values in the one request
         u32x4 v[PER];
 #pragma unroll
-        for (int q = 0; q < PER; ++q) v[q] = src[min(tid + q * 256, n - 1)];
+        for (int q = 0; q < PER; ++q) v[q] = src[min(tid + q * NT, n - 1)];
         // the caller's weights stay behind these loads: moved ahead of them by the scheduler, the staging below waited
         // for weights out of HBM where it needs x out of L2 (loads come back in order)
         __builtin_amdgcn_sched_barrier(VMEM_STAYS);
         after_issue();
 #pragma unroll
-        for (int q = 0; q < PER; ++q) dst[min(tid + q * 256, n - 1)] = v[q];
-        for (int i = tid + PER * 256; i < n; i += 256) dst[i] = src[i];
+        for (int q = 0; q < PER; ++q) dst[min(tid + q * NT, n - 1)] = v[q];
+        for (int i = tid + PER * NT; i < n; i += NT) dst[i] = src[i];
     } else if (XMODE == X_SILU) {
         after_issue();
         const int half = C / 2;  // pairs per row
@@ -287,7 +289,7 @@ __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int
 
 template <int XMODE>
 __device__ __forceinline__ void stage_x(uint32_t* xs, const XArgs& a, int M, int C) {
-    stage_x<XMODE, 0, false>(xs, a, M, C, [] {});
+    stage_x<XMODE, 0, false, 256>(xs, a, M, C, [] {});
 }
 
 // ------------------------------------------------------------------------------------------------------------

@@ -108,8 +108,8 @@ __device__ __forceinline__ void gemv_tile(const typename F::Params& p, const typ
 // been issued, so those (served by L2) are not queued behind the weights: the weights do not depend on x, and their
 // round trip to HBM overlaps the staging (for the add + norm form a block-wide sum and a second pass) instead of
 // following it.
-template <class F, int M, int LPR, int RPW, int U, int XMODE, int EPI>
-__global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs xa, uint16_t* __restrict__ y, int R, int C) {
+template <class F, int M, int LPR, int RPW, int U, int XMODE, int EPI, int NT = 256>
+__global__ void __launch_bounds__(NT) gemv_stream(typename F::Params p, XArgs xa, uint16_t* __restrict__ y, int R, int C) {
     extern __shared__ __align__(16) uint32_t xs[];  // [M][C / 2] packed bf16 pairs
     static_assert(EPI != E_GLU || RPW == 2, "the GLU form pairs a gate row with an up row");
     static_assert(EPI != E_GLU_SPLIT || (RPW == 1 && LPR <= 32), "the split GLU form: gate and up in neighbouring row groups");
@@ -124,7 +124,7 @@ __global__ void __launch_bounds__(256) gemv_stream(typename F::Params p, XArgs x
 
     typename F::Raw first[U][RPW] = {};
     typename F::RowCtx first_ctx[RPW];
-    stage_x<XMODE, M, sizeof(typename F::Raw) != 16>(xs, xa, M, C, [&] {
+    stage_x<XMODE, M, sizeof(typename F::Raw) != 16, NT>(xs, xa, M, C, [&] {
         // a wave with no tile requests the last tile's span and drops it: nothing here is conditional (see
         // load_span_always)
 #pragma unroll
@@ -195,6 +195,28 @@ static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
+    }
+    // One row of x, one tile a wave, plain: a launch is then a single turn over the CUs and ends with the CU that
+    // holds the most waves. Workgroups of four waves put 2560 one-row tiles on the CUs as 640 workgroups, 12 waves on
+    // half the CUs and 8 on the others; workgroups of five put 10 on each (a bf16 matrix of 2048 rows of 9728, which divides evenly, ran
+    // at 8.1 us where 2304 rows took 10.1).
+    if constexpr (M == 1 && XMODE == X_PLAIN && EPI == E_PLAIN) {
+        const int waves = (ntiles + tiles_per_wave - 1) / tiles_per_wave;
+        const int g5 = (waves + 4) / 5;
+        // (measured: pack12 down 9.45 -> 8.45 us and o level, the packed step 1.910 -> 1.893 ms; bf16 o 5.28 -> 5.13 us
+        // but down, whose rows are two spans, 10.1 -> 10.6: bf16 takes five waves only where a row is one span)
+        constexpr bool WIDENS = sizeof(typename F::Raw) != 16;
+        const bool suits = WIDENS || U * LPR >= C / F::UW;
+        if (suits && tiles_per_wave == 1 && tuning("gemv_five_waves") != 0 && evenness(g5) >= evenness(grid) + 0.1) {
+            auto kern5 = gemv_stream<F, M, LPR, RPW, U, XMODE, EPI, 320>;
+            if (lds > 64 * 1024) {
+                hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern5),
+                                                   hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+                if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
+            }
+            hipLaunchKernelGGL(kern5, dim3(g5), dim3(320), lds, st, p, xa, static_cast<uint16_t*>(y), R, C);
+            return hip_status(hipGetLastError(), "gemv launch");
+        }
     }
     hipLaunchKernelGGL(kern, dim3(grid), dim3(256), lds, st, p, xa, static_cast<uint16_t*>(y), R, C);
     return hip_status(hipGetLastError(), "gemv launch");

@@ -266,7 +266,7 @@ __global__ void __launch_bounds__(256) moe_gate_up_kernel(Stack stack, const uin
     // weights do not depend on x, and nothing about these loads is conditional (a wave past the last tile requests the
     // last tile's and drops them)
     typename F::Raw first[U][RPW] = {};
-    stage_x<X_PLAIN, 0, false>(xs, XArgs{x + (size_t)token * C, nullptr, nullptr, nullptr, 0.f, 0}, 1, C, [&] {
+    stage_x<X_PLAIN, 0, false, 256>(xs, XArgs{x + (size_t)token * C, nullptr, nullptr, nullptr, 0.f, 0}, 1, C, [&] {
         typename F::RowCtx c0[RPW];
 #pragma unroll
         for (int j = 0; j < RPW; ++j)
