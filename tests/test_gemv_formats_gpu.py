@@ -86,6 +86,35 @@ def test_gemv_mxfp4(card, R, C, M):
     check(y, ref)
 
 
+@pytest.mark.parametrize("form,R,C", [("bf16", 2560, 4096), ("bf16", 2560, 9728), ("p12", 2560, 4096), ("p12", 2560, 9728),
+                                      ("mxfp4", 9216, 2048), ("bf16", 2304, 1024)])
+def test_the_grid_changes_no_bit(card, form, R, C):
+    """how a launch is cut over the CUs - workgroups of five waves where four leave the CUs uneven, a tile more a wave
+    where that fills the turns evenly - is the launch's own business: with either choice switched off (knobs
+    gemv_five_waves, gemv_even_grid) the one-row matvec gives the same bits"""
+    x = acts_bf16(1, C, seed=402).cuda()
+    if form == "bf16":
+        w = weights_bf16(R, C, seed=401).cuda()
+        run = lambda: card.gemv(w, x)
+    elif form == "p12":
+        pw = P12Weight.pack(weights_bf16(R, C, seed=401).cuda(), card)
+        run = lambda: card.gemv_p12(pw, x)
+    else:
+        blocks, scales = mxfp4.quantize(weights_bf16(R, C, seed=401).float())
+        mw = mxfp4.MxWeight(blocks.reshape(-1).cuda(), scales.reshape(-1).cuda(), R, C)
+        run = lambda: card.gemv_mx4(mw, x)
+    want = run()
+    try:
+        for knob in ("gemv_five_waves", "gemv_even_grid"):
+            card.set_tuning(knob, 0)
+            got = run()
+            card.set_tuning(knob, -1)
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16)), knob
+    finally:
+        card.set_tuning("gemv_five_waves", -1)
+        card.set_tuning("gemv_even_grid", -1)
+
+
 def test_format_refusals(card):
     L = card.lib
     z = torch.zeros(4096, dtype=torch.uint8, device="cuda")
