@@ -238,7 +238,7 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
     if constexpr (EPI == E_GLU) {
         if constexpr (WIDENS && LPR <= 32) {
             // a widening form whose rows take at most 32 lanes: gate and up side by side, one row a lane
-            if constexpr (M == 1 && std::is_base_of<FmtP12, F>::value) {
+            if constexpr (M <= 4 && std::is_base_of<FmtP12, F>::value) {
                 if (per_lane == 5) return launch_variant<F, M, LPR, 1, 5, XMODE, E_GLU_SPLIT>(p, xa, y, R, C, st);
             }
             return launch_variant<F, M, LPR, 1, 4, XMODE, E_GLU_SPLIT>(p, xa, y, R, C, st);
@@ -266,10 +266,11 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
             }
             return launch_variant<F, M, LPR, 2, 2, XMODE, E_PLAIN>(p, xa, y, R, C, st);
         } else {
-            // one row of x over pack12 rows of five units a lane (2560 columns): the five at once, one trip for the row
-            // where four and one were two (the one-row [9728 x 2560] 8.8 -> 8.3 us, qkv + norm 7.3 -> 6.9; rows of four
-            // or ten units a lane lose by it: o 5.06 -> 5.22, down 9.3 -> 9.4)
-            if constexpr (M == 1 && std::is_base_of<FmtP12, F>::value) {
+            // up to four rows of x over pack12 rows of five units a lane (2560 columns): the five at once, one trip for
+            // the row where four and one were two (the one-row [9728 x 2560] 8.8 -> 8.3 us, qkv + norm 7.3 -> 6.9, the
+            // packed pass of two / three rows 2.31 / 2.76 -> 2.18 / 2.65 ms; rows of four or ten units a lane lose by it:
+            // o 5.06 -> 5.22, down 9.3 -> 9.4)
+            if constexpr (M <= 4 && std::is_base_of<FmtP12, F>::value) {
                 if (per_lane == 5) return launch_variant<F, M, LPR, 1, 5, XMODE, E_PLAIN>(p, xa, y, R, C, st);
             }
             return launch_variant<F, M, LPR, 1, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
