@@ -232,7 +232,8 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
     constexpr bool WIDENS = sizeof(typename F::Raw) != 16;  // everything but plain bf16
     // One bf16 row of x (the decode step proper): where a slightly longer span saves a whole round trip to memory - a
     // row of 5 units a lane read as 5, not 4 + 1; 19 as 10 + 9, not 8 + 8 + 3 - the span is stretched to 5 (10 for one
-    // row a wave). Measured a gain for bf16 and a loss for the forms that widen, which keep their spans.
+    // row a wave). The span of 5 at two rows of x as well (the bf16 pass of two rows 2.309 -> 2.2 ms, nearly all of it
+    // the gate / up form's); at three rows it loses (2.59 -> 2.61).
     const int per_lane = (C / F::UW + LPR - 1) / LPR;
     auto fewer = [per_lane](int u_new, int u_base) { return (per_lane + u_new - 1) / u_new < (per_lane + u_base - 1) / u_base; };
     if constexpr (EPI == E_GLU) {
@@ -245,7 +246,7 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
         } else if constexpr (WIDENS) {
             return launch_variant<F, M, LPR, 2, 2, XMODE, E_GLU>(p, xa, y, R, C, st);
         } else {
-            if constexpr (M == 1) {
+            if constexpr (M <= 2) {
                 if (fewer(5, 4)) return launch_variant<F, M, LPR, 2, 5, XMODE, E_GLU>(p, xa, y, R, C, st);
             }
             return launch_variant<F, M, LPR, 2, (M <= 2 ? 4 : 2), XMODE, E_GLU>(p, xa, y, R, C, st);
@@ -278,8 +279,8 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
     } else {
         const bool tall = R >= 4096 * (WAVE / LPR);
         if constexpr (M <= 2) {
+            if (tall && fewer(5, 4)) return launch_variant<F, M, LPR, 2, 5, XMODE, E_PLAIN>(p, xa, y, R, C, st);
             if constexpr (M == 1) {
-                if (tall && fewer(5, 4)) return launch_variant<F, M, LPR, 2, 5, XMODE, E_PLAIN>(p, xa, y, R, C, st);
                 if (!tall && fewer(10, 8)) return launch_variant<F, M, LPR, 1, 10, XMODE, E_PLAIN>(p, xa, y, R, C, st);
             }
             if (tall) return launch_variant<F, M, LPR, 2, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
