@@ -372,11 +372,23 @@ int32_t gemv_mfma_dl_p12(const uint8_t* lo, const uint8_t* hi4, const uint8_t* t
                          const uint8_t* esc_val, const int32_t* row_ptr, const void* x, void* y, int R, int C, int M,
                          hipStream_t st);
 
-// whether a pass of M rows goes to the matrix cores through the LDS-staged kernel
-static bool wide_pass(size_t M, size_t R, size_t C, bool packed) {
-    return M >= 5 && (packed ? mfma_lds_fits_packed((int)R, (int)C) : mfma_lds_fits_bf16((int)R, (int)C)) &&
+// whether a pass of M rows goes to the matrix cores through the LDS-staged kernel: from `from` rows on (the knob
+// gemv_mfma_from, when set, replaces every form's own figure)
+static bool wide_pass(size_t M, size_t R, size_t C, bool packed, size_t from = 5) {
+    if (tuning("gemv_mfma_from") > 0) from = (size_t)tuning("gemv_mfma_from");
+    return M >= from && (packed ? mfma_lds_fits_packed((int)R, (int)C) : mfma_lds_fits_bf16((int)R, (int)C)) &&
            tuning("gemv_no_mfma") <= 0 && tuning("mfma_lds") != 0;
 }
+
+// the block-scaled forms' vector kernels pay for every further row of x in LDS reads and in widening, the matrix-core
+// kernels' time does not move up to 16 rows: on large matrices these take the pass earlier than at five rows
+// (measured: MXFP4 [18432 x 7168] at 2 / 3 / 4 rows 23.6 / 30.0 / 37.8 us on the vector kernel, 19 us on the matrix
+// cores; FP8 33.3 / 45.1 us at 3 / 4 rows against 30.7; under 4 M weights the vector kernel wins to four rows)
+static size_t mx4_matrix_from(size_t R, size_t C) {
+    const size_t n = R * C;
+    return n >= (1u << 25) ? 2 : n >= (1u << 23) ? 3 : n >= (1u << 22) ? 4 : 5;
+}
+static size_t fp8_matrix_from(size_t R, size_t C) { return R * C >= (1u << 25) ? 3 : 5; }
 
 static bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 static bool aligned2(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 1u) == 0; }
@@ -632,7 +644,8 @@ int32_t btb_hip_gemv_fp8(const void* w, const void* scales, size_t sr, size_t sc
     if (rc != OK) return rc;
     if (R % sr != 0 || C % sc != 0 || (C / sc) % FmtF8::UW != 0) return ERR_DOMAIN;
     if (!aligned16(w) || !aligned16(x) || (reinterpret_cast<uintptr_t>(scales) & 3u) || !aligned2(y)) return ERR_DOMAIN;
-    if (wide_pass(M, R, C, true) && mfma_dl_fits_fp8((int)R, (int)C, 16, (int)(R / sr), (int)(C / sc))) {
+    const size_t from = fp8_matrix_from(R, C);
+    if (wide_pass(M, R, C, true, from) && mfma_dl_fits_fp8((int)R, (int)C, 16, (int)(R / sr), (int)(C / sc))) {
         const uint16_t* xp = static_cast<const uint16_t*>(x);  // the long rows: weights straight into LDS, 16 rows a pass
         uint16_t* yp = static_cast<uint16_t*>(y);
         for (size_t m0 = 0; m0 < M; m0 += 16) {
@@ -643,7 +656,7 @@ int32_t btb_hip_gemv_fp8(const void* w, const void* scales, size_t sr, size_t sc
         }
         return OK;
     }
-    if (wide_pass(M, R, C, true)) {  // the verify widths: the matrix cores, 32 rows of x a pass
+    if (wide_pass(M, R, C, true, from)) {  // the verify widths: the matrix cores, 32 rows of x a pass
         const uint16_t* xp = static_cast<const uint16_t*>(x);
         uint16_t* yp = static_cast<uint16_t*>(y);
         for (size_t m0 = 0; m0 < M; m0 += 32) {
@@ -666,7 +679,9 @@ int32_t btb_hip_gemv_mxfp4(const void* blocks, const void* scales, const void* x
     int32_t rc = check_dims(R, C, M, FmtMx4::UW);
     if (rc != OK) return rc;
     if (!aligned16(blocks) || !aligned16(x) || !aligned2(y)) return ERR_DOMAIN;
-    if (wide_pass(M, R, C, true) && mfma_dl_fits((int)R, (int)C, 16) && (reinterpret_cast<uintptr_t>(scales) & 3u) == 0) {
+    const size_t from = mx4_matrix_from(R, C);
+    if (wide_pass(M, R, C, true, from) && mfma_dl_fits((int)R, (int)C, 16) &&
+        (reinterpret_cast<uintptr_t>(scales) & 3u) == 0) {
         const uint16_t* xp = static_cast<const uint16_t*>(x);  // the long rows: weights straight into LDS, 16 rows a pass
         uint16_t* yp = static_cast<uint16_t*>(y);
         for (size_t m0 = 0; m0 < M; m0 += 16) {
@@ -677,7 +692,7 @@ int32_t btb_hip_gemv_mxfp4(const void* blocks, const void* scales, const void* x
         }
         return OK;
     }
-    if (wide_pass(M, R, C, true)) {
+    if (wide_pass(M, R, C, true, from)) {
         const uint16_t* xp = static_cast<const uint16_t*>(x);
         uint16_t* yp = static_cast<uint16_t*>(y);
         for (size_t m0 = 0; m0 < M; m0 += 32) {

@@ -49,7 +49,9 @@ int32_t btb_hip_sms(void);
 const char* btb_hip_last_error(void);
 
 /* Overrides a launch-tuning knob (e.g. "gemv_wgs_per_cu"); value < 0 restores the default. Unknown keys are
- * BTB_ERR_DOMAIN. For measurement only: no knob changes any result bit. No counterpart in the reference. */
+ * BTB_ERR_DOMAIN. For measurement only: no knob changes a result bit within a kernel family ("gemv_no_mfma" and
+ * "gemv_mfma_from" choose between the vector and the matrix-core family, whose sums round in another order).
+ * No counterpart in the reference. */
 int32_t btb_hip_set_tuning(const char* key, int32_t value);
 
 /* A measurement aid: the streaming matvec's loads without the matvec. Reads a [rows, 2560] bf16-shaped matrix (rows

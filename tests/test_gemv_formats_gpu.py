@@ -150,6 +150,20 @@ def _width_law(card, op, w, x, ref):
     check(v, ref)
     peak = float(y.float().abs().max())
     assert float((v.float() - y.float()).abs().max()) <= peak * 2.0**-7
+    # two to four rows: large block-scaled matrices go to the matrix cores from two or three rows on, the others stay
+    # on the vector kernels; whichever family takes the pass, its rows are that family's rows, bit for bit
+    for m in (2, 3, 4):
+        ym = op(w, x[:m].contiguous())
+        check(ym, ref[:m])
+        matrix = torch.equal(ym.view(torch.int16), y[:m].view(torch.int16))
+        vector = torch.equal(ym.view(torch.int16), v[:m].view(torch.int16))
+        assert matrix or vector, m
+    card.set_tuning("gemv_mfma_from", 5)  # every form's threshold back at five rows: the vector family to four
+    try:
+        y4 = op(w, x[:4].contiguous())
+    finally:
+        card.set_tuning("gemv_mfma_from", -1)
+    assert torch.equal(y4.view(torch.int16), v[:4].view(torch.int16))
 
 
 @pytest.mark.parametrize("R,C,block", [(18432, 7168, (128, 128)), (2048, 7168, (128, 128)), (512, 1024, (128, 128)),
@@ -342,7 +356,13 @@ def test_full_shape_one_row_and_linearity(card, form):
     y1 = op(w, x[:1].contiguous().cuda())
     check(y1, ref[:1])
     both = op(w, x.cuda())
-    assert torch.equal(both[:1].view(torch.int16), y1.view(torch.int16))      # row 0 of the 2-row pass: the same bits
+    check(both, ref)
+    if form == "fp8":  # two rows of FP8 stay on the vector kernel: row 0 of the 2-row pass has the one-row pass's bits
+        assert torch.equal(both[:1].view(torch.int16), y1.view(torch.int16))
+    else:  # two rows of MXFP4 on a matrix this large go to the matrix cores: the rows of an 8-row pass, bit for bit
+        y8 = op(w, torch.cat([x, acts_bf16(6, C, seed=352)]).cuda())
+        assert torch.equal(both.view(torch.int16), y8[:2].view(torch.int16))
+        assert not torch.equal(both[:1].view(torch.int16), y1.view(torch.int16))  # (and so not the vector kernel's)
     total = both.float().sum(dim=0).cpu().numpy()
     want = ref.sum(axis=0)
     assert np.abs(total - want).max() <= 1e-2 * np.abs(want).max()
