@@ -61,6 +61,7 @@ struct Knob {
 static Knob g_knobs[] = {
     {"gemv_wgs_per_cu", {-1}},
     {"gemv_even_grid", {-1}},
+    {"gemv_halves", {-1}},
     {"gemv_mfma_from", {-1}},
     {"gemv_five_waves", {-1}},
     {"gemv_no_mfma", {-1}},

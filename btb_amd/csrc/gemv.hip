@@ -144,6 +144,111 @@ __global__ void __launch_bounds__(NT) gemv_stream(typename F::Params p, XArgs xa
         gemv_tile<F, M, LPR, RPW, U, EPI, false>(p, first, first_ctx, tile, xs4, y, R, C, lane);
 }
 
+// A bf16 row too long for one span of a wave (more than ten 16-byte units a lane), by two waves: each takes a half of
+// the row's units in one span, the second half's sum reaches the first half's wave through LDS. Twice the waves,
+// each with one trip to memory where the whole row's wave made two - and 2560 such rows, 2.5 a SIMD, lie on the SIMDs
+// as five halves each where whole rows lay three on some and two on others (a launch ends with its fullest SIMD):
+// down [2560 x 9728] 10.15 -> 9.4 us, the step 1.993 -> 1.973 ms; the pass of 3 / 4 rows 2.575 / 2.780 -> 2.403 /
+// 2.667 ms. A workgroup's waves come in pairs, a row a pair and turn. The
+// split comes from the row length alone and is the same at every M up to four and in every x mode: a row's bits
+// depend on neither.
+template <int M, int U, int XMODE, int NT>
+__global__ void __launch_bounds__(NT) gemv_halves(FmtBf16::Params p, XArgs xa, uint16_t* __restrict__ y, int R, int C) {
+    using F = FmtBf16;
+    extern __shared__ __align__(16) uint32_t xs[];
+    constexpr int RW = NT / (2 * WAVE);  // rows a workgroup's turn
+    __shared__ float part[2][RW][M];  // [turn's parity][row of the workgroup][row of x]
+    const int units = C / F::UW;
+    const int lane = threadIdx.x & (WAVE - 1), wib = threadIdx.x / WAVE;
+    const int mine = wib >> 1, half = wib & 1;
+    const int ua = (units + 1) / 2;  // the first half's units
+    const int u0 = half ? ua : 0, un = half ? units - ua : ua;
+    constexpr int span = U * WAVE;
+    const int xrow4 = C / 8;
+    auto ctx_of = [&](int row) { return F::RowCtx{p.w + (size_t)min(row, R - 1) * units + u0}; };
+
+    F::Raw first[U][1] = {};
+    F::RowCtx ctx[1] = {ctx_of(blockIdx.x * RW + mine)};
+    stage_x<XMODE, M, false, NT>(xs, xa, M, C, [&] { load_span_always<F, WAVE, 1, U>(first, ctx, 0, lane, un); });
+    const uint4* xs4 = reinterpret_cast<const uint4*>(xs) + u0;
+
+    // a half is one span (U * 64 units hold it: launch_halves): the first turn's was requested above, a later turn
+    // requests its own
+    auto products = [&](const F::Raw (&raw)[U][1], float (&acc)[1][M]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int unit = u * WAVE + lane;
+            if (unit < un) fma_unit<F, M, 1>(ctx, raw[u], unit, xs4, xrow4, acc);
+        }
+    };
+    auto finish = [&](const float (&acc)[1][M], int row, int parity) {
+        float s[M];
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+            s[m] = group_sum_last<WAVE>(acc[0][m]);
+            if (half == 1 && lane == WAVE - 1) part[parity][mine][m] = s[m];
+        }
+        __syncthreads();  // one a turn: the next turn writes the other parity's slots
+        if (half == 0 && lane == WAVE - 1 && row < R) {
+#pragma unroll
+            for (int m = 0; m < M; ++m) y[(size_t)m * R + row] = f32_bf16(s[m] + part[parity][mine][m]);
+        }
+    };
+    {
+        float acc[1][M];
+#pragma unroll
+        for (int m = 0; m < M; ++m) acc[0][m] = 0.f;
+        products(first, acc);
+        finish(acc, blockIdx.x * RW + mine, 0);
+    }
+    int parity = 1;
+    for (int base = (blockIdx.x + gridDim.x) * RW; base < R; base += gridDim.x * RW, parity ^= 1) {  // every wave alike
+        ctx[0] = ctx_of(base + mine);
+        F::Raw raw[U][1];
+        load_span<F, WAVE, 1, U, true>(raw, ctx, 0, lane, un);
+        float acc[1][M];
+#pragma unroll
+        for (int m = 0; m < M; ++m) acc[0][m] = 0.f;
+        products(raw, acc);
+        finish(acc, base + mine, parity);
+    }
+}
+
+// the row lengths gemv_halves takes: 11 to 20 units a lane of a whole-row wave
+static bool halves_fit(int C) {
+    const int per_lane = (C / FmtBf16::UW + WAVE - 1) / WAVE;
+    return per_lane > 10 && per_lane <= 20 && tuning("gemv_halves") != 0;
+}
+
+template <int M, int XMODE>
+static int32_t launch_halves(const FmtBf16::Params& p, const XArgs& xa, void* y, int R, int C, hipStream_t st) {
+    const DeviceInfo& dev = device_info();
+    const size_t lds = stage_lds_bytes(XMODE, M, C);
+    if (lds > (size_t)dev.lds_bytes) {
+        set_error("gemv: the x rows do not fit LDS");
+        return ERR_DOMAIN;
+    }
+    const int half_lane = ((C / FmtBf16::UW + 1) / 2 + WAVE - 1) / WAVE;  // 6 to 10
+    // eight waves a workgroup (four rows a turn) from two rows of x on, where the plain copy of x is what a workgroup
+    // pays for first: as many workgroups as the whole-row kernel has
+    // Ten waves a workgroup (five rows a turn) where x is copied as it is: 2560 rows are then two workgroups a CU, and
+    // x is staged twice a CU, not five times (the pass of 2 / 3 / 4 rows with workgroups of four waves 2.28 / 2.63 /
+    // 2.89 ms, of eight 2.20 / 2.46 / 2.66, of ten 2.17 / 2.40 / 2.67; one row level). The other x modes are written
+    // for workgroups of 256 threads. Either way twenty waves a CU and turn.
+    constexpr int NT = XMODE == X_PLAIN ? 640 : 256;
+    constexpr int RW = NT / (2 * WAVE);
+    auto kern = half_lane <= 8 ? gemv_halves<M, 8, XMODE, NT> : gemv_halves<M, 10, XMODE, NT>;
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
+    }
+    int grid = (R + RW - 1) / RW;
+    if (grid > dev.cus * 10 / RW) grid = dev.cus * 10 / RW;
+    hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds, st, p, xa, static_cast<uint16_t*>(y), R, C);
+    return hip_status(hipGetLastError(), "gemv_halves launch");
+}
+
 // ------------------------------------------------------------------------------------------------------------
 // launch
 // ------------------------------------------------------------------------------------------------------------
@@ -277,6 +382,9 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
             return launch_variant<F, M, LPR, 1, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
         }
     } else {
+        if constexpr (LPR == 64 && std::is_same<F, FmtBf16>::value) {
+            if (halves_fit(C)) return launch_halves<M, XMODE>(p, xa, y, R, C, st);
+        }
         const bool tall = R >= 4096 * (WAVE / LPR);
         if constexpr (M <= 2) {
             if (tall && fewer(5, 4)) return launch_variant<F, M, LPR, 2, 5, XMODE, E_PLAIN>(p, xa, y, R, C, st);

@@ -62,6 +62,48 @@ def test_row_of_a_wide_pass_is_its_one_row_pass(card, M):
         assert torch.equal(solo[0].view(torch.int16), y[m].view(torch.int16))
 
 
+@pytest.mark.parametrize("R,C", [(2560, 9728), (2561, 5128), (7, 10240), (1, 6152), (5000, 8192), (3000, 9736)])
+def test_long_rows_by_two_waves(card, R, C):
+    """rows of 5121 .. 10240 values are summed by two waves, a half each (`gemv_halves`): against the oracle at one to
+    four rows of x; row m of a pass is its one-row pass bit for bit; the add + norm in the x load gives the bits of
+    add_rmsnorm followed by the plain matvec; with the split switched off (knob gemv_halves = 0: the whole-row kernel,
+    another order of summation) the outputs stay within one bf16 ulp of the largest. Shapes: the down projection, odd
+    row counts, the shortest and the longest row the split takes, rows of an odd number of units, and a matrix tall
+    enough that workgroups take several turns."""
+    w = weights_bf16(R, C, seed=120)
+    x = acts_bf16(4, C, seed=121)
+    ref = oracle_bf16_out(w, x)
+    wd, xd = w.cuda(), x.cuda()
+    y4 = card.gemv(wd, xd)
+    check(y4, ref)
+    for M in (1, 2, 3):
+        ym = card.gemv(wd, xd[:M].contiguous())
+        assert torch.equal(ym.view(torch.int16), y4[:M].view(torch.int16)), M
+    solo = card.gemv(wd, xd[3:4].contiguous())
+    assert torch.equal(solo[0].view(torch.int16), y4[3].view(torch.int16))
+    # the add + norm form (workgroups of four waves) against the two launches (ten waves): the same bits
+    for M in (1, 3):
+        h = acts_bf16(M, C, seed=122).cuda()
+        d = acts_bf16(M, C, seed=123).cuda()
+        nw = (1.0 + 0.1 * torch.randn(C, generator=torch.Generator().manual_seed(124))).to(torch.bfloat16).cuda()
+        h1, x1 = h.clone(), torch.empty_like(h)
+        card.add_rmsnorm(h1, d, nw, 1e-6, x1)
+        want = card.gemv(wd, x1)
+        h2 = torch.empty_like(h)
+        out = torch.empty(M, R, dtype=torch.bfloat16, device="cuda")
+        card.gemv_norm(wd, h, d, nw, 1e-6, h2, out, glu=False)
+        assert torch.equal(out.view(torch.int16), want.view(torch.int16))
+        assert torch.equal(h2.view(torch.int16), h1.view(torch.int16))
+    card.set_tuning("gemv_halves", 0)
+    try:
+        whole = card.gemv(wd, xd)
+    finally:
+        card.set_tuning("gemv_halves", -1)
+    check(whole, ref)
+    peak = float(np.abs(ref).max())
+    assert float((whole.float() - y4.float()).abs().max()) <= peak * 2.0**-7
+
+
 @pytest.mark.parametrize("R,C", [(9728, 2560), (2560, 9728), (2560, 4096), (1000, 96), (18, 32)])
 @pytest.mark.parametrize("M", [8, 16, 32, 12, 40])
 def test_verify_widths_on_the_matrix_cores(card, R, C, M):
