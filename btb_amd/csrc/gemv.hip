@@ -144,54 +144,79 @@ __global__ void __launch_bounds__(NT) gemv_stream(typename F::Params p, XArgs xa
         gemv_tile<F, M, LPR, RPW, U, EPI, false>(p, first, first_ctx, tile, xs4, y, R, C, lane);
 }
 
-// A bf16 row too long for one span of a wave (more than ten 16-byte units a lane), by two waves: each takes a half of
-// the row's units in one span, the second half's sum reaches the first half's wave through LDS. Twice the waves,
-// each with one trip to memory where the whole row's wave made two - and 2560 such rows, 2.5 a SIMD, lie on the SIMDs
-// as five halves each where whole rows lay three on some and two on others (a launch ends with its fullest SIMD):
-// down [2560 x 9728] 10.15 -> 9.4 us, the step 1.993 -> 1.973 ms; the pass of 3 / 4 rows 2.575 / 2.780 -> 2.403 /
-// 2.667 ms. A workgroup's waves come in pairs, a row a pair and turn. The
-// split comes from the row length alone and is the same at every M up to four and in every x mode: a row's bits
-// depend on neither.
-template <int M, int U, int XMODE, int NT>
-__global__ void __launch_bounds__(NT) gemv_halves(FmtBf16::Params p, XArgs xa, uint16_t* __restrict__ y, int R, int C) {
-    using F = FmtBf16;
+// A bf16 row too long for one span of a wave (5121 .. 10240 values: more than ten 16-byte units a lane), by two waves:
+// each takes a half of the row's units in one span, the second half's sum reaches the first half's wave through LDS.
+// Twice the waves, each with one trip to memory where the whole row's wave made two - and 2560 such rows, 2.5 a SIMD,
+// lie on the SIMDs as five halves each where whole rows lay three on some and two on others (a launch ends with its
+// fullest SIMD): down [2560 x 9728] 10.15 -> 9.4 us, the step 1.993 -> 1.973 ms; the pass of 3 / 4 rows 2.575 / 2.780
+// -> 2.403 / 2.667 ms. A workgroup's waves come in pairs, a row a pair and turn. The split comes from the row length
+// alone and is the same at every M up to four, in every x mode and under the gate / up fold: a row's bits depend on
+// none of them. Written over the format policy (what a form does past the stream is the first half's wave's), taken
+// by bf16 only: pack12 rows of that length gain 0.4 % of the packed step at one row of x and 3 - 4 % of the pass at
+// three and four, and lose 3.3 % at two (2.158 -> 2.230 ms), and every width has to take the same split.
+// E_GLU: a pair of waves on gate row r, the next pair on up row I + r; the four sums meet in LDS and the up pair's
+// first wave writes bf16(bf16(silu(g)) * u), g and u added up as the plain form adds them - the bits of the plain
+// matvec followed by silu_mul.
+template <class F, int M, int U, int XMODE, int EPI, int NT>
+__global__ void __launch_bounds__(NT) gemv_halves(typename F::Params p, XArgs xa, uint16_t* __restrict__ y, int R, int C) {
+    static_assert(EPI == E_PLAIN || EPI == E_GLU, "plain rows, or gate and up rows folded");
+    static_assert(EPI == E_PLAIN || NT % (4 * WAVE) == 0, "the folded form: four waves an output");
     extern __shared__ __align__(16) uint32_t xs[];
-    constexpr int RW = NT / (2 * WAVE);  // rows a workgroup's turn
-    __shared__ float part[2][RW][M];  // [turn's parity][row of the workgroup][row of x]
+    constexpr int NW = NT / WAVE;
+    constexpr int OW = EPI == E_GLU ? NW / 4 : NW / 2;  // outputs a workgroup's turn
+    __shared__ float part[2][NW][M];                    // [turn's parity][wave][row of x]: the waves' sums
+    const int Rout = EPI == E_GLU ? R / 2 : R;
     const int units = C / F::UW;
     const int lane = threadIdx.x & (WAVE - 1), wib = threadIdx.x / WAVE;
-    const int mine = wib >> 1, half = wib & 1;
+    const int half = wib & 1;
+    const int mine = EPI == E_GLU ? wib >> 2 : wib >> 1;  // the wave's output of the turn
+    const bool up = EPI == E_GLU && (wib & 2) != 0;
     const int ua = (units + 1) / 2;  // the first half's units
-    const int u0 = half ? ua : 0, un = half ? units - ua : ua;
-    constexpr int span = U * WAVE;
+    const int u0 = half ? ua : 0, u1 = half ? units : ua;
     const int xrow4 = C / 8;
-    auto ctx_of = [&](int row) { return F::RowCtx{p.w + (size_t)min(row, R - 1) * units + u0}; };
+    auto row_of = [&](int out) { return min(out, Rout - 1) + (up ? Rout : 0); };  // the weight row
+    F::prepare(p);
 
-    F::Raw first[U][1] = {};
-    F::RowCtx ctx[1] = {ctx_of(blockIdx.x * RW + mine)};
-    stage_x<XMODE, M, false, NT>(xs, xa, M, C, [&] { load_span_always<F, WAVE, 1, U>(first, ctx, 0, lane, un); });
-    const uint4* xs4 = reinterpret_cast<const uint4*>(xs) + u0;
+    typename F::Raw first[U][1] = {};
+    typename F::RowCtx ctx[1];
+    stage_x<XMODE, M, sizeof(typename F::Raw) != 16, NT>(xs, xa, M, C, [&] {
+        ctx[0] = F::row_ctx(p, (size_t)row_of((int)blockIdx.x * OW + mine), units, lane);
+        load_span_always<F, WAVE, 1, U>(first, ctx, u0, lane, u1);
+        F::prepare_finish(p);
+    });
+    const uint4* xs4 = reinterpret_cast<const uint4*>(xs);
 
     // a half is one span (U * 64 units hold it: launch_halves): the first turn's was requested above, a later turn
-    // requests its own
-    auto products = [&](const F::Raw (&raw)[U][1], float (&acc)[1][M]) {
+    // requests its own. The x values are read a unit at a time: asked for a span ahead, as the whole-row kernel does
+    // at one row, they cost the registers that decide how many waves a SIMD holds.
+    auto products = [&](const typename F::Raw (&raw)[U][1], float (&acc)[1][M]) {
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int unit = u * WAVE + lane;
-            if (unit < un) fma_unit<F, M, 1>(ctx, raw[u], unit, xs4, xrow4, acc);
+            const int unit = u0 + u * WAVE + lane;
+            if (unit < u1) fma_unit<F, M, 1>(ctx, raw[u], unit, xs4, xrow4, acc);
         }
     };
-    auto finish = [&](const float (&acc)[1][M], int row, int parity) {
+    auto finish = [&](float (&acc)[1][M], int out, int parity) {
+        if (half == 0) F::template tail<M>(p, ctx[0], (size_t)row_of(out), lane, WAVE, C, xs, acc[0]);
         float s[M];
 #pragma unroll
         for (int m = 0; m < M; ++m) {
             s[m] = group_sum_last<WAVE>(acc[0][m]);
-            if (half == 1 && lane == WAVE - 1) part[parity][mine][m] = s[m];
+            if ((EPI == E_GLU || half == 1) && lane == WAVE - 1) part[parity][wib][m] = s[m];
         }
         __syncthreads();  // one a turn: the next turn writes the other parity's slots
-        if (half == 0 && lane == WAVE - 1 && row < R) {
+        if (half == 0 && lane == WAVE - 1 && out < Rout && (EPI == E_PLAIN || up)) {
 #pragma unroll
-            for (int m = 0; m < M; ++m) y[(size_t)m * R + row] = f32_bf16(s[m] + part[parity][mine][m]);
+            for (int m = 0; m < M; ++m) {
+                const float mine_sum = s[m] + part[parity][wib + 1][m];
+                if constexpr (EPI == E_GLU) {
+                    const float g = bfround(part[parity][wib - 2][m] + part[parity][wib - 1][m]), u = bfround(mine_sum);
+                    const float sg = bfround(g / (1.f + expf(-g)));
+                    y[(size_t)m * Rout + out] = f32_bf16(sg * u);
+                } else {
+                    y[(size_t)m * Rout + out] = f32_bf16(mine_sum);
+                }
+            }
         }
     };
     {
@@ -199,13 +224,13 @@ __global__ void __launch_bounds__(NT) gemv_halves(FmtBf16::Params p, XArgs xa, u
 #pragma unroll
         for (int m = 0; m < M; ++m) acc[0][m] = 0.f;
         products(first, acc);
-        finish(acc, blockIdx.x * RW + mine, 0);
+        finish(acc, blockIdx.x * OW + mine, 0);
     }
     int parity = 1;
-    for (int base = (blockIdx.x + gridDim.x) * RW; base < R; base += gridDim.x * RW, parity ^= 1) {  // every wave alike
-        ctx[0] = ctx_of(base + mine);
-        F::Raw raw[U][1];
-        load_span<F, WAVE, 1, U, true>(raw, ctx, 0, lane, un);
+    for (int base = (blockIdx.x + gridDim.x) * OW; base < Rout; base += gridDim.x * OW, parity ^= 1) {  // every wave alike
+        ctx[0] = F::row_ctx(p, (size_t)row_of(base + mine), units, lane);
+        typename F::Raw raw[U][1];
+        load_span<F, WAVE, 1, U, true>(raw, ctx, u0, lane, u1);
         float acc[1][M];
 #pragma unroll
         for (int m = 0; m < M; ++m) acc[0][m] = 0.f;
@@ -214,37 +239,37 @@ __global__ void __launch_bounds__(NT) gemv_halves(FmtBf16::Params p, XArgs xa, u
     }
 }
 
-// the row lengths gemv_halves takes: 11 to 20 units a lane of a whole-row wave
-static bool halves_fit(int C) {
-    const int per_lane = (C / FmtBf16::UW + WAVE - 1) / WAVE;
-    return per_lane > 10 && per_lane <= 20 && tuning("gemv_halves") != 0;
-}
+// the row lengths gemv_halves takes
+static bool halves_fit(int C) { return C > 5120 && C <= 10240 && tuning("gemv_halves") != 0; }
 
-template <int M, int XMODE>
-static int32_t launch_halves(const FmtBf16::Params& p, const XArgs& xa, void* y, int R, int C, hipStream_t st) {
+template <class F, int M, int XMODE, int EPI>
+static int32_t launch_halves(const typename F::Params& p, const XArgs& xa, void* y, int R, int C, hipStream_t st) {
     const DeviceInfo& dev = device_info();
     const size_t lds = stage_lds_bytes(XMODE, M, C);
     if (lds > (size_t)dev.lds_bytes) {
         set_error("gemv: the x rows do not fit LDS");
         return ERR_DOMAIN;
     }
-    const int half_lane = ((C / FmtBf16::UW + 1) / 2 + WAVE - 1) / WAVE;  // 6 to 10
-    // eight waves a workgroup (four rows a turn) from two rows of x on, where the plain copy of x is what a workgroup
-    // pays for first: as many workgroups as the whole-row kernel has
+    // a half's units a lane: 6 to 10 of bf16 (spans of 8 or 10); the 16-weight forms' 3 to 5 would be a span of 5
+    constexpr bool BF = std::is_same<F, FmtBf16>::value;
+    const int half_lane = ((C / F::UW + 1) / 2 + WAVE - 1) / WAVE;
     // Ten waves a workgroup (five rows a turn) where x is copied as it is: 2560 rows are then two workgroups a CU, and
-    // x is staged twice a CU, not five times (the pass of 2 / 3 / 4 rows with workgroups of four waves 2.28 / 2.63 /
-    // 2.89 ms, of eight 2.20 / 2.46 / 2.66, of ten 2.17 / 2.40 / 2.67; one row level). The other x modes are written
-    // for workgroups of 256 threads. Either way twenty waves a CU and turn.
-    constexpr int NT = XMODE == X_PLAIN ? 640 : 256;
-    constexpr int RW = NT / (2 * WAVE);
-    auto kern = half_lane <= 8 ? gemv_halves<M, 8, XMODE, NT> : gemv_halves<M, 10, XMODE, NT>;
+    // x is staged twice a CU, not five times (the bf16 pass of 2 / 3 / 4 rows with workgroups of four waves 2.28 /
+    // 2.63 / 2.89 ms, of eight 2.20 / 2.46 / 2.66, of ten 2.17 / 2.40 / 2.67; one row level); eight for the folded
+    // form, four waves an output. The other x modes are written for workgroups of 256 threads.
+    constexpr int NT = XMODE != X_PLAIN ? 256 : EPI == E_GLU ? 512 : 640;
+    constexpr int OW = EPI == E_GLU ? NT / (4 * WAVE) : NT / (2 * WAVE);
+    const int Rout = EPI == E_GLU ? R / 2 : R;
+    auto kern = !BF ? gemv_halves<F, M, 5, XMODE, EPI, NT>
+                    : half_lane <= 8 ? gemv_halves<F, M, 8, XMODE, EPI, NT> : gemv_halves<F, M, (BF ? 10 : 5), XMODE, EPI, NT>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (e != hipSuccess) return hip_status(e, "hipFuncSetAttribute");
     }
-    int grid = (R + RW - 1) / RW;
-    if (grid > dev.cus * 10 / RW) grid = dev.cus * 10 / RW;
+    int grid = (Rout + OW - 1) / OW;
+    const int cap = dev.cus * 20 * WAVE / NT;  // twenty waves a CU and turn
+    if (grid > cap) grid = cap;
     hipLaunchKernelGGL(kern, dim3(grid), dim3(NT), lds, st, p, xa, static_cast<uint16_t*>(y), R, C);
     return hip_status(hipGetLastError(), "gemv_halves launch");
 }
@@ -342,6 +367,10 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
     const int per_lane = (C / F::UW + LPR - 1) / LPR;
     auto fewer = [per_lane](int u_new, int u_base) { return (per_lane + u_new - 1) / u_new < (per_lane + u_base - 1) / u_base; };
     if constexpr (EPI == E_GLU) {
+        // long bf16 rows (LPR is 64 there): the folded form of the split the plain form makes
+        if constexpr (LPR == 64 && !WIDENS) {
+            if (halves_fit(C)) return launch_halves<F, M, XMODE, E_GLU>(p, xa, y, R, C, st);
+        }
         if constexpr (WIDENS && LPR <= 32) {
             // a widening form whose rows take at most 32 lanes: gate and up side by side, one row a lane
             if constexpr (M <= 4 && std::is_base_of<FmtP12, F>::value) {
@@ -382,8 +411,8 @@ static int32_t launch_stream(const typename F::Params& p, const XArgs& xa, void*
             return launch_variant<F, M, LPR, 1, 4, XMODE, E_PLAIN>(p, xa, y, R, C, st);
         }
     } else {
-        if constexpr (LPR == 64 && std::is_same<F, FmtBf16>::value) {
-            if (halves_fit(C)) return launch_halves<M, XMODE>(p, xa, y, R, C, st);
+        if constexpr (LPR == 64) {
+            if (halves_fit(C)) return launch_halves<F, M, XMODE, E_PLAIN>(p, xa, y, R, C, st);
         }
         const bool tall = R >= 4096 * (WAVE / LPR);
         if constexpr (M <= 2) {

@@ -66,7 +66,8 @@ def test_row_of_a_wide_pass_is_its_one_row_pass(card, M):
 def test_long_rows_by_two_waves(card, R, C):
     """rows of 5121 .. 10240 values are summed by two waves, a half each (`gemv_halves`): against the oracle at one to
     four rows of x; row m of a pass is its one-row pass bit for bit; the add + norm in the x load gives the bits of
-    add_rmsnorm followed by the plain matvec; with the split switched off (knob gemv_halves = 0: the whole-row kernel,
+    add_rmsnorm followed by the plain matvec, the gate / up fold those of the plain matvec followed by silu_mul; with
+    the split switched off (knob gemv_halves = 0: the whole-row kernel,
     another order of summation) the outputs stay within one bf16 ulp of the largest. Shapes: the down projection, odd
     row counts, the shortest and the longest row the split takes, rows of an odd number of units, and a matrix tall
     enough that workgroups take several turns."""
@@ -94,6 +95,14 @@ def test_long_rows_by_two_waves(card, R, C):
         card.gemv_norm(wd, h, d, nw, 1e-6, h2, out, glu=False)
         assert torch.equal(out.view(torch.int16), want.view(torch.int16))
         assert torch.equal(h2.view(torch.int16), h1.view(torch.int16))
+    # the gate / up fold over such rows (four waves an output): the plain matvec, then silu_mul, bit for bit
+    if R % 2 == 0:
+        for M in (1, 3):
+            xm = xd[:M].contiguous()
+            want = torch.empty(M, R // 2, dtype=torch.bfloat16, device="cuda")
+            card.silu_mul(card.gemv(wd, xm), want)
+            got = card.gemv_glu_silu(wd, xm)
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16)), M
     card.set_tuning("gemv_halves", 0)
     try:
         whole = card.gemv(wd, xd)
