@@ -113,6 +113,24 @@ def test_long_rows_by_two_waves(card, R, C):
     assert float((whole.float() - y4.float()).abs().max()) <= peak * 2.0**-7
 
 
+def test_long_rows_by_two_waves_over_drawn_shapes(card):
+    """twenty drawn shapes in and around the split's range of row lengths (any multiple of 8 from 5000 to 10400 values,
+    1 .. 3000 rows, 1 .. 4 rows of x): the oracle's bar, and every row of the pass the bits of its one-row pass"""
+    rng = np.random.default_rng(20261)
+    for i in range(20):
+        R = int(rng.integers(1, 3001))
+        C = 8 * int(rng.integers(625, 1301))
+        M = int(rng.integers(1, 5))
+        w = weights_bf16(R, C, seed=2000 + i)
+        x = acts_bf16(M, C, seed=3000 + i)
+        wd, xd = w.cuda(), x.cuda()
+        y = card.gemv(wd, xd)
+        check(y, oracle_bf16_out(w, x))
+        for m in range(M):
+            solo = card.gemv(wd, xd[m : m + 1].contiguous())
+            assert torch.equal(solo[0].view(torch.int16), y[m].view(torch.int16)), (R, C, M, m)
+
+
 @pytest.mark.parametrize("R,C", [(9728, 2560), (2560, 9728), (2560, 4096), (1000, 96), (18, 32)])
 @pytest.mark.parametrize("M", [8, 16, 32, 12, 40])
 def test_verify_widths_on_the_matrix_cores(card, R, C, M):
