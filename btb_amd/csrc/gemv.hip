@@ -260,8 +260,8 @@ static int32_t launch_halves(const typename F::Params& p, const XArgs& xa, void*
     constexpr int NT = XMODE != X_PLAIN ? 256 : EPI == E_GLU ? 512 : 640;
     constexpr int OW = EPI == E_GLU ? NT / (4 * WAVE) : NT / (2 * WAVE);
     const int Rout = EPI == E_GLU ? R / 2 : R;
-    auto kern = !BF ? gemv_halves<F, M, 5, XMODE, EPI, NT>
-                    : half_lane <= 8 ? gemv_halves<F, M, 8, XMODE, EPI, NT> : gemv_halves<F, M, (BF ? 10 : 5), XMODE, EPI, NT>;
+    constexpr int LONGEST = BF ? 10 : 5;
+    auto kern = BF && half_lane <= 8 ? gemv_halves<F, M, 8, XMODE, EPI, NT> : gemv_halves<F, M, LONGEST, XMODE, EPI, NT>;
     if (lds > 64 * 1024) {
         hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
