@@ -306,7 +306,14 @@ static int32_t launch_variant(const typename F::Params& p, const XArgs& xa, void
     // instead of two: bf16 gate/up 17.55 -> 17.0 us and the step 2.022 -> 2.004 ms, packed 16.3 -> 15.5 us and
     // 1.928 -> 1.914 ms; at three rows the pass loses by it (2.58 -> 2.67 ms), and so does the plain one-row packed
     // [9728 x 2560] (8.25 -> 9.15 us).
-    if (per_cu <= 0) per_cu = (EPI != E_PLAIN && M <= 2) ? 4 : std::is_same<F, FmtP12G>::value ? 5 : 6;
+    // One row of bf16 x with the add + norm in the x load, plain output (qkv, the head): two, which the even cut
+    // below turns into one workgroup a CU whose waves walk three tiles each for qkv's 3072 - the add + norm is then
+    // made once a CU, not three times side by side: qkv 7.36 -> 6.97 us, the step 1.967 -> 1.961 ms (the head level;
+    // from two rows of x on and for the packed form it loses: 2.16 -> 2.21 ms at two rows, packed qkv 6.63 -> 7.42 us).
+    constexpr bool BF16_NORM_ROW =
+        std::is_same<F, FmtBf16>::value && M == 1 && XMODE == X_ADDNORM && EPI == E_PLAIN;
+    if (per_cu <= 0)
+        per_cu = BF16_NORM_ROW ? 2 : (EPI != E_PLAIN && M <= 2) ? 4 : std::is_same<F, FmtP12G>::value ? 5 : 6;
     const int cap_waves = dev.cus * per_cu * 4;
     // ... and of the counts from there to two more, the one whose workgroups fill the CUs' turns most evenly (when it
     // gains a twentieth or more): a launch ends with its fullest CU, and the forms that widen are bound by what a CU
